@@ -1,0 +1,192 @@
+// Row-wise kernels of the step: embedding gather, RMSNorm (optionally on chosen
+// rows), the SiLU-gated product, rotary position encoding fused with the write
+// of keys and values into cache pages.
+//
+// Formulas follow the reference's scalar kernels (src/kernels.cpp:18-31,59-66,
+// 189-203 and the page addressing of src/paged_kv.cpp:88-111); statistics,
+// rotation and activation are evaluated in 32-bit whatever the storage type.
+#include "common.h"
+
+namespace llme {
+
+// ---------------------------------------------------------------------------------
+// out[t, :] = table[tokens[t], :]        (src/kernels.cpp:59-66; no scaling)
+template <typename TW>
+__global__ void embed_gather_kernel(const TW* __restrict__ table, const int* __restrict__ tokens,
+                                    float* __restrict__ out, int H) {
+    const int t = blockIdx.x;
+    const TW* row = table + static_cast<size_t>(tokens[t]) * H;
+    float* o = out + static_cast<size_t>(t) * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_float(row[i]);
+}
+
+// ---------------------------------------------------------------------------------
+// out[r, i] = w[i] * x[row(r), i] * rsqrt(mean_i x^2 + eps)   (src/kernels.cpp:18-24)
+// row(r) = rows ? rows[r] : r. The product is evaluated (w*x)*inv as the reference does.
+template <typename TW, typename TO>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ w,
+                               TO* __restrict__ out, const int* __restrict__ rows, int H, float eps) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int src = rows ? rows[r] : r;
+    const float* xr = x + static_cast<size_t>(src) * H;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < H; i += blockDim.x) {
+        const float v = xr[i];
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch, blockDim.x / kWave);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(H) + eps);
+    TO* o = out + static_cast<size_t>(r) * H;
+    for (int i = threadIdx.x; i < H; i += blockDim.x)
+        o[i] = from_float<TO>((to_float(w[i]) * xr[i]) * inv);
+}
+
+// ---------------------------------------------------------------------------------
+// out[t, j] = silu(gate[t, j]) * up[t, j]      (src/kernels.cpp:26-31, src/engine.cpp:215-216)
+// gu is [T, 2*FF]; gate and up alternate in groups of `group` columns:
+// gate j sits at (j / group) * 2 * group + j % group, up `group` columns later.
+// group == FF is the plain "all gates, then all ups" layout.
+template <typename TI, typename TO>
+__global__ void swiglu_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int FF, int group, size_t total) {
+    const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const size_t t = idx / FF;
+    const int j = static_cast<int>(idx % FF);
+    const size_t base = t * 2 * static_cast<size_t>(FF) + static_cast<size_t>(j / group) * 2 * group + (j % group);
+    const float g = to_float(gu[base]);
+    const float u = to_float(gu[base + group]);
+    out[idx] = from_float<TO>((g / (1.0f + expf(-g))) * u);
+}
+
+// ---------------------------------------------------------------------------------
+// Rotary encoding of q and k heads (pairs (i, i + rot/2), src/kernels.cpp:189-203),
+// q written to q_out, rotated k and plain v written into the token's cache page.
+//   qkv     [T, (n_q + 2 n_kv) * hd] 32-bit: q heads, then k heads, then v heads
+//   cos,sin [max_pos, rot/2] 32-bit (null: no rotation)
+//   k_cache [pages, n_kv, page, hd]      v_cache [pages, n_kv, hd, page]
+//   block_table [n_seq, max_blocks]; the token's page is block_table[seq][pos / page]
+template <typename TQ, typename TC>
+__global__ void rope_kv_write_kernel(const float* __restrict__ qkv, const float* __restrict__ cos_t,
+                                     const float* __restrict__ sin_t, const int* __restrict__ positions,
+                                     const int* __restrict__ seq_idx, const int* __restrict__ block_table,
+                                     int max_blocks, TQ* __restrict__ q_out, TC* __restrict__ k_cache,
+                                     TC* __restrict__ v_cache, int n_q, int n_kv, int hd, int rot,
+                                     int page, int write_cache) {
+    const int t = blockIdx.x;
+    const int pos = positions[t];
+    const int half = rot / 2;
+    const float* row = qkv + static_cast<size_t>(t) * (n_q + 2 * n_kv) * hd;
+    const float* cs = cos_t ? cos_t + static_cast<size_t>(pos) * half : nullptr;
+    const float* sn = sin_t ? sin_t + static_cast<size_t>(pos) * half : nullptr;
+
+    // q heads: pairs inside the rotated span, plain copy behind it
+    TQ* qo = q_out + static_cast<size_t>(t) * n_q * hd;
+    const int pairs_q = n_q * half;
+    for (int e = threadIdx.x; e < pairs_q; e += blockDim.x) {
+        const int h = e / half, i = e % half;
+        const float a = row[h * hd + i], b = row[h * hd + i + half];
+        const float c = cs ? cs[i] : 1.f, s = sn ? sn[i] : 0.f;
+        qo[h * hd + i] = from_float<TQ>(a * c - b * s);
+        qo[h * hd + i + half] = from_float<TQ>(b * c + a * s);
+    }
+    const int tail = hd - rot;
+    for (int e = threadIdx.x; e < n_q * tail; e += blockDim.x) {
+        const int h = e / tail, i = rot + e % tail;
+        qo[h * hd + i] = from_float<TQ>(row[h * hd + i]);
+    }
+    if (!write_cache) return;
+
+    const int s_idx = seq_idx[t];
+    const int pg = block_table[static_cast<size_t>(s_idx) * max_blocks + pos / page];
+    const int off = pos % page;
+    const float* krow = row + n_q * hd;
+    const float* vrow = krow + n_kv * hd;
+    for (int e = threadIdx.x; e < n_kv * half; e += blockDim.x) {
+        const int h = e / half, i = e % half;
+        const float a = krow[h * hd + i], b = krow[h * hd + i + half];
+        const float c = cs ? cs[i] : 1.f, s = sn ? sn[i] : 0.f;
+        TC* kd = k_cache + ((static_cast<size_t>(pg) * n_kv + h) * page + off) * hd;
+        kd[i] = from_float<TC>(a * c - b * s);
+        kd[i + half] = from_float<TC>(b * c + a * s);
+    }
+    for (int e = threadIdx.x; e < n_kv * tail; e += blockDim.x) {
+        const int h = e / tail, i = rot + e % tail;
+        k_cache[((static_cast<size_t>(pg) * n_kv + h) * page + off) * hd + i] = from_float<TC>(krow[h * hd + i]);
+    }
+    for (int e = threadIdx.x; e < n_kv * hd; e += blockDim.x) {
+        const int h = e / hd, d = e % hd;
+        v_cache[((static_cast<size_t>(pg) * n_kv + h) * hd + d) * page + off] = from_float<TC>(vrow[e]);
+    }
+}
+
+}  // namespace llme
+
+using namespace llme;
+
+extern "C" int llme_embed_gather(const void* table, int table_dtype, const int* tokens, float* out, int T,
+                                 int H, hipStream_t stream) {
+    if (T <= 0) return 0;
+    if (table_dtype == kF32)
+        hipLaunchKernelGGL(embed_gather_kernel<float>, dim3(T), dim3(256), 0, stream,
+                           static_cast<const float*>(table), tokens, out, H);
+    else if (table_dtype == kBF16)
+        hipLaunchKernelGGL(embed_gather_kernel<bf16>, dim3(T), dim3(256), 0, stream,
+                           static_cast<const bf16*>(table), tokens, out, H);
+    else
+        return kErrBadArgument;
+    return launch_status();
+}
+
+extern "C" int llme_rmsnorm(const float* x, const void* w, int w_dtype, void* out, int out_dtype,
+                            const int* rows, int R, int H, float eps, hipStream_t stream) {
+    if (R <= 0) return 0;
+#define LLME_NORM(TW, TO)                                                                        \
+    hipLaunchKernelGGL((rmsnorm_kernel<TW, TO>), dim3(R), dim3(256), 0, stream, x,               \
+                       static_cast<const TW*>(w), static_cast<TO*>(out), rows, H, eps)
+    if (w_dtype == kF32 && out_dtype == kF32) LLME_NORM(float, float);
+    else if (w_dtype == kF32 && out_dtype == kBF16) LLME_NORM(float, bf16);
+    else if (w_dtype == kBF16 && out_dtype == kF32) LLME_NORM(bf16, float);
+    else if (w_dtype == kBF16 && out_dtype == kBF16) LLME_NORM(bf16, bf16);
+    else return kErrBadArgument;
+#undef LLME_NORM
+    return launch_status();
+}
+
+extern "C" int llme_swiglu(const void* gu, int in_dtype, void* out, int out_dtype, int T, int FF, int group,
+                           hipStream_t stream) {
+    if (T <= 0) return 0;
+    if (group <= 0 || FF % group != 0) return kErrBadArgument;
+    const size_t total = static_cast<size_t>(T) * FF;
+    const dim3 grid(static_cast<unsigned>((total + 255) / 256));
+#define LLME_SWIGLU(TI, TO)                                                                      \
+    hipLaunchKernelGGL((swiglu_kernel<TI, TO>), grid, dim3(256), 0, stream,                      \
+                       static_cast<const TI*>(gu), static_cast<TO*>(out), FF, group, total)
+    if (in_dtype == kF32 && out_dtype == kF32) LLME_SWIGLU(float, float);
+    else if (in_dtype == kF32 && out_dtype == kBF16) LLME_SWIGLU(float, bf16);
+    else if (in_dtype == kBF16 && out_dtype == kBF16) LLME_SWIGLU(bf16, bf16);
+    else return kErrBadArgument;
+#undef LLME_SWIGLU
+    return launch_status();
+}
+
+extern "C" int llme_rope_kv_write(const float* qkv, const float* cos_t, const float* sin_t,
+                                  const int* positions, const int* seq_idx, const int* block_table,
+                                  int max_blocks, void* q_out, int q_dtype, void* k_cache, void* v_cache,
+                                  int cache_dtype, int T, int n_q, int n_kv, int hd, int rot, int page,
+                                  int write_cache, hipStream_t stream) {
+    if (T <= 0) return 0;
+    if (rot < 0 || rot > hd || rot % 2 != 0 || page <= 0) return kErrBadArgument;
+#define LLME_ROPE(TQ, TC)                                                                        \
+    hipLaunchKernelGGL((rope_kv_write_kernel<TQ, TC>), dim3(T), dim3(256), 0, stream, qkv, cos_t, \
+                       sin_t, positions, seq_idx, block_table, max_blocks, static_cast<TQ*>(q_out), \
+                       static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), n_q, n_kv, hd, rot,  \
+                       page, write_cache)
+    if (q_dtype == kF32 && cache_dtype == kF32) LLME_ROPE(float, float);
+    else if (q_dtype == kBF16 && cache_dtype == kBF16) LLME_ROPE(bf16, bf16);
+    else if (q_dtype == kF32 && cache_dtype == kBF16) LLME_ROPE(float, bf16);
+    else if (q_dtype == kBF16 && cache_dtype == kF32) LLME_ROPE(bf16, float);
+    else return kErrBadArgument;
+#undef LLME_ROPE
+    return launch_status();
+}

@@ -1,0 +1,6 @@
+from .step import CacheContext, CapacityError, ModelRunner, StepContext, StepEntry, Workspace
+from .scheduler import ContinuousBatchScheduler, SequenceResult
+from .engine import BlockManager, Engine, parse_dtype
+
+__all__ = ["CacheContext", "CapacityError", "ModelRunner", "StepContext", "StepEntry", "Workspace",
+           "ContinuousBatchScheduler", "SequenceResult", "BlockManager", "Engine", "parse_dtype"]

@@ -1,0 +1,275 @@
+"""The Python entry point: `Engine(model_dir, dtype).generate(ids, max_new_tokens)`.
+
+Names and meanings follow the reference's binding (src/bindings.cpp:150-266,
+276-335): `Engine(model_dir, dtype="fp32")`, `.generate(prompt_ids,
+max_new_tokens) -> (ids, "stop" | "length")`, `.forward_logits(ids) -> [T, V]`,
+properties `dtype`, `cfg`, `max_pos`, `weight_names()`, `has_weight(name)`, and
+`BlockManager(num_blocks, block_size, ...)` with `num_blocks`, `block_size`,
+`free_blocks`. dtype is "fp32" (everything in true 32-bit) or "bf16" (weights,
+activations and cache in bfloat16; accumulation, norms, softmax, rotation and the
+residual stream in 32-bit; logits 32-bit). All forward passes of an engine are
+serialized by one lock, as the reference's are (include/llmengine/engine.hpp:158).
+"""
+from __future__ import annotations
+
+import threading
+from typing import Sequence
+
+import numpy as np
+import torch
+
+from ..config.base import read_model_json
+from ..config.registry import architecture_name, parse_config, resolve
+from ..parts.base import Placement
+from ..sampling import Sampler
+from ..weights import TensorIndex, load_model_weights, load_state_dict, random_state
+from .step import CacheContext, CapacityError, ModelRunner, StepEntry
+
+_DTYPES = {"fp32": torch.float32, "float32": torch.float32, "bf16": torch.bfloat16,
+           "bfloat16": torch.bfloat16}
+
+
+def parse_dtype(name: str) -> torch.dtype:
+    try:
+        return _DTYPES[name]
+    except KeyError:
+        raise ValueError(f"dtype must be 'fp32' | 'bf16', got: {name}") from None
+
+
+def require_gpu(device: str | torch.device = "cuda:0") -> torch.device:
+    device = torch.device(device)
+    if device.type != "cuda" or not torch.cuda.is_available():
+        raise RuntimeError("this engine runs on an AMD GPU only: no HIP device is visible "
+                           f"(asked for {device}); there is no CPU path")
+    return device
+
+
+class BlockManager:
+    """The geometry of a page pool (the reference's constructor also takes the
+    layer and head sizes, which here come from the model; they are accepted and
+    checked when given)."""
+
+    def __init__(self, num_blocks: int, block_size: int, num_layers: int | None = None,
+                 num_kv_heads: int | None = None, head_dim: int | None = None):
+        for name, v in (("num_blocks", num_blocks), ("block_size", block_size)):
+            if v is None or int(v) <= 0:
+                raise ValueError("BlockManager: non-positive dim")
+        for v in (num_layers, num_kv_heads, head_dim):
+            if v is not None and int(v) <= 0:
+                raise ValueError("BlockManager: non-positive dim")
+        self._num_blocks, self._block_size = int(num_blocks), int(block_size)
+        self.dims = (num_layers, num_kv_heads, head_dim)
+        self._cache: CacheContext | None = None
+
+    num_blocks = property(lambda self: self._num_blocks)
+    block_size = property(lambda self: self._block_size)
+
+    @property
+    def free_blocks(self) -> int:
+        if self._cache is None:
+            return self._num_blocks
+        return min(self._cache.manager.free_pages(g) for g in self._cache.manager.groups)
+
+
+class Engine:
+    def __init__(self, model_dir: str | None, dtype: str = "fp32", *, device: str = "cuda:0",
+                 max_prefill_tokens_per_step: int = 8192, temperature: float = 0.0, seed: int = 0,
+                 block_size: int = 16, _config: dict | None = None, _tensors=None):
+        self._dtype_name = {"float32": "fp32", "bfloat16": "bf16"}.get(dtype, dtype)
+        self._torch_dtype = parse_dtype(dtype)
+        if _config is None:
+            cfg_dict, gen = read_model_json(model_dir)
+        else:
+            cfg_dict, gen = _config, None
+        self.model_dir = model_dir
+        self._cfg_dict = cfg_dict
+        self._arch = resolve(architecture_name(cfg_dict))
+        self.cfg = self._arch.parse_config(cfg_dict, gen, architecture=self._arch.name)
+        self._index_names: list[str] | None = None
+        if model_dir is not None and _tensors is None:
+            index = TensorIndex(model_dir)          # parse headers now: malformed files fail here
+            self._index_names = index.names()
+            index.close()
+        self._tensors = _tensors
+        self._device_name = device
+        self._runner: ModelRunner | None = None
+        self._lock = threading.RLock()
+        self.sampler = Sampler(temperature, seed)
+        self.block_size = int(block_size)
+        self.prefill_chunk = int(max_prefill_tokens_per_step)
+        self._own_cache: CacheContext | None = None
+
+    # ---- construction from random weights ----
+    @classmethod
+    def from_random(cls, config: dict, seed: int = 0, dtype: str = "bf16", *, std: float = 0.02,
+                    norm_mean: float = 1.0, norm_std: float = 0.0, **kwargs) -> "Engine":
+        """An engine over seeded random weights that are never written to disk."""
+        store = torch.float32 if parse_dtype(dtype) == torch.float32 else torch.bfloat16
+        tensors = dict(random_state(config, seed, store, std, norm_mean, norm_std))
+        return cls(None, dtype, _config=config, _tensors=tensors, **kwargs)
+
+    # ---- properties of the reference's binding ----
+    @property
+    def dtype(self) -> str:
+        return self._dtype_name
+
+    @property
+    def max_pos(self) -> int:
+        return self.cfg.max_pos
+
+    @property
+    def vocab_size(self) -> int:
+        return self.cfg.vocab_size
+
+    @property
+    def eos_token_ids(self):
+        return self.cfg.eos_token_ids
+
+    def weight_names(self) -> list[str]:
+        names = set(self._index_names if self._index_names is not None else self._tensors)
+        if getattr(self.cfg, "tie_word_embeddings", False) and "model.embed_tokens.weight" in names:
+            names.add("lm_head.weight")         # the tied head answers to both names
+        return sorted(names)
+
+    def has_weight(self, name: str) -> bool:
+        return name in self.weight_names()
+
+    # ---- the model on the device (made at first use, so that bad requests are
+    #      refused before a bad checkpoint is: src/engine.cpp:719-742) ----
+    @property
+    def runner(self) -> ModelRunner:
+        with self._lock:
+            if self._runner is None:
+                device = require_gpu(self._device_name)
+                from ..ops import library
+                library()                               # fails loudly if the kernels are missing
+                model = self._arch.build_model(self.cfg)
+                placement = Placement(device, self._torch_dtype)
+                with torch.cuda.device(device):
+                    if self._tensors is not None:
+                        load_state_dict(model, self._tensors, placement)
+                        self._tensors = {k: None for k in self._tensors}    # keep the names only
+                    else:
+                        load_model_weights(model, self.model_dir, placement)
+                self._runner = ModelRunner(model, self._torch_dtype, device)
+            return self._runner
+
+    @property
+    def model(self):
+        return self.runner.model
+
+    # ---- caches ----
+    def new_cache(self, num_blocks: int, block_size: int | None = None, max_requests: int = 64) -> CacheContext:
+        with torch.cuda.device(self.runner.device):
+            return self.runner.new_cache(int(num_blocks), int(block_size or self.block_size), int(max_requests))
+
+    def open_cache(self, block_manager: BlockManager, max_requests: int) -> CacheContext:
+        """The device pool behind a `BlockManager` (made once per manager)."""
+        n_layers, n_kv, hd = block_manager.dims
+        for given, have, what in ((n_layers, getattr(self.cfg, "num_hidden_layers", None), "num_layers"),
+                                  (n_kv, getattr(self.cfg, "num_key_value_heads", None), "num_kv_heads"),
+                                  (hd, getattr(self.cfg, "head_dim", None), "head_dim")):
+            if given is not None and have is not None and int(given) != int(have):
+                raise ValueError(f"BlockManager: {what}={given} does not match the model's {have}")
+        if block_manager._cache is None or block_manager._cache.max_requests < max_requests:
+            block_manager._cache = self.new_cache(block_manager.num_blocks, block_manager.block_size, max_requests)
+        return block_manager._cache
+
+    # ---- the step function ----
+    def step(self, cache: CacheContext, entries: Sequence[StepEntry]) -> torch.Tensor | None:
+        with self._lock, torch.cuda.device(self.runner.device):
+            return self.runner.step(cache, entries, max_position=self.max_pos)
+
+    def run_step(self, cache: CacheContext, entries, draws, temperature: float = 0.0, seed: int = 0) -> list[int]:
+        """A step plus the choice of a token for every wanted row (the scheduler's call)."""
+        with self._lock, torch.cuda.device(self.runner.device):
+            logits = self.runner.step(cache, entries, max_position=self.max_pos)
+            if logits is None:
+                return []
+            sampler = self.sampler if (temperature == self.sampler.temperature and seed == self.sampler.seed) \
+                else Sampler(temperature, seed)
+            return sampler.choose(logits, draws)
+
+    # ---- whole-sequence logits (src/engine.cpp:694-716) ----
+    def _validate_ids(self, ids: Sequence[int], what: str) -> list[int]:
+        ids = [int(t) for t in ids]
+        V = self.cfg.vocab_size
+        for t in ids:
+            if t < 0 or t >= V:
+                raise ValueError(f"{what}: token id {t} out of range [0, {V})")
+        return ids
+
+    def _private_cache(self, tokens: int) -> CacheContext:
+        """The engine's own pool for `generate` and `forward_logits`, grown when a
+        call needs more pages than it has."""
+        pages = max(1, (tokens + self.block_size - 1) // self.block_size)
+        c = self._own_cache
+        if c is not None:
+            for r in c.manager.live_requests():
+                c.release(r)
+            if min(c.manager.num_pages(g) for g in c.manager.groups) >= pages:
+                return c
+            self._own_cache = c = None          # drop the small pool before making the larger one
+        self._own_cache = self.new_cache(pages, self.block_size, 1)
+        return self._own_cache
+
+    def forward_logits(self, ids: Sequence[int]) -> np.ndarray:
+        """Logits at every position of a sequence, [T, vocab] float32."""
+        ids = self._validate_ids(ids, "forward_logits")
+        if not ids:
+            raise ValueError("forward_logits: ids is empty")
+        if len(ids) > self.max_pos:
+            raise RuntimeError("forward_logits: sequence exceeds RoPE max_pos")
+        with self._lock:
+            cache = self._private_cache(len(ids))
+            cache.admit("forward_logits")
+            try:
+                out = np.empty((len(ids), self.cfg.vocab_size), dtype=np.float32)
+                for start in range(0, len(ids), self.prefill_chunk):
+                    part = ids[start:start + self.prefill_chunk]
+                    logits = self.step(cache, [StepEntry("forward_logits", part, list(range(len(part))))])
+                    out[start:start + len(part)] = logits.cpu().numpy()
+                return out
+            finally:
+                cache.release("forward_logits")
+
+    # ---- generation (src/engine.cpp:718-774) ----
+    def generate(self, prompt_ids: Sequence[int], max_new_tokens: int) -> tuple[list[int], str]:
+        """Decodes up to max_new_tokens after the prompt, greedily unless the engine
+        was given a temperature; stops at an EOS id, which is not appended. Returns
+        (prompt + generated ids, "stop" | "length")."""
+        if len(prompt_ids) == 0:
+            raise ValueError("generate: prompt_ids is empty")
+        if max_new_tokens < 0:
+            raise ValueError("generate: max_new_tokens negative")
+        ids = self._validate_ids(prompt_ids, "generate")
+        if len(ids) + int(max_new_tokens) > self.max_pos:
+            raise RuntimeError("generate: prompt + max_new_tokens exceeds RoPE max_pos")
+        out = list(ids)
+        if max_new_tokens == 0:
+            return out, "length"
+        eos = set(self.cfg.eos_token_ids)
+        with self._lock:
+            cache = self._private_cache(len(ids) + int(max_new_tokens))
+            rid = "generate"
+            cache.admit(rid)
+            try:
+                logits = None
+                for start in range(0, len(ids), self.prefill_chunk):
+                    part = ids[start:start + self.prefill_chunk]
+                    last = start + len(part) == len(ids)
+                    logits = self.step(cache, [StepEntry(rid, part, [len(part) - 1] if last else [])])
+                finish = "length"
+                generated = 0
+                while generated < max_new_tokens:
+                    nxt = self.sampler.choose(logits, [(0, generated)])[0]
+                    if nxt in eos:
+                        finish = "stop"
+                        break
+                    out.append(nxt)
+                    generated += 1
+                    if generated < max_new_tokens:
+                        logits = self.step(cache, [StepEntry(rid, [nxt], [0])])
+                return out, finish
+            finally:
+                cache.release(rid)

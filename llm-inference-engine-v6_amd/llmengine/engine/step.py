@@ -1,0 +1,257 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+The reference has three forward entry points: one token of one sequence, one
+token of each of B sequences, or a whole sequence token by token
+(src/engine.cpp:273-282,488-493,694-716). Here they are one call. A step is a flat
+batch of T tokens from several requests; each request brings n >= 1 consecutive
+tokens (a whole prompt, a portion of one, or one decoded token) that continue what
+its cache holds. The step runs only these tokens, writes their keys and values into
+the request's pages, and returns 32-bit logits at the wanted places.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Sequence
+
+import torch
+
+from ..cache import CacheManager, CacheStorage, plan_groups
+from ..models.model import DecoderModel
+
+
+class CapacityError(RuntimeError):
+    """The page pool cannot hold the tokens of a step."""
+
+
+@dataclass
+class StepEntry:
+    request_id: object
+    tokens: Sequence[int]
+    want: Sequence[int] = ()        # places among `tokens` whose logits are wanted
+
+
+class Workspace:
+    """Scratch buffers by name, grown on demand and kept, so that steps of the same
+    size reuse the same device addresses."""
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self._buffers: dict[tuple[str, torch.dtype], torch.Tensor] = {}
+
+    def get(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for d in shape:
+            n *= int(d)
+        key = (name, dtype)
+        buf = self._buffers.get(key)
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._buffers[key] = buf
+        return buf[:n].view(shape)
+
+
+@dataclass
+class StepContext:
+    """What the parts see of a step. Device tensors are int32."""
+    num_tokens: int
+    num_seqs: int
+    tokens: torch.Tensor            # [T] token ids
+    positions: torch.Tensor         # [T] position of each token in its request
+    seq_idx: torch.Tensor           # [T] row of the token's request in the per-request arrays
+    q_start: torch.Tensor           # [S + 1] first row of each request's tokens in the batch
+    ctx_len: torch.Tensor           # [S] tokens cached before this step
+    slots: torch.Tensor             # [S] state slot of each request
+    block_tables: dict[str, torch.Tensor]      # group -> [S, max_blocks]
+    act_dtype: torch.dtype
+    workspace: Workspace
+    # host copies, for kernels' launch decisions and checks
+    new_lens: list[int] = field(default_factory=list)
+    ctx_lens: list[int] = field(default_factory=list)
+    slot_list: list[int] = field(default_factory=list)
+    max_position: int = 0
+    extra: dict = field(default_factory=dict)          # per-step notes of kernels (launch plans)
+
+    def buffer(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        return self.workspace.get(name, shape, dtype)
+
+
+class _Staging:
+    """Pinned host buffers for the step's integer arrays, used in rotation; a buffer
+    is rewritten only after the copy that read it has finished."""
+
+    def __init__(self, count: int = 4):
+        self._bufs: list[torch.Tensor | None] = [None] * count
+        self._events: list[torch.cuda.Event | None] = [None] * count
+        self._next = 0
+
+    def take(self, n: int) -> tuple[torch.Tensor, int]:
+        i = self._next
+        self._next = (self._next + 1) % len(self._bufs)
+        if self._events[i] is not None:
+            self._events[i].synchronize()
+        buf = self._bufs[i]
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(n, 1024), dtype=torch.int32, pin_memory=True)
+            self._bufs[i] = buf
+        return buf, i
+
+    def sent(self, i: int) -> None:
+        ev = self._events[i] or torch.cuda.Event()
+        ev.record()
+        self._events[i] = ev
+
+
+class CacheContext:
+    """A page pool with its device memory, for one model: the cache manager's
+    bookkeeping plus the tensors the pages live in."""
+
+    def __init__(self, model: DecoderModel, num_pages, page_size: int, max_requests: int,
+                 dtype: torch.dtype, device: torch.device):
+        specs = model.cache_specs()
+        groups = plan_groups(specs, num_pages)
+        self.manager = CacheManager(groups, page_size, max_requests)
+        self.storage = CacheStorage(specs, groups, page_size, max_requests, dtype, device)
+        self.page_size = page_size
+        self.max_requests = max_requests
+
+    def admit(self, request_id) -> int:
+        slot = self.manager.admit(request_id)
+        self.storage.clear_slot(slot)
+        return slot
+
+    def release(self, request_id) -> None:
+        self.manager.release(request_id)
+
+
+class ModelRunner:
+    """A loaded model on a device plus the scratch memory its steps use."""
+
+    def __init__(self, model: DecoderModel, dtype: torch.dtype, device: torch.device):
+        self.model = model
+        self.dtype = dtype
+        self.device = device
+        self.workspace = Workspace(device)
+        self._staging = _Staging()
+        self._meta_dev: torch.Tensor | None = None
+
+    def new_cache(self, num_pages, page_size: int, max_requests: int) -> CacheContext:
+        return CacheContext(self.model, num_pages, page_size, max_requests, self.dtype, self.device)
+
+    # ------------------------------------------------------------------------------
+    def step(self, cache: CacheContext, entries: Sequence[StepEntry], max_position: int | None = None
+             ) -> torch.Tensor | None:
+        """Runs one step. Every entry's request must be admitted to `cache`. Pages for
+        all entries are reserved first (CapacityError, with nothing changed, if the
+        pools are short); then the tokens run as one batch; then the requests are
+        that much longer. Returns logits [sum(len(want)), vocab] on the device, in
+        the order of the entries and of their `want` lists, or None."""
+        mgr = cache.manager
+        if not entries:
+            return None
+        vocab = self.model.vocab_size
+        seen = set()
+        for e in entries:
+            if len(e.tokens) == 0:
+                raise ValueError(f"request {e.request_id!r}: a step entry needs at least one token")
+            if e.request_id in seen:
+                raise ValueError(f"request {e.request_id!r} appears twice in one step")
+            seen.add(e.request_id)
+            for t in e.tokens:
+                if not 0 <= int(t) < vocab:
+                    raise ValueError(f"token id {t} out of range [0, {vocab})")
+            for w in e.want:
+                if not 0 <= int(w) < len(e.tokens):
+                    raise ValueError(f"request {e.request_id!r}: wanted place {w} is not among "
+                                     f"{len(e.tokens)} tokens")
+            end = mgr.length(e.request_id) + len(e.tokens)
+            if max_position is not None and end > max_position:
+                raise ValueError(f"request {e.request_id!r}: {end} tokens exceed the position limit "
+                                 f"{max_position}")
+        # pages for every entry, or none: count first, then take
+        need = {g: 0 for g in mgr.groups}
+        for e in entries:
+            for g, n in mgr.pages_needed(e.request_id, len(e.tokens)).items():
+                need[g] += n
+        for g, n in need.items():
+            if n > mgr.free_pages(g):
+                raise CapacityError(f"the step needs {n} more pages of group {g!r}, {mgr.free_pages(g)} are free")
+        for e in entries:
+            if not mgr.reserve(e.request_id, len(e.tokens)):
+                raise CapacityError(f"request {e.request_id!r}: pages ran out while reserving")
+
+        ctx, logit_rows = self._build_context(cache, entries)
+        logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
+        for e in entries:
+            mgr.commit(e.request_id, len(e.tokens))
+        return logits
+
+    # ------------------------------------------------------------------------------
+    def _build_context(self, cache: CacheContext, entries: Sequence[StepEntry]):
+        mgr = cache.manager
+        page = cache.page_size
+        S = len(entries)
+        new_lens = [len(e.tokens) for e in entries]
+        ctx_lens = [mgr.length(e.request_id) for e in entries]
+        T = sum(new_lens)
+        groups = list(mgr.groups)
+        max_blocks = max(1, max((c + n + page - 1) // page for c, n in zip(ctx_lens, new_lens)))
+        wanted: list[int] = []
+        row = 0
+        for e, n in zip(entries, new_lens):
+            wanted += [row + int(w) for w in e.want]
+            row += n
+        R = len(wanted)
+
+        # layout of the one integer buffer: tokens, positions, seq_idx, q_start, ctx_len, slots,
+        # one block table per group, logit rows
+        sizes = [T, T, T, S + 1, S, S] + [S * max_blocks] * len(groups) + [R]
+        offsets = [0]
+        for s in sizes:
+            offsets.append(offsets[-1] + s)
+        total = offsets[-1]
+        host, idx = self._staging.take(total)
+        h = host.numpy()
+        pos = 0
+        tok_o, pos_o, seq_o, qs_o, ctx_o, slot_o = offsets[:6]
+        slot_list = []
+        for i, (e, n, c) in enumerate(zip(entries, new_lens, ctx_lens)):
+            h[tok_o + pos:tok_o + pos + n] = e.tokens
+            h[pos_o + pos:pos_o + pos + n] = range(c, c + n)
+            h[seq_o + pos:seq_o + pos + n] = i
+            h[qs_o + i] = pos
+            h[ctx_o + i] = c
+            slot = mgr.slot(e.request_id)
+            h[slot_o + i] = slot
+            slot_list.append(slot)
+            pos += n
+        h[qs_o + S] = T
+        for gi, g in enumerate(groups):
+            base = offsets[6 + gi]
+            for i, e in enumerate(entries):
+                table = mgr.block_table(e.request_id, g)
+                row_base = base + i * max_blocks
+                nb = min(len(table), max_blocks)
+                # pages given back (-1) are never read: every key a token may see has a page
+                h[row_base:row_base + nb] = table[:nb]
+                h[row_base + nb:row_base + max_blocks] = 0
+        if R:
+            h[offsets[-2]:offsets[-1]] = wanted
+
+        if self._meta_dev is None or self._meta_dev.numel() < total:
+            self._meta_dev = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
+        dev = self._meta_dev
+        dev[:total].copy_(host[:total], non_blocking=True)
+        self._staging.sent(idx)
+
+        def view(k: int, shape=None):
+            t = dev[offsets[k]:offsets[k + 1]]
+            return t if shape is None else t.view(shape)
+
+        ctx = StepContext(
+            num_tokens=T, num_seqs=S, tokens=view(0), positions=view(1), seq_idx=view(2), q_start=view(3),
+            ctx_len=view(4), slots=view(5),
+            block_tables={g: view(6 + gi, (S, max_blocks)) for gi, g in enumerate(groups)},
+            act_dtype=self.dtype, workspace=self.workspace, new_lens=new_lens, ctx_lens=ctx_lens,
+            slot_list=slot_list, max_position=max(c + n for c, n in zip(ctx_lens, new_lens)) - 1)
+        logit_rows = view(len(sizes) - 1) if R else None
+        return ctx, logit_rows

@@ -1,0 +1,191 @@
+"""Python faces of the HIP kernels: each checks its operands on the host (device,
+layout, type, shape, the limits the kernel assumes) and then launches on the
+current HIP stream. Nothing here computes on the host and nothing falls back to
+another library: a refused size raises `KernelError`.
+"""
+from __future__ import annotations
+
+import torch
+
+from .lib import BF16, F32, KernelError, check, code, entry, ptr, require, stream
+
+_FLOATS = (torch.float32, torch.bfloat16)
+
+
+class Policy:
+    """Which kernel family the dispatching operations may choose.
+
+    `fast_gemm` / `fast_attention`: allow the MFMA kernels where operand types and
+    sizes fit them; off, every product and every attention goes through the
+    plain-precision kernels (the 32-bit model always does)."""
+
+    fast_gemm = True
+    fast_attention = True
+
+
+policy = Policy()
+
+
+# --- embedding ---------------------------------------------------------------------
+def embed_gather(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, :] = table[tokens[t], :] widened to 32-bit."""
+    require(table, "table", _FLOATS, (None, None))
+    V, H = table.shape
+    T = tokens.shape[0]
+    require(tokens, "tokens", torch.int32, (T,))
+    require(out, "out", torch.float32, (T, H))
+    check(entry("llme_embed_gather")(ptr(table), code(table.dtype), ptr(tokens), ptr(out), T, H, stream()),
+          "embed_gather")
+
+
+# --- norm --------------------------------------------------------------------------
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+            rows: torch.Tensor | None = None) -> None:
+    """out[r] = weight * x[rows[r] or r] / sqrt(mean(x^2) + eps); x is 32-bit."""
+    require(x, "x", torch.float32, (None, None))
+    H = x.shape[1]
+    require(weight, "weight", _FLOATS, (H,))
+    R = x.shape[0] if rows is None else rows.shape[0]
+    if rows is not None:
+        require(rows, "rows", torch.int32, (R,))
+    require(out, "out", _FLOATS, (R, H))
+    check(entry("llme_rmsnorm")(ptr(x), ptr(weight), code(weight.dtype), ptr(out), code(out.dtype),
+                                ptr(rows), R, H, float(eps), stream()), "rmsnorm")
+
+
+# --- feed-forward activation ------------------------------------------------------
+def swiglu(gu: torch.Tensor, out: torch.Tensor, group: int) -> None:
+    """out[t, j] = silu(gate_j) * up_j from gu [T, 2 FF] laid out in alternating groups."""
+    require(out, "out", _FLOATS, (None, None))
+    T, FF = out.shape
+    require(gu, "gu", _FLOATS, (T, 2 * FF))
+    if group <= 0 or FF % group != 0:
+        raise KernelError(f"swiglu: group {group} does not divide the width {FF}")
+    if gu.dtype == torch.bfloat16 and out.dtype != torch.bfloat16:
+        raise KernelError("swiglu: bfloat16 input needs bfloat16 output")
+    check(entry("llme_swiglu")(ptr(gu), code(gu.dtype), ptr(out), code(out.dtype), T, FF, group, stream()),
+          "swiglu")
+
+
+# --- rotary encoding + cache write --------------------------------------------------
+def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor | None,
+                  positions: torch.Tensor, seq_idx: torch.Tensor, block_table: torch.Tensor,
+                  q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  n_q: int, n_kv: int, head_dim: int, rotary_dim: int, write_cache: bool = True,
+                  max_position: int | None = None) -> None:
+    """Rotates q and k heads of qkv [T, (n_q + 2 n_kv) hd] (32-bit) by the tables' rows
+    at `positions`, writes q to q_out and k, v into the pages named by the block table.
+    k_cache [pages, n_kv, page, hd]; v_cache [pages, n_kv, hd, page]."""
+    T = qkv.shape[0]
+    require(qkv, "qkv", torch.float32, (T, (n_q + 2 * n_kv) * head_dim))
+    require(positions, "positions", torch.int32, (T,))
+    require(seq_idx, "seq_idx", torch.int32, (T,))
+    require(block_table, "block_table", torch.int32, (None, None))
+    require(q_out, "q_out", _FLOATS, (T, n_q * head_dim))
+    require(k_cache, "k_cache", _FLOATS, (None, n_kv, None, head_dim))
+    page = k_cache.shape[2]
+    require(v_cache, "v_cache", k_cache.dtype, (k_cache.shape[0], n_kv, head_dim, page))
+    if rotary_dim % 2 or not 0 <= rotary_dim <= head_dim:
+        raise KernelError(f"rope: rotary_dim {rotary_dim} must be even and within head_dim {head_dim}")
+    if (cos is None) != (sin is None):
+        raise KernelError("rope: cos and sin tables come together")
+    if cos is not None:
+        require(cos, "cos", torch.float32, (None, rotary_dim // 2))
+        require(sin, "sin", torch.float32, tuple(cos.shape))
+    check(entry("llme_rope_kv_write")(
+        ptr(qkv), ptr(cos), ptr(sin), ptr(positions), ptr(seq_idx), ptr(block_table), block_table.shape[1],
+        ptr(q_out), code(q_out.dtype), ptr(k_cache), ptr(v_cache), code(k_cache.dtype), T, n_q, n_kv,
+        head_dim, rotary_dim if cos is not None else 0, page, 1 if write_cache else 0, stream()),
+        "rope_kv_write")
+
+
+def rope_q_only(q32: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor | None,
+                positions: torch.Tensor, q_out: torch.Tensor, n_q: int, head_dim: int, rotary_dim: int) -> None:
+    """Rotates query heads only (a layer that reads keys and values another layer cached)."""
+    T = q32.shape[0]
+    require(q32, "q32", torch.float32, (T, n_q * head_dim))
+    require(positions, "positions", torch.int32, (T,))
+    require(q_out, "q_out", _FLOATS, (T, n_q * head_dim))
+    if cos is not None:
+        require(cos, "cos", torch.float32, (None, rotary_dim // 2))
+        require(sin, "sin", torch.float32, tuple(cos.shape))
+    check(entry("llme_rope_kv_write")(
+        ptr(q32), ptr(cos), ptr(sin), ptr(positions), None, None, 0, ptr(q_out), code(q_out.dtype), None, None,
+        code(q_out.dtype), T, n_q, 0, head_dim, rotary_dim if cos is not None else 0, 1, 0, stream()),
+        "rope_q_only")
+
+
+# --- matrix product ------------------------------------------------------------------
+def gemm_generic(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    require(a, "a", _FLOATS, (None, None))
+    M, K = a.shape
+    require(w, "w", _FLOATS, (None, K))
+    N = w.shape[0]
+    require(out, "out", _FLOATS, (M, N))
+    check(entry("llme_gemm_generic")(ptr(a), code(a.dtype), ptr(w), code(w.dtype), ptr(out), code(out.dtype),
+                                     M, N, K, 1 if accumulate else 0, stream()), "gemm_generic")
+
+
+_fast_gemm = None       # set by ops/mfma.py when the MFMA kernels are present
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out[m, n] (+)= sum_k a[m, k] w[n, k]; 32-bit accumulation whatever the types."""
+    if policy.fast_gemm and _fast_gemm is not None and _fast_gemm(a, w, out, accumulate):
+        return
+    gemm_generic(a, w, out, accumulate)
+
+
+# --- attention -----------------------------------------------------------------------
+def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
+                      positions: torch.Tensor, seq_idx: torch.Tensor, block_table: torch.Tensor,
+                      n_q: int, n_kv: int, head_dim: int, scale: float, window: int = 0) -> None:
+    T = q.shape[0]
+    require(q, "q", _FLOATS, (T, n_q * head_dim))
+    require(out, "out", q.dtype, (T, n_q * head_dim))
+    require(k_cache, "k_cache", _FLOATS, (None, n_kv, None, head_dim))
+    page = k_cache.shape[2]
+    require(v_cache, "v_cache", k_cache.dtype, (k_cache.shape[0], n_kv, head_dim, page))
+    require(positions, "positions", torch.int32, (T,))
+    require(seq_idx, "seq_idx", torch.int32, (T,))
+    require(block_table, "block_table", torch.int32, (None, None))
+    if head_dim > 256:
+        raise KernelError(f"attention: head_dim {head_dim} is beyond the kernel's limit of 256")
+    if n_q % n_kv:
+        raise KernelError(f"attention: {n_q} query heads do not divide into {n_kv} key/value heads")
+    check(entry("llme_attention_generic")(
+        ptr(q), code(q.dtype), ptr(k_cache), ptr(v_cache), code(k_cache.dtype), ptr(out), ptr(positions),
+        ptr(seq_idx), ptr(block_table), block_table.shape[1], T, n_q, n_kv, head_dim, page, float(scale),
+        int(window), stream()), "attention_generic")
+
+
+_fast_attention = None  # set by ops/mfma.py when the MFMA kernels are present
+
+
+def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, step,
+              block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int, scale: float,
+              window: int = 0) -> None:
+    """Attention of every token of the step over its request's pages. `step` carries
+    positions, request index per token and, on the host, how the batch is cut."""
+    if policy.fast_attention and _fast_attention is not None and _fast_attention(
+            q, k_cache, v_cache, out, step, block_table, n_q, n_kv, head_dim, scale, window):
+        return
+    attention_generic(q, k_cache, v_cache, out, step.positions, step.seq_idx, block_table, n_q, n_kv,
+                      head_dim, scale, window)
+
+
+# --- sampling ------------------------------------------------------------------------
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    require(logits, "logits", torch.float32, (None, None))
+    R, V = logits.shape
+    require(out, "out", torch.int32, (R,))
+    check(entry("llme_argmax")(ptr(logits), ptr(out), R, V, stream()), "argmax")
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor) -> None:
+    require(logits, "logits", torch.float32, (None, None))
+    R, V = logits.shape
+    require(temperature, "temperature", torch.float32, (R,))
+    require(uniform, "uniform", torch.float32, (R,))
+    require(out, "out", torch.int32, (R,))
+    check(entry("llme_sample")(ptr(logits), ptr(temperature), ptr(uniform), ptr(out), R, V, stream()), "sample")

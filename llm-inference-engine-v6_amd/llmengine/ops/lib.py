@@ -1,0 +1,126 @@
+"""Loads the HIP kernel library and declares its entry points.
+
+There is no other implementation behind these operations: if the library cannot
+be built or loaded, the first use raises `KernelLibraryError`.
+"""
+from __future__ import annotations
+
+import ctypes
+import threading
+
+import torch
+
+from . import build as _build
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+F32, BF16 = 0, 1            # dtype codes of csrc/common.h
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+_lib = None
+_lock = threading.Lock()
+
+_vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+
+_SIGNATURES = {
+    "llme_embed_gather": [_vp, _i, _vp, _vp, _i, _i, _vp],
+    "llme_rmsnorm": [_vp, _vp, _i, _vp, _i, _vp, _i, _i, _f, _vp],
+    "llme_swiglu": [_vp, _i, _vp, _i, _i, _i, _i, _vp],
+    "llme_rope_kv_write": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i,
+                           _i, _i, _i, _i, _i, _i, _i, _vp],
+    "llme_gemm_generic": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
+    "llme_attention_generic": [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
+                               _f, _i, _vp],
+    "llme_argmax": [_vp, _vp, _i, _i, _vp],
+    "llme_sample": [_vp, _vp, _vp, _vp, _i, _i, _vp],
+}
+
+
+def library() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        try:
+            path = _build.ensure_built()
+            lib = ctypes.CDLL(path)
+        except (OSError, _build.BuildError) as e:
+            raise KernelLibraryError(
+                f"the HIP kernel library is not available ({e}); this engine has no other "
+                "implementation of its kernels") from e
+        for name, argtypes in _SIGNATURES.items():
+            try:
+                fn = getattr(lib, name)
+            except AttributeError:
+                continue        # optional entry points are checked where they are used
+            fn.argtypes = argtypes
+            fn.restype = ctypes.c_int
+        _lib = lib
+        return lib
+
+
+def declare(name: str, argtypes: list) -> None:
+    """Adds an entry point's signature (kernel files added later register here)."""
+    _SIGNATURES[name] = argtypes
+    if _lib is not None and hasattr(_lib, name):
+        fn = getattr(_lib, name)
+        fn.argtypes = argtypes
+        fn.restype = ctypes.c_int
+
+
+def entry(name: str):
+    lib = library()
+    try:
+        return getattr(lib, name)
+    except AttributeError:
+        raise KernelLibraryError(f"the kernel library has no entry point {name}") from None
+
+
+def code(dtype: torch.dtype) -> int:
+    try:
+        return _CODES[dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16 tensors, not {dtype}") from None
+
+
+def stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        if status == 10001:
+            raise KernelError(f"{what}: the kernel refused its arguments")
+        if status == 10002:
+            raise KernelError(f"{what}: the kernel does not support this size")
+        raise KernelError(f"{what}: HIP error {status}")
+
+
+def require(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
+    """Host-side check of an operand before a launch: device, layout, type, shape."""
+    if not isinstance(t, torch.Tensor):
+        raise KernelError(f"{name}: expected a tensor, got {type(t).__name__}")
+    if t.device.type != "cuda":
+        raise KernelError(f"{name}: must live on the GPU, is on {t.device}")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: must be contiguous")
+    if dtype is not None:
+        allowed = dtype if isinstance(dtype, (tuple, list)) else (dtype,)
+        if t.dtype not in allowed:
+            raise KernelError(f"{name}: dtype {t.dtype} not in {allowed}")
+    if shape is not None:
+        if len(shape) != t.dim() or any(s is not None and s != d for s, d in zip(shape, t.shape)):
+            raise KernelError(f"{name}: shape {tuple(t.shape)} does not match {tuple(shape)}")

@@ -1,0 +1,88 @@
+"""Grouped-query attention over the paged cache.
+
+q, k, v = x Wq^T, x Wk^T, x Wv^T without biases; head j is the slice
+[j hd, (j+1) hd); q and k are rotated at the token's position and k is cached after
+rotation, v as it is (src/engine.cpp:142-170); query head h reads kv head
+h / (n_q / n_kv); scores scale by head_dim^-1/2, softmax over the keys up to the
+token's own position (src/kernels.cpp:413-474); out = concat(heads) Wo^T
+(src/engine.cpp:193-194).
+
+The three projections are one product against the row-concatenated matrix. The
+step's own keys and values go into the pages first, then every token reads pages
+only: whole prompts, portions with earlier context and single decoded tokens are
+the same case. `window` > 0 restricts a token at position p to keys > p - window.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .base import PAGE, CacheSpec, Getter, Mixer, ParamSpec, Placement, PositionEncoding
+from .registry import register_part
+
+
+class Attention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 position: PositionEncoding | None = None, scale: float | None = None, window: int = 0):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads do not divide into {num_kv_heads} key/value heads")
+        self.hidden_size = int(hidden_size)
+        self.num_heads, self.num_kv_heads, self.head_dim = int(num_heads), int(num_kv_heads), int(head_dim)
+        self.position = position
+        self.scale = float(scale) if scale is not None else float(head_dim) ** -0.5
+        self.window = int(window)
+        self.q_dim = self.num_heads * self.head_dim
+        self.kv_dim = self.num_kv_heads * self.head_dim
+        self.w_qkv: torch.Tensor | None = None
+        self.w_o: torch.Tensor | None = None
+
+    def param_specs(self):
+        H = self.hidden_size
+        return {"q_proj.weight": ParamSpec((self.q_dim, H)), "k_proj.weight": ParamSpec((self.kv_dim, H)),
+                "v_proj.weight": ParamSpec((self.kv_dim, H)), "o_proj.weight": ParamSpec((H, self.q_dim))}
+
+    def load_params(self, get: Getter, placement: Placement) -> None:
+        parts = [get("q_proj.weight"), get("k_proj.weight"), get("v_proj.weight")]
+        dtype = placement.common_dtype(parts)
+        fused = torch.empty((self.q_dim + 2 * self.kv_dim, self.hidden_size), dtype=dtype,
+                            device=placement.device)
+        row = 0
+        for p in parts:
+            fused[row:row + p.shape[0]].copy_(p)
+            row += p.shape[0]
+        self.w_qkv = fused
+        self.w_o = placement.place(get("o_proj.weight"))
+        if self.position is not None and hasattr(self.position, "materialize"):
+            self.position.materialize(placement)
+
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec(kind="window" if self.window > 0 else "full", window=self.window,
+                         paged={"k": (self.num_kv_heads, PAGE, self.head_dim),
+                                "v": (self.num_kv_heads, self.head_dim, PAGE)})
+
+    def forward(self, x, step, cache, out, accumulate, write_cache=True):
+        T = x.shape[0]
+        n_q, n_kv, hd = self.num_heads, self.num_kv_heads, self.head_dim
+        tables = self.position.rotary_tables() if self.position is not None else None
+        cos, sin, rot = tables if tables is not None else (None, None, 0)
+        if cos is not None and step.max_position >= cos.shape[0]:
+            raise ValueError(f"position {step.max_position} is beyond the position table ({cos.shape[0]} rows)")
+        block_table = step.block_tables[cache.group]
+        k_cache, v_cache = cache.paged["k"], cache.paged["v"]
+        q = step.buffer("attn.q", (T, self.q_dim), x.dtype)
+        if write_cache:
+            qkv = step.buffer("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
+            ops.gemm(x, self.w_qkv, qkv)
+            ops.rope_kv_write(qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
+                              n_q, n_kv, hd, rot, write_cache=True)
+        else:
+            # A layer that reads another layer's cache projects queries only.
+            q32 = step.buffer("attn.q32", (T, self.q_dim), torch.float32)
+            ops.gemm(x, self.w_qkv[:self.q_dim], q32)
+            ops.rope_q_only(q32, cos, sin, step.positions, q, n_q, hd, rot)
+        o = step.buffer("attn.o", (T, self.q_dim), x.dtype)
+        ops.attention(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, hd, self.scale, self.window)
+        ops.gemm(o, self.w_o, out, accumulate)
+
+
+register_part("mixer", "attention", Attention)

@@ -1,0 +1,178 @@
+"""Interfaces of the parts a model is put together from.
+
+A part owns its sizes and constants (constructor arguments), names the tensors it
+reads from a checkpoint (`param_specs`), places them on the device in the layout
+its kernels want (`load_params`) and runs on a step's flat batch (`forward`). No
+part knows which model it is in: names under which a model stores a part's
+tensors are given by whoever composes the parts.
+
+Kinds of parts and what each must provide:
+
+* `Norm`:      forward(x32 [T, H], out [R, H], rows=None)
+* `PositionEncoding`: rotary_tables() -> (cos, sin, rotary_dim) or None, and
+               apply(q, k, positions) for encodings that are not rotary tables
+* `Mixer`:     cache_spec(), forward(x [T, H], step, cache, out32 [T, H], accumulate,
+               write_cache)
+* `FeedForward`: forward(x [T, H], step, out32 [T, H], accumulate)
+* `Block`:     the arrangement of the four above around the 32-bit residual stream:
+               forward(h32 [T, H], step, cache, write_cache)
+
+`step` is the engine's `StepContext` (tokens, positions, request index per token,
+block tables, slots, scratch buffers); `cache` is the `LayerCache` that the cache
+manager made from the mixer's `cache_spec`.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable, Mapping
+
+import torch
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """A tensor a part reads from the checkpoint: its exact shape there, and how a
+    random model fills it ("linear": N(0, std); "norm": N(mean, std) around one)."""
+    shape: tuple[int, ...]
+    init: str = "linear"
+
+
+@dataclass(frozen=True)
+class Placement:
+    """Where parameters live and in which precision the model computes."""
+    device: torch.device
+    compute_dtype: torch.dtype          # torch.float32 or torch.bfloat16
+
+    def storage_dtype(self, stored: torch.dtype) -> torch.dtype:
+        """A tensor's dtype on the device, given its dtype in the file. The 32-bit
+        model widens everything; the bfloat16 model keeps bfloat16 tensors as they
+        are and leaves tensors stored in 32-bit (or half, widened exactly) in
+        32-bit; integer tables become int32."""
+        if stored in (torch.int32, torch.int64):
+            return torch.int32
+        if self.compute_dtype == torch.float32:
+            return torch.float32
+        return torch.bfloat16 if stored == torch.bfloat16 else torch.float32
+
+    def place(self, t: torch.Tensor, dtype: torch.dtype | None = None) -> torch.Tensor:
+        dtype = dtype or self.storage_dtype(t.dtype)
+        return t.to(device=self.device, dtype=dtype).contiguous()
+
+    def common_dtype(self, tensors: list[torch.Tensor]) -> torch.dtype:
+        """The storage dtype of a buffer that fuses several checkpoint tensors."""
+        kinds = {self.storage_dtype(t.dtype) for t in tensors}
+        return kinds.pop() if len(kinds) == 1 else torch.float32
+
+
+Getter = Callable[[str], torch.Tensor]      # local tensor name -> CPU tensor as stored
+
+
+class Part:
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {}
+
+    def children(self) -> dict[str, "Part"]:
+        """Sub-parts by the name prefix under which their tensors are stored."""
+        return {}
+
+    def ignored_names(self) -> set[str]:
+        """Tensor names that a checkpoint may hold for this part and that are not read."""
+        return set()
+
+    def load_params(self, get: Getter, placement: Placement) -> None:
+        """Reads the part's own tensors (children are loaded by the walker)."""
+
+    # ---- walking a tree of parts ----
+    def named_specs(self, prefix: str = "") -> dict[str, ParamSpec]:
+        out = {prefix + k: v for k, v in self.param_specs().items()}
+        for name, child in self.children().items():
+            out.update(child.named_specs(f"{prefix}{name}."))
+        return out
+
+    def named_ignored(self, prefix: str = "") -> set[str]:
+        out = {prefix + k for k in self.ignored_names()}
+        for name, child in self.children().items():
+            out |= child.named_ignored(f"{prefix}{name}.")
+        return out
+
+    def load_tree(self, get: Getter, placement: Placement, prefix: str = "") -> None:
+        self.load_params(lambda local: get(prefix + local), placement)
+        for name, child in self.children().items():
+            child.load_tree(get, placement, f"{prefix}{name}.")
+
+
+# --- what a mixer keeps between steps ---------------------------------------------------
+PAGE = -1       # placeholder for the page size in a paged tensor's shape
+
+
+@dataclass(frozen=True)
+class CacheSpec:
+    """What one mixer keeps for a request.
+
+    paged: tensors kept per token, in pages: name -> shape of one page, with `PAGE`
+           where the page size goes. Layers with the same (kind, window) share a
+           page pool and a block table (one page id covers all of them).
+    kind:  "full": every token of the request stays; "window": only the last
+           `window` tokens are ever read, pages behind them are given back.
+    state: tensors of fixed size per request: name -> (shape, dtype), kept in the
+           request's slot, zero when the request is admitted.
+    """
+    kind: str = "full"
+    window: int = 0
+    paged: Mapping[str, tuple[int, ...]] = field(default_factory=dict)
+    state: Mapping[str, tuple[tuple[int, ...], torch.dtype]] = field(default_factory=dict)
+
+    def __post_init__(self):
+        if self.kind not in ("full", "window"):
+            raise ValueError(f"cache kind {self.kind!r} is not 'full' or 'window'")
+        if self.kind == "window" and self.window <= 0:
+            raise ValueError("a window cache needs window > 0")
+
+    @property
+    def group_key(self) -> tuple:
+        return (self.kind, self.window if self.kind == "window" else 0)
+
+
+@dataclass
+class LayerCache:
+    """The device tensors of one mixer's cache, as the mixer sees them in a step."""
+    paged: dict[str, torch.Tensor]          # name -> [num_pages, *page shape]
+    state: dict[str, torch.Tensor]          # name -> [num_slots, *shape]
+    page_size: int
+    group: str | None                       # key into StepContext.block_tables
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def rotary_tables(self):
+        """(cos [P, r/2], sin [P, r/2], r) for rotate-half pairs (i, i + r/2), or None."""
+        return None
+
+    @property
+    def max_position(self) -> int:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self) -> CacheSpec | None:
+        return None
+
+    def forward(self, x: torch.Tensor, step, cache: LayerCache | None, out: torch.Tensor,
+                accumulate: bool, write_cache: bool = True) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, step, out: torch.Tensor, accumulate: bool) -> None:
+        raise NotImplementedError
+
+
+class Block(Part):
+    mixer: Mixer
+
+    def forward(self, h: torch.Tensor, step, cache: LayerCache | None, write_cache: bool = True) -> None:
+        raise NotImplementedError

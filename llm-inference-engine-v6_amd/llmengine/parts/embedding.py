@@ -1,0 +1,54 @@
+"""Token embedding and output head.
+
+Embedding: h = E[token] with no multiplier (src/kernels.cpp:59-66). Head:
+logits = x . W^T in 32-bit (src/engine.cpp:242-249); a tied head is the embedding
+table itself, one buffer under two names (src/weights.cpp:244-267, src/model.cpp:185-190).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .base import Getter, ParamSpec, Part, Placement
+
+
+class Embedding(Part):
+    def __init__(self, vocab_size: int, hidden_size: int):
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.weight: torch.Tensor | None = None
+
+    def param_specs(self):
+        return {"weight": ParamSpec((self.vocab_size, self.hidden_size), "linear")}
+
+    def load_params(self, get: Getter, placement: Placement) -> None:
+        self.weight = placement.place(get("weight"))
+
+    def forward(self, tokens: torch.Tensor, out: torch.Tensor) -> None:
+        ops.embed_gather(self.weight, tokens, out)
+
+
+class OutputHead(Part):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: Embedding | None = None):
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.tied_to = tied_to
+        self._weight: torch.Tensor | None = None
+
+    def param_specs(self):
+        if self.tied_to is not None:
+            return {}
+        return {"weight": ParamSpec((self.vocab_size, self.hidden_size), "linear")}
+
+    def ignored_names(self):
+        # A tied checkpoint may still store the head; the embedding is used either way.
+        return {"weight"} if self.tied_to is not None else set()
+
+    def load_params(self, get: Getter, placement: Placement) -> None:
+        if self.tied_to is None:
+            self._weight = placement.place(get("weight"))
+
+    @property
+    def weight(self) -> torch.Tensor:
+        return self.tied_to.weight if self.tied_to is not None else self._weight
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor) -> None:
+        ops.gemm(x, self.weight, out)
