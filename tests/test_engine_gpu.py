@@ -1,0 +1,197 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16, under every way
+of cutting requests into steps: whole; most in one step and the last 32 tokens one by one;
+portions of changing size down to two tokens; mixed batches of up to four live requests with
+so few pages that they are used again; long decoding; the first tokens of a sequence."""
+import numpy as np
+import pytest
+import torch
+
+import replay
+from plain_llama import bf16_round, load_plain_model, plain_forward
+from tiny_models import (A_INIT, B_INIT, C_INIT, D_INIT, TINY_A, TINY_B, TINY_C, TINY_D, make_model_dir,
+                         random_tokens)
+
+pytestmark = pytest.mark.gpu
+
+# Largest allowed max|engine - plain| per row, relative to the row's largest |logit|.
+TOL = {"fp32": 1e-5, "bf16": 2e-2}
+
+MODELS = {
+    "A": (TINY_A, A_INIT, 4, [5, 11, 17, 40]),
+    "B": (TINY_B, B_INIT, 8, [1, 9, 33, 70]),
+    "D": (TINY_D, D_INIT, 16, [3, 50, 66, 21]),
+}
+
+
+@pytest.fixture(scope="module")
+def zoo(tmp_path_factory):
+    """name -> (model folder, requests, plain logits per dtype), made once."""
+    out = {}
+    for name, (cfg, init, page, lens) in MODELS.items():
+        d = make_model_dir(tmp_path_factory.mktemp(f"tiny{name}"), cfg, init, torch.bfloat16)
+        reqs = {f"r{i}": random_tokens(n, cfg["vocab_size"], 100 + i) for i, n in enumerate(lens)}
+        pcfg, pw = load_plain_model(d)
+        plain = {
+            "fp32": {rid: plain_forward(pcfg, pw, ids).numpy() for rid, ids in reqs.items()},
+            "bf16": {rid: plain_forward(pcfg, pw, ids, rounder=bf16_round).numpy() for rid, ids in reqs.items()},
+        }
+        out[name] = (d, reqs, plain, page)
+    return out
+
+
+_ENGINES = {}
+
+
+def engine_for(model_dir, dtype):
+    from llmengine import Engine
+    key = (model_dir, dtype)
+    if key not in _ENGINES:
+        _ENGINES[key] = Engine(model_dir, dtype)
+    return _ENGINES[key]
+
+
+def check_against_plain(got: dict, plain: dict, reqs: dict, dtype: str):
+    worst = 0.0
+    for rid, ids in reqs.items():
+        assert sorted(got[rid]) == list(range(len(ids))), f"{rid}: positions {sorted(got[rid])}"
+        for pos in range(len(ids)):
+            ref = plain[rid][pos]
+            err = np.abs(got[rid][pos].astype(np.float64) - ref).max() / np.abs(ref).max()
+            worst = max(worst, err)
+            assert err < TOL[dtype], f"request {rid} position {pos}: relative error {err:.3e}"
+    return worst
+
+
+SCHEDULES = {
+    "whole": lambda reqs: replay.whole(reqs),
+    "tail": lambda reqs: replay.tail_one_by_one(reqs, 32),
+    "portions": lambda reqs: replay.portions(reqs),
+    "mixed": lambda reqs: replay.mixed(reqs, max_live=4),
+    "mixed3": lambda reqs: replay.mixed(reqs, max_live=3, prompt_frac=0.3, seed=5),
+}
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+@pytest.mark.parametrize("schedule", list(SCHEDULES))
+@pytest.mark.parametrize("name", list(MODELS))
+def test_schedules_match_plain(zoo, name, schedule, dtype):
+    model_dir, reqs, plain, page = zoo[name]
+    engine = engine_for(model_dir, dtype)
+    steps = SCHEDULES[schedule](reqs)
+    # exactly as many pages as the trace's peak needs, so finished requests' pages are used again
+    pages = replay.trace_peak_tokens(steps, round_to=page) // page
+    cache = engine.new_cache(pages, page, max_requests=4)
+    got = replay.run_trace(engine, cache, steps)
+    check_against_plain(got, plain[dtype], reqs, dtype)
+    assert all(cache.manager.free_pages(g) == cache.manager.num_pages(g) for g in cache.manager.groups)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_page_reuse_leaves_nothing_behind(zoo, dtype):
+    """The same request replayed after other requests have used (and dirtied) every page."""
+    model_dir, reqs, plain, page = zoo["B"]
+    engine = engine_for(model_dir, dtype)
+    cache = engine.new_cache(12, page, max_requests=4)
+    for _ in range(3):
+        got = replay.run_trace(engine, cache, replay.portions(reqs, sizes=(13, 2, 6)))
+        check_against_plain(got, plain[dtype], reqs, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_batch_order_does_not_matter(zoo, dtype):
+    """Rows of a batch are independent of their neighbours: permuting the entries permutes the logits."""
+    model_dir, reqs, plain, page = zoo["A"]
+    engine = engine_for(model_dir, dtype)
+    from llmengine import StepEntry
+    ids = list(reqs)
+    results = []
+    for order in (ids, ids[::-1]):
+        cache = engine.new_cache(64, page, max_requests=4)
+        for rid in order:
+            cache.admit(rid)
+        logits = engine.step(cache, [StepEntry(rid, reqs[rid], [len(reqs[rid]) - 1]) for rid in order])
+        results.append(dict(zip(order, logits.cpu().numpy())))
+    for rid in ids:
+        ref = plain[dtype][rid][-1]
+        for res in results:
+            assert np.abs(res[rid] - ref).max() / np.abs(ref).max() < TOL[dtype]
+    if dtype == "fp32":
+        for rid in ids:
+            assert np.abs(results[0][rid] - results[1][rid]).max() <= 1e-6 * np.abs(results[0][rid]).max()
+
+
+@pytest.fixture(scope="module")
+def model_c(tmp_path_factory):
+    d = make_model_dir(tmp_path_factory.mktemp("tinyC"), TINY_C, C_INIT, torch.bfloat16)
+    return d
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_long_decoding(model_c, dtype):
+    """A 40-token prompt, then 400 tokens decoded one by one: positions far beyond the rope
+    scaling's original length, many pages, logits compared at chosen positions."""
+    ids = random_tokens(440, TINY_C["vocab_size"], 7)
+    pcfg, pw = load_plain_model(model_c)
+    ref = plain_forward(pcfg, pw, ids, rounder=bf16_round if dtype == "bf16" else None).numpy()
+    engine = engine_for(model_c, dtype)
+    steps = replay.tail_one_by_one({"long": ids}, tail=400)
+    cache = engine.new_cache(28, 16, max_requests=1)
+    got = replay.run_trace(engine, cache, steps)["long"]
+    for pos in range(len(ids)):
+        err = np.abs(got[pos] - ref[pos]).max() / np.abs(ref[pos]).max()
+        assert err < TOL[dtype], f"position {pos}: {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_first_tokens(zoo, dtype):
+    """Positions 0, 1, 2 of a sequence, alone and as the start of longer steps."""
+    model_dir, reqs, plain, page = zoo["B"]
+    engine = engine_for(model_dir, dtype)
+    ids = reqs["r3"]
+    for cut in ([1, 1, 1], [1, 2], [2, 1], [3]):
+        steps, pos = [], 0
+        for n in cut:
+            steps.append({"step": len(steps), "entries": [{"id": "x", "tokens": ids[pos:pos + n],
+                                                           "want": list(range(n))}],
+                          "end": ["x"] if pos + n == 3 else []})
+            pos += n
+        cache = engine.new_cache(2, page, max_requests=1)
+        got = replay.run_trace(engine, cache, steps)["x"]
+        for p in range(3):
+            ref = plain[dtype]["r3"][p]
+            assert np.abs(got[p] - ref).max() / np.abs(ref).max() < TOL[dtype], (cut, p)
+
+
+def test_a_far_key_is_found(tmp_path):
+    """Random weights would hide a lost far key among hundreds: here the query of the last token
+    is made to match the key of token 5 so strongly that it takes nearly all the weight, and that
+    token's value decides the logits. Dropping or misplacing that one key changes the answer."""
+    from safetensors.torch import load_file
+    from llmengine.weights import write_state_dict
+    import json
+    import os
+    d = make_model_dir(tmp_path / "base", TINY_C, C_INIT, torch.float32)
+    w = load_file(os.path.join(d, "model.safetensors"))
+    cfg = dict(TINY_C)
+    # make layer 0's keys and queries depend only on the token id through the embedding:
+    # scale q and k projections up so that equal tokens produce a dominant score.
+    for name in ("model.layers.0.self_attn.q_proj.weight", "model.layers.0.self_attn.k_proj.weight"):
+        w[name] = w[name] * 4.0
+    out_dir = str(tmp_path / "sharp")
+    os.makedirs(out_dir)
+    write_state_dict(os.path.join(out_dir, "model.safetensors"), w)
+    with open(os.path.join(out_dir, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    ids = random_tokens(600, cfg["vocab_size"], 21)
+    ids[-1] = ids[5]                       # the last token repeats token 5: its key matches best
+    pcfg, pw = load_plain_model(out_dir)
+    ref = plain_forward(pcfg, pw, ids).numpy()
+    from llmengine import Engine
+    engine = Engine(out_dir, "fp32")
+    for steps in (replay.whole({"s": ids}), replay.tail_one_by_one({"s": ids}, 32),
+                  replay.portions({"s": ids}, sizes=(97, 2, 31, 64))):
+        cache = engine.new_cache(38, 16, max_requests=1)
+        got = replay.run_trace(engine, cache, steps)["s"]
+        for pos in (5, 6, 300, 598, 599):
+            err = np.abs(got[pos] - ref[pos]).max() / np.abs(ref[pos]).max()
+            assert err < 1e-5, (pos, err)

@@ -1,0 +1,218 @@
+"""Each HIP kernel alone against the plain implementation, at sizes other than the
+engine's tiny models: widths and vocabularies that are no power of two, head sizes in
+steps of 16, several page sizes, both storage types."""
+import math
+
+import pytest
+import torch
+
+from plain_llama import (bf16_round, plain_apply_rope, plain_argmax, plain_attention, plain_linear,
+                         plain_rmsnorm, plain_sample_bounds, plain_silu)
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def _rel(a: torch.Tensor, b: torch.Tensor) -> float:
+    return float((a.double() - b.double()).abs().max() / b.double().abs().max().clamp_min(1e-30))
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from llmengine import ops
+    ops.library()
+    return ops
+
+
+@pytest.mark.parametrize("V,H,dtype", [(37, 50, torch.float32), (129, 96, torch.bfloat16)])
+def test_embed_gather(ops, V, H, dtype):
+    table = torch.randn(V, H, generator=_gen(0)).to(dtype)
+    tokens = torch.tensor([0, 1, 7, V - 1, 3, 3], dtype=torch.int32)
+    out = torch.empty(len(tokens), H, dtype=torch.float32, device=DEV)
+    ops.embed_gather(table.to(DEV), tokens.to(DEV), out)
+    assert torch.equal(out.cpu(), table[tokens.long()].float())       # exact row copies
+
+
+@pytest.mark.parametrize("H", [16, 64, 257, 2048, 3000])
+@pytest.mark.parametrize("wdtype,odtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                           (torch.float32, torch.bfloat16)])
+def test_rmsnorm(ops, H, wdtype, odtype):
+    x = torch.randn(5, H, generator=_gen(1)) * 3
+    w = (1 + 0.1 * torch.randn(H, generator=_gen(2))).to(wdtype)
+    out = torch.empty(5, H, dtype=odtype, device=DEV)
+    ops.rmsnorm(x.to(DEV), w.to(DEV), 1e-6, out)
+    ref = plain_rmsnorm(x.double(), w.double(), 1e-6)
+    if odtype == torch.float32:
+        assert _rel(out.cpu(), ref) < 2e-6
+    else:
+        assert torch.equal(out.cpu().float(), ref.float().to(torch.bfloat16).float()) or \
+            _rel(out.cpu().float(), ref) < 8e-3
+    rows = torch.tensor([4, 0, 4], dtype=torch.int32, device=DEV)
+    picked = torch.empty(3, H, dtype=odtype, device=DEV)
+    ops.rmsnorm(x.to(DEV), w.to(DEV), 1e-6, picked, rows)
+    assert torch.equal(picked.cpu(), out.cpu()[[4, 0, 4]])
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 8, 16), (1, 128, 128), (4, 64, 32), (7, 100, 50), (65, 67, 33),
+                                   (130, 331, 144), (3, 96, 176)])
+@pytest.mark.parametrize("adt,wdt,odt", [(torch.float32,) * 3, (torch.bfloat16,) * 3,
+                                         (torch.bfloat16, torch.bfloat16, torch.float32),
+                                         (torch.bfloat16, torch.float32, torch.float32)])
+def test_gemm_generic(ops, M, N, K, adt, wdt, odt):
+    a = torch.randn(M, K, generator=_gen(3)).to(adt)
+    w = torch.randn(N, K, generator=_gen(4)).to(wdt)
+    out = torch.full((M, N), 7.0, dtype=odt, device=DEV)
+    ops.gemm_generic(a.to(DEV), w.to(DEV), out)
+    ref = plain_linear(a.double(), w.double())
+    tol = 2e-6 if odt == torch.float32 else 8e-3
+    assert _rel(out.cpu().double(), ref) < tol
+    # accumulate adds into what is there
+    base = torch.randn(M, N, generator=_gen(5)).to(odt)
+    out2 = base.clone().to(DEV)
+    ops.gemm_generic(a.to(DEV), w.to(DEV), out2, accumulate=True)
+    assert _rel(out2.cpu().double(), ref + base.double()) < (4e-6 if odt == torch.float32 else 1.6e-2)
+
+
+@pytest.mark.parametrize("FF,group", [(176, 16), (50, 50), (384, 16)])
+def test_swiglu(ops, FF, group):
+    T = 3
+    g = 3 * torch.randn(T, FF, generator=_gen(6))
+    u = torch.randn(T, FF, generator=_gen(7))
+    gu = torch.empty(T, 2 * FF)
+    gu.view(T, FF // group, 2, group)[:, :, 0] = g.view(T, FF // group, group)
+    gu.view(T, FF // group, 2, group)[:, :, 1] = u.view(T, FF // group, group)
+    out = torch.empty(T, FF, dtype=torch.float32, device=DEV)
+    ops.swiglu(gu.to(DEV), out, group)
+    ref = plain_silu(g.double()) * u.double()
+    assert (out.cpu().double() - ref).abs().max() < 1e-5
+    z = torch.zeros(1, 2 * FF)
+    z.view(1, FF // group, 2, group)[:, :, 1] = 5.0
+    outz = torch.empty(1, FF, dtype=torch.float32, device=DEV)
+    ops.swiglu(z.to(DEV), outz, group)
+    assert torch.all(outz == 0)                      # gate 0 gives 0 whatever up is
+
+
+def _paged_setup(ops, lens, n_q, n_kv, hd, page, dtype, seed, rotate=True, scramble=True):
+    """Random q/k/v for requests of the given lengths, written through rope_kv_write into
+    scrambled pages. Returns everything attention needs plus the plain per-request q, k, v."""
+    T = sum(lens)
+    g = _gen(seed)
+    qkv = torch.randn(T, (n_q + 2 * n_kv) * hd, generator=g)
+    max_pos = max(lens) + 3
+    half = hd // 2
+    inv = 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float64) * 2 / hd))
+    ang = torch.arange(max_pos, dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = torch.cos(ang).float(), torch.sin(ang).float()
+    nblk = [(n + page - 1) // page for n in lens]
+    total_pages = sum(nblk) + 2
+    perm = torch.randperm(total_pages, generator=g).tolist() if scramble else list(range(total_pages))
+    max_blocks = max(nblk)
+    table = torch.zeros(len(lens), max_blocks, dtype=torch.int32)
+    p = 0
+    for s, nb in enumerate(nblk):
+        for b in range(nb):
+            table[s, b] = perm[p]
+            p += 1
+    positions = torch.cat([torch.arange(n) for n in lens]).to(torch.int32)
+    seq_idx = torch.cat([torch.full((n,), s) for s, n in enumerate(lens)]).to(torch.int32)
+    k_cache = torch.zeros(total_pages, n_kv, page, hd, dtype=dtype, device=DEV)
+    v_cache = torch.zeros(total_pages, n_kv, hd, page, dtype=dtype, device=DEV)
+    q_out = torch.empty(T, n_q * hd, dtype=dtype, device=DEV)
+    ops.rope_kv_write(qkv.to(DEV), cos.to(DEV) if rotate else None, sin.to(DEV) if rotate else None,
+                      positions.to(DEV), seq_idx.to(DEV), table.to(DEV), q_out, k_cache, v_cache,
+                      n_q, n_kv, hd, hd)
+    # plain side
+    plain = []
+    row = 0
+    for n in lens:
+        blk = qkv[row:row + n].double()
+        q = blk[:, :n_q * hd].reshape(n, n_q, hd)
+        k = blk[:, n_q * hd:(n_q + n_kv) * hd].reshape(n, n_kv, hd)
+        v = blk[:, (n_q + n_kv) * hd:].reshape(n, n_kv, hd)
+        if rotate:
+            c = torch.cat([cos[:n], cos[:n]], dim=1).double()
+            s_ = torch.cat([sin[:n], sin[:n]], dim=1).double()
+            q, k = plain_apply_rope(q, c, s_), plain_apply_rope(k, c, s_)
+        if dtype == torch.bfloat16:
+            q, k, v = bf16_round(q), bf16_round(k), bf16_round(v)
+        plain.append((q, k, v))
+        row += n
+    return dict(q=q_out, k_cache=k_cache, v_cache=v_cache, positions=positions.to(DEV),
+                seq_idx=seq_idx.to(DEV), table=table.to(DEV), plain=plain, T=T, qkv=qkv)
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,page,lens", [
+    (4, 2, 32, 4, [1]), (4, 2, 32, 4, [7]), (8, 2, 16, 8, [13, 5]), (3, 1, 48, 16, [33, 2, 17]),
+    (6, 3, 80, 16, [70]), (4, 4, 128, 32, [65, 40]), (2, 1, 256, 16, [20])])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_write_and_attention_generic(ops, n_q, n_kv, hd, page, lens, dtype):
+    s = _paged_setup(ops, lens, n_q, n_kv, hd, page, dtype, seed=11)
+    # the rotated queries
+    q_ref = torch.cat([p[0].reshape(-1, n_q * hd) for p in s["plain"]])
+    assert _rel(s["q"].cpu().double(), q_ref) < (2e-6 if dtype == torch.float32 else 1e-9 + 4e-3)
+    out = torch.empty_like(s["q"])
+    ops.attention_generic(s["q"], s["k_cache"], s["v_cache"], out, s["positions"], s["seq_idx"], s["table"],
+                          n_q, n_kv, hd, 1.0 / math.sqrt(hd))
+    ref = torch.cat([plain_attention(q, k, v).reshape(-1, n_q * hd) for q, k, v in s["plain"]])
+    assert _rel(out.cpu().double(), ref) < (3e-6 if dtype == torch.float32 else 8e-3)
+
+
+def test_attention_generic_window_and_far_key(ops):
+    """A window's edge, and one far key that dominates: the key at position 3 gets a large
+    score for the last query; with a window that excludes it the result must change."""
+    n_q, n_kv, hd, page = 2, 1, 32, 8
+    lens = [300]
+    s = _paged_setup(ops, lens, n_q, n_kv, hd, page, torch.float32, seed=5, rotate=False)
+    q, k, v = s["plain"][0]
+    out = torch.empty_like(s["q"])
+    for window in (0, 64, 297, 298):
+        ops.attention_generic(s["q"], s["k_cache"], s["v_cache"], out, s["positions"], s["seq_idx"],
+                              s["table"], n_q, n_kv, hd, 1.0 / math.sqrt(hd), window)
+        ref = plain_attention(q, k, v, window).reshape(-1, n_q * hd)
+        assert _rel(out.cpu().double(), ref) < 3e-6, window
+
+
+def test_attention_single_key_is_value_row(ops):
+    s = _paged_setup(ops, [1], 4, 2, 32, 4, torch.float32, seed=3)
+    out = torch.empty_like(s["q"])
+    ops.attention_generic(s["q"], s["k_cache"], s["v_cache"], out, s["positions"], s["seq_idx"], s["table"],
+                          4, 2, 32, 0.5)
+    v = s["plain"][0][2]                                     # [1, n_kv, hd]
+    want = torch.stack([v[0, h // 2] for h in range(4)]).reshape(1, -1)
+    assert torch.allclose(out.cpu().double(), want, atol=1e-6)
+
+
+@pytest.mark.parametrize("V", [5, 256, 331, 128256])
+def test_argmax_first_maximum(ops, V):
+    logits = torch.randn(4, V, generator=_gen(9))
+    logits[1, V // 2] = logits[1, V - 1] = 50.0          # tie: the lower id wins
+    logits[2, 0] = 60.0
+    logits[3, V - 1] = 70.0
+    out = torch.empty(4, dtype=torch.int32, device=DEV)
+    ops.argmax(logits.to(DEV), out)
+    assert out.tolist() == [plain_argmax(r) for r in logits]
+    assert out.tolist()[1] == V // 2
+
+
+@pytest.mark.parametrize("V", [7, 300, 5000])
+def test_temperature_sampling_interval(ops, V):
+    R = 64
+    logits = 2 * torch.randn(R, V, generator=_gen(10))
+    u = torch.rand(R, generator=_gen(11))
+    temp = torch.full((R,), 0.8)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    ops.sample(logits.to(DEV), temp.to(DEV), u.to(DEV), out)
+    for r in range(R):
+        cum = plain_sample_bounds(logits[r], 0.8)
+        tok = out[r].item()
+        lo = cum[tok - 1].item() if tok > 0 else 0.0
+        assert lo - 1e-5 <= u[r].item() <= cum[tok].item() + 1e-5, (r, tok)
+    # temperature 0 is greedy
+    zero = torch.zeros(R)
+    ops.sample(logits.to(DEV), zero.to(DEV), u.to(DEV), out)
+    assert out.tolist() == logits.argmax(dim=1).tolist()
