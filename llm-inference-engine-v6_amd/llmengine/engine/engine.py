@@ -73,7 +73,7 @@ class BlockManager:
 
 class Engine:
     def __init__(self, model_dir: str | None, dtype: str = "fp32", *, device: str = "cuda:0",
-                 max_prefill_tokens_per_step: int = 8192, temperature: float = 0.0, seed: int = 0,
+                 max_prefill_tokens_per_step: int = 8192, temperature: float = 0.0, sampler_seed: int = 0,
                  block_size: int = 16, _config: dict | None = None, _tensors=None):
         self._dtype_name = {"float32": "fp32", "bfloat16": "bf16"}.get(dtype, dtype)
         self._torch_dtype = parse_dtype(dtype)
@@ -94,7 +94,7 @@ class Engine:
         self._device_name = device
         self._runner: ModelRunner | None = None
         self._lock = threading.RLock()
-        self.sampler = Sampler(temperature, seed)
+        self.sampler = Sampler(temperature, sampler_seed)
         self.block_size = int(block_size)
         self.prefill_chunk = int(max_prefill_tokens_per_step)
         self._own_cache: CacheContext | None = None

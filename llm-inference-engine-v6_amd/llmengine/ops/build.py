@@ -105,9 +105,9 @@ def built_library() -> str | None:
     return None
 
 
-def _compile_one(hipcc: str, src: str, obj: str, env: dict) -> tuple[str, float]:
+def _compile_one(hipcc: str, src: str, obj: str, env: dict, reuse: bool) -> tuple[str, float]:
     t0 = time.time()
-    if os.path.isfile(obj):          # same source, headers and flags: keep the object
+    if reuse and os.path.isfile(obj):          # same source, headers and flags: keep the object
         return src, 0.0
     cmd = [hipcc, *HIPCC_FLAGS, "-I", CSRC, "-c", src, "-o", obj]
     tmp = obj + f".{os.getpid()}.tmp"
@@ -119,8 +119,9 @@ def _compile_one(hipcc: str, src: str, obj: str, env: dict) -> tuple[str, float]
     return src, time.time() - t0
 
 
-def build(force: bool = True) -> str:
-    """Compiles every kernel source and links the library; returns its path."""
+def build(force: bool = True, reuse_objects: bool = False) -> str:
+    """Compiles every kernel source and links the library; returns its path.
+    reuse_objects keeps objects whose source, headers and flags have not changed."""
     if not force:
         lib = built_library()
         if lib:
@@ -144,7 +145,7 @@ def build(force: bool = True) -> str:
     t0 = last = time.time()
     done = 0
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        futures = [pool.submit(_compile_one, hipcc, s, o, env) for s, o in zip(srcs, objs)]
+        futures = [pool.submit(_compile_one, hipcc, s, o, env, reuse_objects) for s, o in zip(srcs, objs)]
         pending = set(futures)
         while pending:
             finished = {f for f in pending if f.done()}
@@ -180,8 +181,8 @@ def build(force: bool = True) -> str:
 
 def ensure_built() -> str:
     """The library for the current sources: the built one, or a fresh build."""
-    return built_library() or build(force=True)
+    return built_library() or build(force=True, reuse_objects=True)
 
 
 if __name__ == "__main__":
-    print(build(force=True))
+    print(ensure_built())

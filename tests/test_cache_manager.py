@@ -1,0 +1,151 @@
+"""The cache manager's bookkeeping (no GPU): pages are never lost, held twice or freed
+twice, under random orders of requests; window groups give pages back as the window passes;
+slots are unique; reservation is all-or-nothing."""
+import random
+
+import pytest
+
+from llmengine.cache import CacheError, CacheManager, GroupSpec, PagePool
+
+
+def test_pool_fifo_and_double_free():
+    pool = PagePool(3)
+    a, b, c = pool.allocate(), pool.allocate(), pool.allocate()
+    assert (a, b, c) == (0, 1, 2) and pool.allocate() is None and pool.free_pages == 0
+    pool.free(b)
+    pool.free(a)
+    assert pool.allocate() == b and pool.allocate() == a          # first freed, first reused
+    with pytest.raises(CacheError):
+        pool.free(7)
+    pool.free(c)
+    with pytest.raises(CacheError):
+        pool.free(c)                                               # freed twice
+
+
+def test_pages_follow_token_counts():
+    m = CacheManager([GroupSpec("full", "full", 0, 8)], page_size=4, max_requests=2)
+    m.admit("a")
+    assert m.pages_needed("a", 9) == {"full": 3}                   # 9 tokens at 4 a page: 3 pages
+    assert m.reserve("a", 9)
+    m.commit("a", 9)
+    assert m.free_pages() == 5 and len(m.block_table("a", "full")) == 3
+    assert m.pages_needed("a", 3) == {"full": 0}                   # tokens 9..11 fit the third page
+    assert m.pages_needed("a", 4) == {"full": 1}
+    m.release("a")
+    assert m.free_pages() == 8
+    m.check()
+
+
+def test_reservation_is_all_or_nothing():
+    m = CacheManager([GroupSpec("full", "full", 0, 1)], page_size=4, max_requests=2)
+    m.admit("a")
+    assert not m.reserve("a", 6)                                   # needs 2 pages, 1 is there
+    assert m.free_pages() == 1 and m.block_table("a", "full") == []
+    assert m.reserve("a", 4)
+    m.commit("a", 4)
+    assert not m.can_reserve("a", 1)                               # position 4 needs a second page
+    with pytest.raises(CacheError):
+        m.commit("a", 1)                                           # nothing was reserved for it
+    m.release("a")
+    assert m.free_pages() == 1
+
+
+def test_pending_counts_against_free_pages():
+    m = CacheManager([GroupSpec("full", "full", 0, 3)], page_size=4, max_requests=4)
+    m.admit("a")
+    m.admit("b")
+    assert m.can_reserve("a", 8) and m.can_reserve("b", 8)
+    assert not m.can_reserve("b", 8, pending={"full": 2})
+
+
+def test_window_group_gives_pages_back():
+    m = CacheManager([GroupSpec("full", "full", 0, 64), GroupSpec("win", "window", 6, 64)],
+                     page_size=4, max_requests=1)
+    m.admit("r")
+    assert m.reserve("r", 10)
+    m.commit("r", 10)                      # next token at 10 reads keys 5..10: block 0 (keys 0..3) is behind
+    assert m.block_table("r", "win")[0] == -1 and m.block_table("r", "win")[1] >= 0
+    assert m.block_table("r", "full")[0] >= 0
+    for _ in range(30):
+        assert m.reserve("r", 1)
+        m.commit("r", 1)
+        m.check()
+    live = [p for p in m.block_table("r", "win") if p >= 0]
+    assert len(live) <= 3                                          # a 6-token window spans at most 3 pages of 4
+    assert len([p for p in m.block_table("r", "full") if p >= 0]) == 10
+    # a long portion needs pages for all its own tokens, but none behind the window of its first
+    assert m.pages_needed("r", 9)["win"] == len(range(40 // 4, (40 + 9 - 1) // 4 + 1)) - 0
+    m.release("r")
+    assert m.free_pages("win") == 64 and m.free_pages("full") == 64
+
+
+def test_slots():
+    m = CacheManager([GroupSpec("full", "full", 0, 4)], page_size=4, max_requests=2)
+    s0, s1 = m.admit("a"), m.admit("b")
+    assert {s0, s1} == {0, 1}
+    with pytest.raises(CacheError):
+        m.admit("c")
+    with pytest.raises(CacheError):
+        m.admit("a")
+    m.release("a")
+    assert m.admit("c") == s0
+    with pytest.raises(CacheError):
+        m.release("a")
+    with pytest.raises(CacheError):
+        m.length("zzz")
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_orders_keep_the_invariants(seed):
+    rng = random.Random(seed)
+    groups = [GroupSpec("full", "full", 0, 40)]
+    if seed % 2:
+        groups.append(GroupSpec("win", "window", rng.choice([3, 8, 17]), 25))
+    m = CacheManager(groups, page_size=rng.choice([1, 4, 16]), max_requests=5)
+    live: dict[int, int] = {}
+    next_id = 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.25 and m.free_slots():
+            m.admit(next_id)
+            live[next_id] = 0
+            next_id += 1
+        elif op < 0.85 and live:
+            rid = rng.choice(list(live))
+            n = rng.choice([1, 1, 1, 2, 5, 9, 33])
+            before = {g: m.free_pages(g) for g in m.groups}
+            tables = {g: list(m.block_table(rid, g)) for g in m.groups}
+            if m.reserve(rid, n):
+                assert m.can_reserve(rid, n)                      # now nothing more is needed
+                m.commit(rid, n)
+                live[rid] += n
+                assert m.length(rid) == live[rid]
+            else:
+                assert before == {g: m.free_pages(g) for g in m.groups}     # a refusal changes nothing
+                assert tables == {g: list(m.block_table(rid, g)) for g in m.groups}
+        elif live:
+            rid = rng.choice(list(live))
+            m.release(rid)
+            del live[rid]
+        m.check()
+        for rid, n in live.items():                               # every readable key has a page
+            for g in m.groups.values():
+                table = m.block_table(rid, g.name)
+                lo = max(0, n - g.window + 1) if g.kind == "window" else 0   # the next token at n reads keys > n - window
+                for pos in range(lo, n):
+                    assert table[pos // m.page_size] >= 0
+    for rid in list(live):
+        m.release(rid)
+    m.check()
+    assert all(m.free_pages(g) == m.num_pages(g) for g in m.groups)
+
+
+def test_bad_arguments():
+    with pytest.raises(ValueError):
+        CacheManager([GroupSpec("g", "full", 0, 4)], page_size=0, max_requests=1)
+    with pytest.raises(ValueError):
+        CacheManager([GroupSpec("g", "window", 0, 4)], page_size=4, max_requests=1)
+    with pytest.raises(ValueError):
+        CacheManager([GroupSpec("g", "full", 0, 4), GroupSpec("g", "full", 0, 4)], page_size=4, max_requests=1)
+    with pytest.raises(ValueError):
+        PagePool(0)

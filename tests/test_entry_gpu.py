@@ -1,0 +1,254 @@
+"""Generation through the entry points on the GPU: `Engine.generate`, the scheduler with
+greedy and temperature sampling, the command line and bin/trace_run, compared with the plain
+implementation; input validation; the tied head; calls from several threads."""
+import json
+import os
+import subprocess
+import sys
+import threading
+
+import numpy as np
+import pytest
+import torch
+
+import replay
+from plain_llama import (bf16_round, load_plain_model, plain_forward, plain_generate, plain_sample_bounds)
+from tiny_models import A_INIT, B_INIT, TINY_A, TINY_B, make_model_dir, random_tokens
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def dir_a(tmp_path_factory):
+    return make_model_dir(tmp_path_factory.mktemp("A"), TINY_A, A_INIT, torch.bfloat16)
+
+
+@pytest.fixture(scope="module")
+def dir_b(tmp_path_factory):
+    return make_model_dir(tmp_path_factory.mktemp("B"), TINY_B, B_INIT, torch.bfloat16)
+
+
+def test_greedy_generate_equals_plain(dir_a):
+    """Tiny A: prompts of 5, 11 and 17 tokens, 8 greedy tokens each, 32-bit: token for token."""
+    from llmengine import Engine
+    cfg, w = load_plain_model(dir_a)
+    engine = Engine(dir_a, "fp32", block_size=4)
+    for i, n in enumerate((5, 11, 17)):
+        prompt = random_tokens(n, 256, 40 + i)
+        assert engine.generate(prompt, 8) == plain_generate(cfg, w, prompt, 8)
+    assert engine.generate([1, 2, 3], 0) == ([1, 2, 3], "length")
+    assert engine.dtype == "fp32" and engine.max_pos == 128 and engine.cfg.hidden_size == 64
+
+
+def test_bf16_generate_is_greedy_under_its_own_rounding(dir_b):
+    """In bfloat16 a near-tie may fall the other way; every chosen token must still be a
+    maximum of the plain logits up to the bfloat16 tolerance."""
+    from llmengine import Engine
+    cfg, w = load_plain_model(dir_b)
+    engine = Engine(dir_b, "bf16", block_size=8)
+    prompt = random_tokens(9, 384, 3)
+    ids, finish = engine.generate(prompt, 12)
+    assert finish == "length" and len(ids) == 21 and ids[:9] == prompt
+    ref = plain_forward(cfg, w, ids, rounder=bf16_round)
+    for i in range(9, 21):
+        row = ref[i - 1]
+        assert row[ids[i]] >= row.max() - 2e-2 * row.abs().max(), i
+
+
+def test_eos_and_limits(tmp_path, dir_a):
+    from llmengine import Engine
+    cfg, w = load_plain_model(dir_a)
+    prompt = [9, 8, 7, 6]
+    stream, _ = plain_generate(cfg, w, prompt, 6)
+    eos = stream[6]                                              # the third generated token
+    d = str(tmp_path / "eos")
+    os.makedirs(d)
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(dict(TINY_A, eos_token_id=[eos, 255]), f)
+    os.symlink(os.path.join(dir_a, "model.safetensors"), os.path.join(d, "model.safetensors"))
+    engine = Engine(d, "fp32")
+    ids, finish = engine.generate(prompt, 6)
+    assert finish == "stop" and ids == stream[:4 + stream[4:].index(eos)]      # EOS is not appended
+    with pytest.raises(ValueError):
+        engine.generate([], 3)
+    with pytest.raises(ValueError):
+        engine.generate([1], -1)
+    with pytest.raises(ValueError):
+        engine.generate([256], 1)
+    with pytest.raises(ValueError):
+        engine.generate([-1], 1)
+    with pytest.raises(RuntimeError, match="max_pos"):
+        engine.generate([1] * 100, 29)
+    with pytest.raises(RuntimeError, match="max_pos"):
+        engine.generate([1], 2 ** 31 - 1)
+    assert len(engine.generate([1] * 100, 28)[0]) == 128        # exactly max_pos fits
+
+
+def test_requests_are_checked_before_weights(tmp_path):
+    """A checkpoint that lacks a tensor: bad requests are still refused as bad requests, and a good
+    request gets the loader's error with the tensor's name (tests/test_input_validation.py:104-136)."""
+    from llmengine import Engine, WeightError
+    from llmengine.weights import random_state, write_state_dict
+    w = dict(random_state(TINY_A, 0, torch.bfloat16))
+    del w["model.layers.1.mlp.down_proj.weight"]
+    d = str(tmp_path)
+    write_state_dict(os.path.join(d, "model.safetensors"), w)
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(TINY_A, f)
+    engine = Engine(d, "fp32")
+    assert engine.has_weight("lm_head.weight") and not engine.has_weight("model.layers.1.mlp.down_proj.weight")
+    with pytest.raises(ValueError):
+        engine.generate([999], 1)
+    with pytest.raises(WeightError, match="missing weight: model.layers.1.mlp.down_proj.weight"):
+        engine.generate([1], 1)
+
+
+def test_tied_head_shares_the_embedding_on_the_device(dir_a, dir_b):
+    from llmengine import Engine
+    a, b = Engine(dir_a, "bf16"), Engine(dir_b, "bf16")
+    assert a.model.head.weight.data_ptr() == a.model.embedding.weight.data_ptr()
+    assert b.model.head.weight.data_ptr() != b.model.embedding.weight.data_ptr()
+    assert a.model.embedding.weight.dtype == torch.bfloat16 and a.model.embedding.weight.is_cuda
+
+
+def _check_sampled(cfg, w, result, temperature, seed, tol):
+    """Teacher-forced check of a sampled stream: every token's cumulative-probability interval
+    under the plain logits contains the request's draw (within tol)."""
+    from llmengine.sampling import uniform_draw
+    ref = plain_forward(cfg, w, result.token_ids)
+    for i in range(result.prompt_len, len(result.token_ids)):
+        tok = result.token_ids[i]
+        u = uniform_draw(seed, result.seq_id, i - result.prompt_len)
+        cum = plain_sample_bounds(ref[i - 1], temperature)
+        lo = cum[tok - 1].item() if tok > 0 else 0.0
+        assert lo - tol <= u <= cum[tok].item() + tol, (result.seq_id, i, tok, u, lo, cum[tok].item())
+
+
+def test_scheduler_temperature_workload(dir_b):
+    """Tiny B's workload: prompts of 1, 9, 33 and 70 tokens, a 16-token prefill budget, 12 tokens
+    each at temperature 0.8 with sampler seed 7, pages of 8."""
+    from llmengine import BlockManager, ContinuousBatchScheduler, Engine
+    cfg, w = load_plain_model(dir_b)
+    engine = Engine(dir_b, "fp32")
+    blocks = BlockManager(40, 8, 3, 1, 32)
+    sched = ContinuousBatchScheduler(engine, blocks, max_concurrent=4, max_prefill_tokens_per_step=16,
+                                     temperature=0.8, seed=7)
+    prompts = [random_tokens(n, 384, 60 + n) for n in (1, 9, 33, 70)]
+    for p in prompts:
+        sched.enqueue(p, 12)
+    sched.run_until_idle()
+    assert blocks.free_blocks == 40
+    for r, p in zip(sched.results, prompts):
+        assert r.finish_reason == "length" and len(r.token_ids) == len(p) + 12 and r.token_ids[:len(p)] == p
+        _check_sampled(cfg, w, r, 0.8, 7, 1e-4)
+    # the same requests alone, in another order and batch: the same tokens (draws belong to requests)
+    again = ContinuousBatchScheduler(engine, BlockManager(40, 8), max_concurrent=1,
+                                     max_prefill_tokens_per_step=200, temperature=0.8, seed=7)
+    for p in prompts:
+        again.enqueue(p, 12)
+    again.run_until_idle()
+    assert [r.token_ids for r in again.results] == [r.token_ids for r in sched.results]
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_scheduler_greedy_equals_generate(dir_a, dtype):
+    from llmengine import BlockManager, ContinuousBatchScheduler, Engine
+    engine = Engine(dir_a, dtype, block_size=4)
+    prompts = [[1], [2, 3, 4], list(range(5, 12)), [12, 13]] + [random_tokens(n, 256, n) for n in (20, 31)]
+    alone = [engine.generate(p, 12) for p in prompts]
+    blocks = BlockManager(64, 4, 2, 2, 16)
+    sched = ContinuousBatchScheduler(engine, blocks, max_concurrent=3, max_prefill_tokens_per_step=6)
+    for p in prompts:
+        sched.enqueue(p, 12)
+    sched.run_until_idle()
+    if dtype == "fp32":
+        assert [(r.token_ids, r.finish_reason) for r in sched.results] == alone
+    else:
+        assert sum(r.token_ids == a[0] for r, a in zip(sched.results, alone)) >= len(prompts) - 1
+    assert blocks.free_blocks == 64 and [r.seq_id for r in sched.results] == list(range(len(prompts)))
+
+
+def test_scheduler_capacity_on_the_gpu(dir_a):
+    from llmengine import BlockManager, ContinuousBatchScheduler, Engine
+    engine = Engine(dir_a, "fp32")
+    blocks = BlockManager(4, 4)
+    sched = ContinuousBatchScheduler(engine, blocks, max_concurrent=2, max_prefill_tokens_per_step=4)
+    prompts = [[1, 2, 3, 4], [5, 6, 7, 8]]
+    for p in prompts:
+        sched.enqueue(p, 12)
+    sched.run_until_idle()
+    assert "capacity" in [r.finish_reason for r in sched.results]
+    for r, p in zip(sched.results, prompts):
+        full, _ = engine.generate(p, 12)
+        assert r.token_ids == full[:len(r.token_ids)]
+    assert blocks.free_blocks == 4
+
+
+def test_threads_get_the_serial_answers(dir_a):
+    from llmengine import Engine
+    engine = Engine(dir_a, "fp32")
+    prompts = [random_tokens(6 + i, 256, 900 + i) for i in range(6)]
+    serial = [engine.generate(p, 6) for p in prompts]
+    got = [None] * len(prompts)
+
+    def work(i):
+        got[i] = engine.generate(prompts[i], 6)
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(prompts))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert got == serial
+
+
+def test_command_line(dir_a, tmp_path):
+    from llmengine import Engine
+    prompt = [5, 17, 3, 99]
+    want = Engine(dir_a, "fp32").generate(prompt, 5)
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "llmengine-cli"), "--model", dir_a,
+                          "--dtype", "fp32", "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "5"],
+                         capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    rec = json.loads(out.stdout.strip().splitlines()[-1])
+    assert (rec["token_ids"], rec["finish_reason"]) == want
+    pf = tmp_path / "prompts.txt"
+    pf.write_text("1 2 3\n7,8,9,10,11\n")
+    cfgf = tmp_path / "cfg.json"
+    cfgf.write_text(json.dumps(TINY_A))
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "llmengine-cli"), "--random", str(cfgf),
+                          "--seed", "3", "--prompt-file", str(pf), "--max-new-tokens", "4", "--temperature", "0.7",
+                          "--block-size", "4"], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    recs = [json.loads(line) for line in out.stdout.strip().splitlines()]
+    assert [len(r["token_ids"]) for r in recs] == [7, 9] and all(r["finish_reason"] == "length" for r in recs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(dir_b, tmp_path, dtype):
+    """bin/trace_run as a user calls it: a mixed trace over so few pages that they are used again."""
+    reqs = {f"q{i}": random_tokens(n, 384, 300 + i) for i, n in enumerate((70, 40, 3, 55, 64, 18))}
+    steps = replay.mixed(reqs, max_live=4, seed=2)
+    peak = replay.trace_peak_tokens(steps, 64)
+    out_dir = tmp_path / "out"
+    text = "\n".join(json.dumps(s) for s in steps) + "\n"
+    p = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", dir_b, "--dtype", dtype, "--out",
+                        str(out_dir), "--max-tokens", str(peak)], input=text, capture_output=True, text=True,
+                       timeout=600)
+    assert p.returncode == 0, p.stderr[-3000:]
+    assert p.stdout.split() == [w for s in steps for w in ("done", str(s["step"]))]
+    cfg, w = load_plain_model(dir_b)
+    plain = {rid: plain_forward(cfg, w, ids, rounder=bf16_round if dtype == "bfloat16" else None).numpy()
+             for rid, ids in reqs.items()}
+    tol = 1e-5 if dtype == "float32" else 2e-2
+    pos = {rid: 0 for rid in reqs}
+    for s in steps:
+        want_rows = sum(len(e["want"]) for e in s["entries"])
+        rows = np.fromfile(out_dir / f"{s['step']}.f32", dtype="<f4").reshape(want_rows, 384)
+        r = 0
+        for e in s["entries"]:
+            for wnt in e["want"]:
+                ref = plain[e["id"]][pos[e["id"]] + wnt]
+                assert np.abs(rows[r] - ref).max() / np.abs(ref).max() < tol, (s["step"], e["id"], wnt)
+                r += 1
+            pos[e["id"]] += len(e["tokens"])

@@ -1,0 +1,184 @@
+"""The scheduler's decisions (no GPU), against a stand-in engine whose next token is a
+function of the whole history that was fed to it: any token fed twice, skipped, or out of
+order changes the stream. Cases follow the reference's tests/test_scheduler.py."""
+import pytest
+
+from llmengine.cache import CacheManager, GroupSpec
+from llmengine.engine.scheduler import ContinuousBatchScheduler
+
+V = 97
+
+
+def next_token(history):
+    return (sum((i + 1) * t for i, t in enumerate(history)) * 31 + len(history)) % V
+
+
+def single_generate(prompt, max_new, eos=()):
+    ids, finish = list(prompt), "length"
+    for _ in range(max_new):
+        t = next_token(ids)
+        if t in eos:
+            finish = "stop"
+            break
+        ids.append(t)
+    return ids, finish
+
+
+class FakeCache:
+    def __init__(self, pages, page_size, max_requests):
+        self.manager = CacheManager([GroupSpec("full", "full", 0, pages)], page_size, max_requests)
+
+    def admit(self, rid):
+        return self.manager.admit(rid)
+
+    def release(self, rid):
+        self.manager.release(rid)
+
+
+class FakeBlocks:
+    def __init__(self, num_blocks, block_size):
+        self.num_blocks, self.block_size = num_blocks, block_size
+        self.cache = None
+
+    @property
+    def free_blocks(self):
+        return self.cache.manager.free_pages() if self.cache else self.num_blocks
+
+
+class FakeEngine:
+    def __init__(self, eos=(), max_pos=512):
+        self.vocab_size, self.max_pos, self.eos_token_ids = V, max_pos, tuple(eos)
+        self.history = {}
+        self.batches = []           # per step: list of (request, n tokens)
+
+    def open_cache(self, blocks, max_requests):
+        blocks.cache = FakeCache(blocks.num_blocks, blocks.block_size, max_requests)
+        return blocks.cache
+
+    def run_step(self, cache, entries, draws, temperature, seed):
+        out = []
+        self.batches.append([(e.request_id, len(e.tokens)) for e in entries])
+        for e in entries:
+            assert cache.manager.reserve(e.request_id, len(e.tokens)), "the scheduler promised pages"
+            h = self.history.setdefault(e.request_id, [])
+            assert cache.manager.length(e.request_id) == len(h)
+            for i, t in enumerate(e.tokens):
+                h.append(t)
+                if i in e.want:
+                    out.append(next_token(h))
+            cache.manager.commit(e.request_id, len(e.tokens))
+        assert len(draws) == len(out)
+        return out
+
+
+def run(prompts, max_new, blocks=(64, 4), **kw):
+    eng = FakeEngine(eos=kw.pop("eos", ()))
+    bm = FakeBlocks(*blocks)
+    s = ContinuousBatchScheduler(eng, bm, **kw)
+    for p, n in zip(prompts, max_new if isinstance(max_new, list) else [max_new] * len(prompts)):
+        s.enqueue(p, n)
+    s.run_until_idle()
+    return s, eng, bm
+
+
+def test_streams_equal_single_sequence():
+    prompts = [[1], [2, 3, 4], [5, 6, 7, 8, 9, 10, 11], [12, 13]]       # tests/test_scheduler.py:97-124
+    s, eng, bm = run(prompts, 12)
+    for r, p in zip(s.results, prompts):
+        assert (r.token_ids, r.finish_reason) == single_generate(p, 12)
+        assert r.prompt_len == len(p)
+    assert bm.free_blocks == bm.num_blocks and s.idle
+    assert [r.seq_id for r in s.results] == [0, 1, 2, 3]
+
+
+def test_one_mixed_batch_per_step():
+    s, eng, _ = run([[1, 2, 3], list(range(20, 50))], 6, max_prefill_tokens_per_step=8)
+    mixed = [b for b in eng.batches if any(n > 1 for _, n in b) and any(n == 1 and rid == 0 for rid, n in b)]
+    assert mixed, "a prompt portion and a decoded token never shared a step"
+    for b in eng.batches:
+        assert sum(n for rid, n in b if not (n == 1 and len(eng.history[rid]) > 3 and rid == 0)) <= 8 + 1
+    for r, p in zip(s.results, [[1, 2, 3], list(range(20, 50))]):
+        assert (r.token_ids, r.finish_reason) == single_generate(p, 6)
+
+
+def test_budget_is_shared_in_admission_order_and_excludes_decoding():
+    prompts = [list(range(1, 6)), list(range(1, 4)), list(range(1, 10))]
+    s, eng, _ = run(prompts, 3, max_prefill_tokens_per_step=7)
+    assert eng.batches[0] == [(0, 5), (1, 2)]                    # first takes what it needs, next the rest
+    assert eng.batches[1][:2] == [(1, 1), (2, 6)]                # then decoding tokens ride along, uncounted
+    assert (0, 1) in eng.batches[1]
+    for b in eng.batches:
+        decoding = sum(1 for rid, n in b if n == 1 and len(eng.history[rid]) > len(prompts[rid]))
+        assert sum(n for _, n in b) - decoding <= 7
+
+
+@pytest.mark.parametrize("max_new", [0, 1, 2, 5])               # tests/test_scheduler.py:220-280
+def test_exact_counts(max_new):
+    s, _, bm = run([[4, 5, 6]], max_new)
+    r = s.results[0]
+    assert len(r.token_ids) == 3 + max_new and r.finish_reason == "length"
+    assert bm.free_blocks == bm.num_blocks
+
+
+def test_small_budget_long_prompt():
+    s, eng, _ = run([list(range(1, 21))], 4, max_prefill_tokens_per_step=2)   # tests/test_scheduler.py:312-331
+    r = s.results[0]
+    assert len(r.token_ids) == 24 and r.finish_reason == "length"
+    assert [n for b in eng.batches[:10] for _, n in b] == [2] * 10
+
+
+def test_eos_stops_and_is_not_appended():
+    prompt = [3, 1, 4]
+    stream, _ = single_generate(prompt, 8)
+    eos = stream[5]                                               # the third generated token
+    s, _, _ = run([prompt], 8, eos=(eos,))
+    r = s.results[0]
+    first = stream[3:].index(eos)
+    assert r.finish_reason == "stop" and r.token_ids == stream[:3 + first]
+
+
+def test_capacity_termination():
+    # 4 pages of 4 tokens, two requests of 4 + 12 tokens: tests/test_scheduler.py:285-307
+    s, eng, bm = run([[1, 2, 3, 4], [5, 6, 7, 8]], 12, blocks=(4, 4), max_concurrent=2,
+                     max_prefill_tokens_per_step=4)
+    reasons = [r.finish_reason for r in s.results]
+    assert "capacity" in reasons
+    for r, p in zip(s.results, [[1, 2, 3, 4], [5, 6, 7, 8]]):
+        full, _ = single_generate(p, 12)
+        assert r.token_ids == full[:len(r.token_ids)]            # what was generated is kept and right
+        assert len(r.token_ids) >= 4
+    assert bm.free_blocks == 4
+    # a prompt that can never fit ends with capacity and the queue goes on
+    s2, _, bm2 = run([list(range(1, 30)), [1, 2]], 2, blocks=(2, 4))
+    assert [r.finish_reason for r in s2.results] == ["capacity", "length"]
+    assert s2.results[0].token_ids == list(range(1, 30)) and bm2.free_blocks == 2
+
+
+def test_freed_pages_serve_waiting_requests():
+    prompts = [[i + 1] * 6 for i in range(6)]
+    s, _, bm = run(prompts, 5, blocks=(6, 4), max_concurrent=2)
+    assert [r.finish_reason for r in s.results] == ["length"] * 6
+    for r, p in zip(s.results, prompts):
+        assert r.token_ids == single_generate(p, 5)[0]
+    assert bm.free_blocks == 6
+
+
+def test_invalid_knobs_and_requests():
+    eng, bm = FakeEngine(max_pos=16), FakeBlocks(8, 4)
+    for kw in ({"max_concurrent": 0}, {"max_prefill_tokens_per_step": 0}, {"temperature": -1.0}):
+        with pytest.raises(ValueError):
+            ContinuousBatchScheduler(eng, bm, **kw)
+    s = ContinuousBatchScheduler(eng, bm)
+    with pytest.raises(ValueError):
+        s.budget = 0
+    s.budget = 3
+    assert s.budget == 3
+    for prompt, n in (([], 1), ([1], -1), ([V], 1), ([-1], 1), ([1] * 10, 7)):
+        with pytest.raises(ValueError):
+            s.enqueue(prompt, n)
+    assert s.idle and not s.step()
+    s.enqueue([1] * 10, 6)                                        # exactly max_pos is allowed
+    s.run_until_idle()
+    assert len(s.results[0].token_ids) == 16
+    s.clear_results()
+    assert s.results == []
