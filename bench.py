@@ -1,0 +1,194 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers L]
+
+The model has the layer sizes of Llama 3.2 1B (16 layers, width 2048, 32 query / 8 key-value
+heads of 64, feed-forward 8192, vocabulary 128256, llama3 rope scaling, tied head) with seeded
+random bfloat16 weights; token ids are seeded uniform random numbers. A "step" is one decode
+step of the whole batch: the model over one token per request from the paged cache, the choice
+of the next token (greedy) and its way back to the host. Every request holds `context - steps -
+warmup` tokens when decoding starts, put there by real prefill steps, so that the timed steps
+run at the configured context length. One JSON line goes to stdout.
+
+Beside the headline value the line holds: `prefill` (one 2,048-token prompt, logits at its last
+place), `roofline` (bytes the decode step has to read: every weight once plus the live
+requests' cache, over its time, against 8 TB/s), `points` (decode at batch 1 and 64).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "llm-inference-engine-v6_amd"))
+
+HBM_PEAK = 8.0e12            # bytes/s
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+LLAMA_1B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 2048, "intermediate_size": 8192, "num_hidden_layers": 16,
+    "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 64,
+    "vocab_size": 128256, "max_position_embeddings": 131072, "rms_norm_eps": 1e-5,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0,
+                     "high_freq_factor": 4.0, "original_max_position_embeddings": 8192},
+    "tie_word_embeddings": True,
+}
+FULL_LAYERS = 16
+
+
+def log(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def layer_weight_elements(c: dict) -> int:
+    H, FF = c["hidden_size"], c["intermediate_size"]
+    q, kv = c["num_attention_heads"] * c["head_dim"], c["num_key_value_heads"] * c["head_dim"]
+    return (q + 2 * kv) * H + H * q + 2 * FF * H + H * FF + 2 * H
+
+
+def decode_bytes(c: dict, batch: int, ctx: float, wbytes: int) -> float:
+    """Bytes a decode step has to read: every weight once, and the cache of the live requests."""
+    weights = (c["num_hidden_layers"] * layer_weight_elements(c) + c["vocab_size"] * c["hidden_size"]
+               + c["hidden_size"]) * wbytes
+    kv = batch * ctx * 2 * c["num_key_value_heads"] * c["head_dim"] * wbytes * c["num_hidden_layers"]
+    return weights + kv
+
+
+def prefill_flops(c: dict, T: int) -> float:
+    """Flops of one T-token prompt from an empty cache, logits at the last place only."""
+    L, H = c["num_hidden_layers"], c["hidden_size"]
+    q = c["num_attention_heads"] * c["head_dim"]
+    gemm = 2.0 * T * L * (layer_weight_elements(c) - 2 * H)
+    attn = L * 2.0 * 2.0 * q * (T * (T + 1) / 2)            # QK^T and PV over the causal half
+    head = 2.0 * c["vocab_size"] * H
+    return gemm + attn + head
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096, help="context length the decode steps run at")
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from llmengine import Engine, StepEntry
+
+    cfg = dict(LLAMA_1B, num_hidden_layers=args.layers)
+    wbytes = 2 if args.dtype == "bf16" else 4
+    t0 = time.time()
+    log(f"building the model ({args.layers} layers, {args.dtype}) with random weights")
+    engine = Engine.from_random(cfg, args.seed, args.dtype, std=0.02)
+    runner = engine.runner
+    log(f"model on the device after {time.time() - t0:.1f} s")
+    gen = torch.Generator().manual_seed(args.seed + 1)
+    V = cfg["vocab_size"]
+    page = 16
+
+    def sync():
+        torch.cuda.synchronize()
+
+    # ---- prefill: one prompt, logits at its last place ----
+    T = args.prefill_tokens
+    prompt = torch.randint(0, V, (T,), generator=gen).tolist()
+    cache = engine.new_cache((T + page - 1) // page + 1, page, 1)
+    pre_ms = []
+    for rep in range(4):
+        cache.admit("p")
+        sync()
+        t = time.perf_counter()
+        engine.step(cache, [StepEntry("p", prompt, [T - 1])])
+        sync()
+        pre_ms.append((time.perf_counter() - t) * 1e3)
+        cache.release("p")
+    prefill_ms = min(pre_ms[1:])
+    flops = prefill_flops(cfg, T)
+    prefill = {"value": round(T / (prefill_ms / 1e3), 1), "tokens": T, "ms": round(prefill_ms, 3),
+               "frac": round(flops / (prefill_ms / 1e3) / PEAK_FLOPS[args.dtype], 4)}
+    log(f"prefill {T} tokens: {prefill_ms:.2f} ms ({prefill['value']:.0f} tok/s, {prefill['frac']:.3f} of peak)")
+    del cache
+
+    # ---- decode ----
+    def decode_run(batch: int, steps: int, warmup: int):
+        start_ctx = args.context - steps - warmup
+        if start_ctx < 1:
+            raise SystemExit("--context must exceed --steps + --warmup")
+        pages = batch * ((args.context + page - 1) // page)
+        cache = engine.new_cache(pages, page, batch)
+        ids = [f"r{i}" for i in range(batch)]
+        for rid in ids:
+            cache.admit(rid)
+        chunk = 4096
+        for rid in ids:                                        # real prefill fills the pages
+            toks = torch.randint(0, V, (start_ctx,), generator=gen).tolist()
+            for s in range(0, start_ctx, chunk):
+                engine.step(cache, [StepEntry(rid, toks[s:s + chunk], [])])
+        last = torch.randint(0, V, (batch,), generator=gen).tolist()
+
+        def one_step(tokens):
+            return engine.run_step(cache, [StepEntry(rid, [t], [0]) for rid, t in zip(ids, tokens)], None)
+        for _ in range(warmup):
+            last = one_step(last)
+        sync()
+        t = time.perf_counter()
+        for _ in range(steps):
+            last = one_step(last)
+        sync()
+        dt = time.perf_counter() - t
+        for rid in ids:
+            cache.release(rid)
+        mean_ctx = start_ctx + warmup + (steps + 1) / 2.0
+        return dt / steps, mean_ctx
+
+    log(f"decode: batch {args.batch}, context {args.context}")
+    step_s, mean_ctx = decode_run(args.batch, args.steps, args.warmup)
+    value = args.batch / step_s
+    nbytes = decode_bytes(cfg, args.batch, mean_ctx, wbytes)
+    roofline = {"bound": "hbm", "achieved": round(nbytes / step_s / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                "frac": round(nbytes / step_s / HBM_PEAK, 4)}
+    log(f"decode b{args.batch}: {step_s * 1e3:.3f} ms/step, {value:.0f} tok/s, {roofline['frac']:.3f} of HBM peak")
+    points = {}
+    for b in [int(x) for x in args.points.split(",") if x.strip()]:
+        s, c = decode_run(b, max(16, args.steps // 2), max(4, args.warmup // 2))
+        points[f"decode_b{b}"] = round(b / s, 1)
+        points[f"decode_b{b}_hbm_frac"] = round(decode_bytes(cfg, b, c, wbytes) / s / HBM_PEAK, 4)
+        log(f"decode b{b}: {s * 1e3:.3f} ms/step, {b / s:.0f} tok/s")
+
+    line = {
+        "metric": "decode_tokens_per_second", "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic (seeded random weights and token ids)",
+        "config": {
+            "model": "llama-3.2-1b-shape", "global_batch": args.batch, "seq_len": args.context,
+            "parallelism": "single-gpu", "layers": args.layers, "layers_full_model": FULL_LAYERS,
+            "hidden_size": cfg["hidden_size"], "intermediate_size": cfg["intermediate_size"],
+            "num_attention_heads": cfg["num_attention_heads"], "num_key_value_heads": cfg["num_key_value_heads"],
+            "head_dim": cfg["head_dim"], "vocab_size": V, "tie_word_embeddings": True,
+            "rope": "theta 5e5, llama3 scaling 32/1/4/8192", "page_size": page,
+            "prefill_tokens": T, "decode_context": args.context, "sampling": "greedy",
+        },
+        "prefill": prefill, "roofline": roofline, "points": points,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

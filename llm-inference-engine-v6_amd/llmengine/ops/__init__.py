@@ -3,5 +3,8 @@ from .lib import KernelError, KernelLibraryError, library
 from .kernels import (argmax, attention, attention_generic, rope_q_only, embed_gather, gemm, gemm_generic, policy, rmsnorm,
                       rope_kv_write, sample, swiglu)
 
-__all__ = ["KernelError", "KernelLibraryError", "library", "argmax", "attention", "attention_generic", "rope_q_only", "embed_gather",
+from . import mfma                                   # noqa: E402  (installs the MFMA kernels)
+from .mfma import gemm_bf16
+
+__all__ = ["gemm_bf16", "mfma", "KernelError", "KernelLibraryError", "library", "argmax", "attention", "attention_generic", "rope_q_only", "embed_gather",
            "gemm", "gemm_generic", "policy", "rmsnorm", "rope_kv_write", "sample", "swiglu"]

@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import torch
 
-from .lib import BF16, F32, KernelError, check, code, entry, ptr, require, stream
+from .lib import BF16, F32, KernelError, check, code, entry, ptr, require, stream  # noqa: F401
 
 _FLOATS = (torch.float32, torch.bfloat16)
 

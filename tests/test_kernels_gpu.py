@@ -216,3 +216,62 @@ def test_temperature_sampling_interval(ops, V):
     zero = torch.zeros(R)
     ops.sample(logits.to(DEV), zero.to(DEV), u.to(DEV), out)
     assert out.tolist() == logits.argmax(dim=1).tolist()
+
+
+# --- MFMA matrix products ----------------------------------------------------------------
+def _bf16_pair(M, N, K, seed):
+    a = torch.randn(M, K, generator=_gen(seed)).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=_gen(seed + 1)).to(torch.bfloat16)
+    return a, w, a.double() @ w.double().T
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 16, 8), (1, 2048, 2048), (8, 3072, 2048), (3, 100, 176), (16, 331, 144),
+                                   (17, 48, 40), (33, 96, 96), (64, 2048, 8192), (50, 129, 1000)])
+@pytest.mark.parametrize("waves,ksplit", [(0, 0), (4, 1), (8, 1), (16, 1), (4, 3)])
+def test_gemm_skinny(ops, M, N, K, waves, ksplit):
+    a, w, ref = _bf16_pair(M, N, K, 20)
+    base = torch.randn(M, N, generator=_gen(22))
+    if ksplit > 1:
+        out = base.clone().to(DEV)
+        ops.gemm_bf16(a.to(DEV), w.to(DEV), out, accumulate=True, waves=waves, ksplit=ksplit)
+        assert _rel(out.cpu().double(), ref + base.double()) < 2e-5
+        return
+    out = torch.full((M, N), 3.0, device=DEV)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), out, waves=waves)
+    assert _rel(out.cpu().double(), ref) < 2e-5
+    acc = base.clone().to(DEV)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), acc, accumulate=True, waves=waves)
+    assert _rel(acc.cpu().double(), ref + base.double()) < 2e-5
+    half = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), half, waves=waves)
+    assert _rel(half.cpu().double(), ref) < 5e-3
+
+
+@pytest.mark.parametrize("M,N,K", [(65, 128, 64), (128, 128, 128), (200, 331, 144), (129, 100, 176), (257, 500, 72),
+                                   (2048, 3072, 2048), (1000, 2048, 8192), (7, 40, 24)])
+def test_gemm_tile(ops, M, N, K):
+    a, w, ref = _bf16_pair(M, N, K, 30)
+    out = torch.full((M, N), 3.0, device=DEV)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), out, force_tile=True)
+    assert _rel(out.cpu().double(), ref) < 2e-5
+    base = torch.randn(M, N, generator=_gen(32))
+    acc = base.clone().to(DEV)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), acc, accumulate=True, force_tile=True)
+    assert _rel(acc.cpu().double(), ref + base.double()) < 2e-5
+    half = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), half, force_tile=True)
+    assert _rel(half.cpu().double(), ref) < 5e-3
+
+
+def test_gemm_dispatch_and_refusals(ops):
+    from llmengine.ops import KernelError
+    a, w, ref = _bf16_pair(5, 30, 36, 40)               # K = 36 is no multiple of 8: the plain kernel takes it
+    out = torch.empty(5, 30, device=DEV)
+    ops.gemm(a.to(DEV), w.to(DEV), out)
+    assert _rel(out.cpu().double(), ref) < 2e-5
+    with pytest.raises(KernelError):
+        ops.gemm_bf16(a.to(DEV), w.to(DEV), out)
+    with pytest.raises(KernelError):
+        ops.gemm(a.to(DEV), w.to(DEV)[:, :30].contiguous(), out)      # inner sizes differ
+    with pytest.raises(KernelError):
+        ops.gemm(a, w, out.cpu())                                      # not on the GPU
