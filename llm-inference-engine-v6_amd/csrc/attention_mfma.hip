@@ -1,0 +1,409 @@
+// Attention over bfloat16 cache pages on the matrix cores (v_mfma_f32_16x16x32_bf16).
+// Formula as in the plain-precision kernel (src/kernels.cpp:413-474): kv head = q head /
+// (n_q / n_kv), scores scaled by `scale`, softmax over the keys a token may see, weighted
+// sum of values. Softmax statistics and accumulation are 32-bit; probabilities enter the
+// second product rounded to bfloat16.
+//
+// Layouts: k_cache [pages, n_kv, page, hd]; v_cache [pages, n_kv, hd, page] (keys contiguous
+// for a fixed dimension, which is what the second product's operand wants); q, out
+// [T, n_q * hd]; block_table [n_seq, max_blocks].
+//
+// One wavefront handles a tile of 16 query rows against 32 keys at a time:
+//   S^T[key, row] = sum_d K[key, d] Q[row, d]      first operand K (16 keys x 32 d, one
+//                                                   16-byte load per lane), second Q^T
+//   lane l then holds, for row l % 16, the keys 4 (l / 16) + e of both 16-key halves:
+//   exactly the 8 keys this lane must supply as first operand of
+//   O[row, d] += sum_key P[row, key] V[key, d]      second operand V^T read 4 keys (8 bytes)
+//                                                   at a time from the transposed pages
+// so probabilities never pass through LDS. The running maximum m and sum l are kept per
+// lane for row l % 16; O's rows are 4 (l / 16) + e, so rescaling fetches factors by shuffle.
+//
+// Two kernels share this tile code:
+//  * decode: requests that bring one token. The 16 rows are the query heads of one kv
+//    head; grid (request, kv head x head tile, split of the keys); partial results of the
+//    splits are joined by a small second kernel.
+//  * prefill: requests that bring several tokens. The rows are 16 consecutive tokens of one
+//    query head; a wavefront takes QT such tiles so that every K and V load is used QT
+//    times; a workgroup's four wavefronts take four neighbouring heads of the same tokens,
+//    so their K and V loads hit the same cache lines. Causal by position: row at position
+//    p sees keys max(0, p - window + 1) .. p; key blocks past the last row are not visited.
+// Requests are told apart on the device from q_start (first batch row of each request).
+//
+// Limits (the caller checks them and otherwise uses the plain-precision kernel): head size a
+// multiple of 16 up to 128; page size a multiple of 16.
+#include "common.h"
+#include <math.h>
+
+namespace llme {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct PagedKV {
+    const bf16* k;
+    const bf16* v;
+    const int* table;       // this request's row of the block table
+    int page, n_kv, kvh, hd;
+};
+
+__device__ __forceinline__ bf16x8 zero_frag() {
+    bf16x8 z;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = static_cast<__bf16>(0.f);
+    return z;
+}
+
+// One 32-key block for QT row tiles. HD: head size (compile time).
+//   t0: first key of the block (multiple of 32); keys outside [key_lo, key_end) are not
+//   loaded: behind key_end nothing is written yet, before key_lo (the first key any row
+//   of the work item may see) the pages may have been given back. row_pos[qt]: position of this lane's row (l % 16) in tile
+//   qt, or -1 for a row that does not exist; row_lo[qt]: first key the row may see.
+template <int HD, int QT>
+__device__ __forceinline__ void attend_block(const PagedKV& kv, int t0, int key_lo, int key_end, const bf16x8 (&qf)[QT][(HD + 31) / 32],
+                                             const int (&row_pos)[QT], const int (&row_lo)[QT], float scale_log2,
+                                             float (&m)[QT], float (&l)[QT], f32x4 (&o)[QT][HD / 16]) {
+    constexpr int DC = (HD + 31) / 32, DT = HD / 16;
+    const int lane = threadIdx.x & 63;
+    const int r = lane & 15, g4 = lane >> 4;
+
+    // K fragments of the two 16-key halves: row r of each half
+    bf16x8 kf[2][DC];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+        const int t = t0 + hf * 16 + r;
+        const bool ok = t >= key_lo && t < key_end;
+        const bf16* row = nullptr;
+        if (ok) {
+            const int pg = kv.table[t / kv.page];
+            row = kv.k + ((static_cast<size_t>(pg) * kv.n_kv + kv.kvh) * kv.page + t % kv.page) * HD;
+        }
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+            const int d = c * 32 + g4 * 8;
+            kf[hf][c] = (ok && d < HD) ? *reinterpret_cast<const bf16x8*>(row + d) : zero_frag();
+        }
+    }
+    // V fragments: for dimension dt * 16 + r, keys 4 g4 .. 4 g4 + 3 of each half
+    bf16x8 vf[DT];
+    {
+        const bf16* base[2];
+        bool ok[2];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            const int t = t0 + hf * 16 + g4 * 4;
+            ok[hf] = t + 3 >= key_lo && t < key_end;     // the 4 keys share a page with a visible key
+            base[hf] = nullptr;
+            if (ok[hf]) {
+                const int pg = kv.table[t / kv.page];
+                base[hf] = kv.v + (static_cast<size_t>(pg) * kv.n_kv + kv.kvh) * HD * kv.page + t % kv.page;
+            }
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const size_t off = static_cast<size_t>(dt * 16 + r) * kv.page;
+            bf16x4 lo4, hi4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) lo4[e] = hi4[e] = static_cast<__bf16>(0.f);
+            if (ok[0]) lo4 = *reinterpret_cast<const bf16x4*>(base[0] + off);
+            if (ok[1]) hi4 = *reinterpret_cast<const bf16x4*>(base[1] + off);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                vf[dt][e] = lo4[e];
+                vf[dt][4 + e] = hi4[e];
+            }
+        }
+    }
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        f32x4 s[2];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            s[hf] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < DC; ++c)
+                s[hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[hf][c], qf[qt][c], s[hf], 0, 0, 0);
+        }
+        // this lane: row r of tile qt, keys t0 + 16 hf + 4 g4 + e
+        const int pos = row_pos[qt], lo = row_lo[qt];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int t = t0 + hf * 16 + g4 * 4 + e;
+                const bool see = (t <= pos) && (t >= lo);
+                const float v = see ? s[hf][e] * scale_log2 : -INFINITY;
+                s[hf][e] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m[qt], mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;       // nothing seen yet: all p are 0
+        const float alpha = exp2f(m[qt] - m_use);                      // 0 when m was -inf
+        m[qt] = m_new;
+        bf16x8 pf;
+        float psum = 0.f;
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float p = exp2f(s[hf][e] - m_use);
+                psum += p;
+                pf[hf * 4 + e] = static_cast<__bf16>(p);
+            }
+        l[qt] = l[qt] * alpha + psum;
+        float ar[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ar[e] = __shfl(alpha, g4 * 4 + e, 64);     // factor of O's row 4 g4 + e
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[qt][dt][e] *= ar[e];
+            o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf[dt], o[qt][dt], 0, 0, 0);
+        }
+    }
+}
+
+// Loads the query fragments of one 16-row tile: lane holds row r, dims c * 32 + 8 g4 ..
+template <int HD>
+__device__ __forceinline__ void load_q(const bf16* qrow, bool ok, bf16x8 (&qf)[(HD + 31) / 32]) {
+    const int g4 = (threadIdx.x & 63) >> 4;
+#pragma unroll
+    for (int c = 0; c < (HD + 31) / 32; ++c) {
+        const int d = c * 32 + g4 * 8;
+        qf[c] = (ok && d < HD) ? *reinterpret_cast<const bf16x8*>(qrow + d) : zero_frag();
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// decode: one token per request
+template <int HD>
+__global__ __launch_bounds__(64) void attention_decode_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    bf16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const int* __restrict__ q_start, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
+    int max_blocks, int n_q, int n_kv, int page, float scale, int window, int split_len, int nsplit) {
+    constexpr int DC = (HD + 31) / 32, DT = HD / 16;
+    const int s = blockIdx.x;
+    const int row0 = q_start[s];
+    if (q_start[s + 1] - row0 != 1) return;            // not a decoding request
+    const int G = n_q / n_kv;
+    const int gtiles = (G + 15) / 16;
+    const int kvh = blockIdx.y / gtiles, gt = blockIdx.y % gtiles;
+    const int split = blockIdx.z;
+    const int lane = threadIdx.x & 63, r = lane & 15, g4 = lane >> 4;
+
+    const int pos = ctx_len[s];                         // the token's position; it sees keys lo..pos
+    const int lo_all = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    int k_begin = split * split_len, k_end = k_begin + split_len;
+    if (k_end > pos + 1) k_end = pos + 1;
+    if (k_begin < (lo_all & ~31)) k_begin = lo_all & ~31;
+
+    const int head = kvh * G + gt * 16 + r;             // this lane's row is a query head
+    const bool row_ok = (gt * 16 + r) < G;
+    bf16x8 qf[1][DC];
+    load_q<HD>(q + (static_cast<size_t>(row0) * n_q + (row_ok ? head : 0)) * HD, row_ok, qf[0]);
+    const int row_pos[1] = {row_ok ? pos : -1};
+    const int row_lo[1] = {lo_all};
+    float m[1] = {-INFINITY}, l[1] = {0.f};
+    f32x4 o[1][DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD};
+    const float scale_log2 = scale * kLog2e;
+    for (int t0 = k_begin; t0 < k_end; t0 += 32)
+        attend_block<HD, 1>(kv, t0, lo_all, k_end, qf, row_pos, row_lo, scale_log2, m, l, o);
+
+    float lt = l[0];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+    // O's rows are heads gt * 16 + 4 g4 + e; statistics sit in the lanes whose r is that row
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int rr = g4 * 4 + e;
+        const float l_row = __shfl(lt, rr, 64), m_row = __shfl(m[0], rr, 64);
+        if (gt * 16 + rr >= G) continue;
+        const int h = kvh * G + gt * 16 + rr;
+        if (nsplit == 1) {
+            const float inv = 1.0f / l_row;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                out[(static_cast<size_t>(row0) * n_q + h) * HD + dt * 16 + r] = static_cast<bf16>(o[0][dt][e] * inv);
+        } else {
+            const size_t pidx = (static_cast<size_t>(s) * n_q + h) * nsplit + split;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) part_o[pidx * HD + dt * 16 + r] = o[0][dt][e];
+            if (r == 0) {
+                part_ml[pidx * 2] = m_row;
+                part_ml[pidx * 2 + 1] = l_row;
+            }
+        }
+    }
+}
+
+// joins the splits of the decode kernel: grid (request, head), 64 lanes over the head's dims
+__global__ __launch_bounds__(64) void attention_join_kernel(const float* __restrict__ part_o,
+                                                            const float* __restrict__ part_ml, bf16* __restrict__ out,
+                                                            const int* __restrict__ q_start, int n_q, int hd, int nsplit) {
+    const int s = blockIdx.x, h = blockIdx.y;
+    const int row0 = q_start[s];
+    if (q_start[s + 1] - row0 != 1) return;
+    const size_t base = (static_cast<size_t>(s) * n_q + h) * nsplit;
+    float mx = -INFINITY;
+    for (int i = 0; i < nsplit; ++i) mx = fmaxf(mx, part_ml[(base + i) * 2]);
+    float total = 0.f;
+    for (int i = 0; i < nsplit; ++i) {
+        const float mi = part_ml[(base + i) * 2];
+        if (mi != -INFINITY) total += exp2f(mi - mx) * part_ml[(base + i) * 2 + 1];
+    }
+    const float inv = 1.0f / total;
+    for (int d = threadIdx.x; d < hd; d += 64) {
+        float acc = 0.f;
+        for (int i = 0; i < nsplit; ++i) {
+            const float mi = part_ml[(base + i) * 2];
+            if (mi != -INFINITY) acc += exp2f(mi - mx) * part_o[(base + i) * hd + d];
+        }
+        out[(static_cast<size_t>(row0) * n_q + h) * hd + d] = static_cast<bf16>(acc * inv);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// prefill: several tokens per request; a wavefront takes QT tiles of 16 tokens of one head
+template <int HD, int QT>
+__global__ __launch_bounds__(256) void attention_prefill_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    bf16* __restrict__ out, const int* __restrict__ q_start, const int* __restrict__ ctx_len,
+    const int* __restrict__ block_table, int max_blocks, int n_seq, int n_q, int n_kv, int page, float scale,
+    int window) {
+    constexpr int DC = (HD + 31) / 32, DT = HD / 16, ROWS = 16 * QT;
+    // which request and which of its row groups this workgroup has
+    int s = 0, first = 0, n_rows = 0, acc = 0;
+    bool found = false;
+    for (int i = 0; i < n_seq; ++i) {
+        const int a = q_start[i], n = q_start[i + 1] - a;
+        const int nt = (n >= 2) ? (n + ROWS - 1) / ROWS : 0;
+        if (!found && static_cast<int>(blockIdx.x) < acc + nt) {
+            s = i;
+            first = (blockIdx.x - acc) * ROWS;           // first row of the group within the request
+            n_rows = n - first < ROWS ? n - first : ROWS;
+            first += a;                                   // as a batch row
+            found = true;
+        }
+        acc += nt;
+    }
+    if (!found) return;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g4 = lane >> 4;
+    const int head = blockIdx.y * 4 + wave;
+    if (head >= n_q) return;
+    const int kvh = head / (n_q / n_kv);
+    const int pos0 = ctx_len[s] + (first - q_start[s]);  // position of the group's first row
+
+    bf16x8 qf[QT][DC];
+    int row_pos[QT], row_lo[QT];
+    float m[QT], l[QT];
+    f32x4 o[QT][DT];
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int rr = qt * 16 + r;
+        const bool ok = rr < n_rows;
+        load_q<HD>(q + (static_cast<size_t>(first + (ok ? rr : 0)) * n_q + head) * HD, ok, qf[qt]);
+        row_pos[qt] = ok ? pos0 + rr : -1;
+        row_lo[qt] = (window > 0 && pos0 + rr - window + 1 > 0) ? pos0 + rr - window + 1 : 0;
+        m[qt] = -INFINITY;
+        l[qt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    const int key_end = pos0 + n_rows;                    // the last row sees keys < key_end
+    const int key_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;   // the first row's first key
+    const int k_begin = key_lo & ~31;
+    PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD};
+    const float scale_log2 = scale * kLog2e;
+    for (int t0 = k_begin; t0 < key_end; t0 += 32)
+        attend_block<HD, QT>(kv, t0, key_lo, key_end, qf, row_pos, row_lo, scale_log2, m, l, o);
+
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        float lt = l[qt];
+        lt += __shfl_xor(lt, 16, 64);
+        lt += __shfl_xor(lt, 32, 64);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int rr = g4 * 4 + e;
+            const float l_row = __shfl(lt, rr, 64);
+            const int row = qt * 16 + rr;
+            if (row >= n_rows) continue;
+            const float inv = 1.0f / l_row;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+                out[(static_cast<size_t>(first + row) * n_q + head) * HD + dt * 16 + r] =
+                    static_cast<bf16>(o[qt][dt][e] * inv);
+        }
+    }
+}
+
+template <int HD>
+static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, float* part_o, float* part_ml,
+                           const int* q_start, const int* ctx_len, const int* table, int max_blocks, int n_seq,
+                           int n_q, int n_kv, int page, float scale, int window, int n_decode, int split_len,
+                           int nsplit, int prefill_groups, int qt, hipStream_t stream) {
+    if (n_decode > 0) {
+        const int G = n_q / n_kv;
+        const dim3 grid(n_seq, n_kv * ((G + 15) / 16), nsplit);
+        hipLaunchKernelGGL((attention_decode_kernel<HD>), grid, dim3(64), 0, stream, q, kc, vc, out, part_o, part_ml,
+                           q_start, ctx_len, table, max_blocks, n_q, n_kv, page, scale, window, split_len, nsplit);
+        if (nsplit > 1)
+            hipLaunchKernelGGL(attention_join_kernel, dim3(n_seq, n_q), dim3(64), 0, stream, part_o, part_ml, out,
+                               q_start, n_q, HD, nsplit);
+    }
+    if (prefill_groups > 0) {
+        const dim3 grid(prefill_groups, (n_q + 3) / 4);
+#define LLME_PREFILL(QT)                                                                                       \
+    hipLaunchKernelGGL((attention_prefill_kernel<HD, QT>), grid, dim3(256), 0, stream, q, kc, vc, out, q_start, \
+                       ctx_len, table, max_blocks, n_seq, n_q, n_kv, page, scale, window)
+        if (qt == 4 && HD <= 64) LLME_PREFILL(4);
+        else if (qt >= 2 && HD <= 128) LLME_PREFILL(2);
+        else LLME_PREFILL(1);
+#undef LLME_PREFILL
+    }
+    return launch_status();
+}
+
+}  // namespace llme
+
+using namespace llme;
+
+// Rows per prefill work item for a head size: the caller sizes the grid with it.
+extern "C" int llme_attention_bf16_rows(int hd) { return hd <= 64 ? 64 : 32; }
+
+// n_decode: requests with one token (0: none, skip the decode kernels); split_len (multiple of
+// 32) and nsplit: how the decode kernel cuts the keys; part_o [n_seq, n_q, nsplit, hd] and
+// part_ml [n_seq, n_q, nsplit, 2] floats (needed when nsplit > 1). prefill_groups: number of
+// row groups of llme_attention_bf16_rows(hd) rows over the requests with two or more tokens.
+extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const void* v_cache, void* out, float* part_o,
+                                   float* part_ml, const int* q_start, const int* ctx_len, const int* block_table,
+                                   int max_blocks, int n_seq, int n_q, int n_kv, int hd, int page, float scale,
+                                   int window, int n_decode, int split_len, int nsplit, int prefill_groups,
+                                   hipStream_t stream) {
+    if (n_seq <= 0) return 0;
+    if (hd % 16 != 0 || hd > 128 || hd <= 0 || page % 16 != 0 || n_kv <= 0 || n_q % n_kv != 0) return kErrUnsupported;
+    if (n_decode > 0 && (split_len <= 0 || split_len % 32 != 0 || nsplit <= 0)) return kErrBadArgument;
+    const int qt = llme_attention_bf16_rows(hd) / 16;
+#define LLME_HEAD(HD)                                                                                           \
+    case HD:                                                                                                    \
+        return launch_for_head<HD>(static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache),              \
+                                   static_cast<const bf16*>(v_cache), static_cast<bf16*>(out), part_o, part_ml, \
+                                   q_start, ctx_len, block_table, max_blocks, n_seq, n_q, n_kv, page, scale,    \
+                                   window, n_decode, split_len, nsplit, prefill_groups, qt, stream)
+    switch (hd) {
+        LLME_HEAD(16); LLME_HEAD(32); LLME_HEAD(48); LLME_HEAD(64);
+        LLME_HEAD(80); LLME_HEAD(96); LLME_HEAD(112); LLME_HEAD(128);
+        default: return kErrUnsupported;
+    }
+#undef LLME_HEAD
+}

@@ -48,3 +48,84 @@ def _fast_gemm(a, w, out, accumulate) -> bool:
 
 
 kernels._fast_gemm = _fast_gemm
+
+
+# --- attention ---------------------------------------------------------------------------
+declare("llme_attention_bf16_rows", [_i])
+declare("llme_attention_bf16", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i,
+                                _i, _i, _i, _i, _vp])
+
+DECODE_BLOCKS_WANTED = 2048         # workgroups the decode kernel should have to fill the chip
+MIN_SPLIT = 64                      # keys per split at least
+
+
+def attention_bf16_supported(q, k_cache, head_dim: int) -> bool:
+    return (q.dtype == torch.bfloat16 and k_cache.dtype == torch.bfloat16 and head_dim % 16 == 0
+            and head_dim <= 128 and k_cache.shape[2] % 16 == 0 and q.data_ptr() % 16 == 0
+            and k_cache.data_ptr() % 16 == 0)
+
+
+def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int) -> dict:
+    """Launch sizes for a step, from how its batch is cut (host-side numbers only)."""
+    rows = entry("llme_attention_bf16_rows")(head_dim)
+    decode = [c + 1 for n, c in zip(new_lens, ctx_lens) if n == 1]
+    groups = sum((n + rows - 1) // rows for n in new_lens if n >= 2)
+    plan = {"n_decode": len(decode), "groups": groups, "split_len": 32, "nsplit": 1}
+    if decode:
+        longest = max(decode)
+        pairs = len(decode) * n_kv * ((n_q // n_kv + 15) // 16)
+        nsplit = max(1, min((DECODE_BLOCKS_WANTED + pairs - 1) // pairs, (longest + MIN_SPLIT - 1) // MIN_SPLIT))
+        split_len = ((longest + nsplit - 1) // nsplit + 31) // 32 * 32
+        plan["split_len"] = split_len
+        plan["nsplit"] = (longest + split_len - 1) // split_len
+    return plan
+
+
+def attention_bf16(q, k_cache, v_cache, out, q_start, ctx_len, block_table, n_q: int, n_kv: int, head_dim: int,
+                   scale: float, window: int, plan: dict, part_o=None, part_ml=None) -> None:
+    """Attention of a step's tokens over bfloat16 pages. q_start [S + 1], ctx_len [S] int32 on
+    the device; plan from plan_attention; part_o / part_ml: float32 scratch for split decoding."""
+    T = q.shape[0]
+    S = ctx_len.shape[0]
+    require(q, "q", torch.bfloat16, (T, n_q * head_dim))
+    require(out, "out", torch.bfloat16, (T, n_q * head_dim))
+    require(k_cache, "k_cache", torch.bfloat16, (None, n_kv, None, head_dim))
+    page = k_cache.shape[2]
+    require(v_cache, "v_cache", torch.bfloat16, (k_cache.shape[0], n_kv, head_dim, page))
+    require(q_start, "q_start", torch.int32, (S + 1,))
+    require(ctx_len, "ctx_len", torch.int32, (S,))
+    require(block_table, "block_table", torch.int32, (S, None))
+    if not attention_bf16_supported(q, k_cache, head_dim):
+        raise kernels.KernelError(f"attention_bf16: head size {head_dim} must be a multiple of 16 up to 128 and "
+                                  f"the page size {page} a multiple of 16")
+    if n_q % n_kv:
+        raise kernels.KernelError(f"attention: {n_q} query heads do not divide into {n_kv} key/value heads")
+    if plan["n_decode"] and plan["nsplit"] > 1:
+        require(part_o, "part_o", torch.float32)
+        require(part_ml, "part_ml", torch.float32)
+        if part_o.numel() < S * n_q * plan["nsplit"] * head_dim or part_ml.numel() < S * n_q * plan["nsplit"] * 2:
+            raise kernels.KernelError("attention_bf16: the scratch for split decoding is too small")
+    check(entry("llme_attention_bf16")(
+        ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), ptr(part_o), ptr(part_ml), ptr(q_start), ptr(ctx_len),
+        ptr(block_table), block_table.shape[1], S, n_q, n_kv, head_dim, page, float(scale), int(window),
+        plan["n_decode"], plan["split_len"], plan["nsplit"], plan["groups"], stream()), "attention_bf16")
+
+
+def _fast_attention(q, k_cache, v_cache, out, step, block_table, n_q, n_kv, head_dim, scale, window) -> bool:
+    if not attention_bf16_supported(q, k_cache, head_dim) or out.dtype != torch.bfloat16:
+        return False
+    key = ("attention_plan", n_q, n_kv, head_dim)
+    plan = step.extra.get(key)
+    if plan is None:
+        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim)
+    part_o = part_ml = None
+    if plan["n_decode"] and plan["nsplit"] > 1:
+        S = step.num_seqs
+        part_o = step.buffer("attn.part_o", (S * n_q * plan["nsplit"] * head_dim,), torch.float32)
+        part_ml = step.buffer("attn.part_ml", (S * n_q * plan["nsplit"] * 2,), torch.float32)
+    attention_bf16(q, k_cache, v_cache, out, step.q_start, step.ctx_len, block_table, n_q, n_kv, head_dim, scale,
+                   window, plan, part_o, part_ml)
+    return True
+
+
+kernels._fast_attention = _fast_attention

@@ -275,3 +275,103 @@ def test_gemm_dispatch_and_refusals(ops):
         ops.gemm(a.to(DEV), w.to(DEV)[:, :30].contiguous(), out)      # inner sizes differ
     with pytest.raises(KernelError):
         ops.gemm(a, w, out.cpu())                                      # not on the GPU
+
+
+# --- MFMA attention ----------------------------------------------------------------------
+def _attn_case(ops, lens, news, n_q, n_kv, hd, page, window=0, seed=50):
+    """Requests with lens[i] tokens in the cache, of which the last news[i] are this step's."""
+    s = _paged_setup(ops, lens, n_q, n_kv, hd, page, torch.bfloat16, seed=seed)
+    rows, q_start, ctx = [], [0], []
+    base = 0
+    for n, new in zip(lens, news):
+        rows += list(range(base + n - new, base + n))
+        q_start.append(q_start[-1] + new)
+        ctx.append(n - new)
+        base += n
+    q = s["q"][torch.tensor(rows, device=DEV)].contiguous()
+    out = torch.zeros_like(q)
+    i32 = dict(dtype=torch.int32, device=DEV)
+    plan = ops.mfma.plan_attention(news, ctx, n_q, n_kv, hd)
+    S = len(lens)
+    part_o = torch.empty(S * n_q * plan["nsplit"] * hd, device=DEV)
+    part_ml = torch.empty(S * n_q * plan["nsplit"] * 2, device=DEV)
+    ops.mfma.attention_bf16(q, s["k_cache"], s["v_cache"], out, torch.tensor(q_start, **i32), torch.tensor(ctx, **i32),
+                            s["table"], n_q, n_kv, hd, 1.0 / math.sqrt(hd), window, plan, part_o, part_ml)
+    ref = torch.cat([plain_attention(qq, kk, vv, window)[n - new:].reshape(new, n_q * hd)
+                     for (qq, kk, vv), n, new in zip(s["plain"], lens, news)])
+    return out.cpu().double(), ref, plan
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,page", [(4, 2, 16, 16), (3, 1, 32, 16), (6, 2, 48, 32), (32, 8, 64, 16),
+                                              (5, 5, 80, 16), (8, 2, 96, 64), (4, 1, 112, 16), (8, 2, 128, 16),
+                                              (34, 2, 64, 16)])
+def test_attention_mfma_decode(ops, n_q, n_kv, hd, page):
+    lens = [1, 2, 31, 32, 33, 300, 77]
+    out, ref, plan = _attn_case(ops, lens, [1] * len(lens), n_q, n_kv, hd, page)
+    assert plan["n_decode"] == len(lens) and plan["groups"] == 0
+    assert _rel(out, ref) < 8e-3
+
+
+def test_attention_mfma_decode_splits(ops, monkeypatch):
+    """Few requests with a long context: the keys are cut into many splits and joined."""
+    out, ref, plan = _attn_case(ops, [1500, 40], [1, 1], 8, 2, 64, 16)
+    assert plan["nsplit"] > 4
+    assert _rel(out, ref) < 8e-3
+    monkeypatch.setattr(ops.mfma, "DECODE_BLOCKS_WANTED", 1)
+    out1, ref1, plan1 = _attn_case(ops, [1500, 40], [1, 1], 8, 2, 64, 16)
+    assert plan1["nsplit"] == 1 and _rel(out1, ref1) < 8e-3
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,page", [(4, 2, 16, 16), (3, 1, 32, 16), (6, 2, 48, 32), (32, 8, 64, 16),
+                                              (5, 5, 80, 16), (8, 2, 128, 16)])
+def test_attention_mfma_prefill_and_mixed(ops, n_q, n_kv, hd, page):
+    lens = [70, 2, 130, 17, 64, 200, 9]
+    news = [70, 2, 35, 1, 64, 3, 1]                      # whole prompts, portions with context, decoded tokens
+    out, ref, plan = _attn_case(ops, lens, news, n_q, n_kv, hd, page)
+    assert plan["n_decode"] == 2 and plan["groups"] >= 5
+    assert _rel(out, ref) < 8e-3
+
+
+@pytest.mark.parametrize("window", [1, 5, 16, 33, 100])
+def test_attention_mfma_window(ops, window):
+    lens = [150, 40, 90]
+    news = [1, 40, 30]
+    out, ref, _ = _attn_case(ops, lens, news, 4, 2, 32, 16, window=window)
+    assert _rel(out, ref) < 8e-3
+
+
+def test_attention_mfma_finds_one_far_key(ops):
+    """One early key is made to dominate (its query-key score is far above the rest): the output
+    must be that key's value row, for a decoded token and for a row of a prompt portion."""
+    n_q, n_kv, hd, page = 4, 2, 64, 16
+    lens, far = [400, 400], 37
+    T = sum(lens)
+    g = _gen(77)
+    qkv = 0.1 * torch.randn(T, (n_q + 2 * n_kv) * hd, generator=g)
+    for base in (0, 400):
+        qkv[base + 399, :n_q * hd] = 0.0
+        qkv[base + 399, :n_q * hd:hd] = 8.0                          # every head of the last query: e_0 * 8
+        qkv[base + far, n_q * hd:(n_q + n_kv) * hd:hd] = 8.0         # key `far`: e_0 * 8 -> score 64 / 8
+    i32 = dict(dtype=torch.int32, device=DEV)
+    nblk = 400 // page
+    table = torch.arange(2 * nblk, dtype=torch.int32).view(2, nblk)
+    positions = torch.cat([torch.arange(400), torch.arange(400)]).to(torch.int32)
+    seq_idx = torch.cat([torch.zeros(400), torch.ones(400)]).to(torch.int32)
+    k_cache = torch.zeros(2 * nblk, n_kv, page, hd, dtype=torch.bfloat16, device=DEV)
+    v_cache = torch.zeros(2 * nblk, n_kv, hd, page, dtype=torch.bfloat16, device=DEV)
+    q_all = torch.empty(T, n_q * hd, dtype=torch.bfloat16, device=DEV)
+    ops.rope_kv_write(qkv.to(DEV), None, None, positions.to(DEV), seq_idx.to(DEV), table.to(DEV), q_all, k_cache,
+                      v_cache, n_q, n_kv, hd, hd)
+    rows = [399] + list(range(400 + 390, 800))                       # request 0 decodes, request 1 brings 10 rows
+    q = q_all[torch.tensor(rows, device=DEV)].contiguous()
+    out = torch.zeros_like(q)
+    plan = ops.mfma.plan_attention([1, 10], [399, 390], n_q, n_kv, hd)
+    part_o = torch.empty(2 * n_q * plan["nsplit"] * hd, device=DEV)
+    part_ml = torch.empty(2 * n_q * plan["nsplit"] * 2, device=DEV)
+    ops.mfma.attention_bf16(q, k_cache, v_cache, out, torch.tensor([0, 1, 11], **i32),
+                            torch.tensor([399, 390], **i32), table.to(DEV), n_q, n_kv, hd, 1.0, 0, plan, part_o, part_ml)
+    v = qkv[:, (n_q + n_kv) * hd:].to(torch.bfloat16).double().view(T, n_kv, hd)
+    for row, base in ((0, 0), (10, 400)):
+        for h in range(n_q):
+            got = out[row].cpu().double().view(n_q, hd)[h]
+            assert (got - v[base + far, h // 2]).abs().max() < 2e-2, (row, h)
