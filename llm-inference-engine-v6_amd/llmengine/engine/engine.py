@@ -74,7 +74,7 @@ class BlockManager:
 class Engine:
     def __init__(self, model_dir: str | None, dtype: str = "fp32", *, device: str = "cuda:0",
                  max_prefill_tokens_per_step: int = 8192, temperature: float = 0.0, sampler_seed: int = 0,
-                 block_size: int = 16, _config: dict | None = None, _tensors=None):
+                 block_size: int = 16, use_graphs: bool = True, _config: dict | None = None, _tensors=None):
         self._dtype_name = {"float32": "fp32", "bfloat16": "bf16"}.get(dtype, dtype)
         self._torch_dtype = parse_dtype(dtype)
         if _config is None:
@@ -98,6 +98,7 @@ class Engine:
         self.block_size = int(block_size)
         self.prefill_chunk = int(max_prefill_tokens_per_step)
         self._own_cache: CacheContext | None = None
+        self.use_graphs = bool(use_graphs)
 
     # ---- construction from random weights ----
     @classmethod
@@ -151,7 +152,7 @@ class Engine:
                         self._tensors = {k: None for k in self._tensors}    # keep the names only
                     else:
                         load_model_weights(model, self.model_dir, placement)
-                self._runner = ModelRunner(model, self._torch_dtype, device)
+                self._runner = ModelRunner(model, self._torch_dtype, device, use_graphs=self.use_graphs)
             return self._runner
 
     @property

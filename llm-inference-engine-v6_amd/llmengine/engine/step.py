@@ -37,6 +37,8 @@ class Workspace:
     def __init__(self, device: torch.device):
         self.device = device
         self._buffers: dict[tuple[str, torch.dtype], torch.Tensor] = {}
+        self.keep_replaced = False      # set once a recorded graph holds addresses of these buffers
+        self._replaced: list[torch.Tensor] = []
 
     def get(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         n = 1
@@ -45,6 +47,8 @@ class Workspace:
         key = (name, dtype)
         buf = self._buffers.get(key)
         if buf is None or buf.numel() < n:
+            if buf is not None and self.keep_replaced:
+                self._replaced.append(buf)          # a recorded graph may still read and write it
             buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._buffers[key] = buf
         return buf[:n].view(shape)
@@ -69,6 +73,10 @@ class StepContext:
     ctx_lens: list[int] = field(default_factory=list)
     slot_list: list[int] = field(default_factory=list)
     max_position: int = 0
+    # When a step is recorded as a HIP graph and replayed for later steps of the same shape,
+    # launch sizes must not follow the momentary lengths: kernels plan for requests of up to
+    # `plan_len` tokens instead (None: plan from ctx_lens / new_lens).
+    plan_len: int | None = None
     extra: dict = field(default_factory=dict)          # per-step notes of kernels (launch plans)
 
     def buffer(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
@@ -113,6 +121,7 @@ class CacheContext:
         self.storage = CacheStorage(specs, groups, page_size, max_requests, dtype, device)
         self.page_size = page_size
         self.max_requests = max_requests
+        self.graphs: dict = {}          # recorded decode steps over this pool's tensors, by shape
 
     def admit(self, request_id) -> int:
         slot = self.manager.admit(request_id)
@@ -126,13 +135,17 @@ class CacheContext:
 class ModelRunner:
     """A loaded model on a device plus the scratch memory its steps use."""
 
-    def __init__(self, model: DecoderModel, dtype: torch.dtype, device: torch.device):
+    GRAPH_BLOCK_BUCKET = 64         # block-table widths of recorded steps are multiples of this
+
+    def __init__(self, model: DecoderModel, dtype: torch.dtype, device: torch.device, use_graphs: bool = True):
         self.model = model
         self.dtype = dtype
         self.device = device
         self.workspace = Workspace(device)
         self._staging = _Staging()
         self._meta_dev: torch.Tensor | None = None
+        self.use_graphs = bool(use_graphs) and model.tree_graph_safe()
+        self.graph_replays = 0
 
     def new_cache(self, num_pages, page_size: int, max_requests: int) -> CacheContext:
         return CacheContext(self.model, num_pages, page_size, max_requests, self.dtype, self.device)
@@ -179,14 +192,49 @@ class ModelRunner:
             if not mgr.reserve(e.request_id, len(e.tokens)):
                 raise CapacityError(f"request {e.request_id!r}: pages ran out while reserving")
 
-        ctx, logit_rows = self._build_context(cache, entries)
-        logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
+        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            logits = self._decode_step_graphed(cache, entries)
+        else:
+            ctx, logit_rows = self._build_context(cache, entries)
+            logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
         for e in entries:
             mgr.commit(e.request_id, len(e.tokens))
         return logits
 
     # ------------------------------------------------------------------------------
-    def _build_context(self, cache: CacheContext, entries: Sequence[StepEntry]):
+    def _decode_step_graphed(self, cache: CacheContext, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """A step of single decoded tokens, all wanting logits: the launch sequence depends
+        only on the number of requests and on the width of the block tables, so it is
+        recorded once as a HIP graph and replayed; only the integer arrays change."""
+        page = cache.page_size
+        S = len(entries)
+        need = max((cache.manager.length(e.request_id) + page) // page for e in entries)
+        bucket = self.GRAPH_BLOCK_BUCKET
+        width = (need + bucket - 1) // bucket * bucket
+        key = (S, width)
+        rec = cache.graphs.get(key)
+        if rec is None:
+            # First time: run it plainly (this also sizes the scratch buffers), then record.
+            # The recorded step reads its integer arrays from a buffer of its own.
+            groups = len(cache.manager.groups)
+            meta = torch.empty(6 * S + 1 + groups * S * width + S + 64, dtype=torch.int32, device=self.device)
+            ctx, logit_rows = self._build_context(cache, entries, max_blocks=width, plan_len=width * page, dev=meta)
+            self.model.forward(ctx, cache.storage.layers, logit_rows)
+            torch.cuda.synchronize(self.device)
+            self.workspace.keep_replaced = True
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
+            cache.graphs[key] = rec = (graph, logits, ctx, meta)
+        else:
+            self._build_context(cache, entries, max_blocks=width, plan_len=width * page, dev=rec[3])
+        rec[0].replay()
+        self.graph_replays += 1
+        return rec[1]
+
+    # ------------------------------------------------------------------------------
+    def _build_context(self, cache: CacheContext, entries: Sequence[StepEntry], max_blocks: int | None = None,
+                       plan_len: int | None = None, dev: torch.Tensor | None = None):
         mgr = cache.manager
         page = cache.page_size
         S = len(entries)
@@ -194,7 +242,8 @@ class ModelRunner:
         ctx_lens = [mgr.length(e.request_id) for e in entries]
         T = sum(new_lens)
         groups = list(mgr.groups)
-        max_blocks = max(1, max((c + n + page - 1) // page for c, n in zip(ctx_lens, new_lens)))
+        if max_blocks is None:
+            max_blocks = max(1, max((c + n + page - 1) // page for c, n in zip(ctx_lens, new_lens)))
         wanted: list[int] = []
         row = 0
         for e, n in zip(entries, new_lens):
@@ -237,9 +286,12 @@ class ModelRunner:
         if R:
             h[offsets[-2]:offsets[-1]] = wanted
 
-        if self._meta_dev is None or self._meta_dev.numel() < total:
-            self._meta_dev = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
-        dev = self._meta_dev
+        if dev is None:
+            if self._meta_dev is None or self._meta_dev.numel() < total:
+                self._meta_dev = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
+            dev = self._meta_dev
+        elif dev.numel() < total:
+            raise RuntimeError("the recorded step's integer buffer is too small for this step")
         dev[:total].copy_(host[:total], non_blocking=True)
         self._staging.sent(idx)
 
@@ -252,6 +304,7 @@ class ModelRunner:
             ctx_len=view(4), slots=view(5),
             block_tables={g: view(6 + gi, (S, max_blocks)) for gi, g in enumerate(groups)},
             act_dtype=self.dtype, workspace=self.workspace, new_lens=new_lens, ctx_lens=ctx_lens,
-            slot_list=slot_list, max_position=max(c + n for c, n in zip(ctx_lens, new_lens)) - 1)
+            slot_list=slot_list, max_position=max(c + n for c, n in zip(ctx_lens, new_lens)) - 1,
+            plan_len=plan_len)
         logit_rows = view(len(sizes) - 1) if R else None
         return ctx, logit_rows

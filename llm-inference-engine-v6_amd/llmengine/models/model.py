@@ -29,6 +29,8 @@ class LayerCall:
 
 
 class DecoderModel(Part):
+    graph_safe = True
+
     def __init__(self, config, embedding: Embedding, layers: list[Block], final_norm: Norm,
                  head: OutputHead, schedule: list[LayerCall] | None = None, names: dict | None = None):
         self.config = config

@@ -65,14 +65,16 @@ def attention_bf16_supported(q, k_cache, head_dim: int) -> bool:
             and k_cache.data_ptr() % 16 == 0)
 
 
-def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int) -> dict:
-    """Launch sizes for a step, from how its batch is cut (host-side numbers only)."""
+def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_len: int | None = None) -> dict:
+    """Launch sizes for a step, from how its batch is cut (host-side numbers only). plan_len:
+    plan the decode splits for requests of up to this many tokens, whatever their length now
+    (a recorded step is replayed while the requests grow)."""
     rows = entry("llme_attention_bf16_rows")(head_dim)
     decode = [c + 1 for n, c in zip(new_lens, ctx_lens) if n == 1]
     groups = sum((n + rows - 1) // rows for n in new_lens if n >= 2)
     plan = {"n_decode": len(decode), "groups": groups, "split_len": 32, "nsplit": 1}
     if decode:
-        longest = max(decode)
+        longest = max(decode) if plan_len is None else max(plan_len, max(decode))
         pairs = len(decode) * n_kv * ((n_q // n_kv + 15) // 16)
         nsplit = max(1, min((DECODE_BLOCKS_WANTED + pairs - 1) // pairs, (longest + MIN_SPLIT - 1) // MIN_SPLIT))
         split_len = ((longest + nsplit - 1) // nsplit + 31) // 32 * 32
@@ -117,7 +119,7 @@ def _fast_attention(q, k_cache, v_cache, out, step, block_table, n_q, n_kv, head
     key = ("attention_plan", n_q, n_kv, head_dim)
     plan = step.extra.get(key)
     if plan is None:
-        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim)
+        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len)
     part_o = part_ml = None
     if plan["n_decode"] and plan["nsplit"] > 1:
         S = step.num_seqs

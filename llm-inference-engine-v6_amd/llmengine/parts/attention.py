@@ -22,6 +22,8 @@ from .registry import register_part
 
 
 class Attention(Mixer):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: PositionEncoding | None = None, scale: float | None = None, window: int = 0):
         if num_heads % num_kv_heads:

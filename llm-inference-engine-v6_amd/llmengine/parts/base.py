@@ -68,6 +68,12 @@ Getter = Callable[[str], torch.Tensor]      # local tensor name -> CPU tensor as
 
 
 class Part:
+    # True if forward() issues the same launches, with the same arguments, for every step of
+    # the same shape, reading what changes (tokens, positions, tables, slots) from the step's
+    # device arrays only. Steps of such parts can be recorded once and replayed as a HIP graph;
+    # a part that looks at the step's host-side lists while it runs must leave this False.
+    graph_safe = False
+
     def param_specs(self) -> dict[str, ParamSpec]:
         return {}
 
@@ -94,6 +100,9 @@ class Part:
         for name, child in self.children().items():
             out |= child.named_ignored(f"{prefix}{name}.")
         return out
+
+    def tree_graph_safe(self) -> bool:
+        return bool(self.graph_safe) and all(c.tree_graph_safe() for c in self.children().values())
 
     def load_tree(self, get: Getter, placement: Placement, prefix: str = "") -> None:
         self.load_params(lambda local: get(prefix + local), placement)

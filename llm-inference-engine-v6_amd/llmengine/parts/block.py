@@ -11,6 +11,8 @@ from .registry import register_part
 
 
 class PreNormBlock(Block):
+    graph_safe = True
+
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, ffn_norm: Norm,
                  names: dict | None = None):
         self.mixer, self.feed_forward = mixer, feed_forward

@@ -13,6 +13,8 @@ from .base import Getter, ParamSpec, Part, Placement
 
 
 class Embedding(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.weight: torch.Tensor | None = None
@@ -28,6 +30,8 @@ class Embedding(Part):
 
 
 class OutputHead(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int, tied_to: Embedding | None = None):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.tied_to = tied_to

@@ -15,6 +15,8 @@ from .registry import register_part
 
 
 class GatedMLP(FeedForward):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, intermediate_size: int):
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.group = 16 if self.intermediate_size % 16 == 0 else self.intermediate_size

@@ -11,6 +11,8 @@ from .registry import register_part
 
 
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, size: int, eps: float):
         self.size = int(size)
         self.eps = float(eps)

@@ -42,6 +42,8 @@ def inverse_frequencies(rotary_dim: int, theta: float, scaling: dict | None) -> 
 
 
 class RotaryEmbedding(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, rotary_dim: int, theta: float, max_position: int, scaling: dict | None = None):
         if rotary_dim % 2:
             raise ValueError(f"rotary_dim {rotary_dim} must be even")
