@@ -56,21 +56,21 @@ __device__ __forceinline__ bf16x8 zero_frag() {
     return z;
 }
 
-// One 32-key block for QT row tiles. HD: head size (compile time).
-//   t0: first key of the block (multiple of 32); keys outside [key_lo, key_end) are not
-//   loaded: behind key_end nothing is written yet, before key_lo (the first key any row
-//   of the work item may see) the pages may have been given back. row_pos[qt]: position of this lane's row (l % 16) in tile
-//   qt, or -1 for a row that does not exist; row_lo[qt]: first key the row may see.
-template <int HD, int QT>
-__device__ __forceinline__ void attend_block(const PagedKV& kv, int t0, int key_lo, int key_end, const bf16x8 (&qf)[QT][(HD + 31) / 32],
-                                             const int (&row_pos)[QT], const int (&row_lo)[QT], float scale_log2,
-                                             float (&m)[QT], float (&l)[QT], f32x4 (&o)[QT][HD / 16]) {
+// The K and V operands of one 32-key block (keys t0 .. t0 + 31), as one lane holds them.
+template <int HD>
+struct KVFrag {
+    bf16x8 kf[2][(HD + 31) / 32];      // row r of each 16-key half: dims c * 32 + 8 g4 ..
+    bf16x8 vf[HD / 16];                // dim dt * 16 + r: keys 4 g4 .. 4 g4 + 3 of each half
+};
+
+// Loads a block's operands. Keys outside [key_lo, key_end) are not loaded (zeros): behind
+// key_end nothing is written yet, before key_lo (the first key any row of the work item may
+// see) the pages may have been given back.
+template <int HD>
+__device__ __forceinline__ void load_block(const PagedKV& kv, int t0, int key_lo, int key_end, KVFrag<HD>& f) {
     constexpr int DC = (HD + 31) / 32, DT = HD / 16;
     const int lane = threadIdx.x & 63;
     const int r = lane & 15, g4 = lane >> 4;
-
-    // K fragments of the two 16-key halves: row r of each half
-    bf16x8 kf[2][DC];
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
         const int t = t0 + hf * 16 + r;
@@ -83,39 +83,46 @@ __device__ __forceinline__ void attend_block(const PagedKV& kv, int t0, int key_
 #pragma unroll
         for (int c = 0; c < DC; ++c) {
             const int d = c * 32 + g4 * 8;
-            kf[hf][c] = (ok && d < HD) ? *reinterpret_cast<const bf16x8*>(row + d) : zero_frag();
+            f.kf[hf][c] = (ok && d < HD) ? *reinterpret_cast<const bf16x8*>(row + d) : zero_frag();
         }
     }
-    // V fragments: for dimension dt * 16 + r, keys 4 g4 .. 4 g4 + 3 of each half
-    bf16x8 vf[DT];
-    {
-        const bf16* base[2];
-        bool ok[2];
+    const bf16* base[2];
+    bool ok[2];
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-            const int t = t0 + hf * 16 + g4 * 4;
-            ok[hf] = t + 3 >= key_lo && t < key_end;     // the 4 keys share a page with a visible key
-            base[hf] = nullptr;
-            if (ok[hf]) {
-                const int pg = kv.table[t / kv.page];
-                base[hf] = kv.v + (static_cast<size_t>(pg) * kv.n_kv + kv.kvh) * HD * kv.page + t % kv.page;
-            }
-        }
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const size_t off = static_cast<size_t>(dt * 16 + r) * kv.page;
-            bf16x4 lo4, hi4;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) lo4[e] = hi4[e] = static_cast<__bf16>(0.f);
-            if (ok[0]) lo4 = *reinterpret_cast<const bf16x4*>(base[0] + off);
-            if (ok[1]) hi4 = *reinterpret_cast<const bf16x4*>(base[1] + off);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                vf[dt][e] = lo4[e];
-                vf[dt][4 + e] = hi4[e];
-            }
+    for (int hf = 0; hf < 2; ++hf) {
+        const int t = t0 + hf * 16 + g4 * 4;
+        ok[hf] = t + 3 >= key_lo && t < key_end;     // the 4 keys share a page with a visible key
+        base[hf] = nullptr;
+        if (ok[hf]) {
+            const int pg = kv.table[t / kv.page];
+            base[hf] = kv.v + (static_cast<size_t>(pg) * kv.n_kv + kv.kvh) * HD * kv.page + t % kv.page;
         }
     }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        const size_t off = static_cast<size_t>(dt * 16 + r) * kv.page;
+        bf16x4 lo4, hi4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) lo4[e] = hi4[e] = static_cast<__bf16>(0.f);
+        if (ok[0]) lo4 = *reinterpret_cast<const bf16x4*>(base[0] + off);
+        if (ok[1]) hi4 = *reinterpret_cast<const bf16x4*>(base[1] + off);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            f.vf[dt][e] = lo4[e];
+            f.vf[dt][4 + e] = hi4[e];
+        }
+    }
+}
+
+// One 32-key block for QT row tiles. row_pos[qt]: position of this lane's row (l % 16) in
+// tile qt, or -1 for a row that does not exist; row_lo[qt]: first key the row may see.
+template <int HD, int QT>
+__device__ __forceinline__ void attend_block(const KVFrag<HD>& f, int t0, const bf16x8 (&qf)[QT][(HD + 31) / 32],
+                                             const int (&row_pos)[QT], const int (&row_lo)[QT], float scale_log2,
+                                             float (&m)[QT], float (&l)[QT], f32x4 (&o)[QT][HD / 16]) {
+    constexpr int DC = (HD + 31) / 32, DT = HD / 16;
+    const int lane = threadIdx.x & 63;
+    const int g4 = lane >> 4;
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
         f32x4 s[2];
@@ -124,7 +131,7 @@ __device__ __forceinline__ void attend_block(const PagedKV& kv, int t0, int key_
             s[hf] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < DC; ++c)
-                s[hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[hf][c], qf[qt][c], s[hf], 0, 0, 0);
+                s[hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.kf[hf][c], qf[qt][c], s[hf], 0, 0, 0);
         }
         // this lane: row r of tile qt, keys t0 + 16 hf + 4 g4 + e
         const int pos = row_pos[qt], lo = row_lo[qt];
@@ -163,8 +170,26 @@ __device__ __forceinline__ void attend_block(const PagedKV& kv, int t0, int key_
         for (int dt = 0; dt < DT; ++dt) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) o[qt][dt][e] *= ar[e];
-            o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf[dt], o[qt][dt], 0, 0, 0);
+            o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, f.vf[dt], o[qt][dt], 0, 0, 0);
         }
+    }
+}
+
+// Walks the 32-key blocks t0 = first, first + stride, ... < key_end, the next block's loads
+// in flight while the current block is computed.
+template <int HD, int QT>
+__device__ __forceinline__ void attend_range(const PagedKV& kv, int first, int stride, int key_lo, int key_end,
+                                             const bf16x8 (&qf)[QT][(HD + 31) / 32], const int (&row_pos)[QT],
+                                             const int (&row_lo)[QT], float scale_log2, float (&m)[QT],
+                                             float (&l)[QT], f32x4 (&o)[QT][HD / 16]) {
+    if (first >= key_end) return;
+    KVFrag<HD> cur, nxt;
+    load_block<HD>(kv, first, key_lo, key_end, cur);
+    for (int t0 = first; t0 < key_end; t0 += stride) {
+        const bool more = t0 + stride < key_end;
+        if (more) load_block<HD>(kv, t0 + stride, key_lo, key_end, nxt);
+        attend_block<HD, QT>(cur, t0, qf, row_pos, row_lo, scale_log2, m, l, o);
+        if (more) cur = nxt;
     }
 }
 
@@ -180,22 +205,28 @@ __device__ __forceinline__ void load_q(const bf16* qrow, bool ok, bf16x8 (&qf)[(
 }
 
 // ------------------------------------------------------------------------------------------
-// decode: one token per request
+// decode: one token per request. A workgroup of four wavefronts takes one split of the keys
+// of one (request, kv head, tile of 16 query heads); its wavefronts take every fourth
+// 32-key block and add up through LDS.
+constexpr int DEC_WAVES = 4;
+
 template <int HD>
-__global__ __launch_bounds__(64) void attention_decode_kernel(
+__global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     bf16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
     int max_blocks, int n_q, int n_kv, int page, float scale, int window, int split_len, int nsplit) {
     constexpr int DC = (HD + 31) / 32, DT = HD / 16;
+    __shared__ float sh_o[DEC_WAVES][16][HD];
+    __shared__ float sh_m[DEC_WAVES][16], sh_l[DEC_WAVES][16];
     const int s = blockIdx.x;
     const int row0 = q_start[s];
-    if (q_start[s + 1] - row0 != 1) return;            // not a decoding request
+    if (q_start[s + 1] - row0 != 1) return;            // not a decoding request (whole workgroup)
     const int G = n_q / n_kv;
     const int gtiles = (G + 15) / 16;
     const int kvh = blockIdx.y / gtiles, gt = blockIdx.y % gtiles;
     const int split = blockIdx.z;
-    const int lane = threadIdx.x & 63, r = lane & 15, g4 = lane >> 4;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g4 = lane >> 4;
 
     const int pos = ctx_len[s];                         // the token's position; it sees keys lo..pos
     const int lo_all = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
@@ -215,60 +246,80 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD};
-    const float scale_log2 = scale * kLog2e;
-    for (int t0 = k_begin; t0 < k_end; t0 += 32)
-        attend_block<HD, 1>(kv, t0, lo_all, k_end, qf, row_pos, row_lo, scale_log2, m, l, o);
+    attend_range<HD, 1>(kv, k_begin + wave * 32, DEC_WAVES * 32, lo_all, k_end, qf, row_pos, row_lo,
+                        scale * kLog2e, m, l, o);
 
     float lt = l[0];
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
-    // O's rows are heads gt * 16 + 4 g4 + e; statistics sit in the lanes whose r is that row
+    if (g4 == 0) {
+        sh_m[wave][r] = m[0];
+        sh_l[wave][r] = lt;
+    }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const int rr = g4 * 4 + e;
-        const float l_row = __shfl(lt, rr, 64), m_row = __shfl(m[0], rr, 64);
-        if (gt * 16 + rr >= G) continue;
-        const int h = kvh * G + gt * 16 + rr;
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sh_o[wave][g4 * 4 + e][dt * 16 + r] = o[0][dt][e];
+    __syncthreads();
+    // join the wavefronts: thread -> (row, dims)
+    for (int item = threadIdx.x; item < 16 * HD; item += DEC_WAVES * 64) {
+        const int row = item / HD, d = item % HD;
+        if (gt * 16 + row >= G) continue;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; ++w) mx = fmaxf(mx, sh_m[w][row]);
+        float acc = 0.f, lsum = 0.f;
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; ++w) {
+            const float mw = sh_m[w][row];
+            const float f = (mw == -INFINITY) ? 0.f : exp2f(mw - mx);
+            acc += f * sh_o[w][row][d];
+            lsum += f * sh_l[w][row];
+        }
+        const int h = kvh * G + gt * 16 + row;
         if (nsplit == 1) {
-            const float inv = 1.0f / l_row;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-                out[(static_cast<size_t>(row0) * n_q + h) * HD + dt * 16 + r] = static_cast<bf16>(o[0][dt][e] * inv);
+            out[(static_cast<size_t>(row0) * n_q + h) * HD + d] = static_cast<bf16>(acc / lsum);
         } else {
             const size_t pidx = (static_cast<size_t>(s) * n_q + h) * nsplit + split;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) part_o[pidx * HD + dt * 16 + r] = o[0][dt][e];
-            if (r == 0) {
-                part_ml[pidx * 2] = m_row;
-                part_ml[pidx * 2 + 1] = l_row;
+            part_o[pidx * HD + d] = acc;
+            if (d == 0) {
+                part_ml[pidx * 2] = mx;
+                part_ml[pidx * 2 + 1] = lsum;
             }
         }
     }
 }
 
-// joins the splits of the decode kernel: grid (request, head), 64 lanes over the head's dims
+// joins the splits of the decode kernel: grid (request, head); lanes over the splits for the
+// statistics, then over the head's dimensions for the weighted sum. nsplit <= 64.
 __global__ __launch_bounds__(64) void attention_join_kernel(const float* __restrict__ part_o,
                                                             const float* __restrict__ part_ml, bf16* __restrict__ out,
                                                             const int* __restrict__ q_start, int n_q, int hd, int nsplit) {
-    const int s = blockIdx.x, h = blockIdx.y;
+    __shared__ float weight[64];
+    const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int row0 = q_start[s];
     if (q_start[s + 1] - row0 != 1) return;
     const size_t base = (static_cast<size_t>(s) * n_q + h) * nsplit;
-    float mx = -INFINITY;
-    for (int i = 0; i < nsplit; ++i) mx = fmaxf(mx, part_ml[(base + i) * 2]);
-    float total = 0.f;
-    for (int i = 0; i < nsplit; ++i) {
-        const float mi = part_ml[(base + i) * 2];
-        if (mi != -INFINITY) total += exp2f(mi - mx) * part_ml[(base + i) * 2 + 1];
+    float mi = -INFINITY, li = 0.f;
+    if (lane < nsplit) {
+        mi = part_ml[(base + lane) * 2];
+        li = part_ml[(base + lane) * 2 + 1];
     }
-    const float inv = 1.0f / total;
-    for (int d = threadIdx.x; d < hd; d += 64) {
+    const float mx = wave_max(mi);
+    const float f = (mi == -INFINITY) ? 0.f : exp2f(mi - mx);
+    const float total = wave_sum(f * li);
+    weight[lane] = f / total;
+    __syncthreads();
+    for (int d = lane; d < hd; d += 64) {
         float acc = 0.f;
-        for (int i = 0; i < nsplit; ++i) {
-            const float mi = part_ml[(base + i) * 2];
-            if (mi != -INFINITY) acc += exp2f(mi - mx) * part_o[(base + i) * hd + d];
+        int i = 0;
+        for (; i + 4 <= nsplit; i += 4) {
+            const float a0 = part_o[(base + i) * hd + d], a1 = part_o[(base + i + 1) * hd + d];
+            const float a2 = part_o[(base + i + 2) * hd + d], a3 = part_o[(base + i + 3) * hd + d];
+            acc += weight[i] * a0 + weight[i + 1] * a1 + weight[i + 2] * a2 + weight[i + 3] * a3;
         }
-        out[(static_cast<size_t>(row0) * n_q + h) * hd + d] = static_cast<bf16>(acc * inv);
+        for (; i < nsplit; ++i) acc += weight[i] * part_o[(base + i) * hd + d];
+        out[(static_cast<size_t>(row0) * n_q + h) * hd + d] = static_cast<bf16>(acc);
     }
 }
 
@@ -324,8 +375,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     const int k_begin = key_lo & ~31;
     PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD};
     const float scale_log2 = scale * kLog2e;
-    for (int t0 = k_begin; t0 < key_end; t0 += 32)
-        attend_block<HD, QT>(kv, t0, key_lo, key_end, qf, row_pos, row_lo, scale_log2, m, l, o);
+    attend_range<HD, QT>(kv, k_begin, 32, key_lo, key_end, qf, row_pos, row_lo, scale_log2, m, l, o);
 
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
@@ -355,7 +405,7 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
     if (n_decode > 0) {
         const int G = n_q / n_kv;
         const dim3 grid(n_seq, n_kv * ((G + 15) / 16), nsplit);
-        hipLaunchKernelGGL((attention_decode_kernel<HD>), grid, dim3(64), 0, stream, q, kc, vc, out, part_o, part_ml,
+        hipLaunchKernelGGL((attention_decode_kernel<HD>), grid, dim3(DEC_WAVES * 64), 0, stream, q, kc, vc, out, part_o, part_ml,
                            q_start, ctx_len, table, max_blocks, n_q, n_kv, page, scale, window, split_len, nsplit);
         if (nsplit > 1)
             hipLaunchKernelGGL(attention_join_kernel, dim3(n_seq, n_q), dim3(64), 0, stream, part_o, part_ml, out,
@@ -392,7 +442,7 @@ extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const voi
                                    hipStream_t stream) {
     if (n_seq <= 0) return 0;
     if (hd % 16 != 0 || hd > 128 || hd <= 0 || page % 16 != 0 || n_kv <= 0 || n_q % n_kv != 0) return kErrUnsupported;
-    if (n_decode > 0 && (split_len <= 0 || split_len % 32 != 0 || nsplit <= 0)) return kErrBadArgument;
+    if (n_decode > 0 && (split_len <= 0 || split_len % 32 != 0 || nsplit <= 0 || nsplit > 64)) return kErrBadArgument;
     const int qt = llme_attention_bf16_rows(hd) / 16;
 #define LLME_HEAD(HD)                                                                                           \
     case HD:                                                                                                    \

@@ -30,16 +30,41 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict
     const int r = blockIdx.x;
     const int src = rows ? rows[r] : r;
     const float* xr = x + static_cast<size_t>(src) * H;
+    TO* o = out + static_cast<size_t>(r) * H;
+    // Rows of up to 8 * blockDim values whose length is a multiple of 4 stay in registers
+    // between the two passes (two 16-byte loads per thread); others are read twice.
+    const bool in_regs = (H % 4 == 0) && (H <= 8 * static_cast<int>(blockDim.x));
+    float4 v[2];
     float ss = 0.f;
-    for (int i = threadIdx.x; i < H; i += blockDim.x) {
-        const float v = xr[i];
-        ss += v * v;
+    if (in_regs) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int i = (threadIdx.x + j * blockDim.x) * 4;
+            v[j] = (i < H) ? *reinterpret_cast<const float4*>(xr + i) : float4{0.f, 0.f, 0.f, 0.f};
+            ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+        }
+    } else {
+        for (int i = threadIdx.x; i < H; i += blockDim.x) {
+            const float t = xr[i];
+            ss += t * t;
+        }
     }
     ss = block_sum(ss, scratch, blockDim.x / kWave);
     const float inv = 1.0f / sqrtf(ss / static_cast<float>(H) + eps);
-    TO* o = out + static_cast<size_t>(r) * H;
-    for (int i = threadIdx.x; i < H; i += blockDim.x)
-        o[i] = from_float<TO>((to_float(w[i]) * xr[i]) * inv);
+    if (in_regs) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int i = (threadIdx.x + j * blockDim.x) * 4;
+            if (i >= H) continue;
+            o[i] = from_float<TO>((to_float(w[i]) * v[j].x) * inv);
+            o[i + 1] = from_float<TO>((to_float(w[i + 1]) * v[j].y) * inv);
+            o[i + 2] = from_float<TO>((to_float(w[i + 2]) * v[j].z) * inv);
+            o[i + 3] = from_float<TO>((to_float(w[i + 3]) * v[j].w) * inv);
+        }
+    } else {
+        for (int i = threadIdx.x; i < H; i += blockDim.x)
+            o[i] = from_float<TO>((to_float(w[i]) * xr[i]) * inv);
+    }
 }
 
 // ---------------------------------------------------------------------------------

@@ -32,15 +32,40 @@ __device__ __forceinline__ void block_argmax(float& bv, int& bi, float* sv, int*
     for (int i = 1; i < kSampleThreads / kWave; ++i) argmax_combine(bv, bi, sv[i], si[i]);
 }
 
-__global__ __launch_bounds__(kSampleThreads) void argmax_kernel(const float* __restrict__ logits,
-                                                                int* __restrict__ out, int V) {
+// Greedy choice in two stages, so that a few rows of a large vocabulary still fill the chip:
+// grid (row, part): each workgroup takes a contiguous part of the row and writes its
+// (maximum, first index); a second small kernel joins the parts.
+__global__ __launch_bounds__(kSampleThreads) void argmax_part_kernel(const float* __restrict__ logits,
+                                                                     float* __restrict__ part_val,
+                                                                     int* __restrict__ part_idx, int V, int chunk) {
     __shared__ float sv[kSampleThreads / kWave];
     __shared__ int si[kSampleThreads / kWave];
     const float* row = logits + static_cast<size_t>(blockIdx.x) * V;
+    const int begin = blockIdx.y * chunk;
+    const int end = (begin + chunk < V) ? begin + chunk : V;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += kSampleThreads) argmax_combine(bv, bi, row[i], i);
+    for (int i = begin + threadIdx.x; i < end; i += kSampleThreads) argmax_combine(bv, bi, row[i], i);
     block_argmax(bv, bi, sv, si);
+    if (threadIdx.x == 0) {
+        part_val[blockIdx.x * gridDim.y + blockIdx.y] = bv;
+        part_idx[blockIdx.x * gridDim.y + blockIdx.y] = bi;
+    }
+}
+
+__global__ __launch_bounds__(kWave) void argmax_join_kernel(const float* __restrict__ part_val,
+                                                            const int* __restrict__ part_idx, int* __restrict__ out,
+                                                            int parts) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int p = threadIdx.x; p < parts; p += kWave)
+        argmax_combine(bv, bi, part_val[blockIdx.x * parts + p], part_idx[blockIdx.x * parts + p]);
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, kWave);
+        const int oi = __shfl_xor(bi, off, kWave);
+        argmax_combine(bv, bi, ov, oi);
+    }
     if (threadIdx.x == 0) out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
 }
 
@@ -101,10 +126,22 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __r
 
 using namespace llme;
 
-extern "C" int llme_argmax(const float* logits, int* out, int R, int V, hipStream_t stream) {
+// Parts per row that llme_argmax uses for a vocabulary size: the caller provides scratch for
+// R * parts floats and ints.
+extern "C" int llme_argmax_parts(int V) {
+    const int parts = (V + 2047) / 2048;
+    return parts < 1 ? 1 : (parts > 64 ? 64 : parts);
+}
+
+extern "C" int llme_argmax(const float* logits, int* out, float* part_val, int* part_idx, int R, int V,
+                           hipStream_t stream) {
     if (R <= 0) return 0;
     if (V <= 0) return kErrBadArgument;
-    hipLaunchKernelGGL(argmax_kernel, dim3(R), dim3(kSampleThreads), 0, stream, logits, out, V);
+    const int parts = llme_argmax_parts(V);
+    const int chunk = (V + parts - 1) / parts;
+    hipLaunchKernelGGL(argmax_part_kernel, dim3(R, parts), dim3(kSampleThreads), 0, stream, logits, part_val,
+                       part_idx, V, chunk);
+    hipLaunchKernelGGL(argmax_join_kernel, dim3(R), dim3(kWave), 0, stream, part_val, part_idx, out, parts);
     return launch_status();
 }
 

@@ -175,11 +175,21 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out
 
 
 # --- sampling ------------------------------------------------------------------------
+_argmax_scratch: dict = {}
+
+
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    """out[r] = first index of the maximum of logits[r, :]."""
     require(logits, "logits", torch.float32, (None, None))
     R, V = logits.shape
     require(out, "out", torch.int32, (R,))
-    check(entry("llme_argmax")(ptr(logits), ptr(out), R, V, stream()), "argmax")
+    need = R * entry("llme_argmax_parts")(V)
+    scratch = _argmax_scratch.get(logits.device)
+    if scratch is None or scratch[0].numel() < need:
+        scratch = (torch.empty(max(need, 4096), dtype=torch.float32, device=logits.device),
+                   torch.empty(max(need, 4096), dtype=torch.int32, device=logits.device))
+        _argmax_scratch[logits.device] = scratch
+    check(entry("llme_argmax")(ptr(logits), ptr(out), ptr(scratch[0]), ptr(scratch[1]), R, V, stream()), "argmax")
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor) -> None:

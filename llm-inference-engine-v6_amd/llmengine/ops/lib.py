@@ -38,7 +38,8 @@ _SIGNATURES = {
     "llme_gemm_generic": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
     "llme_attention_generic": [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
                                _f, _i, _vp],
-    "llme_argmax": [_vp, _vp, _i, _i, _vp],
+    "llme_argmax": [_vp, _vp, _vp, _vp, _i, _i, _vp],
+    "llme_argmax_parts": [_i],
     "llme_sample": [_vp, _vp, _vp, _vp, _i, _i, _vp],
 }
 

@@ -55,8 +55,9 @@ declare("llme_attention_bf16_rows", [_i])
 declare("llme_attention_bf16", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i,
                                 _i, _i, _i, _i, _vp])
 
-DECODE_BLOCKS_WANTED = 2048         # workgroups the decode kernel should have to fill the chip
-MIN_SPLIT = 64                      # keys per split at least
+DECODE_BLOCKS_WANTED = 1024         # workgroups (of four wavefronts) the decode kernel should have
+MIN_SPLIT = 128                     # keys per split at least: one 32-key block per wavefront
+MAX_SPLITS = 64                     # the join kernel's limit
 
 
 def attention_bf16_supported(q, k_cache, head_dim: int) -> bool:
@@ -76,7 +77,8 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
     if decode:
         longest = max(decode) if plan_len is None else max(plan_len, max(decode))
         pairs = len(decode) * n_kv * ((n_q // n_kv + 15) // 16)
-        nsplit = max(1, min((DECODE_BLOCKS_WANTED + pairs - 1) // pairs, (longest + MIN_SPLIT - 1) // MIN_SPLIT))
+        nsplit = max(1, min((DECODE_BLOCKS_WANTED + pairs - 1) // pairs, (longest + MIN_SPLIT - 1) // MIN_SPLIT,
+                            MAX_SPLITS))
         split_len = ((longest + nsplit - 1) // nsplit + 31) // 32 * 32
         plan["split_len"] = split_len
         plan["nsplit"] = (longest + split_len - 1) // split_len
