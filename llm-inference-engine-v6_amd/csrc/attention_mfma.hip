@@ -63,11 +63,29 @@ struct KVFrag {
     bf16x8 vf[HD / 16];                // dim dt * 16 + r: keys 4 g4 .. 4 g4 + 3 of each half
 };
 
-// Loads a block's operands. Keys outside [key_lo, key_end) are not loaded (zeros): behind
-// key_end nothing is written yet, before key_lo (the first key any row of the work item may
-// see) the pages may have been given back.
+// The pages of a block's two 16-key halves (a half never straddles pages: the page size is a
+// multiple of 16). A half none of whose keys lies in [key_lo, key_end) is not looked up: behind
+// key_end nothing is written yet (and the table may end), before key_lo (the first key any
+// row of the work item may see) the pages may have been given back.
+struct BlockPages {
+    int pg[2];
+};
+
+__device__ __forceinline__ BlockPages lookup_pages(const PagedKV& kv, int t0, int key_lo, int key_end) {
+    BlockPages b;
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+        const int h0 = t0 + hf * 16;
+        b.pg[hf] = (h0 < key_end && h0 + 15 >= key_lo) ? kv.table[h0 / kv.page] : 0;
+    }
+    return b;
+}
+
+// Loads a block's operands from the pages looked up before. Keys outside [key_lo, key_end)
+// are not loaded (zeros).
 template <int HD>
-__device__ __forceinline__ void load_block(const PagedKV& kv, int t0, int key_lo, int key_end, KVFrag<HD>& f) {
+__device__ __forceinline__ void load_block(const PagedKV& kv, int t0, const BlockPages& pages, int key_lo, int key_end,
+                                           KVFrag<HD>& f) {
     constexpr int DC = (HD + 31) / 32, DT = HD / 16;
     const int lane = threadIdx.x & 63;
     const int r = lane & 15, g4 = lane >> 4;
@@ -75,11 +93,7 @@ __device__ __forceinline__ void load_block(const PagedKV& kv, int t0, int key_lo
     for (int hf = 0; hf < 2; ++hf) {
         const int t = t0 + hf * 16 + r;
         const bool ok = t >= key_lo && t < key_end;
-        const bf16* row = nullptr;
-        if (ok) {
-            const int pg = kv.table[t / kv.page];
-            row = kv.k + ((static_cast<size_t>(pg) * kv.n_kv + kv.kvh) * kv.page + t % kv.page) * HD;
-        }
+        const bf16* row = kv.k + ((static_cast<size_t>(pages.pg[hf]) * kv.n_kv + kv.kvh) * kv.page + t % kv.page) * HD;
 #pragma unroll
         for (int c = 0; c < DC; ++c) {
             const int d = c * 32 + g4 * 8;
@@ -92,11 +106,7 @@ __device__ __forceinline__ void load_block(const PagedKV& kv, int t0, int key_lo
     for (int hf = 0; hf < 2; ++hf) {
         const int t = t0 + hf * 16 + g4 * 4;
         ok[hf] = t + 3 >= key_lo && t < key_end;     // the 4 keys share a page with a visible key
-        base[hf] = nullptr;
-        if (ok[hf]) {
-            const int pg = kv.table[t / kv.page];
-            base[hf] = kv.v + (static_cast<size_t>(pg) * kv.n_kv + kv.kvh) * HD * kv.page + t % kv.page;
-        }
+        base[hf] = kv.v + (static_cast<size_t>(pages.pg[hf]) * kv.n_kv + kv.kvh) * HD * kv.page + t % kv.page;
     }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
@@ -115,11 +125,15 @@ __device__ __forceinline__ void load_block(const PagedKV& kv, int t0, int key_lo
 }
 
 // One 32-key block for QT row tiles. row_pos[qt]: position of this lane's row (l % 16) in
-// tile qt, or -1 for a row that does not exist; row_lo[qt]: first key the row may see.
+// tile qt, or -1 for a row that does not exist; row_lo[qt]: first key the row may see;
+// tile_free[qt]: the last key every row of tile qt sees without a check (the position of its
+// first row if all 16 rows exist and there is no window, else -1): blocks that end at or
+// before it skip the masking.
 template <int HD, int QT>
 __device__ __forceinline__ void attend_block(const KVFrag<HD>& f, int t0, const bf16x8 (&qf)[QT][(HD + 31) / 32],
-                                             const int (&row_pos)[QT], const int (&row_lo)[QT], float scale_log2,
-                                             float (&m)[QT], float (&l)[QT], f32x4 (&o)[QT][HD / 16]) {
+                                             const int (&row_pos)[QT], const int (&row_lo)[QT],
+                                             const int (&tile_free)[QT], float scale_log2, float (&m)[QT],
+                                             float (&l)[QT], f32x4 (&o)[QT][HD / 16]) {
     constexpr int DC = (HD + 31) / 32, DT = HD / 16;
     const int lane = threadIdx.x & 63;
     const int g4 = lane >> 4;
@@ -134,18 +148,28 @@ __device__ __forceinline__ void attend_block(const KVFrag<HD>& f, int t0, const 
                 s[hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.kf[hf][c], qf[qt][c], s[hf], 0, 0, 0);
         }
         // this lane: row r of tile qt, keys t0 + 16 hf + 4 g4 + e
-        const int pos = row_pos[qt], lo = row_lo[qt];
         float mx = -INFINITY;
+        if (t0 + 31 <= tile_free[qt]) {
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf)
+            for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int t = t0 + hf * 16 + g4 * 4 + e;
-                const bool see = (t <= pos) && (t >= lo);
-                const float v = see ? s[hf][e] * scale_log2 : -INFINITY;
-                s[hf][e] = v;
-                mx = fmaxf(mx, v);
-            }
+                for (int e = 0; e < 4; ++e) {
+                    s[hf][e] *= scale_log2;
+                    mx = fmaxf(mx, s[hf][e]);
+                }
+        } else {
+            const int pos = row_pos[qt], lo = row_lo[qt];
+#pragma unroll
+            for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int t = t0 + hf * 16 + g4 * 4 + e;
+                    const bool see = (t <= pos) && (t >= lo);
+                    const float v = see ? s[hf][e] * scale_log2 : -INFINITY;
+                    s[hf][e] = v;
+                    mx = fmaxf(mx, v);
+                }
+        }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m[qt], mx);
@@ -163,33 +187,40 @@ __device__ __forceinline__ void attend_block(const KVFrag<HD>& f, int t0, const 
                 pf[hf * 4 + e] = static_cast<__bf16>(p);
             }
         l[qt] = l[qt] * alpha + psum;
-        float ar[4];
+        if (__any(alpha != 1.0f)) {                    // some row's maximum moved: rescale what is summed
+            float ar[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) ar[e] = __shfl(alpha, g4 * 4 + e, 64);     // factor of O's row 4 g4 + e
+            for (int e = 0; e < 4; ++e) ar[e] = __shfl(alpha, g4 * 4 + e, 64);     // factor of O's row 4 g4 + e
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
+            for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[qt][dt][e] *= ar[e];
-            o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, f.vf[dt], o[qt][dt], 0, 0, 0);
+                for (int e = 0; e < 4; ++e) o[qt][dt][e] *= ar[e];
         }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, f.vf[dt], o[qt][dt], 0, 0, 0);
     }
 }
 
-// Walks the 32-key blocks t0 = first, first + stride, ... < key_end, the next block's loads
-// in flight while the current block is computed.
+// Walks the 32-key blocks t0 = first, first + stride, ... < key_end: the next block's loads
+// are in flight while the current block is computed, and the page ids are looked up one block
+// further ahead, so that no load waits for a table entry.
 template <int HD, int QT>
 __device__ __forceinline__ void attend_range(const PagedKV& kv, int first, int stride, int key_lo, int key_end,
                                              const bf16x8 (&qf)[QT][(HD + 31) / 32], const int (&row_pos)[QT],
-                                             const int (&row_lo)[QT], float scale_log2, float (&m)[QT],
-                                             float (&l)[QT], f32x4 (&o)[QT][HD / 16]) {
+                                             const int (&row_lo)[QT], const int (&tile_free)[QT], float scale_log2,
+                                             float (&m)[QT], float (&l)[QT], f32x4 (&o)[QT][HD / 16]) {
     if (first >= key_end) return;
     KVFrag<HD> cur, nxt;
-    load_block<HD>(kv, first, key_lo, key_end, cur);
+    BlockPages pg_next = lookup_pages(kv, first + stride, key_lo, key_end);
+    load_block<HD>(kv, first, lookup_pages(kv, first, key_lo, key_end), key_lo, key_end, cur);
     for (int t0 = first; t0 < key_end; t0 += stride) {
         const bool more = t0 + stride < key_end;
-        if (more) load_block<HD>(kv, t0 + stride, key_lo, key_end, nxt);
-        attend_block<HD, QT>(cur, t0, qf, row_pos, row_lo, scale_log2, m, l, o);
+        const BlockPages pg_after = lookup_pages(kv, t0 + 2 * stride, key_lo, key_end);
+        if (more) load_block<HD>(kv, t0 + stride, pg_next, key_lo, key_end, nxt);
+        attend_block<HD, QT>(cur, t0, qf, row_pos, row_lo, tile_free, scale_log2, m, l, o);
         if (more) cur = nxt;
+        pg_next = pg_after;
     }
 }
 
@@ -240,14 +271,16 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     load_q<HD>(q + (static_cast<size_t>(row0) * n_q + (row_ok ? head : 0)) * HD, row_ok, qf[0]);
     const int row_pos[1] = {row_ok ? pos : -1};
     const int row_lo[1] = {lo_all};
+    const int tile_free[1] = {-1};                      // few blocks, heads may be missing: always checked
     float m[1] = {-INFINITY}, l[1] = {0.f};
     f32x4 o[1][DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD};
-    attend_range<HD, 1>(kv, k_begin + wave * 32, DEC_WAVES * 32, lo_all, k_end, qf, row_pos, row_lo,
-                        scale * kLog2e, m, l, o);
+    const int first = k_begin + __builtin_amdgcn_readfirstlane(wave) * 32;
+    attend_range<HD, 1>(kv, first, DEC_WAVES * 32, lo_all, k_end, qf, row_pos, row_lo, tile_free, scale * kLog2e,
+                        m, l, o);
 
     float lt = l[0];
     lt += __shfl_xor(lt, 16, 64);
@@ -340,7 +373,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
         const int nt = (n >= 2) ? (n + ROWS - 1) / ROWS : 0;
         if (!found && static_cast<int>(blockIdx.x) < acc + nt) {
             s = i;
-            first = (blockIdx.x - acc) * ROWS;           // first row of the group within the request
+            first = (nt - 1 - (blockIdx.x - acc)) * ROWS; // first row of the group within the request; the
+                                                          // last groups see the most keys and start first
             n_rows = n - first < ROWS ? n - first : ROWS;
             first += a;                                   // as a batch row
             found = true;
@@ -355,7 +389,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     const int pos0 = ctx_len[s] + (first - q_start[s]);  // position of the group's first row
 
     bf16x8 qf[QT][DC];
-    int row_pos[QT], row_lo[QT];
+    int row_pos[QT], row_lo[QT], tile_free[QT];
     float m[QT], l[QT];
     f32x4 o[QT][DT];
 #pragma unroll
@@ -365,6 +399,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
         load_q<HD>(q + (static_cast<size_t>(first + (ok ? rr : 0)) * n_q + head) * HD, ok, qf[qt]);
         row_pos[qt] = ok ? pos0 + rr : -1;
         row_lo[qt] = (window > 0 && pos0 + rr - window + 1 > 0) ? pos0 + rr - window + 1 : 0;
+        tile_free[qt] = (window == 0 && qt * 16 + 16 <= n_rows) ? pos0 + qt * 16 : -1;
         m[qt] = -INFINITY;
         l[qt] = 0.f;
 #pragma unroll
@@ -375,7 +410,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     const int k_begin = key_lo & ~31;
     PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD};
     const float scale_log2 = scale * kLog2e;
-    attend_range<HD, QT>(kv, k_begin, 32, key_lo, key_end, qf, row_pos, row_lo, scale_log2, m, l, o);
+    attend_range<HD, QT>(kv, k_begin, 32, key_lo, key_end, qf, row_pos, row_lo, tile_free, scale_log2, m, l, o);
 
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {

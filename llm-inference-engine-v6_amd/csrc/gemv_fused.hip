@@ -1,0 +1,236 @@
+// Decode-time projections fused with the RMSNorm in front of them (and, for the gated
+// feed-forward, with the activation behind them), for up to 16 rows:
+//
+//   plain:  out[m, n]  = inv_m * sum_k bf16(w_norm[k] * h[row(m), k]) * W[n, k]
+//   gated:  out[m, j]  = silu(g) * u,  g, u = the same sums over the gate and the up row of unit j
+//   inv_m = 1 / sqrt(mean_k h[row(m), k]^2 + eps)          (src/kernels.cpp:18-24, 26-31, 33-57)
+//
+// The norm's scale is a factor per row, so it is applied to the 32-bit sums after the product;
+// the activations enter the product as bf16(w_norm * h). h is the 32-bit residual stream,
+// row(m) = rows ? rows[m] : m (the output head reads the wanted rows only).
+//
+// A workgroup first puts bf16(w_norm * h) of all rows into LDS, each wavefront summing the
+// squares of its rows, while its first weight loads are already in flight. It then works
+// through tiles of 16 output columns (gated: the 16 gate and the 16 up rows of 16 units, which
+// lie next to each other in the interleaved weight matrix), TPR tiles at a time: NW / TPR
+// wavefronts share a tile, each streaming every (NW / TPR)-th 128-element chunk of k of the
+// tile's weight rows from HBM straight into MFMA operand registers, the next chunk's loads
+// issued before the current chunk's products; the partial sums are added through LDS, scaled
+// by inv_m and stored. The grid is sized so that the prologue is paid once per several tiles.
+//
+// Limits (checked by the caller): M <= 16, K a multiple of 8, 16 * (K + 8) * 2 bytes of LDS.
+#include "common.h"
+#include <math.h>
+
+namespace llme {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int GV_U = 4;                 // 32-element k steps per chunk
+constexpr int GV_CHUNK = 32 * GV_U;     // 128
+
+__device__ __forceinline__ bf16x8 gv_zero8() {
+    bf16x8 z;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) z[i] = static_cast<__bf16>(0.f);
+    return z;
+}
+
+template <int NW, int TPR, bool GATED, typename TNW>
+__global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restrict__ h, const int* __restrict__ rows,
+                                                            const TNW* __restrict__ norm_w, float eps,
+                                                            const bf16* __restrict__ w, void* __restrict__ out,
+                                                            int M, int N, int K, int tiles) {
+    constexpr int NT = GATED ? 2 : 1;                   // weight fragments per k step
+    constexpr int KS = NW / TPR;                        // wavefronts that share a tile, splitting k
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    const int XS = K + 8;                               // padded row of the activation tile (elements)
+    bf16* xs = reinterpret_cast<bf16*>(lds_raw);                                    // [16][XS]
+    f32x4* red = reinterpret_cast<f32x4*>(lds_raw + static_cast<size_t>(16) * XS * 2);   // [NW][NT][64]
+    float* ssum = reinterpret_cast<float*>(red + NW * NT * 64);                      // [16]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane & 15, q = lane >> 4;
+    const int slot = wave / KS, kpart = wave % KS;      // which of the round's tiles, which share of k
+    const int n_rows_w = GATED ? 2 * N : N;             // rows of the weight matrix
+    const int n_chunks = (K + GV_CHUNK - 1) / GV_CHUNK;
+    const int rounds = (tiles + gridDim.x * TPR - 1) / (gridDim.x * TPR);
+
+    // two sets of weight fragments, used in turn (named apart so that both stay in registers)
+    bf16x8 fwa[NT][GV_U], fwb[NT][GV_U];
+    auto load_w = [&](bf16x8 (&fw)[NT][GV_U], int tile, int chunk) {
+        // weight rows of this lane: plain: n = 16 tile + r; gated: gate row 32 tile + r, up row 16 further
+        const int wr0 = GATED ? tile * 32 + r : tile * 16 + r;
+        const int k0 = chunk * GV_CHUNK;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            const bool w_ok = tile < tiles && (wr0 + 16 * t) < n_rows_w;
+            const bf16* wp = w + static_cast<size_t>(w_ok ? wr0 + 16 * t : 0) * K + q * 8;
+#pragma unroll
+            for (int u = 0; u < GV_U; ++u) {
+                const int kk = k0 + u * 32;
+                fw[t][u] = (w_ok && (kk + q * 8) < K) ? *reinterpret_cast<const bf16x8*>(wp + kk) : gv_zero8();
+            }
+        }
+    };
+    const int first_tile = blockIdx.x * TPR + slot;
+    if (kpart < n_chunks) load_w(fwa, first_tile, kpart);       // in flight during the norm prologue
+
+    // ---- prologue: xs[m][k] = bf16(w_norm[k] * h[row(m)][k]); ssum[m] = sum_k h^2 ----
+    for (int m = wave; m < 16; m += NW) {
+        bf16* xrow = xs + static_cast<size_t>(m) * XS;
+        if (m < M) {
+            const float* hrow = h + static_cast<size_t>(rows ? rows[m] : m) * K;
+            float ss = 0.f;
+            for (int k = lane * 4; k < K; k += 64 * 4) {      // K % 8 == 0: whole groups of 4
+                const float4 v = *reinterpret_cast<const float4*>(hrow + k);
+                ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+                bf16x4 o;
+                o[0] = static_cast<__bf16>(to_float(norm_w[k]) * v.x);
+                o[1] = static_cast<__bf16>(to_float(norm_w[k + 1]) * v.y);
+                o[2] = static_cast<__bf16>(to_float(norm_w[k + 2]) * v.z);
+                o[3] = static_cast<__bf16>(to_float(norm_w[k + 3]) * v.w);
+                *reinterpret_cast<bf16x4*>(xrow + k) = o;
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) ssum[m] = ss;
+        } else {
+            bf16x4 z;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) z[e] = static_cast<__bf16>(0.f);
+            for (int k = lane * 4; k < K; k += 64 * 4) *reinterpret_cast<bf16x4*>(xrow + k) = z;
+            if (lane == 0) ssum[m] = 0.f;
+        }
+    }
+    __syncthreads();
+
+    const bf16* xlane = xs + static_cast<size_t>(r) * XS + q * 8;      // row m = r of the activation tile
+    f32x4 acc[NT];
+    auto multiply = [&](const bf16x8 (&fw)[NT][GV_U], int chunk) {
+        const int k0 = chunk * GV_CHUNK;
+#pragma unroll
+        for (int u = 0; u < GV_U; ++u) {
+            const int kk = k0 + u * 32;
+            const bf16x8 fx = ((kk + q * 8) < K) ? *reinterpret_cast<const bf16x8*>(xlane + kk) : gv_zero8();
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[t][u], fx, acc[t], 0, 0, 0);
+        }
+    };
+
+    for (int round = 0; round < rounds; ++round) {
+        const int tile = (round * gridDim.x + blockIdx.x) * TPR + slot;
+        if (round > 0 && kpart < n_chunks) load_w(fwa, tile, kpart);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int chunk = kpart; chunk < n_chunks;) {
+            if (chunk + KS < n_chunks) load_w(fwb, tile, chunk + KS);
+            multiply(fwa, chunk);
+            chunk += KS;
+            if (chunk >= n_chunks) break;
+            if (chunk + KS < n_chunks) load_w(fwa, tile, chunk + KS);
+            multiply(fwb, chunk);
+            chunk += KS;
+        }
+#pragma unroll
+        for (int t = 0; t < NT; ++t) red[(wave * NT + t) * 64 + lane] = acc[t];
+        __syncthreads();
+        // the first wavefront of each tile adds up: lane l holds row m = l % 16, columns 4 (l / 16) + e
+        if (kpart == 0 && tile < tiles) {
+            f32x4 s[NT];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                s[t] = acc[t];
+                for (int wv = 1; wv < KS; ++wv) {
+                    const f32x4 p = red[((wave + wv) * NT + t) * 64 + lane];
+                    s[t][0] += p[0]; s[t][1] += p[1]; s[t][2] += p[2]; s[t][3] += p[3];
+                }
+            }
+            const int m = lane & 15;
+            if (m < M) {
+                const float inv = 1.0f / sqrtf(ssum[m] / static_cast<float>(K) + eps);
+                const int c0 = tile * 16 + (lane >> 4) * 4;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int c = c0 + e;
+                    if (c >= N) continue;
+                    if (GATED) {
+                        const float g = s[0][e] * inv, u = s[1][e] * inv;
+                        static_cast<bf16*>(out)[static_cast<size_t>(m) * N + c] =
+                            static_cast<bf16>((g / (1.0f + expf(-g))) * u);
+                    } else {
+                        static_cast<float*>(out)[static_cast<size_t>(m) * N + c] = s[0][e] * inv;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+template <int NW, int TPR, bool GATED, typename TNW>
+static int launch_gemv_norm(const float* h, const int* rows, const void* norm_w, float eps, const bf16* w, void* out,
+                            int M, int N, int K, int grid, hipStream_t stream) {
+    const size_t lds = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(NW) * (GATED ? 2 : 1) * 64 * 16 + 64;
+    if (lds > 160 * 1024) return kErrUnsupported;
+    auto kernel = gemv_norm_kernel<NW, TPR, GATED, TNW>;
+    static size_t granted = 0;                          // per instantiation
+    if (lds > granted) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+        if (e != hipSuccess) return static_cast<int>(e);
+        granted = lds;
+    }
+    const int tiles = (N + 15) / 16;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(NW * 64), lds, stream, h, rows, static_cast<const TNW*>(norm_w), eps,
+                       w, out, M, N, K, tiles);
+    return launch_status();
+}
+
+template <bool GATED, typename TNW>
+static int launch_gemv_norm_shape(int tpr, const float* h, const int* rows, const void* norm_w, float eps,
+                                  const bf16* w, void* out, int M, int N, int K, int grid, hipStream_t stream) {
+    if (tpr >= 4) return launch_gemv_norm<8, 4, GATED, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, stream);
+    if (tpr == 2) return launch_gemv_norm<8, 2, GATED, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, stream);
+    return launch_gemv_norm<8, 1, GATED, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, stream);
+}
+
+}  // namespace llme
+
+using namespace llme;
+
+// h [*, K] float32; rows: M indices into h or null; norm_w [K] (norm_dtype 0 float32, 1 bfloat16);
+// w bfloat16: plain [N, K], gated [2 N, K] with gate and up rows interleaved in groups of 16;
+// out: plain float32 [M, N], gated bfloat16 [M, N]. tpr (tiles a workgroup of 8 wavefronts works
+// on at a time: 1, 2 or 4) and grid (workgroups): 0 lets the entry point choose.
+extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_w, int norm_dtype, float eps,
+                              const void* w, void* out, int M, int N, int K, int gated, int tpr, int grid,
+                              hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K <= 0 || K % 8 != 0) return kErrUnsupported;
+    if (static_cast<size_t>(16) * (K + 8) * 2 > 132 * 1024) return kErrUnsupported;
+    if (gated && N % 16 != 0) return kErrUnsupported;
+    const int tiles = (N + 15) / 16;
+    if (tpr <= 0) {
+        // few tiles: all 8 wavefronts on one tile, so that every tile has a workgroup of its own;
+        // more tiles than compute units: 2 tiles at a time, 4 wavefronts each with several chunks of k
+        tpr = tiles <= 256 ? 1 : 2;
+    }
+    if (tpr != 1 && tpr != 2 && tpr != 4) return kErrBadArgument;
+    if (grid <= 0) {
+        grid = (tiles + tpr - 1) / tpr;
+        if (grid > 512) grid = 512;                     // two workgroups per compute unit
+    }
+    const bf16* W = static_cast<const bf16*>(w);
+    if (norm_dtype == kBF16) {
+        return gated ? launch_gemv_norm_shape<true, bf16>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream)
+                     : launch_gemv_norm_shape<false, bf16>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream);
+    }
+    if (norm_dtype == kF32) {
+        return gated ? launch_gemv_norm_shape<true, float>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream)
+                     : launch_gemv_norm_shape<false, float>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream);
+    }
+    return kErrBadArgument;
+}

@@ -86,8 +86,11 @@ class DecoderModel(Part):
         if logit_rows is None or logit_rows.shape[0] == 0:
             return None
         R = logit_rows.shape[0]
-        x = step.buffer("model.head_in", (R, self.hidden_size), step.act_dtype)
-        self.final_norm.forward(h, x, rows=logit_rows)
         logits = step.buffer("model.logits", (R, self.vocab_size), torch.float32)
-        self.head.forward(x, logits)
+        if self.head.fuses_norm(h, self.final_norm, R, step.act_dtype):
+            self.head.forward_normed_rows(h, logit_rows, self.final_norm, logits)
+        else:
+            x = step.buffer("model.head_in", (R, self.hidden_size), step.act_dtype)
+            self.final_norm.forward(h, x, rows=logit_rows)
+            self.head.forward(x, logits)
         return logits

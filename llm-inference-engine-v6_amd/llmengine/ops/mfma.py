@@ -133,3 +133,42 @@ def _fast_attention(q, k_cache, v_cache, out, step, block_table, n_q, n_kv, head
 
 
 kernels._fast_attention = _fast_attention
+
+
+# --- projections fused with the norm in front of them (decoding) ---------------------------
+declare("llme_gemv_norm", [_vp, _vp, _vp, _i, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp])
+
+GEMV_NORM_MAX_ROWS = 16
+
+
+def gemv_norm_supported(h: torch.Tensor, norm_weight: torch.Tensor, w: torch.Tensor, rows_out: int,
+                        gated: bool) -> bool:
+    K = h.shape[1]
+    n_out = w.shape[0] // 2 if gated else w.shape[0]
+    return (kernels.policy.fast_gemm and h.dtype == torch.float32 and w.dtype == torch.bfloat16
+            and norm_weight.dtype in (torch.float32, torch.bfloat16) and 0 < rows_out <= GEMV_NORM_MAX_ROWS
+            and K % 8 == 0 and 16 * (K + 8) * 2 <= 132 * 1024 and w.shape[1] == K
+            and (not gated or n_out % 16 == 0) and w.data_ptr() % 16 == 0 and h.data_ptr() % 16 == 0)
+
+
+def gemv_norm(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor,
+              gated: bool = False, rows: torch.Tensor | None = None, tiles_per_round: int = 0,
+              grid: int = 0) -> None:
+    """out = (rmsnorm(h[rows]) with norm_weight) @ w^T for up to 16 rows of the 32-bit h; gated:
+    w holds gate and up rows interleaved in groups of 16 and out = silu(gate) * up in bfloat16."""
+    require(h, "h", torch.float32, (None, None))
+    K = h.shape[1]
+    M = h.shape[0] if rows is None else rows.shape[0]
+    if rows is not None:
+        require(rows, "rows", torch.int32, (M,))
+    require(norm_weight, "norm_weight", (torch.float32, torch.bfloat16), (K,))
+    require(w, "w", torch.bfloat16, (None, K))
+    N = w.shape[0] // 2 if gated else w.shape[0]
+    require(out, "out", torch.bfloat16 if gated else torch.float32, (M, N))
+    if not gemv_norm_supported(h, norm_weight, w, M, gated):
+        raise kernels.KernelError(f"gemv_norm: {M} rows (at most 16), K={K} (multiple of 8, 16 rows must fit "
+                                  "into LDS) or the operand types are not supported")
+    check(entry("llme_gemv_norm")(ptr(h), ptr(rows), ptr(norm_weight), 0 if norm_weight.dtype == torch.float32 else 1,
+                                  float(eps), ptr(w), ptr(out), M, N, K, 1 if gated else 0, tiles_per_round, grid,
+                                  stream()),
+          "gemv_norm")

@@ -18,6 +18,7 @@ import torch
 
 from .. import ops
 from .base import PAGE, CacheSpec, Getter, Mixer, ParamSpec, Placement, PositionEncoding
+from .norm import RMSNorm
 from .registry import register_part
 
 
@@ -62,7 +63,12 @@ class Attention(Mixer):
                          paged={"k": (self.num_kv_heads, PAGE, self.head_dim),
                                 "v": (self.num_kv_heads, self.head_dim, PAGE)})
 
-    def forward(self, x, step, cache, out, accumulate, write_cache=True):
+    def fuses_norm(self, h, norm, step):
+        # A few rows (decoding): the q/k/v projection applies the norm itself.
+        return (isinstance(norm, RMSNorm) and step.act_dtype == torch.bfloat16
+                and ops.gemv_norm_supported(h, norm.weight, self.w_qkv, h.shape[0], gated=False))
+
+    def forward(self, x, step, cache, out, accumulate, write_cache=True, pre_norm=None):
         T = x.shape[0]
         n_q, n_kv, hd = self.num_heads, self.num_kv_heads, self.head_dim
         tables = self.position.rotary_tables() if self.position is not None else None
@@ -71,18 +77,25 @@ class Attention(Mixer):
             raise ValueError(f"position {step.max_position} is beyond the position table ({cos.shape[0]} rows)")
         block_table = step.block_tables[cache.group]
         k_cache, v_cache = cache.paged["k"], cache.paged["v"]
-        q = step.buffer("attn.q", (T, self.q_dim), x.dtype)
+        act = step.act_dtype
+        q = step.buffer("attn.q", (T, self.q_dim), act)
+
+        def project(weight, dst):
+            if pre_norm is not None:
+                ops.gemv_norm(x, pre_norm.weight, pre_norm.eps, weight, dst)
+            else:
+                ops.gemm(x, weight, dst)
         if write_cache:
             qkv = step.buffer("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
-            ops.gemm(x, self.w_qkv, qkv)
+            project(self.w_qkv, qkv)
             ops.rope_kv_write(qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
                               n_q, n_kv, hd, rot, write_cache=True)
         else:
             # A layer that reads another layer's cache projects queries only.
             q32 = step.buffer("attn.q32", (T, self.q_dim), torch.float32)
-            ops.gemm(x, self.w_qkv[:self.q_dim], q32)
+            project(self.w_qkv[:self.q_dim], q32)
             ops.rope_q_only(q32, cos, sin, step.positions, q, n_q, hd, rot)
-        o = step.buffer("attn.o", (T, self.q_dim), x.dtype)
+        o = step.buffer("attn.o", (T, self.q_dim), act)
         ops.attention(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, hd, self.scale, self.window)
         ops.gemm(o, self.w_o, out, accumulate)
 

@@ -170,12 +170,21 @@ class Mixer(Part):
     def cache_spec(self) -> CacheSpec | None:
         return None
 
+    def fuses_norm(self, h: torch.Tensor, norm: "Norm", step) -> bool:
+        """True if, for this step, the part wants the un-normed 32-bit stream plus the norm in
+        front of it (`forward(h, ..., pre_norm=norm)`) because a kernel of its own applies the
+        norm. Parts that do not know about this are always given normed activations."""
+        return False
+
     def forward(self, x: torch.Tensor, step, cache: LayerCache | None, out: torch.Tensor,
                 accumulate: bool, write_cache: bool = True) -> None:
         raise NotImplementedError
 
 
 class FeedForward(Part):
+    def fuses_norm(self, h: torch.Tensor, norm: "Norm", step) -> bool:
+        return False
+
     def forward(self, x: torch.Tensor, step, out: torch.Tensor, accumulate: bool) -> None:
         raise NotImplementedError
 

@@ -31,10 +31,16 @@ class PreNormBlock(Block):
     def forward(self, h, step, cache, write_cache=True):
         T, H = h.shape
         x = step.buffer("block.normed", (T, H), step.act_dtype)
-        self.mixer_norm.forward(h, x)
-        self.mixer.forward(x, step, cache, h, True, write_cache)
-        self.ffn_norm.forward(h, x)
-        self.feed_forward.forward(x, step, h, True)
+        if self.mixer.fuses_norm(h, self.mixer_norm, step):
+            self.mixer.forward(h, step, cache, h, True, write_cache, pre_norm=self.mixer_norm)
+        else:
+            self.mixer_norm.forward(h, x)
+            self.mixer.forward(x, step, cache, h, True, write_cache)
+        if self.feed_forward.fuses_norm(h, self.ffn_norm, step):
+            self.feed_forward.forward(h, step, h, True, pre_norm=self.ffn_norm)
+        else:
+            self.ffn_norm.forward(h, x)
+            self.feed_forward.forward(x, step, h, True)
 
 
 register_part("block", "prenorm", PreNormBlock)

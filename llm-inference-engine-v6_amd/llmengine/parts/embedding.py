@@ -54,5 +54,14 @@ class OutputHead(Part):
     def weight(self) -> torch.Tensor:
         return self.tied_to.weight if self.tied_to is not None else self._weight
 
+    def fuses_norm(self, h: torch.Tensor, norm, n_rows: int, act_dtype) -> bool:
+        from .norm import RMSNorm
+        return (isinstance(norm, RMSNorm) and act_dtype == torch.bfloat16
+                and ops.gemv_norm_supported(h, norm.weight, self.weight, n_rows, gated=False))
+
     def forward(self, x: torch.Tensor, out: torch.Tensor) -> None:
         ops.gemm(x, self.weight, out)
+
+    def forward_normed_rows(self, h: torch.Tensor, rows: torch.Tensor, norm, out: torch.Tensor) -> None:
+        """Logits of the chosen rows of the 32-bit stream, the final norm applied inside the product."""
+        ops.gemv_norm(h, norm.weight, norm.eps, self.weight, out, rows=rows)

@@ -11,6 +11,7 @@ import torch
 
 from .. import ops
 from .base import FeedForward, Getter, ParamSpec, Placement
+from .norm import RMSNorm
 from .registry import register_part
 
 
@@ -39,13 +40,22 @@ class GatedMLP(FeedForward):
         self.w_gate_up = fused
         self.w_down = placement.place(get("down_proj.weight"))
 
-    def forward(self, x, step, out, accumulate):
+    def fuses_norm(self, h, norm, step):
+        # A few rows (decoding): one kernel applies the norm, both projections and the activation.
+        return (isinstance(norm, RMSNorm) and self.group == 16 and step.act_dtype == torch.bfloat16
+                and ops.gemv_norm_supported(h, norm.weight, self.w_gate_up, h.shape[0], gated=True))
+
+    def forward(self, x, step, out, accumulate, pre_norm=None):
         T = x.shape[0]
         FF = self.intermediate_size
-        gu = step.buffer("mlp.gate_up", (T, 2 * FF), torch.float32)
-        ops.gemm(x, self.w_gate_up, gu)
-        act = step.buffer("mlp.act", (T, FF), x.dtype)
-        ops.swiglu(gu, act, self.group)
+        if pre_norm is not None:
+            act = step.buffer("mlp.act", (T, FF), torch.bfloat16)
+            ops.gemv_norm(x, pre_norm.weight, pre_norm.eps, self.w_gate_up, act, gated=True)
+        else:
+            gu = step.buffer("mlp.gate_up", (T, 2 * FF), torch.float32)
+            ops.gemm(x, self.w_gate_up, gu)
+            act = step.buffer("mlp.act", (T, FF), x.dtype)
+            ops.swiglu(gu, act, self.group)
         ops.gemm(act, self.w_down, out, accumulate)
 
 

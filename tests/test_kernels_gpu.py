@@ -375,3 +375,56 @@ def test_attention_mfma_finds_one_far_key(ops):
         for h in range(n_q):
             got = out[row].cpu().double().view(n_q, hd)[h]
             assert (got - v[base + far, h // 2]).abs().max() < 2e-2, (row, h)
+
+
+# --- projections fused with the norm in front of them -----------------------------------
+@pytest.mark.parametrize("M,N,K", [(1, 48, 64), (8, 3072, 2048), (16, 100, 96), (5, 331, 144), (3, 128256, 2048),
+                                   (7, 64, 4096)])
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("tpr,grid", [(0, 0), (1, 0), (2, 3), (4, 0), (4, 5)])
+def test_gemv_norm(ops, M, N, K, wdtype, tpr, grid):
+    if N > 10000 and (tpr, grid) not in ((0, 0), (4, 0)):
+        pytest.skip("large case twice")
+    h = 2 * torch.randn(M + 3, K, generator=_gen(60))
+    nw = (1 + 0.1 * torch.randn(K, generator=_gen(61))).to(wdtype)
+    w = (0.05 * torch.randn(N, K, generator=_gen(62))).to(torch.bfloat16)
+    rows = torch.tensor([(3 * i + 1) % (M + 3) for i in range(M)], dtype=torch.int32)
+    out = torch.empty(M, N, device=DEV)
+    ops.gemv_norm(h.to(DEV), nw.to(DEV), 1e-5, w.to(DEV), out, rows=rows.to(DEV), tiles_per_round=tpr, grid=grid)
+    x = plain_rmsnorm(h[rows.long()].double(), nw.double(), 1e-5)
+    ref = plain_linear(x, w.double())
+    assert _rel(out.cpu().double(), ref) < 4e-3          # activations enter the product in bfloat16
+    direct = torch.empty(M, N, device=DEV)
+    ops.gemv_norm(h[:M].contiguous().to(DEV), nw.to(DEV), 1e-5, w.to(DEV), direct, tiles_per_round=tpr, grid=grid)
+    ref2 = plain_linear(plain_rmsnorm(h[:M].double(), nw.double(), 1e-5), w.double())
+    assert _rel(direct.cpu().double(), ref2) < 4e-3
+
+
+@pytest.mark.parametrize("M,FF,K", [(1, 176, 64), (8, 8192, 2048), (16, 256, 96), (4, 208, 144)])
+def test_gemv_norm_gated(ops, M, FF, K):
+    h = 2 * torch.randn(M, K, generator=_gen(63))
+    nw = (1 + 0.1 * torch.randn(K, generator=_gen(64))).to(torch.bfloat16)
+    wg = (0.1 * torch.randn(FF, K, generator=_gen(65))).to(torch.bfloat16)
+    wu = (0.1 * torch.randn(FF, K, generator=_gen(66))).to(torch.bfloat16)
+    fused = torch.empty(2 * FF, K, dtype=torch.bfloat16)
+    fused.view(FF // 16, 2, 16, K)[:, 0] = wg.view(FF // 16, 16, K)
+    fused.view(FF // 16, 2, 16, K)[:, 1] = wu.view(FF // 16, 16, K)
+    out = torch.empty(M, FF, dtype=torch.bfloat16, device=DEV)
+    x = plain_rmsnorm(h.double(), nw.double(), 1e-6)
+    ref = plain_silu(plain_linear(x, wg.double())) * plain_linear(x, wu.double())
+    for tpr, grid in ((0, 0), (1, 0), (2, 2), (4, 0)):
+        out.zero_()
+        ops.gemv_norm(h.to(DEV), nw.to(DEV), 1e-6, fused.to(DEV), out, gated=True, tiles_per_round=tpr, grid=grid)
+        assert _rel(out.cpu().double(), ref) < 1e-2, (tpr, grid)
+
+
+def test_gemv_norm_refusals(ops):
+    from llmengine.ops import KernelError
+    h = torch.randn(17, 64, device=DEV)
+    nw = torch.ones(64, device=DEV)
+    w = torch.randn(32, 64, device=DEV).bfloat16()
+    with pytest.raises(KernelError):
+        ops.gemv_norm(h, nw, 1e-5, w, torch.empty(17, 32, device=DEV))          # more than 16 rows
+    with pytest.raises(KernelError):
+        ops.gemv_norm(h[:4, :60].contiguous(), nw[:60].contiguous(), 1e-5, w[:, :60].contiguous(),
+                      torch.empty(4, 32, device=DEV))                              # K no multiple of 8
