@@ -41,6 +41,11 @@ typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLazy = 8.0f;
+
+// 2^x by the hardware instruction alone: arguments here are <= 0, results below the normal
+// range may flush to zero, which is what a softmax weight that small amounts to.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 struct PagedKV {
     const bf16* k;
@@ -76,51 +81,71 @@ __device__ __forceinline__ BlockPages lookup_pages(const PagedKV& kv, int t0, in
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
         const int h0 = t0 + hf * 16;
-        b.pg[hf] = (h0 < key_end && h0 + 15 >= key_lo) ? kv.table[h0 / kv.page] : 0;
+        // the same for every lane: kept in a scalar register, so that page addresses are scalar work
+        b.pg[hf] = (h0 < key_end && h0 + 15 >= key_lo) ? __builtin_amdgcn_readfirstlane(kv.table[h0 / kv.page]) : 0;
     }
     return b;
 }
 
 // Loads a block's operands from the pages looked up before. Keys outside [key_lo, key_end)
-// are not loaded (zeros).
+// are not loaded (zeros); a block that lies inside the range whole takes the path without
+// any per-lane checks.
 template <int HD>
 __device__ __forceinline__ void load_block(const PagedKV& kv, int t0, const BlockPages& pages, int key_lo, int key_end,
                                            KVFrag<HD>& f) {
     constexpr int DC = (HD + 31) / 32, DT = HD / 16;
     const int lane = threadIdx.x & 63;
     const int r = lane & 15, g4 = lane >> 4;
+    const bool inside = t0 >= key_lo && t0 + 32 <= key_end;        // uniform
+    const bf16* krow[2];
+    const bf16* vbase[2];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+        const int h0 = t0 + hf * 16;
+        const size_t page_base = (static_cast<size_t>(pages.pg[hf]) * kv.n_kv + kv.kvh) * kv.page * HD;   // scalar
+        krow[hf] = kv.k + page_base + static_cast<size_t>(h0 % kv.page + r) * HD + g4 * 8;
+        vbase[hf] = kv.v + page_base + static_cast<size_t>(r) * kv.page + (h0 % kv.page + g4 * 4);
+    }
+    if (inside) {
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int c = 0; c < DC; ++c)
+                f.kf[hf][c] = (HD % 32 == 0 || c * 32 + g4 * 8 < HD)
+                                  ? *reinterpret_cast<const bf16x8*>(krow[hf] + c * 32) : zero_frag();
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const size_t off = static_cast<size_t>(dt) * 16 * kv.page;
+            const bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vbase[0] + off);
+            const bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(vbase[1] + off);
+            f.vf[dt] = __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+        return;
+    }
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
         const int t = t0 + hf * 16 + r;
         const bool ok = t >= key_lo && t < key_end;
-        const bf16* row = kv.k + ((static_cast<size_t>(pages.pg[hf]) * kv.n_kv + kv.kvh) * kv.page + t % kv.page) * HD;
 #pragma unroll
-        for (int c = 0; c < DC; ++c) {
-            const int d = c * 32 + g4 * 8;
-            f.kf[hf][c] = (ok && d < HD) ? *reinterpret_cast<const bf16x8*>(row + d) : zero_frag();
-        }
+        for (int c = 0; c < DC; ++c)
+            f.kf[hf][c] = (ok && c * 32 + g4 * 8 < HD) ? *reinterpret_cast<const bf16x8*>(krow[hf] + c * 32)
+                                                       : zero_frag();
     }
-    const bf16* base[2];
     bool ok[2];
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf) {
         const int t = t0 + hf * 16 + g4 * 4;
         ok[hf] = t + 3 >= key_lo && t < key_end;     // the 4 keys share a page with a visible key
-        base[hf] = kv.v + (static_cast<size_t>(pages.pg[hf]) * kv.n_kv + kv.kvh) * HD * kv.page + t % kv.page;
     }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-        const size_t off = static_cast<size_t>(dt * 16 + r) * kv.page;
+        const size_t off = static_cast<size_t>(dt) * 16 * kv.page;
         bf16x4 lo4, hi4;
 #pragma unroll
         for (int e = 0; e < 4; ++e) lo4[e] = hi4[e] = static_cast<__bf16>(0.f);
-        if (ok[0]) lo4 = *reinterpret_cast<const bf16x4*>(base[0] + off);
-        if (ok[1]) hi4 = *reinterpret_cast<const bf16x4*>(base[1] + off);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            f.vf[dt][e] = lo4[e];
-            f.vf[dt][4 + e] = hi4[e];
-        }
+        if (ok[0]) lo4 = *reinterpret_cast<const bf16x4*>(vbase[0] + off);
+        if (ok[1]) hi4 = *reinterpret_cast<const bf16x4*>(vbase[1] + off);
+        f.vf[dt] = __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
     }
 }
 
@@ -172,9 +197,12 @@ __device__ __forceinline__ void attend_block(const KVFrag<HD>& f, int t0, const 
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m[qt], mx);
+        // The reference maximum moves only when a score exceeds it by more than kLazy (in powers
+        // of two): until then weights are at most 2^kLazy, well inside the range, and the sums
+        // need no rescaling. The softmax does not depend on which reference is subtracted.
+        const float m_new = (mx > m[qt] + kLazy) ? mx : m[qt];
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;       // nothing seen yet: all p are 0
-        const float alpha = exp2f(m[qt] - m_use);                      // 0 when m was -inf
+        const float alpha = fast_exp2(m[qt] - m_use);                  // 0 when m was -inf
         m[qt] = m_new;
         bf16x8 pf;
         float psum = 0.f;
@@ -182,7 +210,7 @@ __device__ __forceinline__ void attend_block(const KVFrag<HD>& f, int t0, const 
         for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const float p = exp2f(s[hf][e] - m_use);
+                const float p = fast_exp2(s[hf][e] - m_use);
                 psum += p;
                 pf[hf * 4 + e] = static_cast<__bf16>(p);
             }
@@ -452,7 +480,7 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
     hipLaunchKernelGGL((attention_prefill_kernel<HD, QT>), grid, dim3(256), 0, stream, q, kc, vc, out, q_start, \
                        ctx_len, table, max_blocks, n_seq, n_q, n_kv, page, scale, window)
         if (qt == 4 && HD <= 64) LLME_PREFILL(4);
-        else if (qt >= 2 && HD <= 128) LLME_PREFILL(2);
+        else if (qt == 2) LLME_PREFILL(2);
         else LLME_PREFILL(1);
 #undef LLME_PREFILL
     }
@@ -463,8 +491,22 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
 
 using namespace llme;
 
-// Rows per prefill work item for a head size: the caller sizes the grid with it.
-extern "C" int llme_attention_bf16_rows(int hd) { return hd <= 64 ? 64 : 32; }
+// Rows per prefill work item (16, 32 or 64) for a head size: the caller sizes the grid with it.
+// More rows reuse every K and V load more often; fewer rows give more wavefronts to hide
+// latencies and to even out the causal triangle. llme_attention_bf16_set_rows overrides the
+// choice (0: back to the default) for measurements.
+static int g_rows_override = 0;
+extern "C" int llme_attention_bf16_set_rows(int rows) {
+    if (rows != 0 && rows != 16 && rows != 32 && rows != 64) return kErrBadArgument;
+    g_rows_override = rows;
+    return 0;
+}
+extern "C" int llme_attention_bf16_rows(int hd) {
+    int rows = hd <= 64 ? 32 : 16;
+    if (g_rows_override) rows = g_rows_override;
+    if (hd > 64 && rows > 32) rows = 32;
+    return rows;
+}
 
 // n_decode: requests with one token (0: none, skip the decode kernels); split_len (multiple of
 // 32) and nsplit: how the decode kernel cuts the keys; part_o [n_seq, n_q, nsplit, hd] and

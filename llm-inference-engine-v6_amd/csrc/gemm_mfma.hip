@@ -37,120 +37,180 @@ __device__ __forceinline__ bf16x8 load8(const bf16* p, bool ok) {
     return ok ? *reinterpret_cast<const bf16x8*>(p) : zero8();
 }
 
-enum OutMode : int { kStoreF32 = 0, kAddF32 = 1, kStoreBF16 = 2, kAtomicF32 = 3 };
+enum OutMode : int { kStoreF32 = 0, kAddF32 = 1, kStoreBF16 = 2, kAtomicF32 = 3, kGatedBF16 = 4 };
 
 // ----------------------------------------------------------------------------------------
-// tile kernel
-constexpr int TM = 128, TN = 128, TK = 64;
+// tile kernel: a workgroup of 2 x 2 wavefronts makes a (32 WMT) x (32 WNT) tile of the output,
+// each wavefront WMT x WNT MFMA tiles of 16 x 16. Larger wavefront tiles read fewer LDS bytes
+// per product (the 64 x 64 wavefront tile is bound by LDS reads); smaller tiles give more
+// workgroups when the output is small.
+constexpr int TK = 64;
 constexpr int TSTRIDE = TK + 8;                      // elements; 144 bytes: conflict-free 16-byte reads
-constexpr int TILE_ELEMS = TM * TSTRIDE;             // one operand tile in LDS
-constexpr int TILE_LDS_BYTES = 4 * TILE_ELEMS * 2;   // A and W, two buffers each
 
-template <int MODE>
+template <int WMT, int WNT>
+constexpr int tile_lds_bytes() { return 2 * (32 * WMT + 32 * WNT) * TSTRIDE * 2; }   // A and W, two buffers
+
+// kGatedBF16: w holds gate and up rows interleaved in groups of 16, so that even MFMA tile
+// columns are gates and odd ones the ups of the same 16 units; out [M, N / 2] bfloat16 gets
+// silu(gate) * up (src/engine.cpp:213-216).
+template <int WMT, int WNT, int MODE>
 __global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w,
                                                         void* __restrict__ out, int M, int N, int K,
-                                                        int tiles_m, int tiles_n) {
+                                                        int tiles_m, int tiles_n, int ksplit) {
+    constexpr int BM = 32 * WMT, BN = 32 * WNT;
+    constexpr int A_ELEMS = BM * TSTRIDE, W_ELEMS = BN * TSTRIDE;
+    constexpr int CA = BM / 32, CW = BN / 32;        // 16-byte chunks per thread and slab
     extern __shared__ __align__(16) unsigned char lds_raw[];
     bf16* lds = reinterpret_cast<bf16*>(lds_raw);
-    // buffers: sA[b] = lds + b * TILE_ELEMS, sW[b] = lds + (2 + b) * TILE_ELEMS
+    // buffers: sA[b] = lds + b * A_ELEMS, sW[b] = lds + 2 * A_ELEMS + b * W_ELEMS
 
-    // Tile order: groups of 8 tile rows, columns fastest inside a group, so that workgroups
-    // that run together share rows of A and of W in L2.
+    // Workgroups go to the chip's 8 dies in turn, each die with an L2 of its own: renumber so
+    // that a die gets consecutive tiles; then tiles in groups of 8 tile rows, columns fastest
+    // inside a group, so that workgroups that run together share rows of A and of W.
+    const int per_split = tiles_m * tiles_n;
+    int pid = blockIdx.x % per_split;
+    const int split = blockIdx.x / per_split;
+    if (per_split % 8 == 0) pid = (pid % 8) * (per_split / 8) + pid / 8;
     constexpr int GROUP = 8;
-    const int pid = blockIdx.x;
     const int per_group = GROUP * tiles_n;
     const int g = pid / per_group;
     const int first_m = g * GROUP;
     const int gsize = (tiles_m - first_m < GROUP) ? tiles_m - first_m : GROUP;
     const int tm = first_m + (pid % per_group) % gsize;
     const int tn = (pid % per_group) / gsize;
-    const int m0 = tm * TM, n0 = tn * TN;
+    const int m0 = tm * BM, n0 = tn * BN;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
-    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int wm = (wave >> 1) * (16 * WMT), wn = (wave & 1) * (16 * WNT);
 
-    // global -> LDS mapping: a tile is 128 rows x 8 chunks of 16 bytes; 4 chunks per thread
-    int crow[4], ckq[4];
+    // this workgroup's share of k (whole slabs)
+    const int nk_all = (K + TK - 1) / TK;
+    const int nk_per = (nk_all + ksplit - 1) / ksplit;
+    const int kt_begin = split * nk_per;
+    const int kt_end = (kt_begin + nk_per < nk_all) ? kt_begin + nk_per : nk_all;
+
+    // global -> LDS: a slab of a tile is rows x 8 chunks of 16 bytes; thread t takes chunks t, t + 256, ..
+    const int crow = tid >> 3, ckq = (tid & 7) * 8;   // chunk i of a thread: row crow + 32 i, same k offset
+    bf16x8 ra[CA], rw[CW];
+    auto load_global = [&](int kt) {
+        const int k = kt * TK + ckq;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int c = tid + 256 * i;
-        crow[i] = c >> 3;
-        ckq[i] = c & 7;
-    }
-    bf16x8 ra[4], rw[4];
-    auto load_global = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int k = k0 + ckq[i] * 8;
-            const int am = m0 + crow[i], wr = n0 + crow[i];
+        for (int i = 0; i < CA; ++i) {
+            const int am = m0 + crow + 32 * i;
             ra[i] = load8(a + static_cast<size_t>(am) * K + k, am < M && k < K);
+        }
+#pragma unroll
+        for (int i = 0; i < CW; ++i) {
+            const int wr = n0 + crow + 32 * i;
             rw[i] = load8(w + static_cast<size_t>(wr) * K + k, wr < N && k < K);
         }
     };
     auto store_lds = [&](int buf) {
-        bf16* sA = lds + buf * TILE_ELEMS;
-        bf16* sW = lds + (2 + buf) * TILE_ELEMS;
+        bf16* sA = lds + buf * A_ELEMS;
+        bf16* sW = lds + 2 * A_ELEMS + buf * W_ELEMS;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<bf16x8*>(sA + crow[i] * TSTRIDE + ckq[i] * 8) = ra[i];
-            *reinterpret_cast<bf16x8*>(sW + crow[i] * TSTRIDE + ckq[i] * 8) = rw[i];
-        }
+        for (int i = 0; i < CA; ++i) *reinterpret_cast<bf16x8*>(sA + (crow + 32 * i) * TSTRIDE + ckq) = ra[i];
+#pragma unroll
+        for (int i = 0; i < CW; ++i) *reinterpret_cast<bf16x8*>(sW + (crow + 32 * i) * TSTRIDE + ckq) = rw[i];
     };
 
-    f32x4 acc[4][4];
+    f32x4 acc[WMT][WNT];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < WMT; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < WNT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int nk = (K + TK - 1) / TK;
-    load_global(0);
-    store_lds(0);
+    if (kt_begin < kt_end) {
+        load_global(kt_begin);
+        store_lds(0);
+    }
     __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) load_global((kt + 1) * TK);
-        const bf16* sA = lds + buf * TILE_ELEMS;
-        const bf16* sW = lds + (2 + buf) * TILE_ELEMS;
+    for (int kt = kt_begin; kt < kt_end; ++kt) {
+        const int buf = (kt - kt_begin) & 1;
+        if (kt + 1 < kt_end) load_global(kt + 1);
+        const bf16* sA = lds + buf * A_ELEMS;
+        const bf16* sW = lds + 2 * A_ELEMS + buf * W_ELEMS;
 #pragma unroll
         for (int kk = 0; kk < TK / 32; ++kk) {
-            bf16x8 fa[4], fw[4];
+            bf16x8 fa[WMT], fw[WNT];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < WMT; ++i)
                 fa[i] = *reinterpret_cast<const bf16x8*>(sA + (wm + i * 16 + r) * TSTRIDE + kk * 32 + q * 8);
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < WNT; ++j)
                 fw[j] = *reinterpret_cast<const bf16x8*>(sW + (wn + j * 16 + r) * TSTRIDE + kk * 32 + q * 8);
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < WMT; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                for (int j = 0; j < WNT; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
         }
-        if (kt + 1 < nk) store_lds(buf ^ 1);
+        if (kt + 1 < kt_end) store_lds(buf ^ 1);
         __syncthreads();
     }
 
     // result tile (i, j): column n = wn + 16 j + r, rows m = wm + 16 i + 4 q + e
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < WMT; ++i) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int m = m0 + wm + i * 16 + q * 4 + e;
             if (m >= M) continue;
+            if (MODE == kGatedBF16) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int n = n0 + wn + j * 16 + r;
-                if (n >= N) continue;
-                const size_t idx = static_cast<size_t>(m) * N + n;
-                const float v = acc[i][j][e];
-                if (MODE == kStoreF32) static_cast<float*>(out)[idx] = v;
-                else if (MODE == kAddF32) static_cast<float*>(out)[idx] += v;
-                else static_cast<bf16*>(out)[idx] = static_cast<bf16>(v);
+                for (int j = 0; j + 1 < WNT; j += 2) {
+                    const int unit = (n0 + wn + j * 16) / 2 + r;        // tile column pair (gate, up)
+                    if (2 * unit >= N) continue;
+                    const float gt = acc[i][j][e], up = acc[i][j + 1][e];
+                    static_cast<bf16*>(out)[static_cast<size_t>(m) * (N / 2) + unit] =
+                        static_cast<bf16>((gt / (1.0f + expf(-gt))) * up);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < WNT; ++j) {
+                    const int n = n0 + wn + j * 16 + r;
+                    if (n >= N) continue;
+                    const size_t idx = static_cast<size_t>(m) * N + n;
+                    const float v = acc[i][j][e];
+                    if (MODE == kStoreF32) static_cast<float*>(out)[idx] = v;
+                    else if (MODE == kAddF32) static_cast<float*>(out)[idx] += v;
+                    else if (MODE == kAtomicF32) atomicAdd(static_cast<float*>(out) + idx, v);
+                    else static_cast<bf16*>(out)[idx] = static_cast<bf16>(v);
+                }
             }
         }
+    }
+}
+
+template <int WMT, int WNT, int MODE>
+static int launch_tile_mode(const bf16* A, const bf16* W, void* out, int M, int N, int K, int ksplit,
+                            hipStream_t stream) {
+    constexpr int LDS = tile_lds_bytes<WMT, WNT>();
+    auto kernel = gemm_tile_kernel<WMT, WNT, MODE>;
+    static bool attr_set = false;                      // per instantiation
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        if (e != hipSuccess) return static_cast<int>(e);
+        attr_set = true;
+    }
+    const int tiles_m = (M + 32 * WMT - 1) / (32 * WMT), tiles_n = (N + 32 * WNT - 1) / (32 * WNT);
+    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * ksplit), dim3(256), LDS, stream, A, W, out, M, N, K, tiles_m,
+                       tiles_n, ksplit);
+    return launch_status();
+}
+
+template <int WMT, int WNT>
+static int launch_tile(const bf16* A, const bf16* W, void* out, int M, int N, int K, int mode, int ksplit,
+                       hipStream_t stream) {
+    switch (mode) {
+        case kStoreF32: return launch_tile_mode<WMT, WNT, kStoreF32>(A, W, out, M, N, K, 1, stream);
+        case kAddF32: return launch_tile_mode<WMT, WNT, kAddF32>(A, W, out, M, N, K, 1, stream);
+        case kAtomicF32: return launch_tile_mode<WMT, WNT, kAtomicF32>(A, W, out, M, N, K, ksplit, stream);
+        case kGatedBF16: return launch_tile_mode<WMT, WNT, kGatedBF16>(A, W, out, M, N, K, 1, stream);
+        default: return launch_tile_mode<WMT, WNT, kStoreBF16>(A, W, out, M, N, K, 1, stream);
     }
 }
 
@@ -258,20 +318,32 @@ static void launch_skinny_nw(const bf16* x, const bf16* w, void* out, int M, int
 using namespace llme;
 
 // a [M, K], w [N, K] bfloat16; out [M, N] float32 (out_dtype 0) or bfloat16 (1).
-// accumulate (float32 only) adds into out. nw, ksplit: 0 lets the entry point choose the
-// skinny kernel's wavefronts per workgroup and grid split over k; force_tile != 0 sends
-// small M to the tile kernel too (for tests).
+// accumulate (float32 only) adds into out. gated: w holds gate and up rows interleaved in
+// groups of 16 and out is bfloat16 [M, N / 2] = silu(gate) * up (tile kernel only).
+// nw, ksplit: 0 lets the entry point choose the skinny kernel's wavefronts per workgroup and
+// the split over k; tile_shape: 0 chooses, 64 / 128 / 256 force the tile kernel with that tile
+// edge also for small M (for tests and measurements).
 extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
-                              int accumulate, int nw, int ksplit, int force_tile, hipStream_t stream) {
+                              int accumulate, int gated, int nw, int ksplit, int tile_shape, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (K <= 0 || K % 8 != 0) return kErrUnsupported;
     if (out_dtype != kF32 && out_dtype != kBF16) return kErrBadArgument;
     if (accumulate && out_dtype != kF32) return kErrBadArgument;
+    if (gated && (out_dtype != kBF16 || N % 32 != 0 || accumulate)) return kErrBadArgument;
     const bf16* A = static_cast<const bf16*>(a);
     const bf16* W = static_cast<const bf16*>(w);
     int mode = out_dtype == kBF16 ? kStoreBF16 : (accumulate ? kAddF32 : kStoreF32);
-    if (M <= 64 && !force_tile) {
+    if (M <= 64 && tile_shape <= 0 && !gated) {
         const int tiles = (N + 15) / 16;
+        if (nw <= 0 && ksplit <= 0 && accumulate && out_dtype == kF32 && tiles < 512) {
+            // Few output columns and a sum to join anyway (the residual stream): cut k over
+            // several workgroups that add their parts with atomics, so that the whole chip
+            // streams the matrix. (The order of these additions is not fixed.)
+            ksplit = 512 / tiles;
+            if (ksplit > K / 512) ksplit = K / 512;
+            if (ksplit < 1) ksplit = 1;
+            nw = 4;
+        }
         if (nw <= 0) {
             // enough wavefronts to cover the chip several times, each with at least one chunk of k
             const int chunks = (K + SK_CHUNK - 1) / SK_CHUNK;
@@ -292,23 +364,26 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
         }
         return launch_status();
     }
-    const int tiles_m = (M + TM - 1) / TM, tiles_n = (N + TN - 1) / TN;
-    const dim3 grid(tiles_m * tiles_n), block(256);
-    static bool attr_set[3] = {false, false, false};
-#define LLME_TILE(MODE, SLOT)                                                                              \
-    do {                                                                                                   \
-        if (!attr_set[SLOT]) {                                                                             \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tile_kernel<MODE>),     \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, TILE_LDS_BYTES); \
-            if (e != hipSuccess) return static_cast<int>(e);                                               \
-            attr_set[SLOT] = true;                                                                         \
-        }                                                                                                  \
-        hipLaunchKernelGGL((gemm_tile_kernel<MODE>), grid, block, TILE_LDS_BYTES, stream, A, W, out, M, N, \
-                           K, tiles_m, tiles_n);                                                           \
-    } while (0)
-    if (mode == kStoreF32) LLME_TILE(kStoreF32, 0);
-    else if (mode == kAddF32) LLME_TILE(kAddF32, 1);
-    else LLME_TILE(kStoreBF16, 2);
-#undef LLME_TILE
-    return launch_status();
+    // tile shape: 0 lets the entry point choose: the largest tile that still gives about one
+    // workgroup per compute unit; a small output with a long k is cut over k instead (the
+    // parts are added with atomics, so this needs an accumulating float32 output).
+    if (gated) mode = kGatedBF16;
+    if (tile_shape <= 0) {
+        const long wg128 = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
+        const long wg256 = static_cast<long>((M + 255) / 256) * ((N + 255) / 256);
+        tile_shape = wg256 >= 200 ? 256 : (wg128 >= 64 ? 128 : 64);
+        if (tile_shape == 128 && mode == kAddF32 && wg256 >= 48 && K >= 4096 && ksplit <= 0) {
+            tile_shape = 256;
+            ksplit = 4;
+        }
+    }
+    if (ksplit <= 0) ksplit = 1;
+    if (ksplit > 1) {
+        if (mode != kAddF32) return kErrBadArgument;
+        mode = kAtomicF32;
+    }
+    if (tile_shape == 256) return launch_tile<8, 8>(A, W, out, M, N, K, mode, ksplit, stream);
+    if (tile_shape == 128) return launch_tile<4, 4>(A, W, out, M, N, K, mode, ksplit, stream);
+    if (tile_shape == 64) return launch_tile<2, 2>(A, W, out, M, N, K, mode, ksplit, stream);
+    return kErrBadArgument;
 }

@@ -12,7 +12,7 @@ from .lib import check, declare, entry, ptr, require, stream
 
 _vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 
-declare("llme_gemm_bf16", [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp])
+declare("llme_gemm_bf16", [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp])
 
 
 def gemm_bf16_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool) -> bool:
@@ -24,20 +24,44 @@ def gemm_bf16_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, acc
 
 
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, *,
-              waves: int = 0, ksplit: int = 0, force_tile: bool = False) -> None:
+              gated: bool = False, waves: int = 0, ksplit: int = 0, tile: int = 0, force_tile: bool = False) -> None:
     """bfloat16 a [M, K] and w [N, K] -> out [M, N] (float32 or bfloat16), 32-bit accumulation.
-    K must be a multiple of 8. waves / ksplit / force_tile override the launch choices (tests)."""
+    K must be a multiple of 8. gated: w holds gate and up rows interleaved in groups of 16 and
+    out is bfloat16 [M, N / 2] = silu(gate) * up. waves / ksplit / tile (64, 128, 256) /
+    force_tile override the launch choices (tests and measurements)."""
     require(a, "a", torch.bfloat16, (None, None))
     M, K = a.shape
     require(w, "w", torch.bfloat16, (None, K))
     N = w.shape[0]
-    require(out, "out", (torch.float32, torch.bfloat16), (M, N))
+    if gated:
+        require(out, "out", torch.bfloat16, (M, N // 2))
+        if N % 32 or accumulate:
+            raise kernels.KernelError("gemm_bf16: a gated product needs a multiple of 32 weight rows and no accumulation")
+    else:
+        require(out, "out", (torch.float32, torch.bfloat16), (M, N))
     if not gemm_bf16_supported(a, w, out, accumulate):
         raise kernels.KernelError(f"gemm_bf16: K={K} must be a multiple of 8, pointers 16-byte aligned, and "
                                   "accumulation needs a float32 output")
+    if force_tile and not tile:
+        tile = 128
     check(entry("llme_gemm_bf16")(ptr(a), ptr(w), ptr(out), 0 if out.dtype == torch.float32 else 1, M, N, K,
-                                  1 if accumulate else 0, waves, ksplit, 1 if force_tile else 0, stream()),
+                                  1 if accumulate else 0, 1 if gated else 0, waves, ksplit, tile, stream()),
           "gemm_bf16")
+
+
+def gemm_gated(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, group: int, scratch) -> None:
+    """out [T, FF] = silu(x Wg^T) * (x Wu^T), the gate and up rows interleaved in groups of `group`
+    rows of w_gate_up [2 FF, K]. One MFMA kernel where the types and sizes fit it; otherwise the
+    product into a 32-bit scratch [T, 2 FF] (scratch(shape, dtype) provides it) and the
+    activation kernel."""
+    T, FF = out.shape
+    if (kernels.policy.fast_gemm and group == 16 and out.dtype == torch.bfloat16 and (2 * FF) % 32 == 0
+            and x.dtype == torch.bfloat16 and gemm_bf16_supported(x, w_gate_up, out, False)):
+        gemm_bf16(x, w_gate_up, out, gated=True)
+        return
+    gu = scratch((T, 2 * FF), torch.float32)
+    kernels.gemm(x, w_gate_up, gu)
+    kernels.swiglu(gu, out, group)
 
 
 def _fast_gemm(a, w, out, accumulate) -> bool:
@@ -52,6 +76,7 @@ kernels._fast_gemm = _fast_gemm
 
 # --- attention ---------------------------------------------------------------------------
 declare("llme_attention_bf16_rows", [_i])
+declare("llme_attention_bf16_set_rows", [_i])
 declare("llme_attention_bf16", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i,
                                 _i, _i, _i, _i, _vp])
 

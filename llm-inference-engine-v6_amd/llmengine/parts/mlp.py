@@ -52,10 +52,9 @@ class GatedMLP(FeedForward):
             act = step.buffer("mlp.act", (T, FF), torch.bfloat16)
             ops.gemv_norm(x, pre_norm.weight, pre_norm.eps, self.w_gate_up, act, gated=True)
         else:
-            gu = step.buffer("mlp.gate_up", (T, 2 * FF), torch.float32)
-            ops.gemm(x, self.w_gate_up, gu)
             act = step.buffer("mlp.act", (T, FF), x.dtype)
-            ops.swiglu(gu, act, self.group)
+            ops.gemm_gated(x, self.w_gate_up, act, self.group,
+                           lambda shape, dtype: step.buffer("mlp.gate_up", shape, dtype))
         ops.gemm(act, self.w_down, out, accumulate)
 
 

@@ -249,18 +249,47 @@ def test_gemm_skinny(ops, M, N, K, waves, ksplit):
 
 @pytest.mark.parametrize("M,N,K", [(65, 128, 64), (128, 128, 128), (200, 331, 144), (129, 100, 176), (257, 500, 72),
                                    (2048, 3072, 2048), (1000, 2048, 8192), (7, 40, 24)])
-def test_gemm_tile(ops, M, N, K):
+@pytest.mark.parametrize("tile", [64, 128, 256])
+def test_gemm_tile(ops, M, N, K, tile):
     a, w, ref = _bf16_pair(M, N, K, 30)
     out = torch.full((M, N), 3.0, device=DEV)
-    ops.gemm_bf16(a.to(DEV), w.to(DEV), out, force_tile=True)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), out, tile=tile)
     assert _rel(out.cpu().double(), ref) < 2e-5
     base = torch.randn(M, N, generator=_gen(32))
     acc = base.clone().to(DEV)
-    ops.gemm_bf16(a.to(DEV), w.to(DEV), acc, accumulate=True, force_tile=True)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), acc, accumulate=True, tile=tile)
     assert _rel(acc.cpu().double(), ref + base.double()) < 2e-5
+    for ksplit in (2, 5):
+        acc = base.clone().to(DEV)
+        ops.gemm_bf16(a.to(DEV), w.to(DEV), acc, accumulate=True, tile=tile, ksplit=ksplit)
+        assert _rel(acc.cpu().double(), ref + base.double()) < 2e-5, ksplit
     half = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
-    ops.gemm_bf16(a.to(DEV), w.to(DEV), half, force_tile=True)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), half, tile=tile)
     assert _rel(half.cpu().double(), ref) < 5e-3
+
+
+@pytest.mark.parametrize("T,FF,K,tile", [(5, 176, 64, 0), (130, 256, 96, 64), (300, 208, 144, 128), (2048, 8192, 2048, 0),
+                                         (257, 320, 128, 256), (64, 8192, 2048, 0)])
+def test_gemm_gated(ops, T, FF, K, tile):
+    x = torch.randn(T, K, generator=_gen(33)).to(torch.bfloat16)
+    wg = (0.1 * torch.randn(FF, K, generator=_gen(34))).to(torch.bfloat16)
+    wu = (0.1 * torch.randn(FF, K, generator=_gen(35))).to(torch.bfloat16)
+    fused = torch.empty(2 * FF, K, dtype=torch.bfloat16)
+    fused.view(FF // 16, 2, 16, K)[:, 0] = wg.view(FF // 16, 16, K)
+    fused.view(FF // 16, 2, 16, K)[:, 1] = wu.view(FF // 16, 16, K)
+    out = torch.zeros(T, FF, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16(x.to(DEV), fused.to(DEV), out, gated=True, tile=tile)
+    g, u = x.double() @ wg.double().T, x.double() @ wu.double().T
+    ref = plain_silu(g) * u
+    assert _rel(out.cpu().double(), ref) < 5e-3
+    # the dispatcher's other way: 32-bit product, then the activation kernel
+    ops.policy.fast_gemm = False
+    try:
+        out2 = torch.zeros(T, FF, dtype=torch.bfloat16, device=DEV)
+        ops.gemm_gated(x.to(DEV), fused.to(DEV), out2, 16, lambda shape, dtype: torch.empty(shape, dtype=dtype, device=DEV))
+    finally:
+        ops.policy.fast_gemm = True
+    assert _rel(out2.cpu().double(), ref) < 5e-3
 
 
 def test_gemm_dispatch_and_refusals(ops):
