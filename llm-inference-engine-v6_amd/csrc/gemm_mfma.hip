@@ -333,7 +333,11 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     const bf16* A = static_cast<const bf16*>(a);
     const bf16* W = static_cast<const bf16*>(w);
     int mode = out_dtype == kBF16 ? kStoreBF16 : (accumulate ? kAddF32 : kStoreF32);
-    if (M <= 64 && tile_shape <= 0 && !gated) {
+    // Up to 16 rows: the skinny kernel (one row tile). 17 to 64 rows: the skinny kernel re-reads
+    // the activations from L2 once per 16 output columns, which costs more than the weights
+    // themselves, so wide outputs and sums that can be cut over k go to the 64 x 64 tile kernel.
+    const bool skinny = M <= 16 || (M <= 64 && !accumulate && N < 8192);
+    if (skinny && tile_shape <= 0 && !gated) {
         const int tiles = (N + 15) / 16;
         if (nw <= 0 && ksplit <= 0 && accumulate && out_dtype == kF32 && tiles < 512) {
             // Few output columns and a sum to join anyway (the residual stream): cut k over
@@ -370,11 +374,13 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     if (gated) mode = kGatedBF16;
     if (tile_shape <= 0) {
         const long wg128 = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
-        const long wg256 = static_cast<long>((M + 255) / 256) * ((N + 255) / 256);
-        tile_shape = wg256 >= 200 ? 256 : (wg128 >= 64 ? 128 : 64);
-        if (tile_shape == 128 && mode == kAddF32 && wg256 >= 48 && K >= 4096 && ksplit <= 0) {
-            tile_shape = 256;
-            ksplit = 4;
+        tile_shape = (M > 64 && wg128 >= 64) ? 128 : 64;
+        if (M <= 64 && mode == kAddF32 && ksplit <= 0) {
+            // one row of tiles: cut k so that about two workgroups per compute unit stream the matrix
+            const int tiles = (N + 63) / 64;
+            ksplit = 512 / tiles;
+            if (ksplit > K / 512) ksplit = K / 512;
+            if (ksplit > 8) ksplit = 8;
         }
     }
     if (ksplit <= 0) ksplit = 1;
