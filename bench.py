@@ -82,6 +82,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode"],
+                    help="run only one part (for profiling); the JSON line then lacks the other")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -106,23 +108,29 @@ def main() -> int:
 
     # ---- prefill: one prompt, logits at its last place ----
     T = args.prefill_tokens
-    prompt = torch.randint(0, V, (T,), generator=gen).tolist()
-    cache = engine.new_cache((T + page - 1) // page + 1, page, 1)
-    pre_ms = []
-    for rep in range(4):
-        cache.admit("p")
-        sync()
-        t = time.perf_counter()
-        engine.step(cache, [StepEntry("p", prompt, [T - 1])])
-        sync()
-        pre_ms.append((time.perf_counter() - t) * 1e3)
-        cache.release("p")
-    prefill_ms = min(pre_ms[1:])
-    flops = prefill_flops(cfg, T)
-    prefill = {"value": round(T / (prefill_ms / 1e3), 1), "tokens": T, "ms": round(prefill_ms, 3),
-               "frac": round(flops / (prefill_ms / 1e3) / PEAK_FLOPS[args.dtype], 4)}
-    log(f"prefill {T} tokens: {prefill_ms:.2f} ms ({prefill['value']:.0f} tok/s, {prefill['frac']:.3f} of peak)")
-    del cache
+    prefill = None
+    if args.phase in ("all", "prefill"):
+        prompt = torch.randint(0, V, (T,), generator=gen).tolist()
+        cache = engine.new_cache((T + page - 1) // page + 1, page, 1)
+        pre_ms = []
+        for rep in range(4):
+            cache.admit("p")
+            sync()
+            t = time.perf_counter()
+            engine.step(cache, [StepEntry("p", prompt, [T - 1])])
+            sync()
+            pre_ms.append((time.perf_counter() - t) * 1e3)
+            cache.release("p")
+        prefill_ms = min(pre_ms[1:])
+        flops = prefill_flops(cfg, T)
+        prefill = {"value": round(T / (prefill_ms / 1e3), 1), "tokens": T, "ms": round(prefill_ms, 3),
+                   "frac": round(flops / (prefill_ms / 1e3) / PEAK_FLOPS[args.dtype], 4)}
+        log(f"prefill {T} tokens: {prefill_ms:.2f} ms ({prefill['value']:.0f} tok/s, {prefill['frac']:.3f} of peak)")
+        del cache
+    if args.phase == "prefill":
+        print(json.dumps({"metric": "prefill_tokens_per_second", "value": prefill["value"], "unit": "tokens/s",
+                          "n_gpus": 1, "dtype": args.dtype, "prefill": prefill}), flush=True)
+        return 0
 
     # ---- decode ----
     def decode_run(batch: int, steps: int, warmup: int):
