@@ -170,6 +170,42 @@ class CacheManager:
         req.reserved = max(req.reserved, req.length + n_new)
         return True
 
+    def reserve_batch(self, items: list[tuple[object, int]]) -> bool:
+        """`reserve` for several requests at once: all of them get their pages, or nothing changes."""
+        plans = []
+        need = {name: 0 for name in self.groups}
+        for request_id, n_new in items:
+            if n_new <= 0:
+                raise ValueError("reserve needs n_new >= 1")
+            req = self._req(request_id)
+            last = (req.length + n_new - 1) // self.page_size
+            for g in self.groups.values():
+                table = req.tables[g.name]
+                if g.kind == "full":
+                    if last < len(table):
+                        continue                    # the common case of decoding: the page is there
+                    blocks = list(range(len(table), last + 1))
+                else:
+                    blocks = self._missing(req, g, n_new)
+                    if not blocks:
+                        continue
+                need[g.name] += len(blocks)
+                plans.append((req, g.name, blocks))
+        for name, n in need.items():
+            if n > self.pools[name].free_pages:
+                return False
+        for req, name, blocks in plans:
+            table = req.tables[name]
+            pool = self.pools[name]
+            for b in blocks:
+                while len(table) <= b:
+                    table.append(-1)
+                table[b] = pool.allocate()
+        for request_id, n_new in items:
+            req = self._requests[request_id]
+            req.reserved = max(req.reserved, req.length + n_new)
+        return True
+
     def commit(self, request_id, n_new: int) -> None:
         """The step wrote n_new tokens: the request is that much longer, and window
         groups give back the pages no later token will read."""

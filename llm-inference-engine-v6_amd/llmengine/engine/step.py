@@ -132,6 +132,63 @@ class CacheContext:
         self.manager.release(request_id)
 
 
+class _DecodeRecord:
+    """A recorded decode step: the graph, where its logits appear, and the integer arrays it
+    reads (a device buffer with a pinned host mirror in the layout of `_build_context` for
+    S requests of one token each). Between replays only what changed is rewritten on the host:
+    tokens and lengths every step, a block-table entry when a request gets a new page,
+    everything when other requests take part."""
+
+    def __init__(self, graph, logits, meta: torch.Tensor, S: int, width: int, groups: list[str]):
+        self.graph, self.logits, self.meta = graph, logits, meta
+        self.S, self.width, self.groups = S, width, groups
+        sizes = [S, S, S, S + 1, S, S] + [S * width] * len(groups) + [S]
+        self.offsets = [0]
+        for n in sizes:
+            self.offsets.append(self.offsets[-1] + n)
+        self.total = self.offsets[-1]
+        self.host = torch.zeros(self.total, dtype=torch.int32, pin_memory=True)
+        self.np = self.host.numpy()
+        self.ids: list | None = None
+        self.blocks: list[list[int]] = []        # per group, per request: table entries written so far
+        self.event: torch.cuda.Event | None = None
+
+    def refresh(self, mgr: CacheManager, entries: Sequence[StepEntry], lengths: list[int]) -> None:
+        if self.event is not None:
+            self.event.synchronize()            # the last copy has read the host mirror
+        S, width, o, h = self.S, self.width, self.offsets, self.np
+        ids = [e.request_id for e in entries]
+        if ids != self.ids:
+            h[o[2]:o[3]] = range(S)             # request index of each token
+            h[o[3]:o[4]] = range(S + 1)         # first row of each request
+            h[o[5]:o[6]] = [mgr.slot(r) for r in ids]
+            h[o[6 + len(self.groups)]:o[7 + len(self.groups)]] = range(S)     # wanted rows
+            self.blocks = []
+            for gi, g in enumerate(self.groups):
+                base = o[6 + gi]
+                h[base:base + S * width] = 0
+                self.blocks.append([0] * S)
+            self.ids = ids
+        h[o[0]:o[1]] = [e.tokens[0] for e in entries]
+        h[o[1]:o[2]] = lengths                  # the new token's position
+        h[o[4]:o[5]] = lengths                  # tokens cached before this step
+        for gi, g in enumerate(self.groups):
+            base = o[6 + gi]
+            done = self.blocks[gi]
+            window = mgr.groups[g].kind == "window"
+            for i, rid in enumerate(ids):
+                table = mgr.block_table(rid, g)
+                nb = len(table)
+                if nb != done[i] or window:
+                    lo = 0 if window else done[i]
+                    h[base + i * width + lo:base + i * width + nb] = table[lo:nb]
+                    done[i] = nb
+        self.meta[:self.total].copy_(self.host, non_blocking=True)
+        if self.event is None:
+            self.event = torch.cuda.Event()
+        self.event.record()
+
+
 class ModelRunner:
     """A loaded model on a device plus the scratch memory its steps use."""
 
@@ -180,19 +237,13 @@ class ModelRunner:
             if max_position is not None and end > max_position:
                 raise ValueError(f"request {e.request_id!r}: {end} tokens exceed the position limit "
                                  f"{max_position}")
-        # pages for every entry, or none: count first, then take
-        need = {g: 0 for g in mgr.groups}
-        for e in entries:
-            for g, n in mgr.pages_needed(e.request_id, len(e.tokens)).items():
-                need[g] += n
-        for g, n in need.items():
-            if n > mgr.free_pages(g):
-                raise CapacityError(f"the step needs {n} more pages of group {g!r}, {mgr.free_pages(g)} are free")
-        for e in entries:
-            if not mgr.reserve(e.request_id, len(e.tokens)):
-                raise CapacityError(f"request {e.request_id!r}: pages ran out while reserving")
+        # pages for every entry, or none
+        if not mgr.reserve_batch([(e.request_id, len(e.tokens)) for e in entries]):
+            need = {g: sum(mgr.pages_needed(e.request_id, len(e.tokens))[g] for e in entries) for g in mgr.groups}
+            raise CapacityError(f"the step needs {need} more pages, free are "
+                                f"{({g: mgr.free_pages(g) for g in mgr.groups})}")
 
-        if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+        if self.use_graphs and all(len(e.tokens) == 1 and len(e.want) == 1 and e.want[0] == 0 for e in entries):
             logits = self._decode_step_graphed(cache, entries)
         else:
             ctx, logit_rows = self._build_context(cache, entries)
@@ -207,8 +258,10 @@ class ModelRunner:
         only on the number of requests and on the width of the block tables, so it is
         recorded once as a HIP graph and replayed; only the integer arrays change."""
         page = cache.page_size
+        mgr = cache.manager
         S = len(entries)
-        need = max((cache.manager.length(e.request_id) + page) // page for e in entries)
+        lengths = [mgr.length(e.request_id) for e in entries]
+        need = (max(lengths) + page) // page
         bucket = self.GRAPH_BLOCK_BUCKET
         width = (need + bucket - 1) // bucket * bucket
         key = (S, width)
@@ -216,8 +269,8 @@ class ModelRunner:
         if rec is None:
             # First time: run it plainly (this also sizes the scratch buffers), then record.
             # The recorded step reads its integer arrays from a buffer of its own.
-            groups = len(cache.manager.groups)
-            meta = torch.empty(6 * S + 1 + groups * S * width + S + 64, dtype=torch.int32, device=self.device)
+            groups = len(mgr.groups)
+            meta = torch.empty(7 * S + 1 + groups * S * width + 64, dtype=torch.int32, device=self.device)
             ctx, logit_rows = self._build_context(cache, entries, max_blocks=width, plan_len=width * page, dev=meta)
             self.model.forward(ctx, cache.storage.layers, logit_rows)
             torch.cuda.synchronize(self.device)
@@ -225,12 +278,11 @@ class ModelRunner:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
-            cache.graphs[key] = rec = (graph, logits, ctx, meta)
-        else:
-            self._build_context(cache, entries, max_blocks=width, plan_len=width * page, dev=rec[3])
-        rec[0].replay()
+            cache.graphs[key] = rec = _DecodeRecord(graph, logits, meta, S, width, list(mgr.groups))
+        rec.refresh(mgr, entries, lengths)
+        rec.graph.replay()
         self.graph_replays += 1
-        return rec[1]
+        return rec.logits
 
     # ------------------------------------------------------------------------------
     def _build_context(self, cache: CacheContext, entries: Sequence[StepEntry], max_blocks: int | None = None,

@@ -149,3 +149,26 @@ def test_bad_arguments():
         CacheManager([GroupSpec("g", "full", 0, 4), GroupSpec("g", "full", 0, 4)], page_size=4, max_requests=1)
     with pytest.raises(ValueError):
         PagePool(0)
+
+
+def test_reserve_batch_is_all_or_nothing():
+    m = CacheManager([GroupSpec("full", "full", 0, 6), GroupSpec("win", "window", 6, 6)], page_size=4, max_requests=3)
+    for r in "abc":
+        m.admit(r)
+    assert m.reserve_batch([("a", 8), ("b", 4)])                       # 2 + 1 pages in each group
+    m.commit("a", 8)
+    m.commit("b", 4)
+    m.check()
+    before = {g: m.free_pages(g) for g in m.groups}
+    tables = {r: list(m.block_table(r, "full")) for r in "abc"}
+    assert not m.reserve_batch([("a", 1), ("c", 12)])                  # a needs 1, c needs 3: 4 > 3 free
+    assert before == {g: m.free_pages(g) for g in m.groups}
+    assert tables == {r: list(m.block_table(r, "full")) for r in "abc"}
+    assert m.reserve_batch([("a", 1), ("b", 1), ("c", 4)])             # a and b: a new page each; c: one
+    for r, n in (("a", 1), ("b", 1), ("c", 4)):
+        m.commit(r, n)
+    m.check()
+    assert m.reserve_batch([("a", 3)])                                  # tokens 9..11 fit a's third page
+    assert m.free_pages("full") == 6 - 3 - 2 - 1                        # a 3 pages, b 2, c 1
+    with pytest.raises(ValueError):
+        m.reserve_batch([("a", 0)])
