@@ -18,6 +18,12 @@
 // issued before the current chunk's products; the partial sums are added through LDS, scaled
 // by inv_m and stored. The grid is sized so that the prologue is paid once per several tiles.
 //
+// A third form serves the attention's q/k/v projection: its epilogue rotates q and k heads at
+// the rows' positions (pairs (i, i + hd/2), src/kernels.cpp:189-203) and writes q to the query
+// buffer and k, v straight into the rows' cache pages, so that neither the 32-bit q/k/v rows
+// nor a separate rotation kernel exist. A workgroup then takes the two tiles of 16 columns
+// that hold each other's rotation partners (the same head, hd/2 columns apart) at a time.
+//
 // Limits (checked by the caller): M <= 16, K a multiple of 8, 16 * (K + 8) * 2 bytes of LDS.
 #include "common.h"
 #include <math.h>
@@ -38,11 +44,29 @@ __device__ __forceinline__ bf16x8 gv_zero8() {
     return z;
 }
 
-template <int NW, int TPR, bool GATED, typename TNW>
+enum Epilogue : int { kPlain = 0, kGated = 1, kRope = 2 };
+
+// What the rotating epilogue needs: where rows sit in their requests and where their pages are.
+struct RopeTarget {
+    const int* positions;       // [M] position of each row's token
+    const int* seq_idx;         // [M] request of each row (row of the block table)
+    const int* block_table;     // [n_seq, max_blocks]
+    int max_blocks;
+    const float* cos_t;         // [max_pos, hd / 2]
+    const float* sin_t;
+    bf16* q_out;                // [M, n_q * hd]
+    bf16* k_cache;              // [pages, n_kv, page, hd]
+    bf16* v_cache;              // [pages, n_kv, hd, page]
+    int n_q, n_kv, hd, page;
+};
+
+template <int NW, int TPR, int EPI, typename TNW>
 __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restrict__ h, const int* __restrict__ rows,
                                                             const TNW* __restrict__ norm_w, float eps,
                                                             const bf16* __restrict__ w, void* __restrict__ out,
-                                                            int M, int N, int K, int tiles) {
+                                                            int M, int N, int K, int tiles, RopeTarget rope) {
+    constexpr bool GATED = EPI == kGated;
+    static_assert(EPI != kRope || TPR == 2, "the rotating epilogue works on pairs of tiles");
     constexpr int NT = GATED ? 2 : 1;                   // weight fragments per k step
     constexpr int KS = NW / TPR;                        // wavefronts that share a tile, splitting k
     extern __shared__ __align__(16) unsigned char lds_raw[];
@@ -50,13 +74,13 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
     bf16* xs = reinterpret_cast<bf16*>(lds_raw);                                    // [16][XS]
     f32x4* red = reinterpret_cast<f32x4*>(lds_raw + static_cast<size_t>(16) * XS * 2);   // [NW][NT][64]
     float* ssum = reinterpret_cast<float*>(red + NW * NT * 64);                      // [16]
+    float* ex = ssum + 16;                                                           // [2][16][16] (rope)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
     const int slot = wave / KS, kpart = wave % KS;      // which of the round's tiles, which share of k
     const int n_rows_w = GATED ? 2 * N : N;             // rows of the weight matrix
     const int n_chunks = (K + GV_CHUNK - 1) / GV_CHUNK;
-    const int rounds = (tiles + gridDim.x * TPR - 1) / (gridDim.x * TPR);
 
     // two sets of weight fragments, used in turn (named apart so that both stay in registers)
     bf16x8 fwa[NT][GV_U], fwb[NT][GV_U];
@@ -75,8 +99,19 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
             }
         }
     };
-    const int first_tile = blockIdx.x * TPR + slot;
-    if (kpart < n_chunks) load_w(fwa, first_tile, kpart);       // in flight during the norm prologue
+    // Which tile this wavefront works on in a round. Rotating epilogue: work item p is a pair of
+    // tiles of one head, hd / 2 columns apart; slot 0 takes the first, slot 1 the second.
+    const int tiles_per_head = (EPI == kRope) ? rope.hd / 16 : 1;
+    auto tile_of = [&](int item) {
+        if (EPI == kRope) {
+            const int half_tiles = tiles_per_head / 2;
+            const int tile = (item / half_tiles) * tiles_per_head + item % half_tiles + slot * half_tiles;
+            return item < tiles / 2 ? tile : tiles;        // past the end: a tile that does not exist
+        }
+        return item * TPR + slot;
+    };
+    const int items = (EPI == kRope) ? tiles / 2 : (tiles + TPR - 1) / TPR;
+    if (kpart < n_chunks) load_w(fwa, tile_of(blockIdx.x), kpart);       // in flight during the norm prologue
 
     // ---- prologue: xs[m][k] = bf16(w_norm[k] * h[row(m)][k]); ssum[m] = sum_k h^2 ----
     for (int m = wave; m < 16; m += NW) {
@@ -120,8 +155,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
         }
     };
 
+    const int rounds = (items + gridDim.x - 1) / gridDim.x;
     for (int round = 0; round < rounds; ++round) {
-        const int tile = (round * gridDim.x + blockIdx.x) * TPR + slot;
+        const int item = round * gridDim.x + blockIdx.x;
+        const int tile = tile_of(item);
         if (round > 0 && kpart < n_chunks) load_w(fwa, tile, kpart);
 #pragma unroll
         for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -138,8 +175,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
         for (int t = 0; t < NT; ++t) red[(wave * NT + t) * 64 + lane] = acc[t];
         __syncthreads();
         // the first wavefront of each tile adds up: lane l holds row m = l % 16, columns 4 (l / 16) + e
-        if (kpart == 0 && tile < tiles) {
-            f32x4 s[NT];
+        f32x4 s[NT];
+        const int m = lane & 15;
+        const bool leader = kpart == 0 && tile < tiles;
+        float inv = 0.f;
+        if (leader) {
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 s[t] = acc[t];
@@ -148,21 +188,58 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
                     s[t][0] += p[0]; s[t][1] += p[1]; s[t][2] += p[2]; s[t][3] += p[3];
                 }
             }
-            const int m = lane & 15;
-            if (m < M) {
-                const float inv = 1.0f / sqrtf(ssum[m] / static_cast<float>(K) + eps);
-                const int c0 = tile * 16 + (lane >> 4) * 4;
+            inv = 1.0f / sqrtf(ssum[m] / static_cast<float>(K) + eps);
+        }
+        if (EPI == kRope) {
+            // both tiles of the pair show each other their values, then each rotates its half
+            if (leader) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ex[(slot * 16 + m) * 16 + (lane >> 4) * 4 + e] = s[0][e] * inv;
+            }
+            __syncthreads();
+            if (leader && m < M) {
+                const int hd = rope.hd, half = hd / 2;
+                const int head = tile / tiles_per_head;                 // among q heads, then k heads, then v heads
+                const int i0 = (tile % tiles_per_head) * 16 - slot * half + (lane >> 4) * 4;   // index within the half
+                const int pos = rope.positions[m];
+                const bool is_q = head < rope.n_q, is_k = !is_q && head < rope.n_q + rope.n_kv;
+                const int kvh = is_q ? 0 : (is_k ? head - rope.n_q : head - rope.n_q - rope.n_kv);
+                size_t page_off = 0;
+                int off = 0;
+                if (!is_q) {
+                    const int pg = rope.block_table[static_cast<size_t>(rope.seq_idx[m]) * rope.max_blocks + pos / rope.page];
+                    off = pos % rope.page;
+                    page_off = (static_cast<size_t>(pg) * rope.n_kv + kvh) * rope.page * hd;
+                }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const int c = c0 + e;
-                    if (c >= N) continue;
-                    if (GATED) {
-                        const float g = s[0][e] * inv, u = s[1][e] * inv;
-                        static_cast<bf16*>(out)[static_cast<size_t>(m) * N + c] =
-                            static_cast<bf16>((g / (1.0f + expf(-g))) * u);
-                    } else {
-                        static_cast<float*>(out)[static_cast<size_t>(m) * N + c] = s[0][e] * inv;
+                    const int i = i0 + e;
+                    const float own = s[0][e] * inv;
+                    float v = own;
+                    if (is_q || is_k) {
+                        const float other = ex[((slot ^ 1) * 16 + m) * 16 + (lane >> 4) * 4 + e];
+                        const float c = rope.cos_t[static_cast<size_t>(pos) * half + i];
+                        const float sn = rope.sin_t[static_cast<size_t>(pos) * half + i];
+                        v = slot == 0 ? own * c - other * sn : own * c + other * sn;
                     }
+                    const int d = slot * half + i;
+                    if (is_q) rope.q_out[(static_cast<size_t>(m) * rope.n_q + head) * hd + d] = static_cast<bf16>(v);
+                    else if (is_k) rope.k_cache[page_off + static_cast<size_t>(off) * hd + d] = static_cast<bf16>(v);
+                    else rope.v_cache[page_off + static_cast<size_t>(d) * rope.page + off] = static_cast<bf16>(v);
+                }
+            }
+        } else if (leader && m < M) {
+            const int c0 = tile * 16 + (lane >> 4) * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int c = c0 + e;
+                if (c >= N) continue;
+                if (GATED) {
+                    const float g = s[0][e] * inv, u = s[NT - 1][e] * inv;
+                    static_cast<bf16*>(out)[static_cast<size_t>(m) * N + c] =
+                        static_cast<bf16>((g / (1.0f + expf(-g))) * u);
+                } else {
+                    static_cast<float*>(out)[static_cast<size_t>(m) * N + c] = s[0][e] * inv;
                 }
             }
         }
@@ -170,12 +247,13 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
     }
 }
 
-template <int NW, int TPR, bool GATED, typename TNW>
+template <int NW, int TPR, int EPI, typename TNW>
 static int launch_gemv_norm(const float* h, const int* rows, const void* norm_w, float eps, const bf16* w, void* out,
-                            int M, int N, int K, int grid, hipStream_t stream) {
-    const size_t lds = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(NW) * (GATED ? 2 : 1) * 64 * 16 + 64;
+                            int M, int N, int K, int grid, const RopeTarget& rope, hipStream_t stream) {
+    const size_t lds = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(NW) * (EPI == kGated ? 2 : 1) * 64 * 16 +
+                       64 + 2 * 16 * 16 * 4;
     if (lds > 160 * 1024) return kErrUnsupported;
-    auto kernel = gemv_norm_kernel<NW, TPR, GATED, TNW>;
+    auto kernel = gemv_norm_kernel<NW, TPR, EPI, TNW>;
     static size_t granted = 0;                          // per instantiation
     if (lds > granted) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -185,16 +263,17 @@ static int launch_gemv_norm(const float* h, const int* rows, const void* norm_w,
     }
     const int tiles = (N + 15) / 16;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(NW * 64), lds, stream, h, rows, static_cast<const TNW*>(norm_w), eps,
-                       w, out, M, N, K, tiles);
+                       w, out, M, N, K, tiles, rope);
     return launch_status();
 }
 
-template <bool GATED, typename TNW>
+template <int EPI, typename TNW>
 static int launch_gemv_norm_shape(int tpr, const float* h, const int* rows, const void* norm_w, float eps,
                                   const bf16* w, void* out, int M, int N, int K, int grid, hipStream_t stream) {
-    if (tpr >= 4) return launch_gemv_norm<8, 4, GATED, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, stream);
-    if (tpr == 2) return launch_gemv_norm<8, 2, GATED, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, stream);
-    return launch_gemv_norm<8, 1, GATED, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, stream);
+    const RopeTarget none{};
+    if (tpr >= 4) return launch_gemv_norm<8, 4, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
+    if (tpr == 2) return launch_gemv_norm<8, 2, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
+    return launch_gemv_norm<8, 1, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
 }
 
 }  // namespace llme
@@ -225,12 +304,38 @@ extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_
     }
     const bf16* W = static_cast<const bf16*>(w);
     if (norm_dtype == kBF16) {
-        return gated ? launch_gemv_norm_shape<true, bf16>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream)
-                     : launch_gemv_norm_shape<false, bf16>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream);
+        return gated ? launch_gemv_norm_shape<kGated, bf16>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream)
+                     : launch_gemv_norm_shape<kPlain, bf16>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream);
     }
     if (norm_dtype == kF32) {
-        return gated ? launch_gemv_norm_shape<true, float>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream)
-                     : launch_gemv_norm_shape<false, float>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream);
+        return gated ? launch_gemv_norm_shape<kGated, float>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream)
+                     : launch_gemv_norm_shape<kPlain, float>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream);
     }
+    return kErrBadArgument;
+}
+
+// The q/k/v projection of up to 16 rows with the norm in front and rotation plus cache write
+// behind: h [M, K] float32 (row m is batch row m), w [(n_q + 2 n_kv) hd, K] bfloat16 (q heads, k
+// heads, v heads), cos/sin [max_pos, hd / 2]; writes q_out [M, n_q hd] and the rows' k, v into
+// the pages that block_table[seq_idx[m]] names for positions[m]. Full rotation only (all hd
+// dimensions), hd a multiple of 32.
+extern "C" int llme_gemv_norm_rope(const float* h, const void* norm_w, int norm_dtype, float eps, const void* w,
+                                   const int* positions, const int* seq_idx, const int* block_table, int max_blocks,
+                                   const float* cos_t, const float* sin_t, void* q_out, void* k_cache, void* v_cache,
+                                   int M, int K, int n_q, int n_kv, int hd, int page, int grid, hipStream_t stream) {
+    if (M <= 0) return 0;
+    if (M > 16 || K <= 0 || K % 8 != 0 || hd <= 0 || hd % 32 != 0 || n_q <= 0 || n_kv <= 0 || page <= 0)
+        return kErrUnsupported;
+    if (static_cast<size_t>(16) * (K + 8) * 2 > 132 * 1024) return kErrUnsupported;
+    const int N = (n_q + 2 * n_kv) * hd;
+    const int pairs = N / 32;
+    if (grid <= 0) grid = pairs > 512 ? 512 : pairs;
+    const RopeTarget rope{positions, seq_idx, block_table, max_blocks, cos_t, sin_t, static_cast<bf16*>(q_out),
+                          static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache), n_q, n_kv, hd, page};
+    const bf16* W = static_cast<const bf16*>(w);
+    if (norm_dtype == kBF16)
+        return launch_gemv_norm<8, 2, kRope, bf16>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, rope, stream);
+    if (norm_dtype == kF32)
+        return launch_gemv_norm<8, 2, kRope, float>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, rope, stream);
     return kErrBadArgument;
 }

@@ -4,7 +4,8 @@ from .kernels import (argmax, attention, attention_generic, rope_q_only, embed_g
                       rope_kv_write, sample, swiglu)
 
 from . import mfma                                   # noqa: E402  (installs the MFMA kernels)
-from .mfma import gemm_bf16, gemm_gated, gemv_norm, gemv_norm_supported
+from .mfma import (gemm_bf16, gemm_gated, gemv_norm, gemv_norm_rope, gemv_norm_rope_supported,
+                   gemv_norm_supported)
 
-__all__ = ["gemm_bf16", "gemm_gated", "gemv_norm", "gemv_norm_supported", "mfma", "KernelError", "KernelLibraryError", "library", "argmax", "attention", "attention_generic", "rope_q_only", "embed_gather",
+__all__ = ["gemm_bf16", "gemm_gated", "gemv_norm_rope", "gemv_norm_rope_supported", "gemv_norm", "gemv_norm_supported", "mfma", "KernelError", "KernelLibraryError", "library", "argmax", "attention", "attention_generic", "rope_q_only", "embed_gather",
            "gemm", "gemm_generic", "policy", "rmsnorm", "rope_kv_write", "sample", "swiglu"]

@@ -197,3 +197,41 @@ def gemv_norm(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.T
                                   float(eps), ptr(w), ptr(out), M, N, K, 1 if gated else 0, tiles_per_round, grid,
                                   stream()),
           "gemv_norm")
+
+
+declare("llme_gemv_norm_rope", [_vp, _vp, _i, _f, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp,
+                                _i, _i, _i, _i, _i, _i, _i, _vp])
+
+
+def gemv_norm_rope_supported(h, norm_weight, w_qkv, k_cache, n_tokens: int, head_dim: int, rotary_dim: int) -> bool:
+    return (gemv_norm_supported(h, norm_weight, w_qkv, n_tokens, gated=False) and rotary_dim == head_dim
+            and head_dim % 32 == 0 and k_cache.dtype == torch.bfloat16)
+
+
+def gemv_norm_rope(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv: torch.Tensor,
+                   positions: torch.Tensor, seq_idx: torch.Tensor, block_table: torch.Tensor, cos: torch.Tensor,
+                   sin: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                   n_q: int, n_kv: int, head_dim: int, grid: int = 0) -> None:
+    """For up to 16 rows: rmsnorm(h) @ w_qkv^T, q and k heads rotated at the rows' positions, q
+    written to q_out (bfloat16) and k, v into the rows' cache pages. Full rotation, head size a
+    multiple of 32."""
+    require(h, "h", torch.float32, (None, None))
+    M, K = h.shape
+    require(norm_weight, "norm_weight", (torch.float32, torch.bfloat16), (K,))
+    require(w_qkv, "w_qkv", torch.bfloat16, ((n_q + 2 * n_kv) * head_dim, K))
+    require(positions, "positions", torch.int32, (M,))
+    require(seq_idx, "seq_idx", torch.int32, (M,))
+    require(block_table, "block_table", torch.int32, (None, None))
+    require(cos, "cos", torch.float32, (None, head_dim // 2))
+    require(sin, "sin", torch.float32, tuple(cos.shape))
+    require(q_out, "q_out", torch.bfloat16, (M, n_q * head_dim))
+    require(k_cache, "k_cache", torch.bfloat16, (None, n_kv, None, head_dim))
+    page = k_cache.shape[2]
+    require(v_cache, "v_cache", torch.bfloat16, (k_cache.shape[0], n_kv, head_dim, page))
+    if not gemv_norm_rope_supported(h, norm_weight, w_qkv, k_cache, M, head_dim, head_dim):
+        raise kernels.KernelError(f"gemv_norm_rope: {M} rows (at most 16), head size {head_dim} (multiple of 32) or "
+                                  "the operand types are not supported")
+    check(entry("llme_gemv_norm_rope")(
+        ptr(h), ptr(norm_weight), 0 if norm_weight.dtype == torch.float32 else 1, float(eps), ptr(w_qkv),
+        ptr(positions), ptr(seq_idx), ptr(block_table), block_table.shape[1], ptr(cos), ptr(sin), ptr(q_out),
+        ptr(k_cache), ptr(v_cache), M, K, n_q, n_kv, head_dim, page, grid, stream()), "gemv_norm_rope")

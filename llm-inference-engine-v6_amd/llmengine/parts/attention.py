@@ -85,7 +85,12 @@ class Attention(Mixer):
                 ops.gemv_norm(x, pre_norm.weight, pre_norm.eps, weight, dst)
             else:
                 ops.gemm(x, weight, dst)
-        if write_cache:
+        if (write_cache and pre_norm is not None and cos is not None
+                and ops.gemv_norm_rope_supported(x, pre_norm.weight, self.w_qkv, k_cache, T, hd, rot)):
+            # decoding: norm, projection, rotation and the cache write are one kernel
+            ops.gemv_norm_rope(x, pre_norm.weight, pre_norm.eps, self.w_qkv, step.positions, step.seq_idx,
+                               block_table, cos, sin, q, k_cache, v_cache, n_q, n_kv, hd)
+        elif write_cache:
             qkv = step.buffer("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
             project(self.w_qkv, qkv)
             ops.rope_kv_write(qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,

@@ -457,3 +457,43 @@ def test_gemv_norm_refusals(ops):
     with pytest.raises(KernelError):
         ops.gemv_norm(h[:4, :60].contiguous(), nw[:60].contiguous(), 1e-5, w[:, :60].contiguous(),
                       torch.empty(4, 32, device=DEV))                              # K no multiple of 8
+
+
+@pytest.mark.parametrize("M,n_q,n_kv,hd,K,page", [(1, 4, 2, 32, 64, 16), (8, 32, 8, 64, 2048, 16), (16, 3, 1, 96, 96, 32),
+                                                  (5, 6, 2, 128, 144, 16), (3, 40, 8, 64, 256, 64)])
+@pytest.mark.parametrize("grid", [0, 3])
+def test_gemv_norm_rope(ops, M, n_q, n_kv, hd, K, page, grid):
+    """The fused kernel against its parts: norm, projection, rotation, cache write."""
+    g = _gen(70)
+    h = 2 * torch.randn(M, K, generator=g)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(torch.bfloat16)
+    N = (n_q + 2 * n_kv) * hd
+    w = (0.05 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    positions = torch.randint(0, 5 * page, (M,), generator=g).to(torch.int32)
+    seq_idx = torch.arange(M, dtype=torch.int32)                  # one request per row
+    table = torch.randperm(M * 5, generator=g).to(torch.int32).view(M, 5)
+    half = hd // 2
+    inv = 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float64) * 2 / hd))
+    ang = torch.arange(5 * page, dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = torch.cos(ang).float(), torch.sin(ang).float()
+    k_cache = torch.zeros(M * 5, n_kv, page, hd, dtype=torch.bfloat16, device=DEV)
+    v_cache = torch.zeros(M * 5, n_kv, hd, page, dtype=torch.bfloat16, device=DEV)
+    q_out = torch.zeros(M, n_q * hd, dtype=torch.bfloat16, device=DEV)
+    ops.gemv_norm_rope(h.to(DEV), nw.to(DEV), 1e-5, w.to(DEV), positions.to(DEV), seq_idx.to(DEV), table.to(DEV),
+                       cos.to(DEV), sin.to(DEV), q_out, k_cache, v_cache, n_q, n_kv, hd, grid=grid)
+    x = plain_rmsnorm(h.double(), nw.double(), 1e-5)
+    qkv = plain_linear(x, w.double())
+    c = torch.cat([cos, cos], dim=1)[positions.long()].double()
+    s_ = torch.cat([sin, sin], dim=1)[positions.long()].double()
+    q_ref = plain_apply_rope(qkv[:, :n_q * hd].reshape(M, n_q, hd), c, s_).reshape(M, -1)
+    k_ref = plain_apply_rope(qkv[:, n_q * hd:(n_q + n_kv) * hd].reshape(M, n_kv, hd), c, s_)
+    v_ref = qkv[:, (n_q + n_kv) * hd:].reshape(M, n_kv, hd)
+    assert _rel(q_out.cpu().double(), q_ref) < 8e-3
+    kc, vc = k_cache.cpu().double(), v_cache.cpu().double()
+    scale = qkv.abs().max()
+    for m in range(M):
+        pos = int(positions[m])
+        pg, off = int(table[m, pos // page]), pos % page
+        assert (kc[pg, :, off, :] - k_ref[m]).abs().max() < 8e-3 * scale
+        assert (vc[pg, :, :, off] - v_ref[m]).abs().max() < 8e-3 * scale
+    assert int((kc != 0).sum()) <= M * n_kv * hd and int((vc != 0).sum()) <= M * n_kv * hd   # nothing else written
