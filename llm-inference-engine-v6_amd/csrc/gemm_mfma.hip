@@ -45,7 +45,7 @@ enum OutMode : int { kStoreF32 = 0, kAddF32 = 1, kStoreBF16 = 2, kAtomicF32 = 3,
 // per product (the 64 x 64 wavefront tile is bound by LDS reads); smaller tiles give more
 // workgroups when the output is small.
 constexpr int TK = 64;
-constexpr int TSTRIDE = TK + 8;                      // elements; 144 bytes: conflict-free 16-byte reads
+constexpr int TSTRIDE = TK + 16;                     // elements; 160-byte rows measured fastest (144 had bank conflicts)
 
 template <int WMT, int WNT>
 constexpr int tile_lds_bytes() { return 2 * (32 * WMT + 32 * WNT) * TSTRIDE * 2; }   // A and W, two buffers
@@ -151,7 +151,75 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__
         __syncthreads();
     }
 
-    // result tile (i, j): column n = wn + 16 j + r, rows m = wm + 16 i + 4 q + e
+    // Epilogue. The result tile (i, j) of a lane is column wn + 16 j + r, rows wm + 16 i + 4 q + e:
+    // written straight from there, a store instruction touches 4 rows with 64 bytes each. Where
+    // the tile fits into the LDS that the operand slabs no longer need, it goes through LDS
+    // instead, so that every thread stores 16 contiguous bytes of a row.
+    constexpr int SS = BN + 4;                           // floats per staged row
+    // (Atomic adds are faster scattered than packed into the same cache lines: they stay direct.)
+    constexpr bool STAGED = MODE != kAtomicF32 &&
+                            static_cast<size_t>(BM) * SS * 4 <= static_cast<size_t>(tile_lds_bytes<WMT, WNT>());
+    if (STAGED && N % 8 == 0) {
+        float* stage = reinterpret_cast<float*>(lds_raw);
+#pragma unroll
+        for (int i = 0; i < WMT; ++i)
+#pragma unroll
+            for (int j = 0; j < WNT; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    stage[(wm + i * 16 + q * 4 + e) * SS + wn + j * 16 + r] = acc[i][j][e];
+        __syncthreads();
+        if (MODE == kGatedBF16) {
+            // a thread makes 8 units: their gates and ups lie 16 columns apart in a group of 32
+            constexpr int PER_ROW = BN / 16;             // 8-unit pieces per row
+            for (int idx = tid; idx < BM * PER_ROW; idx += 256) {
+                const int row = idx / PER_ROW, piece = idx % PER_ROW;
+                const int col = (piece / 2) * 32 + (piece % 2) * 8;
+                const int m = m0 + row, n = n0 + col;
+                if (m >= M || n >= N) continue;
+                const float* gp = stage + row * SS + col;
+                bf16x8 o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float gt = gp[e], up = gp[16 + e];
+                    o[e] = static_cast<__bf16>((gt / (1.0f + expf(-gt))) * up);
+                }
+                const int unit = (n0 + (piece / 2) * 32) / 2 + (piece % 2) * 8;
+                *reinterpret_cast<bf16x8*>(static_cast<bf16*>(out) + static_cast<size_t>(m) * (N / 2) + unit) = o;
+            }
+        } else if (MODE == kStoreBF16) {
+            constexpr int PER_ROW = BN / 8;
+            for (int idx = tid; idx < BM * PER_ROW; idx += 256) {
+                const int row = idx / PER_ROW, col = (idx % PER_ROW) * 8;
+                const int m = m0 + row, n = n0 + col;
+                if (m >= M || n >= N) continue;
+                const float* sp = stage + row * SS + col;
+                bf16x8 o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = static_cast<__bf16>(sp[e]);
+                *reinterpret_cast<bf16x8*>(static_cast<bf16*>(out) + static_cast<size_t>(m) * N + n) = o;
+            }
+        } else {
+            constexpr int PER_ROW = BN / 4;
+            for (int idx = tid; idx < BM * PER_ROW; idx += 256) {
+                const int row = idx / PER_ROW, col = (idx % PER_ROW) * 4;
+                const int m = m0 + row, n = n0 + col;
+                if (m >= M || n >= N) continue;
+                const float4 v = *reinterpret_cast<const float4*>(stage + row * SS + col);
+                float* op = static_cast<float*>(out) + static_cast<size_t>(m) * N + n;
+                if (MODE == kStoreF32) {
+                    *reinterpret_cast<float4*>(op) = v;
+                } else if (MODE == kAddF32) {
+                    float4 cur = *reinterpret_cast<const float4*>(op);
+                    cur.x += v.x; cur.y += v.y; cur.z += v.z; cur.w += v.w;
+                    *reinterpret_cast<float4*>(op) = cur;
+                } else {
+                    atomicAdd(op, v.x); atomicAdd(op + 1, v.y); atomicAdd(op + 2, v.z); atomicAdd(op + 3, v.w);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < WMT; ++i) {
 #pragma unroll
@@ -375,6 +443,7 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     if (tile_shape <= 0) {
         const long wg128 = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
         tile_shape = (M > 64 && wg128 >= 64) ? 128 : 64;
+        if (tile_shape == 128 && mode == kAddF32 && ksplit <= 0 && wg128 <= 256 && K >= 4096) ksplit = 2;
         if (M <= 64 && mode == kAddF32 && ksplit <= 0) {
             // one row of tiles: cut k so that about two workgroups per compute unit stream the matrix
             const int tiles = (N + 63) / 64;

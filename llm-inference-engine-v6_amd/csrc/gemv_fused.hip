@@ -271,6 +271,9 @@ template <int EPI, typename TNW>
 static int launch_gemv_norm_shape(int tpr, const float* h, const int* rows, const void* norm_w, float eps,
                                   const bf16* w, void* out, int M, int N, int K, int grid, hipStream_t stream) {
     const RopeTarget none{};
+    // tpr: tiles at a time; 12 and 14: 2 and 4 tiles with 16 wavefronts instead of 8
+    if (tpr == 12) return launch_gemv_norm<16, 2, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
+    if (tpr == 14) return launch_gemv_norm<16, 4, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
     if (tpr >= 4) return launch_gemv_norm<8, 4, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
     if (tpr == 2) return launch_gemv_norm<8, 2, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
     return launch_gemv_norm<8, 1, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
@@ -297,9 +300,10 @@ extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_
         // more tiles than compute units: 2 tiles at a time, 4 wavefronts each with several chunks of k
         tpr = tiles <= 256 ? 1 : 2;
     }
-    if (tpr != 1 && tpr != 2 && tpr != 4) return kErrBadArgument;
+    if (tpr != 1 && tpr != 2 && tpr != 4 && tpr != 12 && tpr != 14) return kErrBadArgument;
     if (grid <= 0) {
-        grid = (tiles + tpr - 1) / tpr;
+        const int at_a_time = tpr > 10 ? tpr - 10 : tpr;
+        grid = (tiles + at_a_time - 1) / at_a_time;
         if (grid > 512) grid = 512;                     // two workgroups per compute unit
     }
     const bf16* W = static_cast<const bf16*>(w);
