@@ -8,8 +8,8 @@ import torch
 
 import replay
 from plain_llama import bf16_round, load_plain_model, plain_forward
-from tiny_models import (A_INIT, B_INIT, C_INIT, D_INIT, TINY_A, TINY_B, TINY_C, TINY_D, make_model_dir,
-                         random_tokens)
+from tiny_models import (A_INIT, B_INIT, C_INIT, D_INIT, E_INIT, TINY_A, TINY_B, TINY_C, TINY_D, TINY_E,
+                         make_model_dir, random_tokens)
 
 pytestmark = pytest.mark.gpu
 
@@ -20,6 +20,7 @@ MODELS = {
     "A": (TINY_A, A_INIT, 4, [5, 11, 17, 40]),
     "B": (TINY_B, B_INIT, 8, [1, 9, 33, 70]),
     "D": (TINY_D, D_INIT, 16, [3, 50, 66, 21]),
+    "E": (TINY_E, E_INIT, 16, [2, 35, 64, 17]),
 }
 
 
@@ -73,7 +74,7 @@ SCHEDULES = {
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
 @pytest.mark.parametrize("schedule", list(SCHEDULES))
-@pytest.mark.parametrize("name,page_override", [("A", 0), ("B", 0), ("D", 0), ("A", 16), ("B", 16), ("D", 32)])
+@pytest.mark.parametrize("name,page_override", [("A", 0), ("B", 0), ("D", 0), ("E", 0), ("A", 16), ("B", 16), ("D", 32)])
 def test_schedules_match_plain(zoo, name, page_override, schedule, dtype):
     """Pages of 4 and 8 tokens go through the plain-precision attention kernel also in
     bfloat16; pages of 16 and 32 through the MFMA kernels."""
@@ -87,6 +88,22 @@ def test_schedules_match_plain(zoo, name, page_override, schedule, dtype):
     got = replay.run_trace(engine, cache, steps)
     check_against_plain(got, plain[dtype], reqs, dtype)
     assert all(cache.manager.free_pages(g) == cache.manager.num_pages(g) for g in cache.manager.groups)
+
+
+@pytest.mark.parametrize("schedule", ["whole", "mixed"])
+def test_weights_stored_in_32_bit_stay_so_in_the_bfloat16_model(tmp_path, schedule):
+    """A checkpoint in float32 run with dtype bf16: activations and cache are bfloat16, the
+    weights keep their 32 bits (the products then take the plain-precision kernel)."""
+    from llmengine import Engine
+    d = make_model_dir(tmp_path, TINY_B, B_INIT, torch.float32)
+    reqs = {f"r{i}": random_tokens(n, TINY_B["vocab_size"], 200 + i) for i, n in enumerate([9, 40, 3, 33])}
+    pcfg, pw = load_plain_model(d)
+    plain = {rid: plain_forward(pcfg, pw, ids, rounder=bf16_round).numpy() for rid, ids in reqs.items()}
+    engine = Engine(d, "bf16")
+    assert engine.model.layers[0].mixer.w_qkv.dtype == torch.float32
+    steps = SCHEDULES[schedule](reqs)
+    cache = engine.new_cache(replay.trace_peak_tokens(steps, 16) // 16, 16, 4)
+    check_against_plain(replay.run_trace(engine, cache, steps), plain, reqs, "bf16")
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])

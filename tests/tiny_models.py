@@ -52,6 +52,18 @@ TINY_D = {
 D_INIT = dict(seed=3, std=0.05, norm_mean=1.0, norm_std=0.1)
 
 
+# E: sizes that no fast kernel takes whole: width 72 with 3 heads of 16 (q_dim 48 != width), feed-forward 100
+# (no multiple of 8 or 16), vocabulary 257, 4 layers, MQA
+TINY_E = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 72, "intermediate_size": 100, "num_hidden_layers": 4,
+    "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 16,
+    "vocab_size": 257, "max_position_embeddings": 300, "rms_norm_eps": 1e-5,
+    "rope_theta": 10000.0, "tie_word_embeddings": True,
+}
+E_INIT = dict(seed=4, std=0.06, norm_mean=1.0, norm_std=0.1)
+
+
 def make_model_dir(tmp_path, cfg: dict, init: dict, dtype=torch.bfloat16) -> str:
     from llmengine.weights import write_random_model
     return write_random_model(cfg, str(tmp_path), init["seed"], dtype, init["std"], init["norm_mean"],
