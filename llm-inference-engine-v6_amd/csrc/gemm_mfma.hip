@@ -443,6 +443,26 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     if (tile_shape <= 0) {
         const long wg128 = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
         tile_shape = (M > 64 && wg128 >= 64) ? 128 : 64;
+        if (tile_shape == 128 && wg128 < 1024 && !(mode == kAddF32 && wg128 <= 256 && K >= 4096)) {
+            // Medium outputs: narrower tiles can fill the 256 compute units (two workgroups
+            // each) more evenly. Estimated time: rounds of 256 workgroups x tile area / measured
+            // efficiency of the shape; a workgroup alone on its compute unit overlaps nothing.
+            const long tm = (M + 127) / 128;
+            const int shapes[3] = {128, 128096, 128064};
+            const int widths[3] = {128, 96, 64};
+            const float eff[3] = {1.0f, 0.9f, 0.85f};
+            float best = 0.f;
+            for (int c = 0; c < 3; ++c) {
+                const long wgs = tm * ((N + widths[c] - 1) / widths[c]);
+                const long rounds = (wgs + 255) / 256;
+                float cost = static_cast<float>(rounds) * 128.f * widths[c] / eff[c];
+                if (wgs <= 256) cost *= 1.25f;
+                if (c == 0 || cost < best) {
+                    best = cost;
+                    tile_shape = shapes[c];
+                }
+            }
+        }
         if (tile_shape == 128 && mode == kAddF32 && ksplit <= 0 && wg128 <= 256 && K >= 4096) ksplit = 2;
         if (M <= 64 && mode == kAddF32 && ksplit <= 0) {
             // one row of tiles: cut k so that about two workgroups per compute unit stream the matrix
@@ -457,6 +477,8 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
         if (mode != kAddF32) return kErrBadArgument;
         mode = kAtomicF32;
     }
+    if (tile_shape == 128096) return launch_tile<4, 3>(A, W, out, M, N, K, mode, ksplit, stream);
+    if (tile_shape == 128064) return launch_tile<4, 2>(A, W, out, M, N, K, mode, ksplit, stream);
     if (tile_shape == 256) return launch_tile<8, 8>(A, W, out, M, N, K, mode, ksplit, stream);
     if (tile_shape == 128) return launch_tile<4, 4>(A, W, out, M, N, K, mode, ksplit, stream);
     if (tile_shape == 64) return launch_tile<2, 2>(A, W, out, M, N, K, mode, ksplit, stream);
