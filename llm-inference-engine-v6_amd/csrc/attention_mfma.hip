@@ -31,237 +31,9 @@
 //
 // Limits (the caller checks them and otherwise uses the plain-precision kernel): head size a
 // multiple of 16 up to 128; page size a multiple of 16.
-#include "common.h"
-#include <math.h>
+#include "attention_tiles.h"
 
 namespace llme {
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLazy = 8.0f;
-
-// 2^x by the hardware instruction alone: arguments here are <= 0, results below the normal
-// range may flush to zero, which is what a softmax weight that small amounts to.
-__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-struct PagedKV {
-    const bf16* k;
-    const bf16* v;
-    const int* table;       // this request's row of the block table
-    int page, n_kv, kvh, hd;
-};
-
-__device__ __forceinline__ bf16x8 zero_frag() {
-    bf16x8 z;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) z[i] = static_cast<__bf16>(0.f);
-    return z;
-}
-
-// The K and V operands of one 32-key block (keys t0 .. t0 + 31), as one lane holds them.
-template <int HD>
-struct KVFrag {
-    bf16x8 kf[2][(HD + 31) / 32];      // row r of each 16-key half: dims c * 32 + 8 g4 ..
-    bf16x8 vf[HD / 16];                // dim dt * 16 + r: keys 4 g4 .. 4 g4 + 3 of each half
-};
-
-// The pages of a block's two 16-key halves (a half never straddles pages: the page size is a
-// multiple of 16). A half none of whose keys lies in [key_lo, key_end) is not looked up: behind
-// key_end nothing is written yet (and the table may end), before key_lo (the first key any
-// row of the work item may see) the pages may have been given back.
-struct BlockPages {
-    int pg[2];
-};
-
-__device__ __forceinline__ BlockPages lookup_pages(const PagedKV& kv, int t0, int key_lo, int key_end) {
-    BlockPages b;
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-        const int h0 = t0 + hf * 16;
-        // the same for every lane: kept in a scalar register, so that page addresses are scalar work
-        b.pg[hf] = (h0 < key_end && h0 + 15 >= key_lo) ? __builtin_amdgcn_readfirstlane(kv.table[h0 / kv.page]) : 0;
-    }
-    return b;
-}
-
-// Loads a block's operands from the pages looked up before. Keys outside [key_lo, key_end)
-// are not loaded (zeros); a block that lies inside the range whole takes the path without
-// any per-lane checks.
-template <int HD>
-__device__ __forceinline__ void load_block(const PagedKV& kv, int t0, const BlockPages& pages, int key_lo, int key_end,
-                                           KVFrag<HD>& f) {
-    constexpr int DC = (HD + 31) / 32, DT = HD / 16;
-    const int lane = threadIdx.x & 63;
-    const int r = lane & 15, g4 = lane >> 4;
-    const bool inside = t0 >= key_lo && t0 + 32 <= key_end;        // uniform
-    const bf16* krow[2];
-    const bf16* vbase[2];
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-        const int h0 = t0 + hf * 16;
-        const size_t page_base = (static_cast<size_t>(pages.pg[hf]) * kv.n_kv + kv.kvh) * kv.page * HD;   // scalar
-        krow[hf] = kv.k + page_base + static_cast<size_t>(h0 % kv.page + r) * HD + g4 * 8;
-        vbase[hf] = kv.v + page_base + static_cast<size_t>(r) * kv.page + (h0 % kv.page + g4 * 4);
-    }
-    if (inside) {
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-            for (int c = 0; c < DC; ++c)
-                f.kf[hf][c] = (HD % 32 == 0 || c * 32 + g4 * 8 < HD)
-                                  ? *reinterpret_cast<const bf16x8*>(krow[hf] + c * 32) : zero_frag();
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const size_t off = static_cast<size_t>(dt) * 16 * kv.page;
-            const bf16x4 lo4 = *reinterpret_cast<const bf16x4*>(vbase[0] + off);
-            const bf16x4 hi4 = *reinterpret_cast<const bf16x4*>(vbase[1] + off);
-            f.vf[dt] = __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-        return;
-    }
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-        const int t = t0 + hf * 16 + r;
-        const bool ok = t >= key_lo && t < key_end;
-#pragma unroll
-        for (int c = 0; c < DC; ++c)
-            f.kf[hf][c] = (ok && c * 32 + g4 * 8 < HD) ? *reinterpret_cast<const bf16x8*>(krow[hf] + c * 32)
-                                                       : zero_frag();
-    }
-    bool ok[2];
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-        const int t = t0 + hf * 16 + g4 * 4;
-        ok[hf] = t + 3 >= key_lo && t < key_end;     // the 4 keys share a page with a visible key
-    }
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-        const size_t off = static_cast<size_t>(dt) * 16 * kv.page;
-        bf16x4 lo4, hi4;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) lo4[e] = hi4[e] = static_cast<__bf16>(0.f);
-        if (ok[0]) lo4 = *reinterpret_cast<const bf16x4*>(vbase[0] + off);
-        if (ok[1]) hi4 = *reinterpret_cast<const bf16x4*>(vbase[1] + off);
-        f.vf[dt] = __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
-}
-
-// One 32-key block for QT row tiles. row_pos[qt]: position of this lane's row (l % 16) in
-// tile qt, or -1 for a row that does not exist; row_lo[qt]: first key the row may see;
-// tile_free[qt]: the last key every row of tile qt sees without a check (the position of its
-// first row if all 16 rows exist and there is no window, else -1): blocks that end at or
-// before it skip the masking.
-template <int HD, int QT>
-__device__ __forceinline__ void attend_block(const KVFrag<HD>& f, int t0, const bf16x8 (&qf)[QT][(HD + 31) / 32],
-                                             const int (&row_pos)[QT], const int (&row_lo)[QT],
-                                             const int (&tile_free)[QT], float scale_log2, float (&m)[QT],
-                                             float (&l)[QT], f32x4 (&o)[QT][HD / 16]) {
-    constexpr int DC = (HD + 31) / 32, DT = HD / 16;
-    const int lane = threadIdx.x & 63;
-    const int g4 = lane >> 4;
-#pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-        f32x4 s[2];
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-            s[hf] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int c = 0; c < DC; ++c)
-                s[hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.kf[hf][c], qf[qt][c], s[hf], 0, 0, 0);
-        }
-        // this lane: row r of tile qt, keys t0 + 16 hf + 4 g4 + e
-        float mx = -INFINITY;
-        if (t0 + 31 <= tile_free[qt]) {
-#pragma unroll
-            for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    s[hf][e] *= scale_log2;
-                    mx = fmaxf(mx, s[hf][e]);
-                }
-        } else {
-            const int pos = row_pos[qt], lo = row_lo[qt];
-#pragma unroll
-            for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int t = t0 + hf * 16 + g4 * 4 + e;
-                    const bool see = (t <= pos) && (t >= lo);
-                    const float v = see ? s[hf][e] * scale_log2 : -INFINITY;
-                    s[hf][e] = v;
-                    mx = fmaxf(mx, v);
-                }
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        // The reference maximum moves only when a score exceeds it by more than kLazy (in powers
-        // of two): until then weights are at most 2^kLazy, well inside the range, and the sums
-        // need no rescaling. The softmax does not depend on which reference is subtracted.
-        const float m_new = (mx > m[qt] + kLazy) ? mx : m[qt];
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;       // nothing seen yet: all p are 0
-        const float alpha = fast_exp2(m[qt] - m_use);                  // 0 when m was -inf
-        m[qt] = m_new;
-        bf16x8 pf;
-        float psum = 0.f;
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float p = fast_exp2(s[hf][e] - m_use);
-                psum += p;
-                pf[hf * 4 + e] = static_cast<__bf16>(p);
-            }
-        l[qt] = l[qt] * alpha + psum;
-        if (__any(alpha != 1.0f)) {                    // some row's maximum moved: rescale what is summed
-            float ar[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) ar[e] = __shfl(alpha, g4 * 4 + e, 64);     // factor of O's row 4 g4 + e
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) o[qt][dt][e] *= ar[e];
-        }
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-            o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, f.vf[dt], o[qt][dt], 0, 0, 0);
-    }
-}
-
-// Walks the 32-key blocks t0 = first, first + stride, ... < key_end: the next block's loads
-// are in flight while the current block is computed, and the page ids are looked up one block
-// further ahead, so that no load waits for a table entry.
-template <int HD, int QT>
-__device__ __forceinline__ void attend_range(const PagedKV& kv, int first, int stride, int key_lo, int key_end,
-                                             const bf16x8 (&qf)[QT][(HD + 31) / 32], const int (&row_pos)[QT],
-                                             const int (&row_lo)[QT], const int (&tile_free)[QT], float scale_log2,
-                                             float (&m)[QT], float (&l)[QT], f32x4 (&o)[QT][HD / 16]) {
-    if (first >= key_end) return;
-    KVFrag<HD> cur, nxt;
-    BlockPages pg_next = lookup_pages(kv, first + stride, key_lo, key_end);
-    load_block<HD>(kv, first, lookup_pages(kv, first, key_lo, key_end), key_lo, key_end, cur);
-    for (int t0 = first; t0 < key_end; t0 += stride) {
-        const bool more = t0 + stride < key_end;
-        const BlockPages pg_after = lookup_pages(kv, t0 + 2 * stride, key_lo, key_end);
-        if (more) load_block<HD>(kv, t0 + stride, pg_next, key_lo, key_end, nxt);
-        attend_block<HD, QT>(cur, t0, qf, row_pos, row_lo, tile_free, scale_log2, m, l, o);
-        if (more) cur = nxt;
-        pg_next = pg_after;
-    }
-}
-
-// Loads the query fragments of one 16-row tile: lane holds row r, dims c * 32 + 8 g4 ..
-template <int HD>
-__device__ __forceinline__ void load_q(const bf16* qrow, bool ok, bf16x8 (&qf)[(HD + 31) / 32]) {
-    const int g4 = (threadIdx.x & 63) >> 4;
-#pragma unroll
-    for (int c = 0; c < (HD + 31) / 32; ++c) {
-        const int d = c * 32 + g4 * 8;
-        qf[c] = (ok && d < HD) ? *reinterpret_cast<const bf16x8*>(qrow + d) : zero_frag();
-    }
-}
 
 // ------------------------------------------------------------------------------------------
 // decode: one token per request. A workgroup of four wavefronts takes one split of the keys
@@ -300,12 +72,13 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     const int row_pos[1] = {row_ok ? pos : -1};
     const int row_lo[1] = {lo_all};
     const int tile_free[1] = {-1};                      // few blocks, heads may be missing: always checked
-    float m[1] = {-INFINITY}, l[1] = {0.f};
+    float m[1] = {kNoMax}, l[1] = {0.f};
     f32x4 o[1][DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD};
+    PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD,
+               page_magic_of(page), static_cast<size_t>(n_kv) * page * HD, static_cast<size_t>(kvh) * page * HD};
     const int first = k_begin + __builtin_amdgcn_readfirstlane(wave) * 32;
     attend_range<HD, 1>(kv, first, DEC_WAVES * 32, lo_all, k_end, qf, row_pos, row_lo, tile_free, scale * kLog2e,
                         m, l, o);
@@ -333,7 +106,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
 #pragma unroll
         for (int w = 0; w < DEC_WAVES; ++w) {
             const float mw = sh_m[w][row];
-            const float f = (mw == -INFINITY) ? 0.f : exp2f(mw - mx);
+            const float f = (mw <= kNoMax) ? 0.f : exp2f(mw - mx);
             acc += f * sh_o[w][row][d];
             lsum += f * sh_l[w][row];
         }
@@ -367,7 +140,7 @@ __global__ __launch_bounds__(64) void attention_join_kernel(const float* __restr
         li = part_ml[(base + lane) * 2 + 1];
     }
     const float mx = wave_max(mi);
-    const float f = (mi == -INFINITY) ? 0.f : exp2f(mi - mx);
+    const float f = (mi <= kNoMax) ? 0.f : exp2f(mi - mx);
     const float total = wave_sum(f * li);
     weight[lane] = f / total;
     __syncthreads();
@@ -410,7 +183,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
         acc += nt;
     }
     if (!found) return;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g4 = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);      // scalar: so are the head's addresses
+    const int lane = threadIdx.x & 63, r = lane & 15, g4 = lane >> 4;
     const int head = blockIdx.y * 4 + wave;
     if (head >= n_q) return;
     const int kvh = head / (n_q / n_kv);
@@ -428,7 +202,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
         row_pos[qt] = ok ? pos0 + rr : -1;
         row_lo[qt] = (window > 0 && pos0 + rr - window + 1 > 0) ? pos0 + rr - window + 1 : 0;
         tile_free[qt] = (window == 0 && qt * 16 + 16 <= n_rows) ? pos0 + qt * 16 : -1;
-        m[qt] = -INFINITY;
+        m[qt] = kNoMax;
         l[qt] = 0.f;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -436,7 +210,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     const int key_end = pos0 + n_rows;                    // the last row sees keys < key_end
     const int key_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;   // the first row's first key
     const int k_begin = key_lo & ~31;
-    PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD};
+    PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD,
+               page_magic_of(page), static_cast<size_t>(n_kv) * page * HD, static_cast<size_t>(kvh) * page * HD};
     const float scale_log2 = scale * kLog2e;
     attend_range<HD, QT>(kv, k_begin, 32, key_lo, key_end, qf, row_pos, row_lo, tile_free, scale_log2, m, l, o);
 
@@ -464,7 +239,7 @@ template <int HD>
 static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, float* part_o, float* part_ml,
                            const int* q_start, const int* ctx_len, const int* table, int max_blocks, int n_seq,
                            int n_q, int n_kv, int page, float scale, int window, int n_decode, int split_len,
-                           int nsplit, int prefill_groups, int qt, hipStream_t stream) {
+                           int nsplit, int prefill_groups, int qt, int shared_rows, hipStream_t stream) {
     if (n_decode > 0) {
         const int G = n_q / n_kv;
         const dim3 grid(n_seq, n_kv * ((G + 15) / 16), nsplit);
@@ -475,6 +250,9 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
                                q_start, n_q, HD, nsplit);
     }
     if (prefill_groups > 0) {
+        if (shared_rows > 0)
+            return launch_prefill_shared(q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, HD,
+                                         page, scale, window, prefill_groups, shared_rows, stream);
         const dim3 grid(prefill_groups, (n_q + 3) / 4);
 #define LLME_PREFILL(QT)                                                                                       \
     hipLaunchKernelGGL((attention_prefill_kernel<HD, QT>), grid, dim3(256), 0, stream, q, kc, vc, out, q_start, \
@@ -491,27 +269,37 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
 
 using namespace llme;
 
-// Rows per prefill work item (16, 32 or 64) for a head size: the caller sizes the grid with it.
-// More rows reuse every K and V load more often; fewer rows give more wavefronts to hide
-// latencies and to even out the causal triangle. llme_attention_bf16_set_rows overrides the
-// choice (0: back to the default) for measurements.
+// Rows per prefill work item for a model's head sizes: the caller sizes the grid with it. More
+// rows reuse every K and V load more often; fewer rows give more wavefronts to hide latencies
+// and to even out the causal triangle. The kernel that shares K and V through LDS is used
+// where it takes the sizes. llme_attention_bf16_set_rows overrides the choice for
+// measurements: rows per item (0: the default), shared -1: as by default, 0: never, 1: if it can.
 static int g_rows_override = 0;
-extern "C" int llme_attention_bf16_set_rows(int rows) {
-    if (rows != 0 && rows != 16 && rows != 32 && rows != 64) return kErrBadArgument;
+static int g_shared_override = -1;
+extern "C" int llme_attention_bf16_set_rows(int rows, int shared) {
+    if (rows < 0 || rows % 16 != 0 || rows > 256 || shared < -1 || shared > 1) return kErrBadArgument;
     g_rows_override = rows;
+    g_shared_override = shared;
     return 0;
 }
-extern "C" int llme_attention_bf16_rows(int hd) {
-    int rows = hd <= 64 ? 32 : 16;
-    if (g_rows_override) rows = g_rows_override;
+static int direct_rows(int hd) {
+    int rows = hd <= 64 ? 64 : 32;
+    if (g_rows_override == 16 || g_rows_override == 32 || g_rows_override == 64) rows = g_rows_override;
     if (hd > 64 && rows > 32) rows = 32;
     return rows;
+}
+static int shared_rows_for(int hd, int n_q, int n_kv) {
+    return g_shared_override == 0 ? 0 : prefill_shared_rows(hd, n_q, n_kv, g_rows_override);
+}
+extern "C" int llme_attention_bf16_rows(int hd, int n_q, int n_kv) {
+    const int shared = shared_rows_for(hd, n_q, n_kv);
+    return shared > 0 ? shared : direct_rows(hd);
 }
 
 // n_decode: requests with one token (0: none, skip the decode kernels); split_len (multiple of
 // 32) and nsplit: how the decode kernel cuts the keys; part_o [n_seq, n_q, nsplit, hd] and
 // part_ml [n_seq, n_q, nsplit, 2] floats (needed when nsplit > 1). prefill_groups: number of
-// row groups of llme_attention_bf16_rows(hd) rows over the requests with two or more tokens.
+// row groups of llme_attention_bf16_rows(hd, n_q, n_kv) rows over the requests with two or more tokens.
 extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const void* v_cache, void* out, float* part_o,
                                    float* part_ml, const int* q_start, const int* ctx_len, const int* block_table,
                                    int max_blocks, int n_seq, int n_q, int n_kv, int hd, int page, float scale,
@@ -519,14 +307,18 @@ extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const voi
                                    hipStream_t stream) {
     if (n_seq <= 0) return 0;
     if (hd % 16 != 0 || hd > 128 || hd <= 0 || page % 16 != 0 || n_kv <= 0 || n_q % n_kv != 0) return kErrUnsupported;
+    if (!(scale > 0.f)) return kErrBadArgument;      // the lazy maximum compares scaled scores
+    // page lookups divide by multiplication, exact while (keys / 16) * (page / 16) < 2^32
+    if (static_cast<double>(max_blocks) * (page / 16) * (page / 16) >= 4294967296.0) return kErrUnsupported;
     if (n_decode > 0 && (split_len <= 0 || split_len % 32 != 0 || nsplit <= 0 || nsplit > 64)) return kErrBadArgument;
-    const int qt = llme_attention_bf16_rows(hd) / 16;
+    const int qt = direct_rows(hd) / 16;
+    const int shared_rows = shared_rows_for(hd, n_q, n_kv);
 #define LLME_HEAD(HD)                                                                                           \
     case HD:                                                                                                    \
         return launch_for_head<HD>(static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache),              \
                                    static_cast<const bf16*>(v_cache), static_cast<bf16*>(out), part_o, part_ml, \
                                    q_start, ctx_len, block_table, max_blocks, n_seq, n_q, n_kv, page, scale,    \
-                                   window, n_decode, split_len, nsplit, prefill_groups, qt, stream)
+                                   window, n_decode, split_len, nsplit, prefill_groups, qt, shared_rows, stream)
     switch (hd) {
         LLME_HEAD(16); LLME_HEAD(32); LLME_HEAD(48); LLME_HEAD(64);
         LLME_HEAD(80); LLME_HEAD(96); LLME_HEAD(112); LLME_HEAD(128);

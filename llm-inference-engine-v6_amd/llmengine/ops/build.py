@@ -27,6 +27,17 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
 ]
+# Flags for single sources. The attention kernels rescale their accumulators with ordinary
+# arithmetic between matrix instructions: with the accumulators in the general registers the
+# compiler does not copy them to and from the accumulation registers around every such step.
+SOURCE_FLAGS = {
+    "attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
+
+
+def flags_for(src: str) -> list[str]:
+    return HIPCC_FLAGS + SOURCE_FLAGS.get(os.path.basename(src), [])
 
 
 class BuildError(RuntimeError):
@@ -52,6 +63,7 @@ def source_digest() -> str:
         with open(path, "rb") as f:
             h.update(f.read())
     h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(repr(sorted(SOURCE_FLAGS.items())).encode())
     return h.hexdigest()[:24]
 
 
@@ -60,7 +72,7 @@ def _object_digest(src: str) -> str:
     for path in [src] + _headers():
         with open(path, "rb") as f:
             h.update(f.read())
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(flags_for(src)).encode())
     return h.hexdigest()[:16]
 
 
@@ -109,7 +121,7 @@ def _compile_one(hipcc: str, src: str, obj: str, env: dict, reuse: bool) -> tupl
     t0 = time.time()
     if reuse and os.path.isfile(obj):          # same source, headers and flags: keep the object
         return src, 0.0
-    cmd = [hipcc, *HIPCC_FLAGS, "-I", CSRC, "-c", src, "-o", obj]
+    cmd = [hipcc, *flags_for(src), "-I", CSRC, "-c", src, "-o", obj]
     tmp = obj + f".{os.getpid()}.tmp"
     cmd[-1] = tmp
     p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)

@@ -75,8 +75,8 @@ kernels._fast_gemm = _fast_gemm
 
 
 # --- attention ---------------------------------------------------------------------------
-declare("llme_attention_bf16_rows", [_i])
-declare("llme_attention_bf16_set_rows", [_i])
+declare("llme_attention_bf16_rows", [_i, _i, _i])
+declare("llme_attention_bf16_set_rows", [_i, _i])
 declare("llme_attention_bf16", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i,
                                 _i, _i, _i, _i, _vp])
 
@@ -95,7 +95,7 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
     """Launch sizes for a step, from how its batch is cut (host-side numbers only). plan_len:
     plan the decode splits for requests of up to this many tokens, whatever their length now
     (a recorded step is replayed while the requests grow)."""
-    rows = entry("llme_attention_bf16_rows")(head_dim)
+    rows = entry("llme_attention_bf16_rows")(head_dim, n_q, n_kv)
     decode = [c + 1 for n, c in zip(new_lens, ctx_lens) if n == 1]
     groups = sum((n + rows - 1) // rows for n in new_lens if n >= 2)
     plan = {"n_decode": len(decode), "groups": groups, "split_len": 32, "nsplit": 1}

@@ -361,6 +361,34 @@ def test_attention_mfma_prefill_and_mixed(ops, n_q, n_kv, hd, page):
     assert _rel(out, ref) < 8e-3
 
 
+@pytest.mark.parametrize("n_q,n_kv,hd,page", [(8, 2, 64, 16), (4, 2, 64, 48), (6, 2, 64, 32), (3, 3, 64, 16),
+                                              (8, 2, 128, 16), (2, 1, 128, 32), (5, 5, 128, 16)])
+@pytest.mark.parametrize("rows,shared", [(0, -1), (64, 1), (0, 0)])
+def test_attention_prefill_shared_and_direct(ops, n_q, n_kv, hd, page, rows, shared):
+    """The prefill kernel that shares K and V through LDS, for 4, 2 and 1 heads of a kv head per
+    workgroup, spans that end inside a 64-key stretch, portions that start deep in a context,
+    and the kernel without LDS at the same sizes."""
+    set_rows = ops.lib.entry("llme_attention_bf16_set_rows")
+    assert set_rows(rows, shared) == 0
+    try:
+        lens = [330, 2, 131, 64, 517, 65, 9]
+        news = [330, 2, 67, 64, 130, 3, 1]
+        out, ref, plan = _attn_case(ops, lens, news, n_q, n_kv, hd, page, seed=61)
+        assert plan["n_decode"] == 1 and plan["groups"] >= 6
+        assert _rel(out, ref) < 8e-3
+    finally:
+        set_rows(0, -1)
+
+
+@pytest.mark.parametrize("window", [1, 7, 64, 65, 200])
+@pytest.mark.parametrize("n_q,n_kv", [(8, 2), (3, 3)])
+def test_attention_prefill_shared_window(ops, window, n_q, n_kv):
+    lens = [300, 70, 190]
+    news = [140, 70, 2]
+    out, ref, _ = _attn_case(ops, lens, news, n_q, n_kv, 64, 16, window=window, seed=62)
+    assert _rel(out, ref) < 8e-3
+
+
 @pytest.mark.parametrize("window", [1, 5, 16, 33, 100])
 def test_attention_mfma_window(ops, window):
     lens = [150, 40, 90]
