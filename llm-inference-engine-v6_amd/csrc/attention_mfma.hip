@@ -78,7 +78,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD,
-               page_magic_of(page), static_cast<size_t>(n_kv) * page * HD, static_cast<size_t>(kvh) * page * HD};
+               page_magic_of(page), static_cast<unsigned>(n_kv) * page * HD, static_cast<unsigned>(kvh) * page * HD};
     const int first = k_begin + __builtin_amdgcn_readfirstlane(wave) * 32;
     attend_range<HD, 1>(kv, first, DEC_WAVES * 32, lo_all, k_end, qf, row_pos, row_lo, tile_free, scale * kLog2e,
                         m, l, o);
@@ -211,7 +211,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     const int key_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;   // the first row's first key
     const int k_begin = key_lo & ~31;
     PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD,
-               page_magic_of(page), static_cast<size_t>(n_kv) * page * HD, static_cast<size_t>(kvh) * page * HD};
+               page_magic_of(page), static_cast<unsigned>(n_kv) * page * HD, static_cast<unsigned>(kvh) * page * HD};
     const float scale_log2 = scale * kLog2e;
     attend_range<HD, QT>(kv, k_begin, 32, key_lo, key_end, qf, row_pos, row_lo, tile_free, scale_log2, m, l, o);
 
@@ -239,7 +239,7 @@ template <int HD>
 static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, float* part_o, float* part_ml,
                            const int* q_start, const int* ctx_len, const int* table, int max_blocks, int n_seq,
                            int n_q, int n_kv, int page, float scale, int window, int n_decode, int split_len,
-                           int nsplit, int prefill_groups, int qt, int shared_rows, hipStream_t stream) {
+                           int nsplit, int prefill_groups, int qt, int shared_rows, int* queue, hipStream_t stream) {
     if (n_decode > 0) {
         const int G = n_q / n_kv;
         const dim3 grid(n_seq, n_kv * ((G + 15) / 16), nsplit);
@@ -252,7 +252,7 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
     if (prefill_groups > 0) {
         if (shared_rows > 0)
             return launch_prefill_shared(q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, HD,
-                                         page, scale, window, prefill_groups, shared_rows, stream);
+                                         page, scale, window, prefill_groups, shared_rows, queue, stream);
         const dim3 grid(prefill_groups, (n_q + 3) / 4);
 #define LLME_PREFILL(QT)                                                                                       \
     hipLaunchKernelGGL((attention_prefill_kernel<HD, QT>), grid, dim3(256), 0, stream, q, kc, vc, out, q_start, \
@@ -273,7 +273,8 @@ using namespace llme;
 // rows reuse every K and V load more often; fewer rows give more wavefronts to hide latencies
 // and to even out the causal triangle. The kernel that shares K and V through LDS is used
 // where it takes the sizes. llme_attention_bf16_set_rows overrides the choice for
-// measurements: rows per item (0: the default), shared -1: as by default, 0: never, 1: if it can.
+// measurements: rows per item of the kernel without LDS (0: the default), shared -1: as by
+// default, 0: never, 1: if it can.
 static int g_rows_override = 0;
 static int g_shared_override = -1;
 extern "C" int llme_attention_bf16_set_rows(int rows, int shared) {
@@ -289,7 +290,7 @@ static int direct_rows(int hd) {
     return rows;
 }
 static int shared_rows_for(int hd, int n_q, int n_kv) {
-    return g_shared_override == 0 ? 0 : prefill_shared_rows(hd, n_q, n_kv, g_rows_override);
+    return g_shared_override == 0 ? 0 : prefill_shared_rows(hd, n_q, n_kv);
 }
 extern "C" int llme_attention_bf16_rows(int hd, int n_q, int n_kv) {
     const int shared = shared_rows_for(hd, n_q, n_kv);
@@ -300,16 +301,19 @@ extern "C" int llme_attention_bf16_rows(int hd, int n_q, int n_kv) {
 // 32) and nsplit: how the decode kernel cuts the keys; part_o [n_seq, n_q, nsplit, hd] and
 // part_ml [n_seq, n_q, nsplit, 2] floats (needed when nsplit > 1). prefill_groups: number of
 // row groups of llme_attention_bf16_rows(hd, n_q, n_kv) rows over the requests with two or more tokens.
+// queue: two integers, zero, for the prefill kernel's work counter (needed when prefill_groups > 0;
+// the kernel leaves them zero; launches that may overlap need separate ones).
 extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const void* v_cache, void* out, float* part_o,
                                    float* part_ml, const int* q_start, const int* ctx_len, const int* block_table,
                                    int max_blocks, int n_seq, int n_q, int n_kv, int hd, int page, float scale,
                                    int window, int n_decode, int split_len, int nsplit, int prefill_groups,
-                                   hipStream_t stream) {
+                                   int* queue, hipStream_t stream) {
     if (n_seq <= 0) return 0;
     if (hd % 16 != 0 || hd > 128 || hd <= 0 || page % 16 != 0 || n_kv <= 0 || n_q % n_kv != 0) return kErrUnsupported;
     if (!(scale > 0.f)) return kErrBadArgument;      // the lazy maximum compares scaled scores
     // page lookups divide by multiplication, exact while (keys / 16) * (page / 16) < 2^32
     if (static_cast<double>(max_blocks) * (page / 16) * (page / 16) >= 4294967296.0) return kErrUnsupported;
+    if (static_cast<double>(n_kv) * page * hd >= 4294967296.0) return kErrUnsupported;   // a page's elements: 32 bits
     if (n_decode > 0 && (split_len <= 0 || split_len % 32 != 0 || nsplit <= 0 || nsplit > 64)) return kErrBadArgument;
     const int qt = direct_rows(hd) / 16;
     const int shared_rows = shared_rows_for(hd, n_q, n_kv);
@@ -318,7 +322,7 @@ extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const voi
         return launch_for_head<HD>(static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache),              \
                                    static_cast<const bf16*>(v_cache), static_cast<bf16*>(out), part_o, part_ml, \
                                    q_start, ctx_len, block_table, max_blocks, n_seq, n_q, n_kv, page, scale,    \
-                                   window, n_decode, split_len, nsplit, prefill_groups, qt, shared_rows, stream)
+                                   window, n_decode, split_len, nsplit, prefill_groups, qt, shared_rows, queue, stream)
     switch (hd) {
         LLME_HEAD(16); LLME_HEAD(32); LLME_HEAD(48); LLME_HEAD(64);
         LLME_HEAD(80); LLME_HEAD(96); LLME_HEAD(112); LLME_HEAD(128);

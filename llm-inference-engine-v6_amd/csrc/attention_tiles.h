@@ -39,8 +39,8 @@ struct PagedKV {
     const int* table;       // this request's row of the block table
     int page, n_kv, kvh, hd;
     unsigned page_magic;    // ceil(2^32 / (page / 16)): key / page without a division, see page_of
-    size_t page_stride;     // elements from one page to the next: n_kv * page * hd
-    size_t head_off;        // elements from a page's start to this kv head's part: kvh * page * hd
+    unsigned page_stride;   // elements from one page to the next: n_kv * page * hd
+    unsigned head_off;      // elements from a page's start to this kv head's part: kvh * page * hd
 };
 
 // Keys come in halves of 16 and the page size is a multiple of 16, so a half's page is
@@ -341,13 +341,13 @@ __device__ __forceinline__ void load_q(const bf16* qrow, bool ok, bf16x8 (&qf)[(
 
 
 // The prefill kernel that shares K and V blocks among a workgroup's wavefronts through LDS
-// (attention_prefill.hip). rows_per_item: rows of one work item, see prefill_shared_rows.
+// (attention_prefill.hip). rows_per_item: rows of one work item, see prefill_shared_rows; queue:
+// two integers that are zero and that no other launch in flight uses.
 int launch_prefill_shared(const bf16* q, const bf16* k_cache, const bf16* v_cache, bf16* out, const int* q_start,
                           const int* ctx_len, const int* block_table, int max_blocks, int n_seq, int n_q, int n_kv,
-                          int hd, int page, float scale, int window, int items, int rows_per_item,
+                          int hd, int page, float scale, int window, int items, int rows_per_item, int* queue,
                           hipStream_t stream);
-// Rows per work item the shared kernel would use for these sizes (`wanted`: 0 or a row count to
-// prefer), or 0 if it does not take them.
-int prefill_shared_rows(int hd, int n_q, int n_kv, int wanted);
+// Rows per work item of the shared kernel for these sizes, or 0 if it does not take them.
+int prefill_shared_rows(int hd, int n_q, int n_kv);
 
 }  // namespace llme

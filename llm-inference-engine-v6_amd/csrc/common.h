@@ -49,6 +49,16 @@ __device__ __forceinline__ float block_sum(float v, float* scratch, int nwaves) 
     return total;
 }
 
+// A workgroup barrier for data exchanged through LDS only: this wavefront's LDS traffic is
+// complete before it and LDS reads start after it, but loads from global memory that are in
+// flight stay in flight (__syncthreads also waits for those, which puts their whole latency
+// in front of every barrier of a loop that prefetches).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // Every entry point returns hipGetLastError() after its launches: 0 on success.
 inline int launch_status() { return static_cast<int>(hipGetLastError()); }
 

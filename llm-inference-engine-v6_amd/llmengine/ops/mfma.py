@@ -78,7 +78,20 @@ kernels._fast_gemm = _fast_gemm
 declare("llme_attention_bf16_rows", [_i, _i, _i])
 declare("llme_attention_bf16_set_rows", [_i, _i])
 declare("llme_attention_bf16", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i,
-                                _i, _i, _i, _i, _vp])
+                                _i, _i, _i, _i, _vp, _vp])
+
+_work_queues: dict = {}
+
+
+def work_queue(device: torch.device) -> torch.Tensor:
+    """Two zeroed integers for the prefill kernel's work counter, one pair per device and
+    stream: launches on one stream run one after the other and leave them zero."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream())
+    q = _work_queues.get(key)
+    if q is None:
+        q = _work_queues[key] = torch.zeros(2, dtype=torch.int32, device=device)
+    return q
+
 
 DECODE_BLOCKS_WANTED = 1024         # workgroups (of four wavefronts) the decode kernel should have
 MIN_SPLIT = 128                     # keys per split at least: one 32-key block per wavefront
@@ -137,7 +150,8 @@ def attention_bf16(q, k_cache, v_cache, out, q_start, ctx_len, block_table, n_q:
     check(entry("llme_attention_bf16")(
         ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), ptr(part_o), ptr(part_ml), ptr(q_start), ptr(ctx_len),
         ptr(block_table), block_table.shape[1], S, n_q, n_kv, head_dim, page, float(scale), int(window),
-        plan["n_decode"], plan["split_len"], plan["nsplit"], plan["groups"], stream()), "attention_bf16")
+        plan["n_decode"], plan["split_len"], plan["nsplit"], plan["groups"],
+        ptr(work_queue(q.device)) if plan["groups"] else None, stream()), "attention_bf16")
 
 
 def _fast_attention(q, k_cache, v_cache, out, step, block_table, n_q, n_kv, head_dim, scale, window) -> bool:
