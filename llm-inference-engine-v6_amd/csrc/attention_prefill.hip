@@ -13,9 +13,10 @@
 // Stretches run from the first key the span's first row sees to the last row's own key; a
 // wavefront skips the 32-key blocks that none of its rows sees and masks the rest by position.
 //
-// LDS: two stages of K [64 keys][hd + 8] (rows 16 bytes longer than the data, so that the
-// 16-byte operand reads of 8 neighbouring keys fall into different banks) and V [hd][64 + 4]
-// (8 bytes longer: the 8-byte reads of 16 neighbouring dims fall into different banks).
+// LDS: two stages of K [64 keys][hd + 16] and V [hd][64 + 8]. The paddings are measured: LDS
+// has 64 banks of 4 bytes; the 16-byte operand reads (lane = key l % 16, dims 8 (l / 16) ..) run
+// at full rate with rows of 2 hd + 32 bytes and at half rate with 2 hd + 16, the 8-byte reads
+// of V (lane = dim l % 16, keys 4 (l / 16) ..) at full rate with rows of 144 bytes.
 // Per stretch one barrier: after it the stage written during the last stretch is read, and
 // the other, which everybody has finished reading, is written from the registers.
 //
@@ -29,8 +30,8 @@ constexpr int KB = 64;                     // keys per stretch
 
 template <int HD>
 struct StageLayout {
-    static constexpr int KS = HD + 8;      // K row stride (elements)
-    static constexpr int VS = KB + 4;      // V row stride (elements)
+    static constexpr int KS = HD + 16;     // K row stride (elements)
+    static constexpr int VS = KB + 8;      // V row stride (elements)
     static constexpr int K_ELEMS = KB * KS;
     static constexpr int V_ELEMS = HD * VS;
     static constexpr int STAGE = K_ELEMS + V_ELEMS;
@@ -128,9 +129,7 @@ __device__ __forceinline__ void store_stretch(bf16* stage, const ChunkPlaces<HD>
 #pragma unroll
     for (int i = 0; i < HD / 32; ++i) {
         *reinterpret_cast<bf16x8*>(stage + c.k_lds[i]) = f.k[i];
-        bf16* dst = stage + c.v_lds[i];                                   // 8-byte aligned
-        *reinterpret_cast<bf16x4*>(dst) = __builtin_shufflevector(f.v[i], f.v[i], 0, 1, 2, 3);
-        *reinterpret_cast<bf16x4*>(dst + 4) = __builtin_shufflevector(f.v[i], f.v[i], 4, 5, 6, 7);
+        *reinterpret_cast<bf16x8*>(stage + c.v_lds[i]) = f.v[i];
     }
 }
 
