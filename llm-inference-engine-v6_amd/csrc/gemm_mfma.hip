@@ -37,6 +37,10 @@ __device__ __forceinline__ bf16x8 load8(const bf16* p, bool ok) {
     return ok ? *reinterpret_cast<const bf16x8*>(p) : zero8();
 }
 
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
+// The fourth word of a buffer descriptor for raw 32-bit data on this chip.
+constexpr int kBufferFlags = 0x00020000;
+
 enum OutMode : int { kStoreF32 = 0, kAddF32 = 1, kStoreBF16 = 2, kAtomicF32 = 3, kGatedBF16 = 4 };
 
 // ----------------------------------------------------------------------------------------
@@ -53,8 +57,8 @@ constexpr int tile_lds_bytes() { return 2 * (32 * WMT + 32 * WNT) * TSTRIDE * 2;
 // kGatedBF16: w holds gate and up rows interleaved in groups of 16, so that even MFMA tile
 // columns are gates and odd ones the ups of the same 16 units; out [M, N / 2] bfloat16 gets
 // silu(gate) * up (src/engine.cpp:213-216).
-template <int WMT, int WNT, int MODE>
-__global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w,
+template <int WMT, int WNT, int MODE, bool KFULL>
+__global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w,
                                                         void* __restrict__ out, int M, int N, int K,
                                                         int tiles_m, int tiles_n, int ksplit) {
     constexpr int BM = 32 * WMT, BN = 32 * WNT;
@@ -92,28 +96,49 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__
     const int kt_end = (kt_begin + nk_per < nk_all) ? kt_begin + nk_per : nk_all;
 
     // global -> LDS: a slab of a tile is rows x 8 chunks of 16 bytes; thread t takes chunks t, t + 256, ..
+    // The loads are buffer loads: a descriptor per matrix that begins at the tile's first row and
+    // ends behind the tile's last row that exists, a 32-bit offset per lane and chunk that never
+    // changes, and the slab's k offset as a scalar. Rows past the matrix lie behind the
+    // descriptor's end and read as zeros without a check; slab numbers past the end read the
+    // last slab again. Every turn of the loop thus issues the same loads, none under a branch,
+    // and the counter of loads in flight tells exactly which slab has arrived. (A tile's rows
+    // span fewer than 2^32 bytes: the entry point checks K.)
     const int crow = tid >> 3, ckq = (tid & 7) * 8;   // chunk i of a thread: row crow + 32 i, same k offset
-    bf16x8 ra[CA], rw[CW];
-    auto load_global = [&](int kt) {
-        const int k = kt * TK + ckq;
+    const int a_rows = M - m0 < BM ? M - m0 : BM, w_rows = N - n0 < BN ? N - n0 : BN;
+    const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16*>(a + static_cast<size_t>(m0) * K), 0, a_rows * K * 2, kBufferFlags);
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16*>(w + static_cast<size_t>(n0) * K), 0, w_rows * K * 2, kBufferFlags);
+    unsigned aoff[CA], woff[CW];                      // bytes
 #pragma unroll
-        for (int i = 0; i < CA; ++i) {
-            const int am = m0 + crow + 32 * i;
-            ra[i] = load8(a + static_cast<size_t>(am) * K + k, am < M && k < K);
-        }
+    for (int i = 0; i < CA; ++i) aoff[i] = (static_cast<unsigned>(crow + 32 * i) * K + ckq) * 2;
 #pragma unroll
-        for (int i = 0; i < CW; ++i) {
-            const int wr = n0 + crow + 32 * i;
-            rw[i] = load8(w + static_cast<size_t>(wr) * K + k, wr < N && k < K);
+    for (int i = 0; i < CW; ++i) woff[i] = (static_cast<unsigned>(crow + 32 * i) * K + ckq) * 2;
+    struct Slab {
+        u32x4 ra[CA], rw[CW];
+    };
+    auto load_global = [&](int kt, Slab& s) {
+        if (kt >= kt_end) kt = kt_end - 1;
+        const int k = kt * TK;
+#pragma unroll
+        for (int i = 0; i < CA; ++i) s.ra[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, aoff[i], k * 2, 0);
+#pragma unroll
+        for (int i = 0; i < CW; ++i) s.rw[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, woff[i], k * 2, 0);
+        if (!KFULL) {                                 // K is a multiple of 8: a chunk is in or out whole
+            const bool ok = k + ckq < K;
+#pragma unroll
+            for (int i = 0; i < CA; ++i) s.ra[i] = ok ? s.ra[i] : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int i = 0; i < CW; ++i) s.rw[i] = ok ? s.rw[i] : u32x4{0u, 0u, 0u, 0u};
         }
     };
-    auto store_lds = [&](int buf) {
+    auto store_lds = [&](int buf, const Slab& s) {
         bf16* sA = lds + buf * A_ELEMS;
         bf16* sW = lds + 2 * A_ELEMS + buf * W_ELEMS;
 #pragma unroll
-        for (int i = 0; i < CA; ++i) *reinterpret_cast<bf16x8*>(sA + (crow + 32 * i) * TSTRIDE + ckq) = ra[i];
+        for (int i = 0; i < CA; ++i) *reinterpret_cast<u32x4*>(sA + (crow + 32 * i) * TSTRIDE + ckq) = s.ra[i];
 #pragma unroll
-        for (int i = 0; i < CW; ++i) *reinterpret_cast<bf16x8*>(sW + (crow + 32 * i) * TSTRIDE + ckq) = rw[i];
+        for (int i = 0; i < CW; ++i) *reinterpret_cast<u32x4*>(sW + (crow + 32 * i) * TSTRIDE + ckq) = s.rw[i];
     };
 
     f32x4 acc[WMT][WNT];
@@ -122,14 +147,10 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__
 #pragma unroll
         for (int j = 0; j < WNT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    if (kt_begin < kt_end) {
-        load_global(kt_begin);
-        store_lds(0);
-    }
-    __syncthreads();
-    for (int kt = kt_begin; kt < kt_end; ++kt) {
-        const int buf = (kt - kt_begin) & 1;
-        if (kt + 1 < kt_end) load_global(kt + 1);
+    // Slab j is computed from LDS buffer j % 2 and travels in register set j % 2. While slab j is
+    // computed, j + 1 sits in its registers and j + 2 is in flight; after the computing, j + 1
+    // goes into the other buffer and its registers ask for j + 3. The barrier waits for LDS only.
+    auto turn = [&](int kt, int buf, Slab& next) {
         const bf16* sA = lds + buf * A_ELEMS;
         const bf16* sW = lds + 2 * A_ELEMS + buf * W_ELEMS;
 #pragma unroll
@@ -146,10 +167,36 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__
 #pragma unroll
                 for (int j = 0; j < WNT; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);        // one k step's operands in registers at a time
         }
-        if (kt + 1 < kt_end) store_lds(buf ^ 1);
-        __syncthreads();
+        // also on the last turn, where nobody reads what is stored: a turn without these would
+        // make the number of loads in flight depend on the path taken
+        store_lds(buf ^ 1, next);
+        load_global(kt + 3, next);
+        lds_barrier();
+    };
+    if (kt_begin < kt_end) {
+        Slab s0, s1;
+        // (the scheduling barriers keep the three slabs' loads in this order: the loop's waits
+        // count on slab j + 1 being older than slab j + 2)
+        load_global(kt_begin, s0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_global(kt_begin + 1, s1);
+        __builtin_amdgcn_sched_barrier(0);
+        store_lds(0, s0);
+        load_global(kt_begin + 2, s0);
+        __builtin_amdgcn_sched_barrier(0);
+        lds_barrier();
+        // pairs of turns in a loop with one way round, then the odd turn: on every path into a
+        // turn the loads in flight are the same, which keeps the compiler's waits exact
+        int kt = kt_begin;
+        for (int pair = (kt_end - kt_begin) / 2; pair > 0; --pair, kt += 2) {
+            turn(kt, 0, s1);
+            turn(kt + 1, 1, s0);
+        }
+        if ((kt_end - kt_begin) & 1) turn(kt, 0, s1);
     }
+    __syncthreads();                                  // the epilogue reuses the slabs' LDS
 
     // Epilogue. The result tile (i, j) of a lane is column wn + 16 j + r, rows wm + 16 i + 4 q + e:
     // written straight from there, a store instruction touches 4 rows with 64 bytes each. Where
@@ -252,22 +299,31 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(const bf16* __restrict__
     }
 }
 
-template <int WMT, int WNT, int MODE>
-static int launch_tile_mode(const bf16* A, const bf16* W, void* out, int M, int N, int K, int ksplit,
-                            hipStream_t stream) {
-    constexpr int LDS = tile_lds_bytes<WMT, WNT>();
-    auto kernel = gemm_tile_kernel<WMT, WNT, MODE>;
-    static bool attr_set = false;                      // per instantiation
+template <auto KERNEL>
+static int launch_tile_kernel(int LDS, int BM, int BN, const bf16* A, const bf16* W, void* out, int M, int N, int K,
+                              int ksplit, hipStream_t stream) {
+    static bool attr_set = false;                      // per kernel
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(KERNEL),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
         if (e != hipSuccess) return static_cast<int>(e);
         attr_set = true;
     }
-    const int tiles_m = (M + 32 * WMT - 1) / (32 * WMT), tiles_n = (N + 32 * WNT - 1) / (32 * WNT);
-    hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n * ksplit), dim3(256), LDS, stream, A, W, out, M, N, K, tiles_m,
+    const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+    hipLaunchKernelGGL(KERNEL, dim3(tiles_m * tiles_n * ksplit), dim3(256), LDS, stream, A, W, out, M, N, K, tiles_m,
                        tiles_n, ksplit);
     return launch_status();
+}
+
+template <int WMT, int WNT, int MODE>
+static int launch_tile_mode(const bf16* A, const bf16* W, void* out, int M, int N, int K, int ksplit,
+                            hipStream_t stream) {
+    constexpr int LDS = tile_lds_bytes<WMT, WNT>();
+    if (K % TK != 0)
+        return launch_tile_kernel<gemm_tile_kernel<WMT, WNT, MODE, false>>(LDS, 32 * WMT, 32 * WNT, A, W, out, M, N, K,
+                                                                           ksplit, stream);
+    return launch_tile_kernel<gemm_tile_kernel<WMT, WNT, MODE, true>>(LDS, 32 * WMT, 32 * WNT, A, W, out, M, N, K,
+                                                                      ksplit, stream);
 }
 
 template <int WMT, int WNT>
@@ -394,7 +450,7 @@ using namespace llme;
 extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
                               int accumulate, int gated, int nw, int ksplit, int tile_shape, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
-    if (K <= 0 || K % 8 != 0) return kErrUnsupported;
+    if (K <= 0 || K % 8 != 0 || K >= (1 << 23)) return kErrUnsupported;   // 256 rows of K must stay below 2^32 bytes
     if (out_dtype != kF32 && out_dtype != kBF16) return kErrBadArgument;
     if (accumulate && out_dtype != kF32) return kErrBadArgument;
     if (gated && (out_dtype != kBF16 || N % 32 != 0 || accumulate)) return kErrBadArgument;
