@@ -167,7 +167,6 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
 #pragma unroll
                 for (int j = 0; j < WNT; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);        // one k step's operands in registers at a time
         }
         // also on the last turn, where nobody reads what is stored: a turn without these would
         // make the number of loads in flight depend on the path taken

@@ -46,6 +46,17 @@ __device__ __forceinline__ bf16x8 gv_zero8() {
 
 enum Epilogue : int { kPlain = 0, kGated = 1, kRope = 2 };
 
+// Four neighbouring norm weights in one load (the entry point checks the vector's alignment).
+__device__ __forceinline__ void load_norm4(const float* p, float (&o)[4]) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+__device__ __forceinline__ void load_norm4(const bf16* p, float (&o)[4]) {
+    const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = static_cast<float>(v[i]);
+}
+
 // What the rotating epilogue needs: where rows sit in their requests and where their pages are.
 struct RopeTarget {
     const int* positions;       // [M] position of each row's token
@@ -114,30 +125,26 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
     if (kpart < n_chunks) load_w(fwa, tile_of(blockIdx.x), kpart);       // in flight during the norm prologue
 
     // ---- prologue: xs[m][k] = bf16(w_norm[k] * h[row(m)][k]); ssum[m] = sum_k h^2 ----
-    for (int m = wave; m < 16; m += NW) {
+    // Rows m >= M stay as they are: a product's row m depends on activation row m alone, and
+    // the results of the rows that do not exist are never stored.
+    for (int m = wave; m < M; m += NW) {
         bf16* xrow = xs + static_cast<size_t>(m) * XS;
-        if (m < M) {
-            const float* hrow = h + static_cast<size_t>(rows ? rows[m] : m) * K;
-            float ss = 0.f;
-            for (int k = lane * 4; k < K; k += 64 * 4) {      // K % 8 == 0: whole groups of 4
-                const float4 v = *reinterpret_cast<const float4*>(hrow + k);
-                ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-                bf16x4 o;
-                o[0] = static_cast<__bf16>(to_float(norm_w[k]) * v.x);
-                o[1] = static_cast<__bf16>(to_float(norm_w[k + 1]) * v.y);
-                o[2] = static_cast<__bf16>(to_float(norm_w[k + 2]) * v.z);
-                o[3] = static_cast<__bf16>(to_float(norm_w[k + 3]) * v.w);
-                *reinterpret_cast<bf16x4*>(xrow + k) = o;
-            }
-            ss = wave_sum(ss);
-            if (lane == 0) ssum[m] = ss;
-        } else {
-            bf16x4 z;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) z[e] = static_cast<__bf16>(0.f);
-            for (int k = lane * 4; k < K; k += 64 * 4) *reinterpret_cast<bf16x4*>(xrow + k) = z;
-            if (lane == 0) ssum[m] = 0.f;
+        const float* hrow = h + static_cast<size_t>(rows ? rows[m] : m) * K;
+        float ss = 0.f;
+        for (int k = lane * 4; k < K; k += 64 * 4) {      // K % 8 == 0: whole groups of 4
+            const float4 v = *reinterpret_cast<const float4*>(hrow + k);
+            float nw4[4];
+            load_norm4(norm_w + k, nw4);
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+            bf16x4 o;
+            o[0] = static_cast<__bf16>(nw4[0] * v.x);
+            o[1] = static_cast<__bf16>(nw4[1] * v.y);
+            o[2] = static_cast<__bf16>(nw4[2] * v.z);
+            o[3] = static_cast<__bf16>(nw4[3] * v.w);
+            *reinterpret_cast<bf16x4*>(xrow + k) = o;
         }
+        ss = wave_sum(ss);
+        if (lane == 0) ssum[m] = ss;
     }
     __syncthreads();
 
@@ -292,6 +299,7 @@ extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_
                               hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 16 || K <= 0 || K % 8 != 0) return kErrUnsupported;
+    if (reinterpret_cast<uintptr_t>(norm_w) % 16 != 0 || reinterpret_cast<uintptr_t>(h) % 16 != 0) return kErrUnsupported;
     if (static_cast<size_t>(16) * (K + 8) * 2 > 132 * 1024) return kErrUnsupported;
     if (gated && N % 16 != 0) return kErrUnsupported;
     const int tiles = (N + 15) / 16;
@@ -328,6 +336,7 @@ extern "C" int llme_gemv_norm_rope(const float* h, const void* norm_w, int norm_
                                    const float* cos_t, const float* sin_t, void* q_out, void* k_cache, void* v_cache,
                                    int M, int K, int n_q, int n_kv, int hd, int page, int grid, hipStream_t stream) {
     if (M <= 0) return 0;
+    if (reinterpret_cast<uintptr_t>(norm_w) % 16 != 0 || reinterpret_cast<uintptr_t>(h) % 16 != 0) return kErrUnsupported;
     if (M > 16 || K <= 0 || K % 8 != 0 || hd <= 0 || hd % 32 != 0 || n_q <= 0 || n_kv <= 0 || page <= 0)
         return kErrUnsupported;
     if (static_cast<size_t>(16) * (K + 8) * 2 > 132 * 1024) return kErrUnsupported;

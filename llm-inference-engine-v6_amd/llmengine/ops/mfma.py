@@ -187,7 +187,8 @@ def gemv_norm_supported(h: torch.Tensor, norm_weight: torch.Tensor, w: torch.Ten
     return (kernels.policy.fast_gemm and h.dtype == torch.float32 and w.dtype == torch.bfloat16
             and norm_weight.dtype in (torch.float32, torch.bfloat16) and 0 < rows_out <= GEMV_NORM_MAX_ROWS
             and K % 8 == 0 and 16 * (K + 8) * 2 <= 132 * 1024 and w.shape[1] == K
-            and (not gated or n_out % 16 == 0) and w.data_ptr() % 16 == 0 and h.data_ptr() % 16 == 0)
+            and (not gated or n_out % 16 == 0) and w.data_ptr() % 16 == 0 and h.data_ptr() % 16 == 0
+            and norm_weight.data_ptr() % 16 == 0)
 
 
 def gemv_norm(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor,
