@@ -8,8 +8,8 @@ import torch
 
 import replay
 from plain_llama import bf16_round, load_plain_model, plain_forward
-from tiny_models import (A_INIT, B_INIT, C_INIT, D_INIT, E_INIT, TINY_A, TINY_B, TINY_C, TINY_D, TINY_E,
-                         make_model_dir, random_tokens)
+from tiny_models import (A_INIT, B_INIT, C_INIT, D_INIT, E_INIT, F_INIT, TINY_A, TINY_B, TINY_C, TINY_D, TINY_E,
+                         TINY_F, make_model_dir, random_tokens)
 
 pytestmark = pytest.mark.gpu
 
@@ -21,6 +21,10 @@ MODELS = {
     "B": (TINY_B, B_INIT, 8, [1, 9, 33, 70]),
     "D": (TINY_D, D_INIT, 16, [3, 50, 66, 21]),
     "E": (TINY_E, E_INIT, 16, [2, 35, 64, 17]),
+    # head sizes 64 and 128: the prefill attention that shares K and V through LDS, with prompts of
+    # several 64-key stretches
+    "C": (TINY_C, C_INIT, 16, [150, 7, 66, 200]),
+    "F": (TINY_F, F_INIT, 16, [131, 64, 2, 97]),
 }
 
 
@@ -74,7 +78,8 @@ SCHEDULES = {
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
 @pytest.mark.parametrize("schedule", list(SCHEDULES))
-@pytest.mark.parametrize("name,page_override", [("A", 0), ("B", 0), ("D", 0), ("E", 0), ("A", 16), ("B", 16), ("D", 32)])
+@pytest.mark.parametrize("name,page_override", [("A", 0), ("B", 0), ("D", 0), ("E", 0), ("C", 0), ("F", 0), ("A", 16),
+                                                ("B", 16), ("D", 32), ("F", 48)])
 def test_schedules_match_plain(zoo, name, page_override, schedule, dtype):
     """Pages of 4 and 8 tokens go through the plain-precision attention kernel also in
     bfloat16; pages of 16 and 32 through the MFMA kernels."""

@@ -64,6 +64,21 @@ TINY_E = {
 E_INIT = dict(seed=4, std=0.06, norm_mean=1.0, norm_std=0.1)
 
 
+# F: head size 128 with four query heads per key/value head (the sizes of the larger Llama models'
+# attention), untied head, rope scaling with another factor
+TINY_F = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "hidden_size": 192, "intermediate_size": 272, "num_hidden_layers": 2,
+    "num_attention_heads": 4, "num_key_value_heads": 1, "head_dim": 128,
+    "vocab_size": 409, "max_position_embeddings": 1024, "rms_norm_eps": 1e-6,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 16.0, "low_freq_factor": 1.0,
+                     "high_freq_factor": 4.0, "original_max_position_embeddings": 256},
+    "tie_word_embeddings": False,
+}
+F_INIT = dict(seed=6, std=0.04, norm_mean=1.0, norm_std=0.1)
+
+
 def make_model_dir(tmp_path, cfg: dict, init: dict, dtype=torch.bfloat16) -> str:
     from llmengine.weights import write_random_model
     return write_random_model(cfg, str(tmp_path), init["seed"], dtype, init["std"], init["norm_mean"],
