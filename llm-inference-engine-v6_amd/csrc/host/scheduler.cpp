@@ -1,0 +1,270 @@
+// Continuous batching above the step function: who is admitted, which tokens a step carries, who
+// finishes and why.
+//
+// State machine, knobs and finish reasons are the reference's ContinuousBatchScheduler
+// (src/scheduler.cpp:136-319): requests wait in a FIFO, are admitted while fewer than
+// max_concurrent are live (no page check at admission), prefill under one token budget per step
+// shared in admission order, then decode one token per step; a sequence ends with "stop" (an EOS
+// id was sampled; it is not appended), "length" (max_new_tokens reached, or 0 asked) or
+// "capacity" (the page pool cannot hold its next tokens; what it generated so far is kept;
+// nothing is preempted or recomputed). Results come back in enqueue order.
+//
+// What differs from the reference: a step is ONE mixed batch. Prompt portions and the single
+// tokens of decoding requests go through the model together, and because pages are reserved
+// before the batch runs, running out of pages is decided here, on the host, in the reference's
+// order (prompt portions take pages first, then decoding requests). A request whose prompt ends
+// in step k decodes first in step k + 1 (the reference does both in step k); token streams are
+// the same. Pages of a finished request go back at the end of the step in which it finished,
+// which is when the reference's next step would find them.
+//
+// This file decides; it runs nothing. A step is plan() (admission, the batch), then the caller
+// runs the batch through the model and samples, then complete() (the sampled tokens arrive,
+// sequences move on or finish, pages go back). The cache manager is the one the step function
+// reserves and commits in; sequence ids are its request keys.
+#include "host_api.h"
+
+#include <algorithm>
+#include <cstdint>
+#include <deque>
+#include <memory>
+#include <vector>
+
+extern "C" {
+int llme_cm_admit(void* h, int64_t key);
+int llme_cm_num_groups(void* h);
+int llme_cm_pages_needed(void* h, int64_t key, long n_new, int* out);
+int llme_cm_can_reserve(void* h, int64_t key, long n_new, const int* pending);
+int llme_cm_release(void* h, int64_t key);
+}
+
+namespace llme_host {
+
+enum State : int { kWaiting = 0, kPrefilling = 1, kRunning = 2, kFinished = 3 };
+enum Reason : int { kNone = 0, kStop = 1, kLength = 2, kCapacity = 3 };
+
+struct Seq {
+    int64_t id = 0;
+    std::vector<int> tokens;                // prompt, then what was generated
+    long prompt_len = 0;
+    long max_new = 0;
+    State state = kWaiting;
+    long cursor = 0;                        // prompt tokens that have gone through the model
+    Reason reason = kNone;
+    long generated() const { return static_cast<long>(tokens.size()) - prompt_len; }
+};
+
+class Scheduler {
+public:
+    Scheduler(void* cm, int max_concurrent, long budget) : cm_(cm), max_concurrent_(max_concurrent), budget_(budget) {}
+
+    void set_budget(long b) { budget_ = b; }
+    long budget() const { return budget_; }
+    int max_concurrent() const { return max_concurrent_; }
+
+    int64_t enqueue(const int* prompt, long n, long max_new) {
+        auto s = std::make_unique<Seq>();
+        s->id = next_id_++;
+        s->tokens.assign(prompt, prompt + n);
+        s->prompt_len = n;
+        s->max_new = max_new;
+        const int64_t id = s->id;
+        waiting_.push_back(std::move(s));
+        return id;
+    }
+
+    bool idle() const { return waiting_.empty() && prefilling_.empty() && running_.empty(); }
+    void counts(int* out) const {
+        out[0] = static_cast<int>(waiting_.size());
+        out[1] = static_cast<int>(prefilling_.size());
+        out[2] = static_cast<int>(running_.size());
+    }
+
+    // Admission, then the step's batch. Returns the number of entries, or an error code.
+    int plan(int* n_admitted, int* admitted_slots, int64_t* entry_seq, int* entry_count, int* entry_want,
+             long* entry_gen, int* tokens, long tokens_cap) {
+        owners_.clear();
+        prompt_ends_.clear();
+        *n_admitted = 0;
+        // admission: no page check, as in the reference
+        while (!waiting_.empty() && static_cast<int>(prefilling_.size() + running_.size()) < max_concurrent_) {
+            const int slot = llme_cm_admit(cm_, waiting_.front()->id);
+            if (slot < 0) return slot;
+            std::unique_ptr<Seq> s = std::move(waiting_.front());
+            waiting_.pop_front();
+            s->state = kPrefilling;
+            admitted_slots[(*n_admitted)++] = slot;
+            prefilling_.push_back(std::move(s));
+        }
+        const int G = llme_cm_num_groups(cm_);
+        std::vector<int> pending(static_cast<size_t>(G), 0), need(static_cast<size_t>(G), 0);
+        auto take_pages = [&](Seq& s, long n) {
+            if (llme_cm_can_reserve(cm_, s.id, n, pending.data()) != 1) return false;
+            llme_cm_pages_needed(cm_, s.id, n, need.data());
+            for (int g = 0; g < G; ++g) pending[static_cast<size_t>(g)] += need[static_cast<size_t>(g)];
+            return true;
+        };
+        int E = 0;
+        long used = 0;
+        auto add_entry = [&](Seq& s, long first, long n, bool want, long gen) {
+            if (used + n > tokens_cap) return false;
+            entry_seq[E] = s.id;
+            entry_count[E] = static_cast<int>(n);
+            entry_want[E] = want ? 1 : 0;
+            entry_gen[E] = gen;
+            std::copy(s.tokens.begin() + first, s.tokens.begin() + first + n, tokens + used);
+            used += n;
+            ++E;
+            if (want) owners_.push_back(&s);
+            return true;
+        };
+        // prompt portions under the step's token budget, in admission order
+        long budget = budget_;
+        for (auto& sp : prefilling_) {
+            Seq& s = *sp;
+            if (budget <= 0) break;
+            const long n = std::min(budget, s.prompt_len - s.cursor);
+            if (n <= 0 || s.state == kFinished) continue;
+            if (!take_pages(s, n)) {
+                finish(s, kCapacity);
+                continue;
+            }
+            const bool ends = s.cursor + n == s.prompt_len;
+            if (!add_entry(s, s.cursor, n, ends && s.max_new > 0, 0)) return LLME_HOST_BAD_ARGUMENT;
+            if (ends) prompt_ends_.push_back(&s);
+            s.cursor += n;
+            budget -= n;
+        }
+        // one token for every decoding request
+        for (auto& sp : running_) {
+            Seq& s = *sp;
+            if (s.state != kRunning) continue;
+            if (!take_pages(s, 1)) {
+                finish(s, kCapacity);
+                continue;
+            }
+            if (!add_entry(s, static_cast<long>(s.tokens.size()) - 1, 1, true, s.generated())) return LLME_HOST_BAD_ARGUMENT;
+        }
+        planned_ = true;
+        return E;
+    }
+
+    // The sampled tokens of the wanted rows, in the order of the entries that wanted one.
+    int complete(const int* sampled, int n, const int* eos, int n_eos) {
+        if (!planned_ || n != static_cast<int>(owners_.size())) return LLME_HOST_BAD_ARGUMENT;
+        planned_ = false;
+        for (int i = 0; i < n; ++i) {
+            Seq& s = *owners_[static_cast<size_t>(i)];
+            // a sampled token arrives for a sequence (src/scheduler.cpp:208-227, 271-282)
+            if (std::find(eos, eos + n_eos, sampled[i]) != eos + n_eos) {
+                finish(s, kStop);
+                continue;
+            }
+            s.tokens.push_back(sampled[i]);
+            if (s.generated() >= s.max_new) finish(s, kLength);
+        }
+        for (Seq* sp : prompt_ends_) {
+            Seq& s = *sp;
+            if (s.state == kFinished) continue;
+            if (s.max_new == 0) {
+                finish(s, kLength);             // nothing is sampled (src/scheduler.cpp:203-207)
+                continue;
+            }
+            s.state = kRunning;
+            auto it = std::find_if(prefilling_.begin(), prefilling_.end(),
+                                   [&](const std::unique_ptr<Seq>& p) { return p.get() == sp; });
+            running_.push_back(std::move(*it));
+            prefilling_.erase(it);
+        }
+        int finished = 0;
+        for (auto* list : {&prefilling_, &running_}) {
+            std::vector<std::unique_ptr<Seq>> keep;
+            for (auto& sp : *list) {
+                if (sp->state == kFinished) {
+                    llme_cm_release(cm_, sp->id);
+                    results_.push_back(std::move(sp));
+                    ++finished;
+                } else {
+                    keep.push_back(std::move(sp));
+                }
+            }
+            list->swap(keep);
+        }
+        if (finished)
+            std::sort(results_.begin(), results_.end(),
+                      [](const std::unique_ptr<Seq>& a, const std::unique_ptr<Seq>& b) { return a->id < b->id; });
+        owners_.clear();
+        prompt_ends_.clear();
+        return finished;
+    }
+
+    int num_results() const { return static_cast<int>(results_.size()); }
+    const Seq* result(int i) const {
+        return i >= 0 && i < num_results() ? results_[static_cast<size_t>(i)].get() : nullptr;
+    }
+    void clear_results() { results_.clear(); }
+
+private:
+    static void finish(Seq& s, Reason r) {
+        s.state = kFinished;
+        s.reason = r;
+    }
+    void* cm_;
+    int max_concurrent_;
+    long budget_;
+    int64_t next_id_ = 0;
+    bool planned_ = false;
+    std::deque<std::unique_ptr<Seq>> waiting_;
+    std::vector<std::unique_ptr<Seq>> prefilling_, running_, results_;
+    std::vector<Seq*> owners_, prompt_ends_;       // between plan() and complete()
+};
+
+}  // namespace llme_host
+
+using llme_host::Scheduler;
+
+extern "C" {
+
+void* llme_sched_create(void* cache_manager, int max_concurrent, long budget) {
+    if (!cache_manager || max_concurrent <= 0 || budget <= 0) return nullptr;
+    return new Scheduler(cache_manager, max_concurrent, budget);
+}
+void llme_sched_destroy(void* h) { delete static_cast<Scheduler*>(h); }
+int llme_sched_set_budget(void* h, long budget) {
+    if (budget <= 0) return LLME_HOST_BAD_ARGUMENT;
+    static_cast<Scheduler*>(h)->set_budget(budget);
+    return 0;
+}
+long llme_sched_enqueue(void* h, const int* prompt, long n, long max_new_tokens) {
+    if (n <= 0 || max_new_tokens < 0) return LLME_HOST_BAD_ARGUMENT;
+    return static_cast<long>(static_cast<Scheduler*>(h)->enqueue(prompt, n, max_new_tokens));
+}
+int llme_sched_idle(void* h) { return static_cast<Scheduler*>(h)->idle() ? 1 : 0; }
+void llme_sched_counts(void* h, int* out) { static_cast<Scheduler*>(h)->counts(out); }
+int llme_sched_plan(void* h, int* n_admitted, int* admitted_slots, int64_t* entry_seq, int* entry_count, int* entry_want,
+                    long* entry_gen, int* tokens, long tokens_cap) {
+    return static_cast<Scheduler*>(h)->plan(n_admitted, admitted_slots, entry_seq, entry_count, entry_want, entry_gen,
+                                            tokens, tokens_cap);
+}
+int llme_sched_complete(void* h, const int* sampled, int n, const int* eos, int n_eos) {
+    return static_cast<Scheduler*>(h)->complete(sampled, n, eos, n_eos);
+}
+int llme_sched_num_results(void* h) { return static_cast<Scheduler*>(h)->num_results(); }
+// reason: 1 "stop", 2 "length", 3 "capacity"
+int llme_sched_result_info(void* h, int i, int64_t* seq_id, long* prompt_len, long* n_tokens, int* reason) {
+    const auto* s = static_cast<Scheduler*>(h)->result(i);
+    if (!s) return LLME_HOST_BAD_ARGUMENT;
+    *seq_id = s->id;
+    *prompt_len = s->prompt_len;
+    *n_tokens = static_cast<long>(s->tokens.size());
+    *reason = static_cast<int>(s->reason);
+    return 0;
+}
+int llme_sched_result_tokens(void* h, int i, int* out) {
+    const auto* s = static_cast<Scheduler*>(h)->result(i);
+    if (!s) return LLME_HOST_BAD_ARGUMENT;
+    std::copy(s->tokens.begin(), s->tokens.end(), out);
+    return 0;
+}
+void llme_sched_clear_results(void* h) { static_cast<Scheduler*>(h)->clear_results(); }
+
+}  // extern "C"

@@ -11,11 +11,17 @@ Layers with the same needs form a group with a page pool and block tables of its
 own: a "full" group keeps every token of a request; a "window" group gives pages
 back once every position in them lies behind the window of the next token. Beside
 the pages, every live request holds a slot: a row in each fixed-size state tensor.
+
+The bookkeeping itself is C++ (csrc/host/cache_manager.cpp); the classes here name
+groups and requests (any hashable; the C++ side knows them by 64-bit keys) and turn
+its codes into exceptions.
 """
 from __future__ import annotations
 
-from collections import deque
-from dataclasses import dataclass, field
+import ctypes
+from dataclasses import dataclass
+
+from ..runtime import native
 
 
 class CacheError(RuntimeError):
@@ -30,28 +36,28 @@ class PagePool:
         if num_pages <= 0:
             raise ValueError("a page pool needs at least one page")
         self.num_pages = int(num_pages)
-        self._free: deque[int] = deque(range(self.num_pages))
-        self._held: set[int] = set()
+        self._lib = native.library()
+        self._h = self._lib.llme_pool_create(self.num_pages)
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.llme_pool_destroy(self._h)
+            self._h = None
 
     @property
     def free_pages(self) -> int:
-        return len(self._free)
+        return self._lib.llme_pool_free_pages(self._h)
 
     def allocate(self) -> int | None:
-        if not self._free:
-            return None
-        page = self._free.popleft()
-        self._held.add(page)
-        return page
+        page = self._lib.llme_pool_allocate(self._h)
+        return None if page < 0 else page
 
     def free(self, page: int) -> None:
-        if page not in self._held:
+        if self._lib.llme_pool_free(self._h, int(page)) != 0:
             raise CacheError(f"page {page} is freed but not held")
-        self._held.remove(page)
-        self._free.append(page)
 
     def held(self) -> set[int]:
-        return set(self._held)
+        return {p for p in range(self.num_pages) if self._lib.llme_pool_is_held(self._h, p)}
 
 
 @dataclass(frozen=True)
@@ -62,12 +68,7 @@ class GroupSpec:
     num_pages: int = 0
 
 
-@dataclass
-class _Request:
-    slot: int
-    length: int = 0                                             # tokens committed
-    reserved: int = 0                                           # tokens with pages reserved (>= length)
-    tables: dict[str, list[int]] = field(default_factory=dict)  # group -> page per logical block, -1 = given back
+_TEXT_KEYS = 1 << 62            # keys of requests that are not named by a small integer
 
 
 class CacheManager:
@@ -84,187 +85,159 @@ class CacheManager:
                 raise ValueError(f"group {g.name}: kind {g.kind!r} is not 'full' or 'window'")
             if g.kind == "window" and g.window <= 0:
                 raise ValueError(f"group {g.name}: a window group needs window > 0")
+            if g.num_pages <= 0:
+                raise ValueError("a page pool needs at least one page")
         self.page_size = int(page_size)
         self.max_requests = int(max_requests)
         self.groups = {g.name: g for g in groups}
-        self.pools = {g.name: PagePool(g.num_pages) for g in groups}
-        self._free_slots: list[int] = list(range(self.max_requests - 1, -1, -1))
-        self._requests: dict[object, _Request] = {}
+        self._index = {g.name: i for i, g in enumerate(groups)}
+        self._lib = native.library()
+        n = len(groups)
+        arr = ctypes.c_int * max(n, 1)
+        self._h = self._lib.llme_cm_create(n, arr(*[int(g.kind == "window") for g in groups]),
+                                           arr(*[int(g.window) for g in groups]),
+                                           arr(*[int(g.num_pages) for g in groups]), self.page_size, self.max_requests)
+        if not self._h:
+            raise ValueError("the cache manager refused its sizes")
+        self._keys: dict[object, int] = {}          # request id -> key on the C++ side
+        self._ids: dict[int, object] = {}
+        self._next_key = _TEXT_KEYS
+        self._counts = arr()
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.llme_cm_destroy(self._h)
+            self._h = None
+
+    @property
+    def handle(self) -> int:
+        """The C++ object, for the other parts of the host runtime (the scheduler)."""
+        return self._h
+
+    # ---- names ----
+    def key_of(self, request_id, create: bool = False) -> int:
+        """The 64-bit key of a request: a non-negative integer below 2^62 is its own key (so a
+        request that the C++ scheduler admitted under its sequence id is found by that id),
+        anything else gets a key of its own while it is live."""
+        if isinstance(request_id, int) and not isinstance(request_id, bool) and 0 <= request_id < _TEXT_KEYS:
+            return request_id
+        key = self._keys.get(request_id)
+        if key is None and create:
+            key = self._next_key
+            self._next_key += 1
+        return -1 if key is None else key
+
+    def _key(self, request_id) -> int:
+        key = self.key_of(request_id)
+        if key < 0 or not self._lib.llme_cm_is_live(self._h, key):
+            raise CacheError(f"request {request_id!r} is not live")
+        return key
+
+    def _group(self, group: str | None) -> int:
+        if group is None:
+            if len(self.groups) != 1:
+                raise ValueError("name the group: there are several")
+            return 0
+        return self._index[group]
 
     # ---- requests and slots ----
     def admit(self, request_id) -> int:
-        if request_id in self._requests:
+        key = self.key_of(request_id, create=True)
+        slot = self._lib.llme_cm_admit(self._h, key)
+        if slot == native.ALREADY_LIVE:
             raise CacheError(f"request {request_id!r} is already live")
-        if not self._free_slots:
+        if slot == native.NO_SLOT:
             raise CacheError(f"no free slot: {self.max_requests} requests are live")
-        slot = self._free_slots.pop()
-        self._requests[request_id] = _Request(slot=slot, tables={g: [] for g in self.groups})
+        if key >= _TEXT_KEYS:
+            self._keys[request_id] = key
+            self._ids[key] = request_id
         return slot
 
     def is_live(self, request_id) -> bool:
-        return request_id in self._requests
+        key = self.key_of(request_id)
+        return key >= 0 and bool(self._lib.llme_cm_is_live(self._h, key))
 
     def live_requests(self) -> list:
-        return list(self._requests)
+        buf = (ctypes.c_int64 * self.max_requests)()
+        n = self._lib.llme_cm_live(self._h, buf, self.max_requests)
+        return [self._ids.get(buf[i], buf[i]) for i in range(n)]
 
     def slot(self, request_id) -> int:
-        return self._req(request_id).slot
+        return self._lib.llme_cm_slot(self._h, self._key(request_id))
 
     def length(self, request_id) -> int:
-        return self._req(request_id).length
+        return self._lib.llme_cm_length(self._h, self._key(request_id))
 
     def free_slots(self) -> int:
-        return len(self._free_slots)
-
-    def _req(self, request_id) -> _Request:
-        try:
-            return self._requests[request_id]
-        except KeyError:
-            raise CacheError(f"request {request_id!r} is not live") from None
+        return self._lib.llme_cm_free_slots(self._h)
 
     # ---- pages ----
-    def _first_needed_block(self, group: GroupSpec, position: int) -> int:
-        """First logical block that a token at `position` reads in this group."""
-        if group.kind == "window":
-            return max(0, position - group.window + 1) // self.page_size
-        return 0
-
-    def _missing(self, req: _Request, group: GroupSpec, n_new: int) -> list[int]:
-        """Logical blocks that must get a page before n_new tokens are appended."""
-        table = req.tables[group.name]
-        start, end = req.length, req.length + n_new
-        first = self._first_needed_block(group, start)
-        last = (end - 1) // self.page_size
-        return [b for b in range(first, last + 1) if b >= len(table) or table[b] < 0]
-
     def pages_needed(self, request_id, n_new: int) -> dict[str, int]:
-        req = self._req(request_id)
-        return {g.name: len(self._missing(req, g, n_new)) for g in self.groups.values()}
+        self._lib.llme_cm_pages_needed(self._h, self._key(request_id), int(n_new), self._counts)
+        return {name: self._counts[i] for name, i in self._index.items()}
 
     def can_reserve(self, request_id, n_new: int, pending: dict[str, int] | None = None) -> bool:
         """True if pages for n_new more tokens are free; `pending` counts pages that
         other reservations of the same step will take first."""
-        for name, need in self.pages_needed(request_id, n_new).items():
-            if need + (pending or {}).get(name, 0) > self.pools[name].free_pages:
-                return False
-        return True
+        arr = None
+        if pending:
+            arr = (ctypes.c_int * max(len(self.groups), 1))(*[int(pending.get(name, 0)) for name in self.groups])
+        return self._lib.llme_cm_can_reserve(self._h, self._key(request_id), int(n_new), arr) == 1
 
     def reserve(self, request_id, n_new: int) -> bool:
         """Gives the request pages for positions [length, length + n_new) in every
         group, or changes nothing and returns False if any pool is short."""
-        if n_new <= 0:
-            raise ValueError("reserve needs n_new >= 1")
-        req = self._req(request_id)
-        missing = {g.name: self._missing(req, g, n_new) for g in self.groups.values()}
-        for name, blocks in missing.items():
-            if len(blocks) > self.pools[name].free_pages:
-                return False
-        for name, blocks in missing.items():
-            table = req.tables[name]
-            for b in blocks:
-                while len(table) <= b:
-                    table.append(-1)
-                page = self.pools[name].allocate()
-                assert page is not None
-                table[b] = page
-        req.reserved = max(req.reserved, req.length + n_new)
-        return True
+        return self.reserve_batch([(request_id, n_new)])
 
     def reserve_batch(self, items: list[tuple[object, int]]) -> bool:
         """`reserve` for several requests at once: all of them get their pages, or nothing changes."""
-        plans = []
-        need = {name: 0 for name in self.groups}
-        for request_id, n_new in items:
+        n = len(items)
+        for _, n_new in items:
             if n_new <= 0:
                 raise ValueError("reserve needs n_new >= 1")
-            req = self._req(request_id)
-            last = (req.length + n_new - 1) // self.page_size
-            for g in self.groups.values():
-                table = req.tables[g.name]
-                if g.kind == "full":
-                    if last < len(table):
-                        continue                    # the common case of decoding: the page is there
-                    blocks = list(range(len(table), last + 1))
-                else:
-                    blocks = self._missing(req, g, n_new)
-                    if not blocks:
-                        continue
-                need[g.name] += len(blocks)
-                plans.append((req, g.name, blocks))
-        for name, n in need.items():
-            if n > self.pools[name].free_pages:
-                return False
-        for req, name, blocks in plans:
-            table = req.tables[name]
-            pool = self.pools[name]
-            for b in blocks:
-                while len(table) <= b:
-                    table.append(-1)
-                table[b] = pool.allocate()
-        for request_id, n_new in items:
-            req = self._requests[request_id]
-            req.reserved = max(req.reserved, req.length + n_new)
-        return True
+        keys = (ctypes.c_int64 * max(n, 1))(*[self._key(r) for r, _ in items])
+        counts = (ctypes.c_long * max(n, 1))(*[int(k) for _, k in items])
+        rc = self._lib.llme_cm_reserve_batch(self._h, n, keys, counts)
+        if rc < 0:
+            raise ValueError("reserve_batch: a request appears twice")
+        return rc == 1
 
     def commit(self, request_id, n_new: int) -> None:
         """The step wrote n_new tokens: the request is that much longer, and window
         groups give back the pages no later token will read."""
-        req = self._req(request_id)
-        if req.length + n_new > req.reserved:
+        rc = self._lib.llme_cm_commit(self._h, self._key(request_id), int(n_new))
+        if rc == native.NOT_RESERVED:
             raise CacheError(f"request {request_id!r}: commit of {n_new} tokens beyond the reserved pages")
-        req.length += n_new
-        for g in self.groups.values():
-            if g.kind != "window":
-                continue
-            table = req.tables[g.name]
-            keep_from = self._first_needed_block(g, req.length)     # next token's first block
-            for b in range(min(keep_from, len(table))):
-                if table[b] >= 0:
-                    self.pools[g.name].free(table[b])
-                    table[b] = -1
 
     def release(self, request_id) -> None:
         """The request is over: all its pages and its slot are given back."""
-        req = self._req(request_id)
-        for name, table in req.tables.items():
-            for page in table:
-                if page >= 0:
-                    self.pools[name].free(page)
-        self._free_slots.append(req.slot)
-        del self._requests[request_id]
+        key = self._key(request_id)
+        self._lib.llme_cm_release(self._h, key)
+        if key >= _TEXT_KEYS:
+            self._keys.pop(self._ids.pop(key), None)
+
+    def forget(self, request_id) -> None:
+        """Drops the name of a request that the C++ side has released on its own."""
+        key = self._keys.pop(request_id, None)
+        if key is not None:
+            self._ids.pop(key, None)
 
     def block_table(self, request_id, group: str) -> list[int]:
-        return self._req(request_id).tables[group]
+        key, g = self._key(request_id), self._index[group]
+        n = self._lib.llme_cm_table_len(self._h, key, g)
+        buf = (ctypes.c_int * max(n, 1))()
+        self._lib.llme_cm_table_copy(self._h, key, g, 0, n, buf)
+        return list(buf[:n])
 
     def free_pages(self, group: str | None = None) -> int:
-        if group is None:
-            if len(self.pools) != 1:
-                raise ValueError("name the group: there are several")
-            group = next(iter(self.pools))
-        return self.pools[group].free_pages
+        return self._lib.llme_cm_free_pages(self._h, self._group(group))
 
     def num_pages(self, group: str | None = None) -> int:
-        if group is None:
-            if len(self.pools) != 1:
-                raise ValueError("name the group: there are several")
-            group = next(iter(self.pools))
-        return self.pools[group].num_pages
+        return self._lib.llme_cm_num_pages(self._h, self._group(group))
 
     # ---- invariants, for tests and debugging ----
     def check(self) -> None:
         """No page is lost or held twice, no slot is held twice."""
-        for name, pool in self.pools.items():
-            owned: list[int] = []
-            for req in self._requests.values():
-                owned += [p for p in req.tables[name] if p >= 0]
-            if len(owned) != len(set(owned)):
-                raise CacheError(f"group {name}: a page is in two block tables")
-            if set(owned) != pool.held():
-                raise CacheError(f"group {name}: pages held {sorted(pool.held())} != pages in tables {sorted(owned)}")
-            if len(owned) + pool.free_pages != pool.num_pages:
-                raise CacheError(f"group {name}: {pool.num_pages - len(owned) - pool.free_pages} pages lost")
-        slots = [r.slot for r in self._requests.values()]
-        if len(slots) != len(set(slots)) or set(slots) & set(self._free_slots):
-            raise CacheError("a slot is held twice")
-        if len(slots) + len(self._free_slots) != self.max_requests:
-            raise CacheError("a slot is lost")
+        rc = self._lib.llme_cm_check(self._h)
+        if rc != 0:
+            raise CacheError(native.CHECK_MESSAGES.get(rc, f"inconsistent (code {rc})"))

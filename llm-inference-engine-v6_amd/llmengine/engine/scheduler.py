@@ -20,13 +20,14 @@ when the reference's next step would find them.
 """
 from __future__ import annotations
 
-from collections import deque
-from dataclasses import dataclass, field
+import ctypes
+from dataclasses import dataclass
 from typing import Protocol, Sequence
 
+from ..runtime import native
 from .step import StepEntry
 
-WAITING, PREFILLING, RUNNING, FINISHED = "WAITING", "PREFILLING", "RUNNING", "FINISHED"
+_REASONS = {1: "stop", 2: "length", 3: "capacity"}
 
 
 @dataclass
@@ -40,33 +41,25 @@ class SequenceResult:
         return f"<SequenceResult seq_id={self.seq_id} finish={self.finish_reason} len={len(self.token_ids)}>"
 
 
-@dataclass
-class Sequence_:
-    seq_id: int
-    token_ids: list[int]
-    prompt_len: int
-    max_new_tokens: int
-    state: str = WAITING
-    prefill_cursor: int = 0
-    finish_reason: str = ""
-
-    @property
-    def generated(self) -> int:
-        return len(self.token_ids) - self.prompt_len
-
-
 class StepBackend(Protocol):
     """What the scheduler needs of an engine."""
     vocab_size: int
     max_pos: int
     eos_token_ids: Sequence[int]
 
-    def open_cache(self, block_manager, max_requests: int): ...           # -> object with .manager, .admit, .release
+    def open_cache(self, block_manager, max_requests: int): ...           # -> object with .manager (a CacheManager)
     def run_step(self, cache, entries: list[StepEntry], draws: list[tuple[int, int]],
                  temperature: float, seed: int) -> list[int]: ...          # next token per wanted row
 
 
 class ContinuousBatchScheduler:
+    """The decisions are made in C++ (csrc/host/scheduler.cpp: admission, the step's batch under
+    the token budget, what happens when pages run out, who finishes and why); this class checks
+    the requests, carries each planned batch to the engine's step function and brings the
+    sampled tokens back. The cache the engine opens must have a `manager` that is the C++ cache
+    manager's face; if it has a `slot_admitted(slot)` method, it is told the slot of every
+    request that is admitted (to clear its fixed-size state)."""
+
     def __init__(self, engine: StepBackend, block_manager, max_concurrent: int = 64,
                  max_prefill_tokens_per_step: int = 256, temperature: float = 0.0, seed: int = 0):
         if max_concurrent <= 0:
@@ -82,12 +75,28 @@ class ContinuousBatchScheduler:
         self.temperature = float(temperature)
         self.seed = int(seed)
         self._cache = engine.open_cache(block_manager, self.max_concurrent)
-        self._waiting: deque[Sequence_] = deque()
-        self._prefilling: list[Sequence_] = []
-        self._running: list[Sequence_] = []
-        self._results: list[SequenceResult] = []
-        self._next_id = 0
+        self._lib = native.library()
+        self._h = self._lib.llme_sched_create(self._cache.manager.handle, self.max_concurrent, self._budget)
+        if not self._h:
+            raise ValueError("ContinuousBatchScheduler: the scheduler refused its sizes")
+        n = self.max_concurrent
+        self._admitted = (ctypes.c_int * n)()
+        self._entry_seq = (ctypes.c_int64 * n)()
+        self._entry_count = (ctypes.c_int * n)()
+        self._entry_want = (ctypes.c_int * n)()
+        self._entry_gen = (ctypes.c_long * n)()
+        self._tokens = None
+        self._size_tokens()
         self.steps = 0
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.llme_sched_destroy(self._h)
+            self._h = None
+
+    def _size_tokens(self) -> None:
+        self._tokens_cap = self._budget + self.max_concurrent
+        self._tokens = (ctypes.c_int * self._tokens_cap)()
 
     # ---- knobs ----
     @property
@@ -99,6 +108,8 @@ class ContinuousBatchScheduler:
         if value <= 0:
             raise ValueError("ContinuousBatchScheduler: max_prefill_tokens_per_step must be >= 1")
         self._budget = int(value)
+        self._lib.llme_sched_set_budget(self._h, self._budget)
+        self._size_tokens()
 
     # ---- requests ----
     def enqueue(self, prompt: Sequence[int], max_new_tokens: int) -> int:
@@ -113,121 +124,63 @@ class ContinuousBatchScheduler:
                 raise ValueError(f"enqueue: token id {t} out of range [0, {V})")
         if len(prompt) + int(max_new_tokens) > self.engine.max_pos:
             raise ValueError("enqueue: prompt + max_new_tokens exceeds RoPE max_pos")
-        seq = Sequence_(self._next_id, prompt, len(prompt), int(max_new_tokens))
-        self._next_id += 1
-        self._waiting.append(seq)
-        return seq.seq_id
+        arr = (ctypes.c_int * len(prompt))(*prompt)
+        return int(self._lib.llme_sched_enqueue(self._h, arr, len(prompt), int(max_new_tokens)))
 
     @property
     def idle(self) -> bool:
-        return not (self._waiting or self._prefilling or self._running)
+        return bool(self._lib.llme_sched_idle(self._h))
 
     @property
     def results(self) -> list[SequenceResult]:
-        return sorted(self._results, key=lambda r: r.seq_id)
+        out = []
+        seq_id, plen, ntok, reason = ctypes.c_int64(), ctypes.c_long(), ctypes.c_long(), ctypes.c_int()
+        for i in range(self._lib.llme_sched_num_results(self._h)):
+            self._lib.llme_sched_result_info(self._h, i, ctypes.byref(seq_id), ctypes.byref(plen), ctypes.byref(ntok),
+                                             ctypes.byref(reason))
+            toks = (ctypes.c_int * max(ntok.value, 1))()
+            self._lib.llme_sched_result_tokens(self._h, i, toks)
+            out.append(SequenceResult(int(seq_id.value), int(plen.value), list(toks[:ntok.value]),
+                                      _REASONS.get(reason.value, "")))
+        return out
 
     def clear_results(self) -> None:
-        self._results.clear()
+        self._lib.llme_sched_clear_results(self._h)
 
     # ---- one step ----
-    def _finish(self, seq: Sequence_, reason: str) -> None:
-        seq.state = FINISHED
-        seq.finish_reason = reason
-
-    def _retire(self) -> None:
-        for lst in (self._prefilling, self._running):
-            keep = []
-            for seq in lst:
-                if seq.state == FINISHED:
-                    self._cache.release(seq.seq_id)
-                    self._results.append(SequenceResult(seq.seq_id, seq.prompt_len, list(seq.token_ids),
-                                                        seq.finish_reason))
-                else:
-                    keep.append(seq)
-            lst[:] = keep
-
-    def _accept(self, seq: Sequence_, token: int) -> None:
-        """A sampled token arrives for a sequence (src/scheduler.cpp:208-227,271-282)."""
-        if token in self._eos:
-            self._finish(seq, "stop")
-            return
-        seq.token_ids.append(int(token))
-        if seq.generated >= seq.max_new_tokens:
-            self._finish(seq, "length")
-
     def step(self) -> bool:
-        self._eos = set(self.engine.eos_token_ids)
-        mgr = self._cache.manager
-        # admission: no page check, as in the reference
-        while self._waiting and len(self._prefilling) + len(self._running) < self.max_concurrent:
-            seq = self._waiting.popleft()
-            seq.state = PREFILLING
-            self._cache.admit(seq.seq_id)
-            self._prefilling.append(seq)
-
+        n_admitted = ctypes.c_int()
+        E = self._lib.llme_sched_plan(self._h, ctypes.byref(n_admitted), self._admitted, self._entry_seq,
+                                      self._entry_count, self._entry_want, self._entry_gen, self._tokens,
+                                      self._tokens_cap)
+        if E < 0:
+            raise RuntimeError(f"the scheduler could not plan a step (code {E}): the cache it was given has fewer "
+                               f"slots than max_concurrent = {self.max_concurrent}")
+        told = getattr(self._cache, "slot_admitted", None)
+        if told is not None:
+            for i in range(n_admitted.value):
+                told(self._admitted[i])
         entries: list[StepEntry] = []
-        owners: list[Sequence_] = []            # sequence of each wanted row
         draws: list[tuple[int, int]] = []
-        pending = {g: 0 for g in mgr.groups}
-
-        def take_pages(seq: Sequence_, n: int) -> bool:
-            if not mgr.can_reserve(seq.seq_id, n, pending):
-                return False
-            for g, k in mgr.pages_needed(seq.seq_id, n).items():
-                pending[g] += k
-            return True
-
-        # prompt portions under the step's token budget, in admission order
-        budget = self._budget
-        prompt_ends: list[Sequence_] = []
-        for seq in self._prefilling:
-            if budget <= 0:
-                break
-            n = min(budget, seq.prompt_len - seq.prefill_cursor)
-            if n <= 0:
-                continue
-            if not take_pages(seq, n):
-                self._finish(seq, "capacity")
-                continue
-            ends = seq.prefill_cursor + n == seq.prompt_len
-            want = [n - 1] if ends and seq.max_new_tokens > 0 else []
-            entries.append(StepEntry(seq.seq_id, seq.token_ids[seq.prefill_cursor:seq.prefill_cursor + n], want))
+        pos = 0
+        for i in range(E):
+            n, seq_id = self._entry_count[i], int(self._entry_seq[i])
+            want = [n - 1] if self._entry_want[i] else []
+            entries.append(StepEntry(seq_id, self._tokens[pos:pos + n], want))
             if want:
-                owners.append(seq)
-                draws.append((seq.seq_id, 0))
-            if ends:
-                prompt_ends.append(seq)
-            seq.prefill_cursor += n
-            budget -= n
-        # one token for every decoding request
-        for seq in self._running:
-            if seq.state != RUNNING:
-                continue
-            if not take_pages(seq, 1):
-                self._finish(seq, "capacity")
-                continue
-            entries.append(StepEntry(seq.seq_id, [seq.token_ids[-1]], [0]))
-            owners.append(seq)
-            draws.append((seq.seq_id, seq.generated))
-
+                draws.append((seq_id, int(self._entry_gen[i])))
+            pos += n
+        sampled: list[int] = []
         if entries:
-            tokens = self.engine.run_step(self._cache, entries, draws, self.temperature, self.seed)
-            if len(tokens) != len(owners):
-                raise RuntimeError(f"the step returned {len(tokens)} tokens for {len(owners)} wanted rows")
-            for seq, tok in zip(owners, tokens):
-                self._accept(seq, tok)
+            sampled = self.engine.run_step(self._cache, entries, draws, self.temperature, self.seed)
+            if len(sampled) != len(draws):
+                raise RuntimeError(f"the step returned {len(sampled)} tokens for {len(draws)} wanted rows")
             self.steps += 1
-
-        for seq in prompt_ends:
-            if seq.state == FINISHED:
-                continue
-            if seq.max_new_tokens == 0:
-                self._finish(seq, "length")         # nothing is sampled (src/scheduler.cpp:203-207)
-            else:
-                seq.state = RUNNING
-                self._prefilling.remove(seq)
-                self._running.append(seq)
-        self._retire()
+        eos = [int(t) for t in self.engine.eos_token_ids]
+        rc = self._lib.llme_sched_complete(self._h, (ctypes.c_int * max(len(sampled), 1))(*[int(t) for t in sampled]),
+                                           len(sampled), (ctypes.c_int * max(len(eos), 1))(*eos), len(eos))
+        if rc < 0:
+            raise RuntimeError(f"the scheduler could not take the step's tokens (code {rc})")
         return not self.idle
 
     def run_until_idle(self) -> None:

@@ -10,6 +10,8 @@ the request's pages, and returns 32-bit logits at the wanted places.
 """
 from __future__ import annotations
 
+import ctypes
+
 from dataclasses import dataclass, field
 from typing import Sequence
 
@@ -128,6 +130,10 @@ class CacheContext:
         self.storage.clear_slot(slot)
         return slot
 
+    def slot_admitted(self, slot: int) -> None:
+        """A request was admitted by the host runtime itself (the scheduler): its state starts empty."""
+        self.storage.clear_slot(slot)
+
     def release(self, request_id) -> None:
         self.manager.release(request_id)
 
@@ -148,41 +154,34 @@ class _DecodeRecord:
             self.offsets.append(self.offsets[-1] + n)
         self.total = self.offsets[-1]
         self.host = torch.zeros(self.total, dtype=torch.int32, pin_memory=True)
-        self.np = self.host.numpy()
-        self.ids: list | None = None
-        self.blocks: list[list[int]] = []        # per group, per request: table entries written so far
+        self.np = h = self.host.numpy()
+        o, G = self.offsets, len(groups)
+        h[o[2]:o[3]] = range(S)                 # request index of each token
+        h[o[3]:o[4]] = range(S + 1)             # first row of each request
+        h[o[6 + G]:o[7 + G]] = range(S)         # wanted rows
+        self.key_list: list[int] | None = None
+        self.keys = None
+        self.done = (ctypes.c_int * max(G * S, 1))()        # per group and request: table entries written so far
+        self.serials = (ctypes.c_int64 * S)()               # which admission of its key sits in each place
         self.event: torch.cuda.Event | None = None
 
-    def refresh(self, mgr: CacheManager, entries: Sequence[StepEntry], lengths: list[int]) -> None:
+    def refresh(self, mgr: CacheManager, entries: Sequence[StepEntry]) -> None:
         if self.event is not None:
             self.event.synchronize()            # the last copy has read the host mirror
         S, width, o, h = self.S, self.width, self.offsets, self.np
-        ids = [e.request_id for e in entries]
-        if ids != self.ids:
-            h[o[2]:o[3]] = range(S)             # request index of each token
-            h[o[3]:o[4]] = range(S + 1)         # first row of each request
-            h[o[5]:o[6]] = [mgr.slot(r) for r in ids]
-            h[o[6 + len(self.groups)]:o[7 + len(self.groups)]] = range(S)     # wanted rows
-            self.blocks = []
-            for gi, g in enumerate(self.groups):
-                base = o[6 + gi]
-                h[base:base + S * width] = 0
-                self.blocks.append([0] * S)
-            self.ids = ids
+        keys = [mgr.key_of(e.request_id) for e in entries]
+        if keys != self.key_list:
+            self.key_list = keys
+            self.keys = (ctypes.c_int64 * S)(*keys)
         h[o[0]:o[1]] = [e.tokens[0] for e in entries]
-        h[o[1]:o[2]] = lengths                  # the new token's position
-        h[o[4]:o[5]] = lengths                  # tokens cached before this step
-        for gi, g in enumerate(self.groups):
-            base = o[6 + gi]
-            done = self.blocks[gi]
-            window = mgr.groups[g].kind == "window"
-            for i, rid in enumerate(ids):
-                table = mgr.block_table(rid, g)
-                nb = len(table)
-                if nb != done[i] or window:
-                    lo = 0 if window else done[i]
-                    h[base + i * width + lo:base + i * width + nb] = table[lo:nb]
-                    done[i] = nb
+        # lengths (tokens cached before this step), slots and the block-table entries that are new,
+        # straight from the C++ manager into the pinned mirror
+        base = h.ctypes.data
+        rc = mgr._lib.llme_cm_fill_decode(mgr.handle, S, self.keys, width, base + 4 * o[4], base + 4 * o[5],
+                                          base + 4 * o[6], self.done, self.serials)
+        if rc != 0:
+            raise RuntimeError(f"a request of the recorded step is not live (code {rc})")
+        h[o[1]:o[2]] = h[o[4]:o[5]]             # the new token's position
         self.meta[:self.total].copy_(self.host, non_blocking=True)
         if self.event is None:
             self.event = torch.cuda.Event()
@@ -279,7 +278,7 @@ class ModelRunner:
             with torch.cuda.graph(graph):
                 logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
             cache.graphs[key] = rec = _DecodeRecord(graph, logits, meta, S, width, list(mgr.groups))
-        rec.refresh(mgr, entries, lengths)
+        rec.refresh(mgr, entries)
         rec.graph.replay()
         self.graph_replays += 1
         return rec.logits

@@ -172,3 +172,49 @@ def test_reserve_batch_is_all_or_nothing():
     assert m.free_pages("full") == 6 - 3 - 2 - 1                        # a 3 pages, b 2, c 1
     with pytest.raises(ValueError):
         m.reserve_batch([("a", 0)])
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_native_manager_agrees_with_the_plain_one(seed):
+    """The C++ manager and the plain Python one, fed the same random requests, give the same
+    answers at every turn: slots, lengths, pages needed, refusals, block tables, free pages."""
+    import plain_cache
+    rng = random.Random(100 + seed)
+    specs = [("full", "full", 0, rng.choice([9, 30])), ("win", "window", rng.choice([2, 7, 20]), rng.choice([6, 18]))]
+    if seed % 3 == 0:
+        specs = specs[:1]
+    page = rng.choice([1, 4, 16])
+    a = CacheManager([GroupSpec(*s) for s in specs], page, 4)
+    b = plain_cache.CacheManager([plain_cache.GroupSpec(*s) for s in specs], page, 4)
+    live, next_id = [], 0
+    for _ in range(500):
+        op = rng.random()
+        if op < 0.2 and a.free_slots():
+            rid = next_id if next_id % 2 else f"r{next_id}"         # integer and other names
+            next_id += 1
+            assert a.admit(rid) == b.admit(rid)
+            live.append(rid)
+        elif op < 0.8 and live:
+            items = [(rid, rng.choice([1, 1, 2, 6, 19])) for rid in rng.sample(live, rng.randint(1, len(live)))]
+            for rid, n in items:
+                assert a.pages_needed(rid, n) == b.pages_needed(rid, n)
+                pending = {g: rng.randint(0, 3) for g in a.groups}
+                assert a.can_reserve(rid, n, pending) == b.can_reserve(rid, n, pending)
+            ok = a.reserve_batch(items)
+            assert ok == b.reserve_batch(items)
+            if ok:
+                for rid, n in items:
+                    a.commit(rid, n)
+                    b.commit(rid, n)
+        elif live:
+            rid = live.pop(rng.randrange(len(live)))
+            a.release(rid)
+            b.release(rid)
+        a.check()
+        assert a.free_slots() == b.free_slots() and a.live_requests() == b.live_requests()
+        for g in a.groups:
+            assert a.free_pages(g) == b.free_pages(g)
+        for rid in live:
+            assert (a.slot(rid), a.length(rid)) == (b.slot(rid), b.length(rid))
+            for g in a.groups:
+                assert a.block_table(rid, g) == b.block_table(rid, g)

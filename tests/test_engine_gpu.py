@@ -122,6 +122,22 @@ def test_page_reuse_leaves_nothing_behind(zoo, dtype):
         check_against_plain(got, plain[dtype], reqs, dtype)
 
 
+def test_a_request_id_used_again_gets_its_own_pages(zoo):
+    """Integer ids that come back after their release, decoding through the same recorded steps:
+    the second holder of an id has other pages than the first, and the recorded step must not
+    keep the first one's block table."""
+    model_dir, reqs, plain, page = zoo["B"]
+    engine = engine_for(model_dir, "bf16")
+    by_number = {i: ids for i, ids in enumerate(reqs.values())}
+    plain_by_number = {i: plain["bf16"][rid] for i, rid in enumerate(reqs)}
+    cache = engine.new_cache(40, page, max_requests=4)
+    for shift in range(3):
+        renamed = {(i + shift) % len(by_number): ids for i, ids in by_number.items()}      # ids change hands
+        wanted = {(i + shift) % len(by_number): p for i, p in plain_by_number.items()}
+        got = replay.run_trace(engine, cache, replay.tail_one_by_one(renamed, 32))
+        check_against_plain(got, wanted, renamed, "bf16")
+
+
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
 def test_batch_order_does_not_matter(zoo, dtype):
     """Rows of a batch are independent of their neighbours: permuting the entries permutes the logits."""
