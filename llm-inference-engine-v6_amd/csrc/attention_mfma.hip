@@ -278,9 +278,11 @@ using namespace llme;
 static int g_rows_override = 0;
 static int g_shared_override = -1;
 extern "C" int llme_attention_bf16_set_rows(int rows, int shared) {
-    if (rows < 0 || rows % 16 != 0 || rows > 256 || shared < -1 || shared > 1) return kErrBadArgument;
+    // shared 2 and 3: the kernel with LDS with one or two wavefronts per tile, whatever the batch
+    if (rows < 0 || rows % 16 != 0 || rows > 256 || shared < -1 || shared > 3) return kErrBadArgument;
     g_rows_override = rows;
-    g_shared_override = shared;
+    g_shared_override = shared > 1 ? 1 : shared;
+    prefill_shared_key_waves(shared > 1 ? shared - 1 : 0);
     return 0;
 }
 static int direct_rows(int hd) {

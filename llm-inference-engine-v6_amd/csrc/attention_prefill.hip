@@ -39,40 +39,40 @@ struct StageLayout {
 };
 
 // What one thread fetches of a stretch: NC chunks of 16 bytes of K and as many of V. Chunk i
-// of thread tid has the running number tid + 256 i; of K it is key idx / (hd / 8), dims
+// of thread tid has the running number tid + threads i; of K it is key idx / (hd / 8), dims
 // 8 (idx % (hd / 8)) ..; of V the 16-key half idx / (2 hd), dim (idx % (2 hd)) / 2, keys
 // 8 (idx % 2) .. of the half. For head sizes 64 and 128 the 64 chunks of a wavefront then lie
-// in one 16-key half, the same for K and V: (64 wave + 256 i) / (2 hd). A half has one page,
+// in one 16-key half, the same for K and V: (64 wave + threads i) / (2 hd). A half has one page,
 // so the page's id, whether the half is to be read at all and the page's address are the
 // same for the whole wavefront: scalar work, and the loads take a scalar base and a 32-bit
 // offset per lane that never changes.
-template <int HD>
+template <int HD, int THREADS>
 struct Fetched {
-    static constexpr int NC = HD / 32;     // 64 keys x hd / 8 chunks over 256 threads
+    static constexpr int NC = HD * 8 / THREADS;    // 64 keys x hd / 8 chunks over the workgroup's threads
     bf16x8 k[NC];
     bf16x8 v[NC];
 };
 
-template <int HD>
-__device__ __forceinline__ int chunk_half(int wave, int i) { return (64 * wave + 256 * i) / (2 * HD); }
+template <int HD, int THREADS>
+__device__ __forceinline__ int chunk_half(int wave, int i) { return (64 * wave + THREADS * i) / (2 * HD); }
 
 // Per lane and chunk, fixed for the kernel: offsets (elements) from the start of the half's
 // keys in its page (K) or of the kv head's part of the page (V), and the places in a stage.
-template <int HD>
+template <int HD, int THREADS>
 struct ChunkPlaces {
-    static constexpr int NC = HD / 32;
+    static constexpr int NC = HD * 8 / THREADS;
     unsigned k_off[NC], v_off[NC];         // global, in elements
     unsigned k_lds[NC], v_lds[NC];         // in a stage, in elements
 };
 
-template <int HD>
-__device__ __forceinline__ ChunkPlaces<HD> chunk_places(int tid, int page) {
+template <int HD, int THREADS>
+__device__ __forceinline__ ChunkPlaces<HD, THREADS> chunk_places(int tid, int page) {
     using L = StageLayout<HD>;
     constexpr int CK = HD / 8;
-    ChunkPlaces<HD> c;
+    ChunkPlaces<HD, THREADS> c;
 #pragma unroll
-    for (int i = 0; i < HD / 32; ++i) {
-        const int idx = tid + 256 * i;
+    for (int i = 0; i < HD * 8 / THREADS; ++i) {
+        const int idx = tid + THREADS * i;
         const int key = idx / CK, dim = (idx % CK) * 8;
         c.k_off[i] = (key & 15) * HD + dim;
         c.k_lds[i] = key * L::KS + dim;
@@ -87,18 +87,19 @@ __device__ __forceinline__ ChunkPlaces<HD> chunk_places(int tid, int page) {
 // The pages of the NC halves that this wavefront fetches of the stretch at t0: page id (or -1:
 // the half has no key in [key_lo, key_end), nothing is read for it) and the first key's place
 // in the page. All scalar.
-template <int HD>
+template <int HD, int THREADS>
 struct StretchPages {
-    int pg[HD / 32];
-    int off[HD / 32];
+    int pg[HD * 8 / THREADS];
+    int off[HD * 8 / THREADS];
 };
 
-template <int HD>
-__device__ __forceinline__ StretchPages<HD> lookup_stretch(const PagedKV& kv, int t0, int key_lo, int key_end, int wave) {
-    StretchPages<HD> p;
+template <int HD, int THREADS>
+__device__ __forceinline__ StretchPages<HD, THREADS> lookup_stretch(const PagedKV& kv, int t0, int key_lo, int key_end,
+                                                                    int wave) {
+    StretchPages<HD, THREADS> p;
 #pragma unroll
-    for (int i = 0; i < HD / 32; ++i) {
-        const int h0 = t0 + 16 * chunk_half<HD>(wave, i);
+    for (int i = 0; i < HD * 8 / THREADS; ++i) {
+        const int h0 = t0 + 16 * chunk_half<HD, THREADS>(wave, i);
         const PagePlace pl = page_of(kv, h0);
         p.off[i] = pl.offset;
         p.pg[i] = (h0 < key_end && h0 + 15 >= key_lo) ? __builtin_amdgcn_readfirstlane(kv.table[pl.block]) : -1;
@@ -108,11 +109,11 @@ __device__ __forceinline__ StretchPages<HD> lookup_stretch(const PagedKV& kv, in
 
 // Every turn issues the same loads: a half that is not to be read reads the pool's first page
 // instead and counts as zeros.
-template <int HD>
-__device__ __forceinline__ void fetch_stretch(const PagedKV& kv, const StretchPages<HD>& p, const ChunkPlaces<HD>& c,
-                                              Fetched<HD>& f) {
+template <int HD, int THREADS>
+__device__ __forceinline__ void fetch_stretch(const PagedKV& kv, const StretchPages<HD, THREADS>& p,
+                                              const ChunkPlaces<HD, THREADS>& c, Fetched<HD, THREADS>& f) {
 #pragma unroll
-    for (int i = 0; i < HD / 32; ++i) {
+    for (int i = 0; i < HD * 8 / THREADS; ++i) {
         const bool ok = p.pg[i] >= 0;                                                     // scalar
         const size_t base = static_cast<size_t>(ok ? p.pg[i] : 0) * kv.page_stride + kv.head_off;   // scalar
         const bf16* ksrc = kv.k + base + static_cast<size_t>(ok ? p.off[i] : 0) * HD;
@@ -124,10 +125,11 @@ __device__ __forceinline__ void fetch_stretch(const PagedKV& kv, const StretchPa
     }
 }
 
-template <int HD>
-__device__ __forceinline__ void store_stretch(bf16* stage, const ChunkPlaces<HD>& c, const Fetched<HD>& f) {
+template <int HD, int THREADS>
+__device__ __forceinline__ void store_stretch(bf16* stage, const ChunkPlaces<HD, THREADS>& c,
+                                              const Fetched<HD, THREADS>& f) {
 #pragma unroll
-    for (int i = 0; i < HD / 32; ++i) {
+    for (int i = 0; i < HD * 8 / THREADS; ++i) {
         *reinterpret_cast<bf16x8*>(stage + c.k_lds[i]) = f.k[i];
         *reinterpret_cast<bf16x8*>(stage + c.v_lds[i]) = f.v[i];
     }
@@ -155,7 +157,7 @@ __device__ __forceinline__ void read_block(const bf16* stage, int sb, KFrag<HD>&
 
 // One work item: span `bx` (counted over the requests with two or more tokens, the last spans of
 // a request first) for head group `by`.
-template <int HD, int QT, int HPW>
+template <int HD, int QT, int HPW, int KW>
 __device__ __forceinline__ void prefill_item(int bx, int by, bf16* lds, const bf16* __restrict__ q,
                                              const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
                                              bf16* __restrict__ out, const int* __restrict__ q_start,
@@ -163,6 +165,7 @@ __device__ __forceinline__ void prefill_item(int bx, int by, bf16* lds, const bf
                                              int max_blocks, int n_seq, int n_q, int n_kv, int page, float scale,
                                              int window) {
     constexpr int DC = HD / 32, DT = HD / 16, ROWS = 16 * QT, RG = 4 / HPW, SPAN = RG * ROWS;
+    constexpr int THREADS = 256 * KW;
     using L = StageLayout<HD>;
 
     // which request and which of its spans this workgroup has
@@ -185,9 +188,11 @@ __device__ __forceinline__ void prefill_item(int bx, int by, bf16* lds, const bf
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63, r = lane & 15, g4 = lane >> 4;
     const int G = n_q / n_kv;
-    const int head = by * HPW + wave % HPW;                // HPW divides G: one kv head per workgroup
+    const int tile = wave % 4;                             // which rows and head; KW wavefronts share a tile
+    const int ks = wave / 4;                               // and take the 32-key blocks sb with sb % KW == ks
+    const int head = by * HPW + tile % HPW;                // HPW divides G: one kv head per workgroup
     const int kvh = (by * HPW) / G;
-    const int rg = wave / HPW;
+    const int rg = tile / HPW;
     const int pos_span = ctx_len[s] + (first - q_start[s]); // position of the span's first row
 
     // this wavefront's rows
@@ -223,14 +228,14 @@ __device__ __forceinline__ void prefill_item(int bx, int by, bf16* lds, const bf
                page_magic_of(page), static_cast<unsigned>(n_kv) * page * HD, static_cast<unsigned>(kvh) * page * HD};
     const float scale_log2 = scale * kLog2e;
 
-    const ChunkPlaces<HD> places = chunk_places<HD>(tid, page);
-    Fetched<HD> fetched;
-    StretchPages<HD> pages = lookup_stretch<HD>(kv, k_begin, key_lo, key_end, wave);
-    fetch_stretch<HD>(kv, pages, places, fetched);
-    pages = lookup_stretch<HD>(kv, k_begin + KB, key_lo, key_end, wave);
-    store_stretch<HD>(lds, places, fetched);
-    fetch_stretch<HD>(kv, pages, places, fetched);         // past key_end: no page ids, zeros
-    pages = lookup_stretch<HD>(kv, k_begin + 2 * KB, key_lo, key_end, wave);
+    const ChunkPlaces<HD, THREADS> places = chunk_places<HD, THREADS>(tid, page);
+    Fetched<HD, THREADS> fetched;
+    StretchPages<HD, THREADS> pages = lookup_stretch<HD, THREADS>(kv, k_begin, key_lo, key_end, wave);
+    fetch_stretch<HD, THREADS>(kv, pages, places, fetched);
+    pages = lookup_stretch<HD, THREADS>(kv, k_begin + KB, key_lo, key_end, wave);
+    store_stretch<HD, THREADS>(lds, places, fetched);
+    fetch_stretch<HD, THREADS>(kv, pages, places, fetched);           // past key_end: no page ids, zeros
+    pages = lookup_stretch<HD, THREADS>(kv, k_begin + 2 * KB, key_lo, key_end, wave);
     lds_barrier();
     int st = 0;
     for (int t0 = k_begin; t0 < key_end; t0 += KB, st ^= 1) {
@@ -238,7 +243,7 @@ __device__ __forceinline__ void prefill_item(int bx, int by, bf16* lds, const bf
 #pragma unroll
         for (int sb = 0; sb < 2; ++sb) {
             const int tb = t0 + 32 * sb;
-            if (tb < my_end && tb + 32 > my_lo) {           // the same for the whole wavefront
+            if (sb % KW == ks && tb < my_end && tb + 32 > my_lo) {         // the same for the whole wavefront
                 KFrag<HD> kf;
                 VFrag<HD> vf;
                 read_block<HD>(stage, sb, kf, vf);
@@ -254,10 +259,53 @@ __device__ __forceinline__ void prefill_item(int bx, int by, bf16* lds, const bf
             }
         }
         if (t0 + KB < key_end) {                            // the same for the whole workgroup
-            store_stretch<HD>(lds + (st ^ 1) * L::STAGE, places, fetched);
-            fetch_stretch<HD>(kv, pages, places, fetched);
-            pages = lookup_stretch<HD>(kv, t0 + 3 * KB, key_lo, key_end, wave);
+            store_stretch<HD, THREADS>(lds + (st ^ 1) * L::STAGE, places, fetched);
+            fetch_stretch<HD, THREADS>(kv, pages, places, fetched);
+            pages = lookup_stretch<HD, THREADS>(kv, t0 + 3 * KB, key_lo, key_end, wave);
             lds_barrier();
+        }
+    }
+
+    if (KW == 2) {
+        // The two wavefronts of a tile have seen every other 32-key block each: the second hands
+        // its maxima, sums and accumulators over through LDS (the stages are done with), the
+        // first brings both to the common maximum and adds them.
+        constexpr int PER_QT = 2 + DT * 4;                 // floats per lane and row tile
+        float* hand = reinterpret_cast<float*>(lds) + tile * (QT * PER_QT * 64);
+        static_assert(4 * QT * PER_QT * 64 * 4 <= L::BYTES, "the hand-over must fit into the stages");
+        __syncthreads();                                   // everybody has read its last stage
+        if (ks == 1) {
+#pragma unroll
+            for (int qt = 0; qt < QT; ++qt) {
+                float* p = hand + qt * PER_QT * 64 + lane;
+                p[0] = m[qt];
+                p[64] = l[qt];
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) p[(2 + dt * 4 + e) * 64] = o[qt][dt][e];
+            }
+        }
+        __syncthreads();
+        if (ks == 1) return;
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+            const float* p = hand + qt * PER_QT * 64 + lane;
+            const float m1 = p[0], l1 = p[64];
+            const float mx = fmaxf(m[qt], m1);
+            const float a0 = fast_exp2(m[qt] - mx), a1 = fast_exp2(m1 - mx);
+            m[qt] = mx;
+            l[qt] = l[qt] * a0 + l1 * a1;
+            float ar0[4], ar1[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {                   // factors of O's row 4 g4 + e
+                ar0[e] = __shfl(a0, g4 * 4 + e, 64);
+                ar1[e] = __shfl(a1, g4 * 4 + e, 64);
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[qt][dt][e] = o[qt][dt][e] * ar0[e] + p[(2 + dt * 4 + e) * 64] * ar1[e];
         }
     }
 
@@ -286,8 +334,10 @@ __device__ __forceinline__ void prefill_item(int bx, int by, bf16* lds, const bf
 // leaves most of the chip idle while the few longest finish. queue[0] counts the items taken,
 // queue[1] the workgroups that have left; both are zero before and after the kernel (the last
 // workgroup to leave clears them), so the same two integers serve every launch on a stream.
-template <int HD, int QT, int HPW>
-__global__ __launch_bounds__(256) void attention_prefill_shared_kernel(
+// KW = 2: eight wavefronts, two per tile, each taking every other 32-key block: half the time
+// for a work item, for batches with too few items to fill the chip.
+template <int HD, int QT, int HPW, int KW>
+__global__ __launch_bounds__(256 * KW) void attention_prefill_shared_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     bf16* __restrict__ out, const int* __restrict__ q_start, const int* __restrict__ ctx_len,
     const int* __restrict__ block_table, int max_blocks, int n_seq, int n_q, int n_kv, int page, float scale,
@@ -303,7 +353,7 @@ __global__ __launch_bounds__(256) void attention_prefill_shared_kernel(
         __syncthreads();
         const int item = __builtin_amdgcn_readfirstlane(next_item);
         if (item >= n_items) break;                        // the counter only grows: every workgroup gets here
-        prefill_item<HD, QT, HPW>(item / head_groups, item % head_groups, lds, q, k_cache, v_cache, out, q_start,
+        prefill_item<HD, QT, HPW, KW>(item / head_groups, item % head_groups, lds, q, k_cache, v_cache, out, q_start,
                                   ctx_len, block_table, max_blocks, n_seq, n_q, n_kv, page, scale, window);
     }
     if (threadIdx.x == 0) {
@@ -315,6 +365,9 @@ __global__ __launch_bounds__(256) void attention_prefill_shared_kernel(
         }
     }
 }
+
+constexpr long kSplitBelowItems = 768;
+static int g_key_waves = 0;                 // 0: by the number of items; 1, 2: forced (measurements, tests)
 
 static int heads_per_workgroup(int n_q, int n_kv) {
     const int G = n_q / n_kv;
@@ -328,12 +381,12 @@ int prefill_shared_rows(int hd, int n_q, int n_kv) {
     return 32 * (4 / heads_per_workgroup(n_q, n_kv));
 }
 
-template <int HD, int QT, int HPW>
+template <int HD, int QT, int HPW, int KW>
 static int launch_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, const int* q_start,
                          const int* ctx_len, const int* table, int max_blocks, int n_seq, int n_q, int n_kv, int page,
                          float scale, int window, int items, int* queue, hipStream_t stream) {
     constexpr int LDS = StageLayout<HD>::BYTES;
-    auto kernel = attention_prefill_shared_kernel<HD, QT, HPW>;
+    auto kernel = attention_prefill_shared_kernel<HD, QT, HPW, KW>;
     static bool attr_set = false;                      // per instantiation
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -347,12 +400,13 @@ static int launch_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* ou
         hipError_t e = hipGetDevice(&dev);
         if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
         if (e == hipSuccess)
-            e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel), 256, LDS);
+            e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel), 256 * KW,
+                                                             LDS);
         if (e != hipSuccess) return static_cast<int>(e);
         resident = cus * (per_cu > 0 ? per_cu : 1);
     }
     const int n_items = items * (n_q / HPW);
-    hipLaunchKernelGGL(kernel, dim3(n_items < resident ? n_items : resident), dim3(256), LDS, stream, q, kc, vc, out,
+    hipLaunchKernelGGL(kernel, dim3(n_items < resident ? n_items : resident), dim3(256 * KW), LDS, stream, q, kc, vc, out,
                        q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, page, scale, window, items, queue);
     return launch_status();
 }
@@ -364,14 +418,22 @@ int launch_prefill_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* o
     if (queue == nullptr) return kErrBadArgument;
     const int hpw = heads_per_workgroup(n_q, n_kv);
     const int rows = rows_per_item / (4 / hpw);            // per row group
-#define LLME_SHARED(HD, QT, HPW)                                                                               \
-    if (hd == HD && rows == 16 * QT && hpw == HPW)                                                             \
-        return launch_shared<HD, QT, HPW>(q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, \
-                                          page, scale, window, items, queue, stream)
+    // Two wavefronts per tile while the items are too few to keep three workgroups of four
+    // wavefronts on every compute unit: then an item's length, not the chip, sets the time.
+    int kw = static_cast<long>(items) * (n_q / hpw) <= kSplitBelowItems ? 2 : 1;
+    if (g_key_waves == 1 || g_key_waves == 2) kw = g_key_waves;
+#define LLME_SHARED(HD, QT, HPW)                                                                                   \
+    if (hd == HD && rows == 16 * QT && hpw == HPW)                                                                 \
+        return kw == 2 ? launch_shared<HD, QT, HPW, 2>(q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, \
+                                                       n_q, n_kv, page, scale, window, items, queue, stream)       \
+                       : launch_shared<HD, QT, HPW, 1>(q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, \
+                                                       n_q, n_kv, page, scale, window, items, queue, stream)
     LLME_SHARED(64, 2, 4); LLME_SHARED(64, 2, 2); LLME_SHARED(64, 2, 1);
     LLME_SHARED(128, 2, 4); LLME_SHARED(128, 2, 2); LLME_SHARED(128, 2, 1);
 #undef LLME_SHARED
     return kErrUnsupported;
 }
+
+void prefill_shared_key_waves(int kw) { g_key_waves = kw; }
 
 }  // namespace llme

@@ -349,5 +349,7 @@ int launch_prefill_shared(const bf16* q, const bf16* k_cache, const bf16* v_cach
                           hipStream_t stream);
 // Rows per work item of the shared kernel for these sizes, or 0 if it does not take them.
 int prefill_shared_rows(int hd, int n_q, int n_kv);
+// Wavefronts that share a tile's keys: 0 lets the launcher choose by the number of items, 1 or 2 forces it.
+void prefill_shared_key_waves(int kw);
 
 }  // namespace llme

@@ -363,7 +363,7 @@ def test_attention_mfma_prefill_and_mixed(ops, n_q, n_kv, hd, page):
 
 @pytest.mark.parametrize("n_q,n_kv,hd,page", [(8, 2, 64, 16), (4, 2, 64, 48), (6, 2, 64, 32), (3, 3, 64, 16),
                                               (8, 2, 128, 16), (2, 1, 128, 32), (5, 5, 128, 16)])
-@pytest.mark.parametrize("rows,shared", [(0, -1), (32, 0), (0, 0)])
+@pytest.mark.parametrize("rows,shared", [(0, -1), (0, 2), (0, 3), (32, 0), (0, 0)])
 def test_attention_prefill_shared_and_direct(ops, n_q, n_kv, hd, page, rows, shared):
     """The prefill kernel that shares K and V through LDS, for 4, 2 and 1 heads of a kv head per
     workgroup, spans that end inside a 64-key stretch, portions that start deep in a context,
