@@ -347,6 +347,29 @@ int llme_cm_num_pages(void* h, int group) {
 }
 int llme_cm_check(void* h) { return static_cast<CacheManager*>(h)->check(); }
 
+// A step of one new token per request, in one call: the requests' lengths, and a page for each
+// new token where it starts a page (all or none). Returns 1, 0 (pools short, nothing changed) or
+// an error code.
+int llme_cm_decode_begin(void* h, int S, const int64_t* keys, int* lengths) {
+    auto* m = static_cast<CacheManager*>(h);
+    std::vector<long> ones(static_cast<size_t>(S), 1);
+    for (int i = 0; i < S; ++i) {
+        auto* r = m->find(keys[i]);
+        if (!r) return LLME_HOST_NOT_LIVE;
+        lengths[i] = static_cast<int>(r->length);
+    }
+    return m->reserve_batch(S, keys, ones.data());
+}
+// commit for several requests: n_new tokens each
+int llme_cm_commit_batch(void* h, int S, const int64_t* keys, long n_new) {
+    auto* m = static_cast<CacheManager*>(h);
+    for (int i = 0; i < S; ++i) {
+        const int rc = m->commit(keys[i], n_new);
+        if (rc != 0) return rc;
+    }
+    return 0;
+}
+
 // What a recorded decode step needs before every replay, in one call: for each of the S requests
 // its length (the new token's position) and slot, and into the block tables of every group
 // (rows of `width` entries, group after group) the entries [done, blocks) that are not there

@@ -184,6 +184,10 @@ class Engine:
     def run_step(self, cache: CacheContext, entries, draws, temperature: float = 0.0, seed: int = 0) -> list[int]:
         """A step plus the choice of a token for every wanted row (the scheduler's call)."""
         with self._lock, torch.cuda.device(self.runner.device):
+            if temperature == 0.0:
+                tokens = self.runner.step_greedy(cache, entries, max_position=self.max_pos)
+                if tokens is not None:
+                    return tokens
             logits = self.runner.step(cache, entries, max_position=self.max_pos)
             if logits is None:
                 return []

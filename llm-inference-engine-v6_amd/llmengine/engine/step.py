@@ -17,6 +17,8 @@ from typing import Sequence
 
 import torch
 
+from .. import ops
+
 from ..cache import CacheManager, CacheStorage, plan_groups
 from ..models.model import DecoderModel
 
@@ -145,8 +147,11 @@ class _DecodeRecord:
     tokens and lengths every step, a block-table entry when a request gets a new page,
     everything when other requests take part."""
 
-    def __init__(self, graph, logits, meta: torch.Tensor, S: int, width: int, groups: list[str]):
+    def __init__(self, graph, logits, meta: torch.Tensor, S: int, width: int, groups: list[str],
+                 tok_host: torch.Tensor | None = None):
         self.graph, self.logits, self.meta = graph, logits, meta
+        self.tok_host = tok_host                # pinned: where a greedy recording leaves the chosen tokens
+        self.tok_event = torch.cuda.Event() if tok_host is not None else None
         self.S, self.width, self.groups = S, width, groups
         sizes = [S, S, S, S + 1, S, S] + [S * width] * len(groups) + [S]
         self.offsets = [0]
@@ -165,14 +170,17 @@ class _DecodeRecord:
         self.serials = (ctypes.c_int64 * S)()               # which admission of its key sits in each place
         self.event: torch.cuda.Event | None = None
 
-    def refresh(self, mgr: CacheManager, entries: Sequence[StepEntry]) -> None:
+    def refresh(self, mgr: CacheManager, entries: Sequence[StepEntry], keys=None) -> None:
         if self.event is not None:
             self.event.synchronize()            # the last copy has read the host mirror
         S, width, o, h = self.S, self.width, self.offsets, self.np
-        keys = [mgr.key_of(e.request_id) for e in entries]
-        if keys != self.key_list:
-            self.key_list = keys
-            self.keys = (ctypes.c_int64 * S)(*keys)
+        if keys is not None:                    # the caller has them as an array already
+            self.keys, self.key_list = keys, None
+        else:
+            keys = [mgr.key_of(e.request_id) for e in entries]
+            if keys != self.key_list:
+                self.key_list = keys
+                self.keys = (ctypes.c_int64 * S)(*keys)
         h[o[0]:o[1]] = [e.tokens[0] for e in entries]
         # lengths (tokens cached before this step), slots and the block-table entries that are new,
         # straight from the C++ manager into the pinned mirror
@@ -256,14 +264,25 @@ class ModelRunner:
         """A step of single decoded tokens, all wanting logits: the launch sequence depends
         only on the number of requests and on the width of the block tables, so it is
         recorded once as a HIP graph and replayed; only the integer arrays change."""
+        mgr = cache.manager
+        lengths = [mgr.length(e.request_id) for e in entries]
+        rec = self._decode_record(cache, entries, max(lengths), greedy=False)
+        rec.refresh(mgr, entries)
+        rec.graph.replay()
+        self.graph_replays += 1
+        return rec.logits
+
+    def _decode_record(self, cache: CacheContext, entries: Sequence[StepEntry], longest: int, greedy: bool):
+        """The recording for this many requests and this width of block tables (and, greedy, with
+        the argmax behind the model and its result written into pinned host memory); made at its
+        first use."""
         page = cache.page_size
         mgr = cache.manager
         S = len(entries)
-        lengths = [mgr.length(e.request_id) for e in entries]
-        need = (max(lengths) + page) // page
+        need = (longest + page) // page
         bucket = self.GRAPH_BLOCK_BUCKET
         width = (need + bucket - 1) // bucket * bucket
-        key = (S, width)
+        key = (S, width, greedy)
         rec = cache.graphs.get(key)
         if rec is None:
             # First time: run it plainly (this also sizes the scratch buffers), then record.
@@ -271,17 +290,63 @@ class ModelRunner:
             groups = len(mgr.groups)
             meta = torch.empty(7 * S + 1 + groups * S * width + 64, dtype=torch.int32, device=self.device)
             ctx, logit_rows = self._build_context(cache, entries, max_blocks=width, plan_len=width * page, dev=meta)
-            self.model.forward(ctx, cache.storage.layers, logit_rows)
+            logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
+            tok_host = None
+            if greedy:
+                # pinned host memory is mapped into the device's address space: the kernel writes
+                # the tokens where the host reads them, without a copy of its own
+                tok_host = torch.zeros(S, dtype=torch.int32, pin_memory=True)
+                ops.argmax_into(logits, tok_host.data_ptr())
             torch.cuda.synchronize(self.device)
             self.workspace.keep_replaced = True
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
-            cache.graphs[key] = rec = _DecodeRecord(graph, logits, meta, S, width, list(mgr.groups))
-        rec.refresh(mgr, entries)
+                if greedy:
+                    ops.argmax_into(logits, tok_host.data_ptr())
+            cache.graphs[key] = rec = _DecodeRecord(graph, logits, meta, S, width, list(mgr.groups), tok_host)
+        return rec
+
+    def step_greedy(self, cache: CacheContext, entries: Sequence[StepEntry], max_position: int | None = None
+                    ) -> list[int] | None:
+        """The greedy next token of every entry, for a step of single decoded tokens that all want
+        one: bookkeeping in two calls into the host runtime, the argmax inside the recorded graph,
+        its result read from pinned memory. None if the step is not of that kind (then `step`
+        and a sampler do it)."""
+        if not self.use_graphs or not entries:
+            return None
+        vocab = self.model.vocab_size
+        ids = []
+        for e in entries:
+            if len(e.tokens) != 1 or len(e.want) != 1 or e.want[0] != 0:
+                return None
+            if not 0 <= int(e.tokens[0]) < vocab:
+                raise ValueError(f"token id {e.tokens[0]} out of range [0, {vocab})")
+            ids.append(e.request_id)
+        S = len(ids)
+        if len(set(ids)) != S:
+            raise ValueError("a request appears twice in one step")
+        mgr = cache.manager
+        keys = (ctypes.c_int64 * S)(*[mgr.key_of(r) for r in ids])
+        lengths = (ctypes.c_int * S)()
+        rc = mgr._lib.llme_cm_decode_begin(mgr.handle, S, keys, lengths)
+        if rc < 0:
+            raise RuntimeError(f"a request of the step is not live (code {rc})")
+        longest = max(lengths)
+        if rc == 0:
+            need = {g: sum(mgr.pages_needed(r, 1)[g] for r in ids) for g in mgr.groups}
+            raise CapacityError(f"the step needs {need} more pages, free are "
+                                f"{({g: mgr.free_pages(g) for g in mgr.groups})}")
+        if max_position is not None and longest + 1 > max_position:
+            raise ValueError(f"{longest + 1} tokens exceed the position limit {max_position}")
+        rec = self._decode_record(cache, entries, longest, greedy=True)
+        rec.refresh(mgr, entries, keys)
         rec.graph.replay()
+        rec.tok_event.record()
         self.graph_replays += 1
-        return rec.logits
+        mgr._lib.llme_cm_commit_batch(mgr.handle, S, keys, 1)
+        rec.tok_event.synchronize()
+        return rec.tok_host.tolist()
 
     # ------------------------------------------------------------------------------
     def _build_context(self, cache: CacheContext, entries: Sequence[StepEntry], max_blocks: int | None = None,

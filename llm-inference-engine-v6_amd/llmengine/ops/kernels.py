@@ -183,13 +183,21 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     require(logits, "logits", torch.float32, (None, None))
     R, V = logits.shape
     require(out, "out", torch.int32, (R,))
+    argmax_into(logits, ptr(out))
+
+
+def argmax_into(logits: torch.Tensor, out_ptr: int) -> None:
+    """argmax with the result (one int32 per row) written to an address the device can reach:
+    device memory, or pinned host memory, which the device sees at the same address."""
+    require(logits, "logits", torch.float32, (None, None))
+    R, V = logits.shape
     need = R * entry("llme_argmax_parts")(V)
     scratch = _argmax_scratch.get(logits.device)
     if scratch is None or scratch[0].numel() < need:
         scratch = (torch.empty(max(need, 4096), dtype=torch.float32, device=logits.device),
                    torch.empty(max(need, 4096), dtype=torch.int32, device=logits.device))
         _argmax_scratch[logits.device] = scratch
-    check(entry("llme_argmax")(ptr(logits), ptr(out), ptr(scratch[0]), ptr(scratch[1]), R, V, stream()), "argmax")
+    check(entry("llme_argmax")(ptr(logits), out_ptr, ptr(scratch[0]), ptr(scratch[1]), R, V, stream()), "argmax")
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor) -> None:

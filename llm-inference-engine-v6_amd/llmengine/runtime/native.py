@@ -127,6 +127,7 @@ _SIGNATURES = {
     "llme_cm_commit": (_i, [_vp, _i64, _l]), "llme_cm_release": (_i, [_vp, _i64]),
     "llme_cm_table_len": (_i, [_vp, _i64, _i]), "llme_cm_table_copy": (_i, [_vp, _i64, _i, _i, _i, _pi]),
     "llme_cm_free_pages": (_i, [_vp, _i]), "llme_cm_num_pages": (_i, [_vp, _i]), "llme_cm_check": (_i, [_vp]),
+    "llme_cm_decode_begin": (_i, [_vp, _i, _pi64, _pi]), "llme_cm_commit_batch": (_i, [_vp, _i, _pi64, _l]),
     "llme_cm_fill_decode": (_i, [_vp, _i, _pi64, _i, _vp, _vp, _vp, _pi, _pi64]),
     "llme_sched_create": (_vp, [_vp, _i, _l]), "llme_sched_destroy": (None, [_vp]),
     "llme_sched_set_budget": (_i, [_vp, _l]), "llme_sched_enqueue": (_l, [_vp, _pi, _l, _l]),
