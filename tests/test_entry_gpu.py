@@ -169,6 +169,43 @@ def test_scheduler_greedy_equals_generate(dir_a, dtype):
     assert blocks.free_blocks == 64 and [r.seq_id for r in sched.results] == list(range(len(prompts)))
 
 
+def test_greedy_step_with_the_argmax_in_the_recording(dir_b):
+    """run_step at temperature 0 takes decode steps through a recording that ends in the argmax:
+    same tokens as the logits' own argmax, a clear error when the pages run out, and requests
+    that come and go between the steps."""
+    from llmengine import CapacityError, Engine, StepEntry
+    engine = Engine(dir_b, "bf16")
+    a = Engine(dir_b, "bf16")
+    prompts = {"x": random_tokens(19, 384, 1), "y": random_tokens(8, 384, 2), 7: random_tokens(33, 384, 3)}
+    caches = [e.new_cache(12, 8, 3) for e in (engine, a)]
+    last = {}
+    for rid, p in prompts.items():
+        for c, e in zip(caches, (engine, a)):
+            c.admit(rid)
+            lg = e.step(c, [StepEntry(rid, p, [len(p) - 1])])
+        last[rid] = int(lg.argmax())
+    for turn in range(12):
+        ids = list(last) if turn % 4 else list(last)[::-1]
+        entries = [StepEntry(r, [last[r]], [0]) for r in ids]
+        got = engine.run_step(caches[0], entries, None)
+        want = a.step(caches[1], entries).argmax(dim=1).tolist()
+        assert got == want
+        last = dict(zip(ids, got))
+        if turn == 5:                                        # one leaves, the others go on
+            for c in caches:
+                c.release("y")
+            del last["y"]
+    assert engine.runner.graph_replays >= 10
+    with pytest.raises(CapacityError):                       # 12 pages of 8: the three requests outgrow them
+        for _ in range(40):
+            got = engine.run_step(caches[0], [StepEntry(r, [last[r]], [0]) for r in last], None)
+            last = dict(zip(last, got))
+    before = {r: caches[0].manager.length(r) for r in last}
+    with pytest.raises(CapacityError):
+        engine.run_step(caches[0], [StepEntry(r, [last[r]], [0]) for r in last], None)
+    assert before == {r: caches[0].manager.length(r) for r in last}      # a refused step changes nothing
+
+
 def test_scheduler_capacity_on_the_gpu(dir_a):
     from llmengine import BlockManager, ContinuousBatchScheduler, Engine
     engine = Engine(dir_a, "fp32")
