@@ -145,6 +145,86 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, const float*
     }
 }
 
+// The same for the usual case (all of a head's dims rotated, head size a multiple of 16), eight
+// dims per thread: 32-byte loads of the projection's row and of the tables, 16-byte stores of q
+// and k. One workgroup per token; a thread takes 8 dims of one half of a q or k head together
+// with their partners in the other half, or 8 dims of a v head.
+template <typename T>
+__device__ __forceinline__ void store8(T* dst, const float (&v)[8]);
+template <>
+__device__ __forceinline__ void store8<float>(float* dst, const float (&v)[8]) {
+    *reinterpret_cast<float4*>(dst) = float4{v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<float4*>(dst + 4) = float4{v[4], v[5], v[6], v[7]};
+}
+template <>
+__device__ __forceinline__ void store8<bf16>(bf16* dst, const float (&v)[8]) {
+    typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+    bf16x8 o;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = static_cast<__bf16>(v[j]);
+    *reinterpret_cast<bf16x8*>(dst) = o;
+}
+__device__ __forceinline__ void load8(const float* src, float (&v)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(src), b = *reinterpret_cast<const float4*>(src + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+template <typename TQ, typename TC>
+__global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
+    const float* __restrict__ qkv, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ positions, const int* __restrict__ seq_idx, const int* __restrict__ block_table,
+    int max_blocks, TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache, int n_q, int n_kv,
+    int hd, int page, int write_cache) {
+    const int t = blockIdx.x;
+    const int pos = positions[t];
+    int pg = 0, off = 0;
+    if (write_cache) {
+        pg = block_table[static_cast<size_t>(seq_idx[t]) * max_blocks + pos / page];
+        off = pos % page;
+    }
+    const int half = hd / 2, hv = half / 8, dv = hd / 8;
+    const float* row = qkv + static_cast<size_t>(t) * (n_q + 2 * n_kv) * hd;
+    const float* cs = cos_t + static_cast<size_t>(pos) * half;
+    const float* sn = sin_t + static_cast<size_t>(pos) * half;
+    const int q_items = n_q * hv, k_items = n_kv * hv, v_items = n_kv * dv;
+    const int items = q_items + (write_cache ? k_items + v_items : 0);
+    for (int it = threadIdx.x; it < items; it += blockDim.x) {
+        if (it < q_items + k_items) {
+            const bool is_q = it < q_items;
+            const int e = is_q ? it : it - q_items;
+            const int h = e / hv, i = (e % hv) * 8;
+            const float* src = row + (is_q ? 0 : n_q * hd) + h * hd + i;
+            float a[8], b[8], c[8], sv[8], lo[8], hi[8];
+            load8(src, a);
+            load8(src + half, b);
+            load8(cs + i, c);
+            load8(sn + i, sv);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                lo[j] = a[j] * c[j] - b[j] * sv[j];
+                hi[j] = b[j] * c[j] + a[j] * sv[j];
+            }
+            if (is_q) {
+                TQ* dst = q_out + (static_cast<size_t>(t) * n_q + h) * hd + i;
+                store8<TQ>(dst, lo);
+                store8<TQ>(dst + half, hi);
+            } else {
+                TC* dst = k_cache + ((static_cast<size_t>(pg) * n_kv + h) * page + off) * hd + i;
+                store8<TC>(dst, lo);
+                store8<TC>(dst + half, hi);
+            }
+        } else {
+            const int e = it - q_items - k_items;
+            const int h = e / dv, d0 = (e % dv) * 8;
+            float v[8];
+            load8(row + (n_q + n_kv) * hd + h * hd + d0, v);
+            TC* dst = v_cache + ((static_cast<size_t>(pg) * n_kv + h) * hd + d0) * page + off;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) dst[static_cast<size_t>(j) * page] = from_float<TC>(v[j]);
+        }
+    }
+}
+
 }  // namespace llme
 
 using namespace llme;
@@ -202,11 +282,24 @@ extern "C" int llme_rope_kv_write(const float* qkv, const float* cos_t, const fl
                                   int write_cache, hipStream_t stream) {
     if (T <= 0) return 0;
     if (rot < 0 || rot > hd || rot % 2 != 0 || page <= 0) return kErrBadArgument;
-#define LLME_ROPE(TQ, TC)                                                                        \
-    hipLaunchKernelGGL((rope_kv_write_kernel<TQ, TC>), dim3(T), dim3(256), 0, stream, qkv, cos_t, \
-                       sin_t, positions, seq_idx, block_table, max_blocks, static_cast<TQ*>(q_out), \
-                       static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), n_q, n_kv, hd, rot,  \
-                       page, write_cache)
+    // all dims rotated and head sizes in steps of 16: the kernel that moves 8 dims per thread
+    const bool vec = rot == hd && hd % 16 == 0 && cos_t != nullptr && sin_t != nullptr &&
+                     reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(q_out) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(cos_t) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(sin_t) % 16 == 0;
+#define LLME_ROPE(TQ, TC)                                                                                   \
+    do {                                                                                                    \
+        if (vec)                                                                                            \
+            hipLaunchKernelGGL((rope_kv_write_vec_kernel<TQ, TC>), dim3(T), dim3(256), 0, stream, qkv, cos_t, \
+                               sin_t, positions, seq_idx, block_table, max_blocks, static_cast<TQ*>(q_out), \
+                               static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), n_q, n_kv, hd, page,   \
+                               write_cache);                                                                \
+        else                                                                                                \
+            hipLaunchKernelGGL((rope_kv_write_kernel<TQ, TC>), dim3(T), dim3(256), 0, stream, qkv, cos_t,   \
+                               sin_t, positions, seq_idx, block_table, max_blocks, static_cast<TQ*>(q_out), \
+                               static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), n_q, n_kv, hd, rot,    \
+                               page, write_cache);                                                          \
+    } while (0)
     if (q_dtype == kF32 && cache_dtype == kF32) LLME_ROPE(float, float);
     else if (q_dtype == kBF16 && cache_dtype == kBF16) LLME_ROPE(bf16, bf16);
     else if (q_dtype == kF32 && cache_dtype == kBF16) LLME_ROPE(float, bf16);
