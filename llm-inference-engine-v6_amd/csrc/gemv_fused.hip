@@ -347,8 +347,8 @@ extern "C" int llme_gemv_norm_rope(const float* h, const void* norm_w, int norm_
                           static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache), n_q, n_kv, hd, page};
     const bf16* W = static_cast<const bf16*>(w);
     if (norm_dtype == kBF16)
-        return launch_gemv_norm<8, 2, kRope, bf16>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, rope, stream);
+        return launch_gemv_norm<16, 2, kRope, bf16>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, rope, stream);
     if (norm_dtype == kF32)
-        return launch_gemv_norm<8, 2, kRope, float>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, rope, stream);
+        return launch_gemv_norm<16, 2, kRope, float>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, rope, stream);
     return kErrBadArgument;
 }
