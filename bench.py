@@ -1,15 +1,18 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 4096] [--layers L] [--shape 1b|3b|8b]
 
-The model has the layer sizes of Llama 3.2 1B (16 layers, width 2048, 32 query / 8 key-value
+By default the model has the layer sizes of Llama 3.2 1B (16 layers, width 2048, 32 query / 8 key-value
 heads of 64, feed-forward 8192, vocabulary 128256, llama3 rope scaling, tied head) with seeded
 random bfloat16 weights; token ids are seeded uniform random numbers. A "step" is one decode
 step of the whole batch: the model over one token per request from the paged cache, the choice
 of the next token (greedy) and its way back to the host. Every request holds `context - steps -
 warmup` tokens when decoding starts, put there by real prefill steps, so that the timed steps
 run at the configured context length. One JSON line goes to stdout.
+
+`--shape 3b` and `--shape 8b` take the layer sizes of Llama 3.2 3B and Llama 3.1 8B instead (for
+measurements at further sizes and context lengths; the default run is the 1B shape).
 
 Beside the headline value the line holds: `prefill` (one 2,048-token prompt, logits at its last
 place), `roofline` (bytes the decode step has to read: every weight once plus the live
@@ -39,7 +42,16 @@ LLAMA_1B = {
                      "high_freq_factor": 4.0, "original_max_position_embeddings": 8192},
     "tie_word_embeddings": True,
 }
-FULL_LAYERS = 16
+
+# Further shapes of the same architecture (--shape), for measurements beside the default one.
+SHAPES = {
+    "1b": LLAMA_1B,
+    "3b": dict(LLAMA_1B, hidden_size=3072, intermediate_size=8192, num_hidden_layers=28, num_attention_heads=24,
+               num_key_value_heads=8, head_dim=128),
+    "8b": dict(LLAMA_1B, hidden_size=4096, intermediate_size=14336, num_hidden_layers=32, num_attention_heads=32,
+               num_key_value_heads=8, head_dim=128, tie_word_embeddings=False,
+               rope_scaling=dict(LLAMA_1B["rope_scaling"], factor=8.0)),
+}
 
 
 def log(msg: str) -> None:
@@ -54,6 +66,8 @@ def layer_weight_elements(c: dict) -> int:
 
 def decode_bytes(c: dict, batch: int, ctx: float, wbytes: int) -> float:
     """Bytes a decode step has to read: every weight once, and the cache of the live requests."""
+    # the output head's matrix once (tied or not, a decode step reads one vocabulary-sized matrix: the
+    # embedding is only gathered from)
     weights = (c["num_hidden_layers"] * layer_weight_elements(c) + c["vocab_size"] * c["hidden_size"]
                + c["hidden_size"]) * wbytes
     kv = batch * ctx * 2 * c["num_key_value_heads"] * c["head_dim"] * wbytes * c["num_hidden_layers"]
@@ -78,7 +92,8 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096, help="context length the decode steps run at")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (named in config)")
+    ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes: Llama 3.2 1B (the default), 3.2 3B, 3.1 8B")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (named in config)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--seed", type=int, default=0)
@@ -92,7 +107,9 @@ def main() -> int:
     import torch
     from llmengine import Engine, StepEntry
 
-    cfg = dict(LLAMA_1B, num_hidden_layers=args.layers)
+    full_layers = SHAPES[args.shape]["num_hidden_layers"]
+    args.layers = args.layers or full_layers
+    cfg = dict(SHAPES[args.shape], num_hidden_layers=args.layers)
     wbytes = 2 if args.dtype == "bf16" else 4
     t0 = time.time()
     log(f"building the model ({args.layers} layers, {args.dtype}) with random weights")
@@ -184,12 +201,13 @@ def main() -> int:
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic (seeded random weights and token ids)",
         "config": {
-            "model": "llama-3.2-1b-shape", "global_batch": args.batch, "seq_len": args.context,
-            "parallelism": "single-gpu", "layers": args.layers, "layers_full_model": FULL_LAYERS,
+            "model": {"1b": "llama-3.2-1b-shape", "3b": "llama-3.2-3b-shape", "8b": "llama-3.1-8b-shape"}[args.shape],
+            "global_batch": args.batch, "seq_len": args.context,
+            "parallelism": "single-gpu", "layers": args.layers, "layers_full_model": full_layers,
             "hidden_size": cfg["hidden_size"], "intermediate_size": cfg["intermediate_size"],
             "num_attention_heads": cfg["num_attention_heads"], "num_key_value_heads": cfg["num_key_value_heads"],
-            "head_dim": cfg["head_dim"], "vocab_size": V, "tie_word_embeddings": True,
-            "rope": "theta 5e5, llama3 scaling 32/1/4/8192", "page_size": page,
+            "head_dim": cfg["head_dim"], "vocab_size": V, "tie_word_embeddings": cfg["tie_word_embeddings"],
+            "rope": f"theta 5e5, llama3 scaling {cfg['rope_scaling']['factor']:g}/1/4/8192", "page_size": page,
             "prefill_tokens": T, "decode_context": args.context, "sampling": "greedy",
         },
         "prefill": prefill, "roofline": roofline, "points": points,
