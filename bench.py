@@ -159,11 +159,17 @@ def main() -> int:
         ids = [f"r{i}" for i in range(batch)]
         for rid in ids:
             cache.admit(rid)
-        chunk = 4096
+        chunk = 8192
+        sync()
+        t_fill = time.perf_counter()
         for rid in ids:                                        # real prefill fills the pages
             toks = torch.randint(0, V, (start_ctx,), generator=gen).tolist()
             for s in range(0, start_ctx, chunk):
                 engine.step(cache, [StepEntry(rid, toks[s:s + chunk], [])])
+        sync()
+        t_fill = time.perf_counter() - t_fill
+        log(f"filled the cache: {batch} x {start_ctx} tokens in portions of {chunk} in {t_fill:.2f} s "
+            f"({batch * start_ctx / t_fill:.0f} tok/s, token generation on the host included)")
         last = torch.randint(0, V, (batch,), generator=gen).tolist()
 
         def one_step(tokens):
