@@ -1,7 +1,8 @@
 """Each part of a layer alone on the GPU against its plain formula, and the generality of
 the composition: a schedule that names a layer twice and lets a layer read another layer's
-cache, a windowed attention with pages given back, and a toy mixer with state of its own
-that is defined here, registered, built and stepped without a change to the framework."""
+cache, a windowed attention with pages given back, and toy parts that are defined here,
+registered, built and stepped without a change to the framework: a mixer with state of its own,
+a feed-forward with routing, another position encoding and another arrangement of a block."""
 import math
 from dataclasses import dataclass
 
@@ -339,3 +340,163 @@ def test_a_toy_mixer_with_state_registers_builds_and_steps():
                 assert _rel(got[rid][pos], plain[rid][pos]) < 1e-5, (rid, pos)
     out, finish = engine.generate(reqs["t1"], 5)
     assert finish == "length" and len(out) == 13
+
+
+# --- a toy feed-forward with routing, another position encoding, another arrangement -------
+def test_toy_routed_feed_forward_position_encoding_and_arrangement():
+    """Three more kinds of part, defined here and registered through the public registries: a
+    feed-forward that routes each token to one of E small experts, a rotary encoding over a part
+    of the head with interpolated positions (p / stretch), and an arrangement in which mixer and
+    feed-forward read the same normed input. Layer 0 uses all three, layer 1 is ordinary."""
+    from llmengine import Engine
+    from llmengine.config import register_architecture
+    from llmengine.models.model import DecoderModel
+    from llmengine.parts import (Block, Embedding, FeedForward, LayerSpec, OutputHead, ParamSpec, PartChoice,
+                                 PositionEncoding, RMSNorm, build_layer, register_part)
+    from llmengine.weights import random_state
+
+    class Top1Experts(FeedForward):
+        def __init__(self, hidden_size, expert_size, num_experts):
+            self.h, self.f, self.e = hidden_size, expert_size, num_experts
+            self.p = {}
+
+        def param_specs(self):
+            specs = {"router.weight": ParamSpec((self.e, self.h))}
+            for e in range(self.e):
+                specs[f"experts.{e}.up.weight"] = ParamSpec((self.f, self.h))
+                specs[f"experts.{e}.down.weight"] = ParamSpec((self.h, self.f))
+            return specs
+
+        def load_params(self, get, placement):
+            self.p = {name: placement.place(get(name), torch.float32) for name in self.param_specs()}
+
+        def forward(self, x, step, out, accumulate):
+            xs = x.float()
+            prob = torch.softmax(xs @ self.p["router.weight"].T, dim=-1)
+            weight, choice = prob.max(dim=-1)
+            y = torch.zeros_like(xs)
+            for e in range(self.e):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    hid = torch.relu(xs[rows] @ self.p[f"experts.{e}.up.weight"].T)
+                    y[rows] = weight[rows, None] * (hid @ self.p[f"experts.{e}.down.weight"].T)
+            if accumulate:
+                out += y
+            else:
+                out.copy_(y)
+
+    class StretchedRotary(PositionEncoding):
+        def __init__(self, rotary_dim, theta, stretch, max_position):
+            self.rotary_dim, self.theta, self.stretch, self._max = rotary_dim, theta, stretch, max_position
+            self.cos = self.sin = None
+
+        @property
+        def max_position(self):
+            return self._max
+
+        def materialize(self, placement):
+            i = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
+            freq = self.theta ** (-2.0 * i / self.rotary_dim)
+            angle = (torch.arange(self._max, dtype=torch.float64) / self.stretch)[:, None] * freq[None, :]
+            self.cos = torch.cos(angle).float().to(placement.device).contiguous()
+            self.sin = torch.sin(angle).float().to(placement.device).contiguous()
+
+        def rotary_tables(self):
+            return self.cos, self.sin, self.rotary_dim
+
+    class ParallelBlock(Block):
+        """h += mixer(norm(h)) + feed_forward(norm(h)): one norm, both read it."""
+
+        def __init__(self, mixer, feed_forward, mixer_norm, ffn_norm):
+            self.mixer, self.feed_forward, self.norm = mixer, feed_forward, mixer_norm
+
+        def children(self):
+            return {"norm": self.norm, "attn": self.mixer, "moe": self.feed_forward}
+
+        def forward(self, h, step, cache, write_cache=True):
+            x = step.buffer("parallel.normed", tuple(h.shape), step.act_dtype)
+            self.norm.forward(h, x)
+            self.mixer.forward(x, step, cache, h, True, write_cache)
+            self.feed_forward.forward(x, step, h, True)
+
+    register_part("feed_forward", "top1_experts", Top1Experts, replace=True)
+    register_part("position", "stretched_rotary", StretchedRotary, replace=True)
+    register_part("block", "parallel", ParallelBlock, replace=True)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        max_pos: int
+        eos_token_ids: tuple = ()
+
+    H, V, FF, E, EF, HD, ROT, NQ, NKV = 40, 77, 56, 3, 24, 16, 8, 2, 2
+    THETA, STRETCH, EPS = 100.0, 2.5, 1e-4
+
+    def build(c):
+        norm = PartChoice("rmsnorm", {"size": H, "eps": EPS})
+        att = PartChoice("attention", {"hidden_size": H, "num_heads": NQ, "num_kv_heads": NKV, "head_dim": HD})
+        first = LayerSpec(PartChoice("parallel"), att,
+                          PartChoice("top1_experts", {"hidden_size": H, "expert_size": EF, "num_experts": E}),
+                          norm, norm, PartChoice("stretched_rotary", {"rotary_dim": ROT, "theta": THETA,
+                                                                      "stretch": STRETCH, "max_position": c.max_pos}))
+        second = LayerSpec(PartChoice("prenorm"), att,
+                           PartChoice("gated_mlp", {"hidden_size": H, "intermediate_size": FF}), norm, norm,
+                           PartChoice("rotary", {"rotary_dim": HD, "theta": THETA, "max_position": c.max_pos}))
+        emb = Embedding(V, H)
+        return DecoderModel(c, emb, [build_layer(first), build_layer(second)], RMSNorm(H, EPS),
+                            OutputHead(V, H, tied_to=emb))
+
+    register_architecture("ToyRoutedForCausalLM", lambda cfg, gen=None, architecture="":
+                          ToyConfig(cfg["max_position_embeddings"]), build, replace=True)
+    cfg = {"architectures": ["ToyRoutedForCausalLM"], "max_position_embeddings": 128}
+    tensors = dict(random_state(cfg, 23, torch.float32, 0.2, 1.0, 0.1))
+    assert "model.layers.0.moe.experts.2.down.weight" in tensors and "model.layers.0.norm.weight" in tensors
+    assert "model.layers.0.post_attention_layernorm.weight" not in tensors
+    engine = Engine(None, "fp32", _config=cfg, _tensors=dict(tensors), block_size=8)
+
+    def plain_attn(x, w, p, cos, sin, rot):
+        n = x.shape[0]
+        q = plain_linear(x, w[p + "q_proj.weight"]).view(n, NQ, HD).clone()
+        k = plain_linear(x, w[p + "k_proj.weight"]).view(n, NKV, HD).clone()
+        v = plain_linear(x, w[p + "v_proj.weight"]).view(n, NKV, HD)
+        q[..., :rot] = plain_apply_rope(q[..., :rot], cos, sin)          # the rest of a head is not rotated
+        k[..., :rot] = plain_apply_rope(k[..., :rot], cos, sin)
+        return plain_linear(plain_attention(q, k, v).reshape(n, -1), w[p + "o_proj.weight"])
+
+    used = set()
+
+    def plain_toy(ids):
+        w = {k: v.double() for k, v in tensors.items()}
+        n = len(ids)
+        h = w["model.embed_tokens.weight"][ids]
+        p = "model.layers.0."
+        x = plain_rmsnorm(h, w[p + "norm.weight"], EPS)
+        freq = [THETA ** (-2.0 * i / ROT) for i in range(ROT // 2)]
+        cos, sin = plain_rope_tables(freq, [t / STRETCH for t in range(n)], ROT)
+        mixed = plain_attn(x, w, p + "attn.", cos, sin, ROT)
+        routed = torch.zeros_like(h)
+        for t in range(n):
+            logits = plain_linear(x[t:t + 1], w[p + "moe.router.weight"])[0]
+            prob = torch.exp(logits - logits.max())
+            prob = prob / prob.sum()
+            e = int(prob.argmax())
+            used.add(e)
+            hid = torch.clamp(plain_linear(x[t:t + 1], w[p + f"moe.experts.{e}.up.weight"]), min=0.0)
+            routed[t] = prob[e] * plain_linear(hid, w[p + f"moe.experts.{e}.down.weight"])[0]
+        h = h + mixed + routed
+        p = "model.layers.1."
+        cos, sin = plain_rope_tables(plain_inv_freq(HD, THETA, None), range(n), HD)
+        h = h + plain_attn(plain_rmsnorm(h, w[p + "input_layernorm.weight"], EPS), w, p + "self_attn.", cos, sin, HD)
+        h = h + plain_mlp(plain_rmsnorm(h, w[p + "post_attention_layernorm.weight"], EPS),
+                          w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+        return plain_linear(plain_rmsnorm(h, w["model.norm.weight"], EPS), w["model.embed_tokens.weight"]).numpy()
+
+    reqs = {f"m{i}": random_tokens(n, V, 90 + i) for i, n in enumerate((45, 9, 33, 70))}
+    plain = {k: plain_toy(v) for k, v in reqs.items()}
+    assert used == set(range(E))                                         # every expert took some token
+    for steps in (replay.whole(reqs), replay.tail_one_by_one(reqs, 12), replay.portions(reqs),
+                  replay.mixed(reqs, max_live=3, seed=9)):
+        cache = engine.new_cache(replay.trace_peak_tokens(steps, 8) // 8, 8, 3)
+        got = replay.run_trace(engine, cache, steps)
+        for rid, ids in reqs.items():
+            for pos in range(len(ids)):
+                assert _rel(got[rid][pos], plain[rid][pos]) < 1e-5, (rid, pos)
