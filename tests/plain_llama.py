@@ -76,12 +76,18 @@ def plain_rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
     return (w * x) * inv_rms
 
 
-def plain_linear(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+def plain_linear_by_rows(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """out[m, n] = sum_k a[m, k] * w[n, k], W stored [N, K]; no bias (src/kernels.cpp:33-57)."""
     out = torch.zeros(a.shape[0], w.shape[0], dtype=a.dtype)
     for n in range(w.shape[0]):
         out[:, n] = (a * w[n]).sum(dim=-1)
     return out
+
+
+def plain_linear(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """The same sum as `plain_linear_by_rows` through the library's matrix product on the CPU
+    (tests pin the two to each other): fast enough for layers of real width."""
+    return a @ w.T
 
 
 def plain_silu(x: torch.Tensor) -> torch.Tensor:
@@ -178,9 +184,9 @@ def bf16_round(x: torch.Tensor) -> torch.Tensor:
 
 
 def plain_forward(cfg: dict, weights: dict, tokens, dtype=torch.float64, rounder=None, positions=None,
-                  schedule=None, window: int = 0) -> torch.Tensor:
-    """Logits [T, V] at every position of one sequence (src/engine.cpp:105-261 per token, applied
-    to the whole sequence at once). `positions` shifts the sequence (default 0..T-1). `schedule`:
+                  schedule=None, window: int = 0, rows=None) -> torch.Tensor:
+    """Logits [T, V] at every position of one sequence, or at the positions `rows` only
+    (src/engine.cpp:105-261 per token, applied to the whole sequence at once). `positions` shifts the sequence (default 0..T-1). `schedule`:
     list of (layer, cache id, writes) in running order (default: each layer once, own cache);
     a call that does not write reads the keys and values of the cache id's writer."""
     c = plain_config(cfg)
@@ -209,6 +215,8 @@ def plain_forward(cfg: dict, weights: dict, tokens, dtype=torch.float64, rounder
         x = rnd(plain_rmsnorm(h, w[p + "post_attention_layernorm.weight"], c["eps"]))  # engine.cpp:208
         h = h + plain_mlp(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                           w[p + "mlp.down_proj.weight"], rounder)                     # engine.cpp:213-239
+    if rows is not None:
+        h = h[list(rows)]
     x = rnd(plain_rmsnorm(h, w["model.norm.weight"], c["eps"]))                       # engine.cpp:243
     head = w["model.embed_tokens.weight"] if c["tie"] else w["lm_head.weight"]        # model.cpp:185-195
     return plain_linear(x, head)                                                      # engine.cpp:247

@@ -100,6 +100,21 @@ def trace_peak_tokens(steps: list[dict], round_to: int = 64) -> int:
     return peak
 
 
+def want_only(steps: list[dict], places: dict) -> list[dict]:
+    """The same steps with logits wanted only at `places[request id]` (positions in the request)."""
+    out, done = [], {}
+    for st in steps:
+        entries = []
+        for e in st["entries"]:
+            start = done.get(e["id"], 0)
+            keep = set(places[e["id"]])
+            entries.append({"id": e["id"], "tokens": e["tokens"],
+                            "want": [w for w in e["want"] if start + w in keep]})
+            done[e["id"]] = start + len(e["tokens"])
+        out.append({"step": st["step"], "entries": entries, "end": st["end"]})
+    return out
+
+
 def run_trace(engine, cache, steps: list[dict]) -> dict:
     """Drives engine.step; returns {request id: {position: logits row (numpy)}}."""
     from llmengine import StepEntry

@@ -245,3 +245,57 @@ def test_a_far_key_is_found(tmp_path):
         for pos in (5, 6, 300, 598, 599):
             err = np.abs(got[pos] - ref[pos]).max() / np.abs(ref[pos]).max()
             assert err < 1e-5, (pos, err)
+
+
+# A layer or two with the sizes of Llama 3.2 1B, 3.2 3B and 3.1 8B: the kernels that serving picks at
+# real widths (tiled products over several row tiles, the prefill attention with many work items, the
+# fused decode kernels at widths 2048, 3072 and 4096, the output head over the whole vocabulary).
+def _wide(hidden, ffn, heads, head_dim, layers, factor, tie):
+    return {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": hidden,
+            "intermediate_size": ffn, "num_hidden_layers": layers, "num_attention_heads": heads,
+            "num_key_value_heads": 8, "head_dim": head_dim, "vocab_size": 128256, "max_position_embeddings": 8192,
+            "rms_norm_eps": 1e-5, "rope_theta": 500000.0, "tie_word_embeddings": tie,
+            "rope_scaling": {"rope_type": "llama3", "factor": factor, "low_freq_factor": 1.0,
+                             "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}}
+
+
+WIDE = {"1b": _wide(2048, 8192, 32, 64, 2, 32.0, True), "3b": _wide(3072, 8192, 24, 128, 1, 32.0, True),
+        "8b": _wide(4096, 14336, 32, 128, 1, 8.0, False)}
+
+
+@pytest.fixture(scope="module", params=list(WIDE))
+def wide(request):
+    from llmengine.weights import random_state
+    cfg = WIDE[request.param]
+    tensors = dict(random_state(cfg, 3, torch.bfloat16, 0.02))
+    reqs = {"w0": random_tokens(333, cfg["vocab_size"], 31), "w1": random_tokens(70, cfg["vocab_size"], 32),
+            "w2": random_tokens(150, cfg["vocab_size"], 33)}
+    rows = {rid: sorted({0, 1, 63, 64, len(ids) // 2} | set(range(len(ids) - 34, len(ids)))) for rid, ids in reqs.items()}
+    plain, wide64 = {}, {k: v.double() for k, v in tensors.items()}
+    for dtype, rounder in (("fp32", None), ("bf16", bf16_round)):
+        plain[dtype] = {rid: plain_forward(cfg, wide64, ids, rounder=rounder, rows=rows[rid]).numpy()
+                        for rid, ids in reqs.items()}
+    return cfg, tensors, reqs, rows, plain
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_real_layer_sizes_match_plain(wide, dtype):
+    from llmengine import Engine
+    cfg, tensors, reqs, rows, plain = wide
+    engine = Engine(None, dtype, _config=cfg, _tensors=dict(tensors), block_size=16)
+    for name in ("whole", "tail", "mixed3"):
+        steps = replay.want_only(SCHEDULES[name](reqs), rows)
+        pages = replay.trace_peak_tokens(steps, round_to=16) // 16
+        cache = engine.new_cache(pages, 16, max_requests=4)
+        got = replay.run_trace(engine, cache, steps)
+        for rid in reqs:
+            assert sorted(got[rid]) == rows[rid]
+            for i, pos in enumerate(rows[rid]):
+                ref = plain[dtype][rid][i]
+                err = np.abs(got[rid][pos].astype(np.float64) - ref).max() / np.abs(ref).max()
+                assert err < TOL[dtype], f"{name}: request {rid} position {pos}: relative error {err:.3e}"
+            if dtype == "fp32":                        # the same greedy token as the plain implementation
+                last = rows[rid][-1]
+                assert int(got[rid][last].argmax()) == int(plain[dtype][rid][-1].argmax())
+    del engine
+    torch.cuda.empty_cache()

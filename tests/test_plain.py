@@ -9,7 +9,7 @@ import torch
 import torch.nn.functional as F
 
 from plain_llama import (plain_apply_rope, plain_argmax, plain_attention, plain_config, plain_forward,
-                         plain_inv_freq, plain_linear, plain_mlp, plain_rmsnorm, plain_rope_tables,
+                         plain_inv_freq, plain_linear, plain_linear_by_rows, plain_mlp, plain_rmsnorm, plain_rope_tables,
                          plain_sample_bounds, plain_silu)
 from tiny_models import TINY_A, TINY_B
 
@@ -45,7 +45,11 @@ def test_rmsnorm_special_cases():
 def test_linear_is_F_linear(M, N, K):
     a = torch.randn(M, K, generator=_gen(4), dtype=D)
     w = torch.randn(N, K, generator=_gen(5), dtype=D)
-    assert torch.allclose(plain_linear(a, w), F.linear(a, w), atol=1e-12)
+    assert torch.allclose(plain_linear_by_rows(a, w), F.linear(a, w), atol=1e-12)
+    assert torch.allclose(plain_linear(a, w), plain_linear_by_rows(a, w), atol=1e-12)
+    # W is [N, K]: the transposed reading gives another result (and another shape unless N == K)
+    if N == K:
+        assert not torch.allclose(plain_linear(a, w), a @ w, atol=1e-6)
 
 
 # --- inverse frequencies -------------------------------------------------------------
