@@ -299,3 +299,59 @@ def test_real_layer_sizes_match_plain(wide, dtype):
                 assert int(got[rid][last].argmax()) == int(plain[dtype][rid][-1].argmax())
     del engine
     torch.cuda.empty_cache()
+
+
+def _random_configuration(case: int):
+    import random
+    r = random.Random(case)
+    n_kv, group = r.choice([1, 2, 3, 5]), r.choice([1, 2, 3, 4, 7])
+    cfg = {"architectures": ["LlamaForCausalLM"], "model_type": "llama",
+           "head_dim": r.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 256]),
+           "hidden_size": r.choice([34, 50, 72, 100, 136, 200, 264]),
+           "intermediate_size": r.choice([50, 98, 176, 264, 400]), "num_hidden_layers": r.choice([1, 2, 3]),
+           "num_attention_heads": n_kv * group, "num_key_value_heads": n_kv,
+           "vocab_size": r.choice([50, 257, 384, 701]), "max_position_embeddings": 512,
+           "rms_norm_eps": r.choice([1e-5, 1e-6]), "rope_theta": r.choice([1e4, 5e5]),
+           "tie_word_embeddings": r.random() < 0.5}
+    if r.random() < 0.5:
+        cfg["rope_scaling"] = {"rope_type": "llama3", "factor": r.choice([8.0, 32.0]), "low_freq_factor": 1.0,
+                               "high_freq_factor": 4.0, "original_max_position_embeddings": r.choice([64, 128])}
+    return cfg, r.choice([4, 8, 16, 16, 32, 48, 64]), [r.randint(1, 220) for _ in range(4)]
+
+
+@pytest.mark.parametrize("case", range(10))
+def test_random_configurations(case):
+    """Sizes drawn at random from what a configuration allows: head sizes in steps of 16 up to 256,
+    odd numbers of heads and groups, widths that are no multiple of 8, any page size. 32-bit against
+    the plain implementation; bfloat16 must be as near to the exact result as the plain
+    implementation with bfloat16 rounding is (its rounding places differ between prompt and decode
+    kernels, so it is measured against the exact logits, not against one particular rounding)."""
+    from llmengine import Engine
+    from llmengine.weights import random_state
+    cfg, page, lens = _random_configuration(case)
+    tensors = dict(random_state(cfg, case, torch.bfloat16, 0.08, 1.0, 0.1))
+    wide = {k: v.double() for k, v in tensors.items()}
+    reqs = {f"r{i}": random_tokens(n, cfg["vocab_size"], 100 + i) for i, n in enumerate(lens)}
+    exact = {rid: plain_forward(cfg, wide, ids).numpy() for rid, ids in reqs.items()}
+    rounded = {rid: plain_forward(cfg, wide, ids, rounder=bf16_round).numpy() for rid, ids in reqs.items()}
+
+    def errors(got, rid):
+        ref = exact[rid]
+        return np.array([np.abs(np.asarray(got[rid][p], dtype=np.float64) - ref[p]).max() / np.abs(ref[p]).max()
+                         for p in range(len(ref))])
+
+    for dtype in ("fp32", "bf16"):
+        engine = Engine(None, dtype, _config=cfg, _tensors=dict(tensors), block_size=page)
+        for name, steps in (("whole", replay.whole(reqs)), ("tail", replay.tail_one_by_one(reqs, 20)),
+                            ("mixed", replay.mixed(reqs, max_live=3, seed=case))):
+            cache = engine.new_cache(replay.trace_peak_tokens(steps, round_to=page) // page, page, max_requests=3)
+            got = replay.run_trace(engine, cache, steps)
+            for rid in reqs:
+                err = errors(got, rid)
+                if dtype == "fp32":
+                    assert err.max() < TOL["fp32"], (cfg, page, name, rid, int(err.argmax()), float(err.max()))
+                else:
+                    base = errors(rounded, rid)
+                    assert err.mean() < 1.3 * base.mean() + 1e-3 and err.max() < 2.0 * base.max() + 1e-3, (
+                        cfg, page, name, rid, int(err.argmax()), float(err.max()), float(base.max()))
+        del engine
