@@ -148,31 +148,45 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
         for (int j = 0; j < WNT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // Slab j is computed from LDS buffer j % 2 and travels in register set j % 2. While slab j is
-    // computed, j + 1 sits in its registers and j + 2 is in flight; after the computing, j + 1
-    // goes into the other buffer and its registers ask for j + 3. The barrier waits for LDS only.
-    auto turn = [&](int kt, int buf, Slab& next) {
+    // computed, j + 1 sits in its registers and j + 2 is in flight. A turn first puts j + 1 into
+    // the other buffer and asks for j + 3, reads the fragments of its second half, multiplies the
+    // first half (whose fragments the turn before has read), and only then meets the others at the
+    // barrier: behind it, it reads the first fragments of slab j + 1 and multiplies its own second
+    // half meanwhile. So no product waits for an LDS read that was issued right in front of it,
+    // and the barrier (which waits for LDS only) is met with products still in the pipe.
+    static_assert(TK == 64, "a turn is two halves of 32");
+    bf16x8 fa0[WMT], fw0[WNT];                        // fragments of a slab's first half
+    auto read_frags = [&](int buf, int kk, bf16x8 (&fa)[WMT], bf16x8 (&fw)[WNT]) {
         const bf16* sA = lds + buf * A_ELEMS;
         const bf16* sW = lds + 2 * A_ELEMS + buf * W_ELEMS;
 #pragma unroll
-        for (int kk = 0; kk < TK / 32; ++kk) {
-            bf16x8 fa[WMT], fw[WNT];
+        for (int i = 0; i < WMT; ++i)
+            fa[i] = *reinterpret_cast<const bf16x8*>(sA + (wm + i * 16 + r) * TSTRIDE + kk * 32 + q * 8);
 #pragma unroll
-            for (int i = 0; i < WMT; ++i)
-                fa[i] = *reinterpret_cast<const bf16x8*>(sA + (wm + i * 16 + r) * TSTRIDE + kk * 32 + q * 8);
+        for (int j = 0; j < WNT; ++j)
+            fw[j] = *reinterpret_cast<const bf16x8*>(sW + (wn + j * 16 + r) * TSTRIDE + kk * 32 + q * 8);
+    };
+    auto multiply = [&](const bf16x8 (&fa)[WMT], const bf16x8 (&fw)[WNT]) {
+#pragma unroll
+        for (int i = 0; i < WMT; ++i)
 #pragma unroll
             for (int j = 0; j < WNT; ++j)
-                fw[j] = *reinterpret_cast<const bf16x8*>(sW + (wn + j * 16 + r) * TSTRIDE + kk * 32 + q * 8);
-#pragma unroll
-            for (int i = 0; i < WMT; ++i)
-#pragma unroll
-                for (int j = 0; j < WNT; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
-        }
-        // also on the last turn, where nobody reads what is stored: a turn without these would
-        // make the number of loads in flight depend on the path taken
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
+    };
+    auto turn = [&](int kt, int buf, Slab& next) {
+        // (the store and the loads also on the last turn, where nobody uses them: a turn without
+        // them would make the number of loads in flight depend on the path taken)
         store_lds(buf ^ 1, next);
         load_global(kt + 3, next);
+        bf16x8 fa1[WMT], fw1[WNT];
+        read_frags(buf, 1, fa1, fw1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(fa0, fw0);
+        __builtin_amdgcn_sched_barrier(0);            // (the products stay in front of the barrier)
         lds_barrier();
+        read_frags(buf ^ 1, 0, fa0, fw0);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(fa1, fw1);
     };
     if (kt_begin < kt_end) {
         Slab s0, s1;
@@ -186,6 +200,7 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
         load_global(kt_begin + 2, s0);
         __builtin_amdgcn_sched_barrier(0);
         lds_barrier();
+        read_frags(0, 0, fa0, fw0);
         // pairs of turns in a loop with one way round, then the odd turn: on every path into a
         // turn the loads in flight are the same, which keeps the compiler's waits exact
         int kt = kt_begin;
