@@ -54,6 +54,18 @@ constexpr int TSTRIDE = TK + 16;                     // elements; 160-byte rows 
 template <int WMT, int WNT>
 constexpr int tile_lds_bytes() { return 2 * (32 * WMT + 32 * WNT) * TSTRIDE * 2; }   // A and W, two buffers
 
+// Kinds of instruction for the compiler's scheduler, and a hint for it: the next COUNT matrix
+// products with one instruction of KIND behind each.
+constexpr int kMfma = 0x008, kVmemRead = 0x020, kDsRead = 0x100, kDsWrite = 0x200;
+template <int KIND, int COUNT>
+__device__ __forceinline__ void deal_between_products() {
+#pragma unroll
+    for (int i = 0; i < COUNT; ++i) {
+        __builtin_amdgcn_sched_group_barrier(kMfma, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(KIND, 1, 0);
+    }
+}
+
 // kGatedBF16: w holds gate and up rows interleaved in groups of 16, so that even MFMA tile
 // columns are gates and odd ones the ups of the same 16 units; out [M, N / 2] bfloat16 gets
 // silu(gate) * up (src/engine.cpp:213-216).
@@ -173,20 +185,27 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
             for (int j = 0; j < WNT; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
     };
+    // Within a half, the compiler is told to deal the memory instructions out between the
+    // products, one after each: a wavefront then uses LDS, the loads' path and the matrix pipe at
+    // the same time all along, instead of in phases that the two workgroups of a compute unit
+    // fall into together (measured: in phases, a call took the sum of the four pipes' times).
     auto turn = [&](int kt, int buf, Slab& next) {
         // (the store and the loads also on the last turn, where nobody uses them: a turn without
         // them would make the number of loads in flight depend on the path taken)
-        store_lds(buf ^ 1, next);
-        load_global(kt + 3, next);
         bf16x8 fa1[WMT], fw1[WNT];
         read_frags(buf, 1, fa1, fw1);
-        __builtin_amdgcn_sched_barrier(0);
+        store_lds(buf ^ 1, next);
         multiply(fa0, fw0);
+        deal_between_products<kDsRead, (WMT * WNT) / 2>();
+        deal_between_products<kDsWrite, (WMT * WNT) / 2>();
         __builtin_amdgcn_sched_barrier(0);            // (the products stay in front of the barrier)
         lds_barrier();
         read_frags(buf ^ 1, 0, fa0, fw0);
-        __builtin_amdgcn_sched_barrier(0);
+        load_global(kt + 3, next);
         multiply(fa1, fw1);
+        deal_between_products<kDsRead, (WMT * WNT) / 2>();
+        deal_between_products<kVmemRead, (WMT * WNT) / 2>();
+        __builtin_amdgcn_sched_barrier(0);
     };
     if (kt_begin < kt_end) {
         Slab s0, s1;
