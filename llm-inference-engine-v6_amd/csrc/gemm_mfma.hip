@@ -478,7 +478,7 @@ using namespace llme;
 // accumulate (float32 only) adds into out. gated: w holds gate and up rows interleaved in
 // groups of 16 and out is bfloat16 [M, N / 2] = silu(gate) * up (tile kernel only).
 // nw, ksplit: 0 lets the entry point choose the skinny kernel's wavefronts per workgroup and
-// the split over k; tile_shape: 0 chooses, 64 / 128 / 256 force the tile kernel with that tile
+// the split over k; tile_shape: 0 chooses, 64 / 128 force the tile kernel with that tile
 // edge also for small M (for tests and measurements).
 extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
                               int accumulate, int gated, int nw, int ksplit, int tile_shape, hipStream_t stream) {
@@ -568,7 +568,6 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     }
     if (tile_shape == 128096) return launch_tile<4, 3>(A, W, out, M, N, K, mode, ksplit, stream);
     if (tile_shape == 128064) return launch_tile<4, 2>(A, W, out, M, N, K, mode, ksplit, stream);
-    if (tile_shape == 256) return launch_tile<8, 8>(A, W, out, M, N, K, mode, ksplit, stream);
     if (tile_shape == 128) return launch_tile<4, 4>(A, W, out, M, N, K, mode, ksplit, stream);
     if (tile_shape == 64) return launch_tile<2, 2>(A, W, out, M, N, K, mode, ksplit, stream);
     return kErrBadArgument;

@@ -27,7 +27,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
               gated: bool = False, waves: int = 0, ksplit: int = 0, tile: int = 0, force_tile: bool = False) -> None:
     """bfloat16 a [M, K] and w [N, K] -> out [M, N] (float32 or bfloat16), 32-bit accumulation.
     K must be a multiple of 8. gated: w holds gate and up rows interleaved in groups of 16 and
-    out is bfloat16 [M, N / 2] = silu(gate) * up. waves / ksplit / tile (64, 128, 256) /
+    out is bfloat16 [M, N / 2] = silu(gate) * up. waves / ksplit / tile (64, 128, 128096, 128064) /
     force_tile override the launch choices (tests and measurements)."""
     require(a, "a", torch.bfloat16, (None, None))
     M, K = a.shape

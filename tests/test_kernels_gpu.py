@@ -249,7 +249,7 @@ def test_gemm_skinny(ops, M, N, K, waves, ksplit):
 
 @pytest.mark.parametrize("M,N,K", [(65, 128, 64), (128, 128, 128), (200, 331, 144), (129, 100, 176), (257, 500, 72),
                                    (2048, 3072, 2048), (1000, 2048, 8192), (7, 40, 24)])
-@pytest.mark.parametrize("tile", [64, 128, 256])
+@pytest.mark.parametrize("tile", [64, 128, 128096, 128064])
 def test_gemm_tile(ops, M, N, K, tile):
     a, w, ref = _bf16_pair(M, N, K, 30)
     out = torch.full((M, N), 3.0, device=DEV)
@@ -269,7 +269,7 @@ def test_gemm_tile(ops, M, N, K, tile):
 
 
 @pytest.mark.parametrize("T,FF,K,tile", [(5, 176, 64, 0), (130, 256, 96, 64), (300, 208, 144, 128), (2048, 8192, 2048, 0),
-                                         (257, 320, 128, 256), (64, 8192, 2048, 0)])
+                                         (257, 320, 128, 128096), (190, 352, 72, 128064), (64, 8192, 2048, 0)])
 def test_gemm_gated(ops, T, FF, K, tile):
     x = torch.randn(T, K, generator=_gen(33)).to(torch.bfloat16)
     wg = (0.1 * torch.randn(FF, K, generator=_gen(34))).to(torch.bfloat16)
