@@ -225,6 +225,84 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
     }
 }
 
+// The same for many tokens (prompts): a workgroup takes 16 consecutive tokens. Where they are 16
+// consecutive positions of one request that begin at a multiple of 16 (the usual case in a
+// prompt: they then lie in one page, whose size is a multiple of 16), a thread writes the 16
+// values of one v dim as one contiguous piece; otherwise value by value as above. ROPE_PARTS
+// workgroups share a group's work so that a prompt of a few thousand tokens fills the chip.
+constexpr int ROPE_GROUP = 16, ROPE_PARTS = 4;
+template <typename TQ, typename TC>
+__global__ __launch_bounds__(256) void rope_kv_write_group_kernel(
+    const float* __restrict__ qkv, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ positions, const int* __restrict__ seq_idx, const int* __restrict__ block_table,
+    int max_blocks, TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache, int n_q, int n_kv,
+    int hd, int page, int write_cache, int T) {
+    const int t0 = blockIdx.x * ROPE_GROUP;
+    const int nt = T - t0 < ROPE_GROUP ? T - t0 : ROPE_GROUP;
+    const int first = blockIdx.y * blockDim.x + threadIdx.x, stride = gridDim.y * blockDim.x;   // the group's work is dealt to gridDim.y workgroups
+    const int half = hd / 2, hv = half / 8;
+    const size_t row_len = static_cast<size_t>(n_q + 2 * n_kv) * hd;
+    const int q_items = n_q * hv, k_items = write_cache ? n_kv * hv : 0;
+    const int per_token = q_items + k_items;
+    for (int it = first; it < nt * per_token; it += stride) {
+        const int t = t0 + it / per_token, e0 = it % per_token;
+        const bool is_q = e0 < q_items;
+        const int e = is_q ? e0 : e0 - q_items;
+        const int h = e / hv, i = (e % hv) * 8;
+        const int pos = positions[t];
+        const float* src = qkv + t * row_len + (is_q ? 0 : n_q * hd) + h * hd + i;
+        float a[8], b[8], c[8], sv[8], lo[8], hi[8];
+        load8(src, a);
+        load8(src + half, b);
+        load8(cos_t + static_cast<size_t>(pos) * half + i, c);
+        load8(sin_t + static_cast<size_t>(pos) * half + i, sv);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            lo[j] = a[j] * c[j] - b[j] * sv[j];
+            hi[j] = b[j] * c[j] + a[j] * sv[j];
+        }
+        if (is_q) {
+            TQ* dst = q_out + (static_cast<size_t>(t) * n_q + h) * hd + i;
+            store8<TQ>(dst, lo);
+            store8<TQ>(dst + half, hi);
+        } else {
+            const int pg = block_table[static_cast<size_t>(seq_idx[t]) * max_blocks + pos / page];
+            TC* dst = k_cache + ((static_cast<size_t>(pg) * n_kv + h) * page + pos % page) * hd + i;
+            store8<TC>(dst, lo);
+            store8<TC>(dst + half, hi);
+        }
+    }
+    if (!write_cache) return;
+    const int v_dims = n_kv * hd;
+    const float* vsrc = qkv + t0 * row_len + static_cast<size_t>(n_q + n_kv) * hd;
+    const int pos0 = positions[t0];
+    const bool together = nt == ROPE_GROUP && seq_idx[t0] == seq_idx[t0 + ROPE_GROUP - 1] &&
+                          pos0 % ROPE_GROUP == 0 && page % ROPE_GROUP == 0;    // the same for the whole workgroup
+    if (together) {
+        const int pg = block_table[static_cast<size_t>(seq_idx[t0]) * max_blocks + pos0 / page];
+        const int off0 = pos0 % page;
+        for (int e = first; e < v_dims; e += stride) {
+            float lo[8], hi[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                lo[j] = vsrc[j * row_len + e];
+                hi[j] = vsrc[(j + 8) * row_len + e];
+            }
+            TC* dst = v_cache + ((static_cast<size_t>(pg) * n_kv + e / hd) * hd + e % hd) * page + off0;
+            store8<TC>(dst, lo);
+            store8<TC>(dst + 8, hi);
+        }
+    } else {
+        for (int it = first; it < nt * v_dims; it += stride) {
+            const int tt = it / v_dims, e = it % v_dims;
+            const int pos = positions[t0 + tt];
+            const int pg = block_table[static_cast<size_t>(seq_idx[t0 + tt]) * max_blocks + pos / page];
+            v_cache[((static_cast<size_t>(pg) * n_kv + e / hd) * hd + e % hd) * page + pos % page] =
+                from_float<TC>(vsrc[tt * row_len + e]);
+        }
+    }
+}
+
 }  // namespace llme
 
 using namespace llme;
@@ -287,9 +365,17 @@ extern "C" int llme_rope_kv_write(const float* qkv, const float* cos_t, const fl
                      reinterpret_cast<uintptr_t>(qkv) % 16 == 0 && reinterpret_cast<uintptr_t>(q_out) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(cos_t) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(sin_t) % 16 == 0;
+    // many tokens: 16 per workgroup, v written in pieces of 16 positions where they lie together
+    const bool grouped = vec && T >= 4 * ROPE_GROUP && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
 #define LLME_ROPE(TQ, TC)                                                                                   \
     do {                                                                                                    \
-        if (vec)                                                                                            \
+        if (grouped)                                                                                        \
+            hipLaunchKernelGGL((rope_kv_write_group_kernel<TQ, TC>),                                       \
+                               dim3((T + ROPE_GROUP - 1) / ROPE_GROUP, ROPE_PARTS),                         \
+                               dim3(256), 0, stream, qkv, cos_t, sin_t, positions, seq_idx, block_table,    \
+                               max_blocks, static_cast<TQ*>(q_out), static_cast<TC*>(k_cache),              \
+                               static_cast<TC*>(v_cache), n_q, n_kv, hd, page, write_cache, T);             \
+        else if (vec)                                                                                       \
             hipLaunchKernelGGL((rope_kv_write_vec_kernel<TQ, TC>), dim3(T), dim3(256), 0, stream, qkv, cos_t, \
                                sin_t, positions, seq_idx, block_table, max_blocks, static_cast<TQ*>(q_out), \
                                static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), n_q, n_kv, hd, page,   \

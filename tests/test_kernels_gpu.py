@@ -525,3 +525,56 @@ def test_gemv_norm_rope(ops, M, n_q, n_kv, hd, K, page, grid):
         assert (kc[pg, :, off, :] - k_ref[m]).abs().max() < 8e-3 * scale
         assert (vc[pg, :, :, off] - v_ref[m]).abs().max() < 8e-3 * scale
     assert int((kc != 0).sum()) <= M * n_kv * hd and int((vc != 0).sum()) <= M * n_kv * hd   # nothing else written
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,page", [(4, 2, 64, 16), (3, 1, 128, 48), (6, 3, 80, 32), (2, 2, 16, 16)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_write_of_many_tokens(ops, n_q, n_kv, hd, page, dtype):
+    """Rotation and cache write for a step of many tokens (16 tokens per workgroup, v written in
+    pieces of 16 positions where they lie together in a page): portions that start at multiples
+    of 16, portions that do not, a request shorter than a group, and groups that span two
+    requests. Every written place of both caches is compared, and no other place is touched."""
+    ctx = [32, 5, 0, 48, 16]                      # tokens already cached
+    new = [40, 50, 3, 16, 33]                     # tokens of this step
+    T, S = sum(new), len(new)
+    g = _gen(71)
+    qkv = torch.randn(T, (n_q + 2 * n_kv) * hd, generator=g)
+    half = hd // 2
+    max_pos = max(c + n for c, n in zip(ctx, new))
+    inv = 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float64) * 2 / hd))
+    ang = torch.arange(max_pos, dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = torch.cos(ang).float(), torch.sin(ang).float()
+    nblk = [(c + n + page - 1) // page for c, n in zip(ctx, new)]
+    total_pages = sum(nblk) + 3
+    perm = torch.randperm(total_pages, generator=g).tolist()
+    table = torch.zeros(S, max(nblk), dtype=torch.int32)
+    p = 0
+    for s, nb in enumerate(nblk):
+        for b in range(nb):
+            table[s, b] = perm[p]
+            p += 1
+    positions = torch.cat([torch.arange(c, c + n) for c, n in zip(ctx, new)]).to(torch.int32)
+    seq_idx = torch.cat([torch.full((n,), s) for s, n in enumerate(new)]).to(torch.int32)
+    mark = 7.0                                    # what the caches hold before
+    k_cache = torch.full((total_pages, n_kv, page, hd), mark, dtype=dtype, device=DEV)
+    v_cache = torch.full((total_pages, n_kv, hd, page), mark, dtype=dtype, device=DEV)
+    q_out = torch.empty(T, n_q * hd, dtype=dtype, device=DEV)
+    ops.rope_kv_write(qkv.to(DEV), cos.to(DEV), sin.to(DEV), positions.to(DEV), seq_idx.to(DEV), table.to(DEV),
+                      q_out, k_cache, v_cache, n_q, n_kv, hd, hd)
+    blk = qkv.double()
+    c2 = torch.cat([cos[positions.long()], cos[positions.long()]], dim=1).double()
+    s2 = torch.cat([sin[positions.long()], sin[positions.long()]], dim=1).double()
+    q = plain_apply_rope(blk[:, :n_q * hd].reshape(T, n_q, hd), c2, s2)
+    k = plain_apply_rope(blk[:, n_q * hd:(n_q + n_kv) * hd].reshape(T, n_kv, hd), c2, s2)
+    v = blk[:, (n_q + n_kv) * hd:].reshape(T, n_kv, hd)
+    tol = 2e-6 if dtype == torch.float32 else 4e-3
+    assert _rel(q_out.cpu().double(), q.reshape(T, -1)) < tol
+    k_ref = torch.full(k_cache.shape, mark, dtype=torch.float64)
+    v_ref = torch.full(v_cache.shape, mark, dtype=torch.float64)
+    for t in range(T):
+        pos, s = int(positions[t]), int(seq_idx[t])
+        pg, off = int(table[s, pos // page]), pos % page
+        k_ref[pg, :, off, :] = k[t]
+        v_ref[pg, :, :, off] = v[t]
+    assert float((k_cache.cpu().double() - k_ref).abs().max()) < tol * 8
+    assert float((v_cache.cpu().double() - v_ref).abs().max()) < tol * 8
