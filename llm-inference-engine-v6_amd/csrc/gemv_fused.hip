@@ -14,9 +14,9 @@
 // through tiles of 16 output columns (gated: the 16 gate and the 16 up rows of 16 units, which
 // lie next to each other in the interleaved weight matrix), TPR tiles at a time: NW / TPR
 // wavefronts share a tile, each streaming every (NW / TPR)-th 128-element chunk of k of the
-// tile's weight rows from HBM straight into MFMA operand registers, the next chunk's loads
-// issued before the current chunk's products; the partial sums are added through LDS, scaled
-// by inv_m and stored. The grid is sized so that the prologue is paid once per several tiles.
+// tile's weight rows from HBM straight into MFMA operand registers, four chunks ahead (two with 16
+// wavefronts), also across tiles; the partial sums are added through LDS, scaled by inv_m and stored. The grid
+// is sized so that the prologue is paid once per several tiles.
 //
 // A third form serves the attention's q/k/v projection: its epilogue rotates q and k heads at
 // the rows' positions (pairs (i, i + hd/2), src/kernels.cpp:189-203) and writes q to the query
@@ -33,6 +33,7 @@ namespace llme {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
 
 constexpr int GV_U = 4;                 // 32-element k steps per chunk
 constexpr int GV_CHUNK = 32 * GV_U;     // 128
@@ -46,16 +47,22 @@ __device__ __forceinline__ bf16x8 gv_zero8() {
 
 enum Epilogue : int { kPlain = 0, kGated = 1, kRope = 2 };
 
-// Four neighbouring norm weights in one load (the entry point checks the vector's alignment).
-__device__ __forceinline__ void load_norm4(const float* p, float (&o)[4]) {
-    const float4 v = *reinterpret_cast<const float4*>(p);
-    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
-}
-__device__ __forceinline__ void load_norm4(const bf16* p, float (&o)[4]) {
-    const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+// Four neighbouring norm weights in one load (the entry point checks the vector's alignment),
+// kept as loaded until they are used: a conversion right behind the load would wait for it.
+template <typename T> struct Norm4;
+template <> struct Norm4<float> {
+    float4 v;
+    __device__ __forceinline__ void load(const float* p) { v = *reinterpret_cast<const float4*>(p); }
+    __device__ __forceinline__ void get(float (&o)[4]) const { o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; }
+};
+template <> struct Norm4<bf16> {
+    bf16x4 v;
+    __device__ __forceinline__ void load(const bf16* p) { v = *reinterpret_cast<const bf16x4*>(p); }
+    __device__ __forceinline__ void get(float (&o)[4]) const {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = static_cast<float>(v[i]);
-}
+        for (int i = 0; i < 4; ++i) o[i] = static_cast<float>(v[i]);
+    }
+};
 
 // What the rotating epilogue needs: where rows sit in their requests and where their pages are.
 struct RopeTarget {
@@ -80,6 +87,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
     static_assert(EPI != kRope || TPR == 2, "the rotating epilogue works on pairs of tiles");
     constexpr int NT = GATED ? 2 : 1;                   // weight fragments per k step
     constexpr int KS = NW / TPR;                        // wavefronts that share a tile, splitting k
+    constexpr int GV_DEPTH = NW > 8 ? 2 : 4;            // chunks of weights a wavefront has in flight (registers: 128 or 256)
     extern __shared__ __align__(16) unsigned char lds_raw[];
     const int XS = K + 8;                               // padded row of the activation tile (elements)
     bf16* xs = reinterpret_cast<bf16*>(lds_raw);                                    // [16][XS]
@@ -93,20 +101,32 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
     const int n_rows_w = GATED ? 2 * N : N;             // rows of the weight matrix
     const int n_chunks = (K + GV_CHUNK - 1) / GV_CHUNK;
 
-    // two sets of weight fragments, used in turn (named apart so that both stay in registers)
-    bf16x8 fwa[NT][GV_U], fwb[NT][GV_U];
-    auto load_w = [&](bf16x8 (&fw)[NT][GV_U], int tile, int chunk) {
+    // The weights come by buffer loads: one descriptor over the whole matrix, a 32-bit byte offset
+    // per lane. A tile or chunk that does not exist gets an offset behind the descriptor's end:
+    // such a load returns zeros and fetches nothing, so loads can be issued without a condition.
+    // (The matrix is smaller than 4 GB: the entry points check it.)
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16*>(w), 0, static_cast<unsigned>(static_cast<size_t>(n_rows_w) * K * 2), 0x00020000);
+    constexpr unsigned kNowhere = 0xFFFFFFF0u;
+    // GV_DEPTH sets of weight fragments, in use one after the other
+    bf16x8 fw[GV_DEPTH][NT][GV_U];
+    auto load_w = [&](bf16x8 (&f)[NT][GV_U], int tile, int chunk) {
         // weight rows of this lane: plain: n = 16 tile + r; gated: gate row 32 tile + r, up row 16 further
         const int wr0 = GATED ? tile * 32 + r : tile * 16 + r;
         const int k0 = chunk * GV_CHUNK;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
-            const bool w_ok = tile < tiles && (wr0 + 16 * t) < n_rows_w;
-            const bf16* wp = w + static_cast<size_t>(w_ok ? wr0 + 16 * t : 0) * K + q * 8;
+            const bool w_ok = tile < tiles && chunk < n_chunks && (wr0 + 16 * t) < n_rows_w;
+            const unsigned base = (static_cast<unsigned>(wr0 + 16 * t) * K + q * 8) * 2;
 #pragma unroll
             for (int u = 0; u < GV_U; ++u) {
                 const int kk = k0 + u * 32;
-                fw[t][u] = (w_ok && (kk + q * 8) < K) ? *reinterpret_cast<const bf16x8*>(wp + kk) : gv_zero8();
+                // (all ones or zero, and the offset put together from both: written as a condition, the
+                // compiler made two loads under a branch out of it, with a wait for everything between)
+                const unsigned in = 0u - static_cast<unsigned>(w_ok && (kk + q * 8) < K);
+                const unsigned off = ((base + static_cast<unsigned>(kk) * 2) & in) | (kNowhere & ~in);
+                const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, off, 0, 0);
+                f[t][u] = __builtin_bit_cast(bf16x8, v);
             }
         }
     };
@@ -122,35 +142,77 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
         return item * TPR + slot;
     };
     const int items = (EPI == kRope) ? tiles / 2 : (tiles + TPR - 1) / TPR;
-    if (kpart < n_chunks) load_w(fwa, tile_of(blockIdx.x), kpart);       // in flight during the norm prologue
-
+    // A wavefront's work in order: unit j is chunk kpart + (j % cpw) KS of the tile of round j / cpw.
+    // Every wavefront has the same number of units (chunks past the end of k are zeros that cost
+    // nothing), GV_DEPTH of them in flight: a unit's loads are issued GV_DEPTH units ahead, also
+    // across rounds and before the prologue, so that the trip to memory is waited for once and not
+    // once per chunk.
+    const int rounds = (items + gridDim.x - 1) / gridDim.x;
+    const int cpw = (n_chunks + KS - 1) / KS;
+    const int units = rounds * cpw;
+    auto unit_tile = [&](int j) { return j < units ? tile_of((j / cpw) * gridDim.x + blockIdx.x) : tiles; };
+    auto unit_chunk = [&](int j) { return kpart + (j % cpw) * KS; };
     // ---- prologue: xs[m][k] = bf16(w_norm[k] * h[row(m)][k]); ssum[m] = sum_k h^2 ----
     // Rows m >= M stay as they are: a product's row m depends on activation row m alone, and
     // the results of the rows that do not exist are never stored.
-    for (int m = wave; m < M; m += NW) {
-        bf16* xrow = xs + static_cast<size_t>(m) * XS;
+    // A row's loads are asked for eight at a time (one after the other, each trip to memory took
+    // as long as the row's whole share of the products), and the first row's before the first
+    // weights: loads come back in the order they were asked for, and the weights' come from far.
+    constexpr int PU = 8;
+    float4 hv[PU];
+    Norm4<TNW> nw4[PU];
+    auto ask = [&](int m, int kb) {
         const float* hrow = h + static_cast<size_t>(rows ? rows[m] : m) * K;
-        float ss = 0.f;
-        for (int k = lane * 4; k < K; k += 64 * 4) {      // K % 8 == 0: whole groups of 4
-            const float4 v = *reinterpret_cast<const float4*>(hrow + k);
-            float nw4[4];
-            load_norm4(norm_w + k, nw4);
-            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-            bf16x4 o;
-            o[0] = static_cast<__bf16>(nw4[0] * v.x);
-            o[1] = static_cast<__bf16>(nw4[1] * v.y);
-            o[2] = static_cast<__bf16>(nw4[2] * v.z);
-            o[3] = static_cast<__bf16>(nw4[3] * v.w);
-            *reinterpret_cast<bf16x4*>(xrow + k) = o;
+#pragma unroll
+        for (int u = 0; u < PU; ++u) {
+            const int k = kb + u * 64 * 4;
+            const int ks = k < K ? k : 0;                          // past the row: a place that exists
+            hv[u] = *reinterpret_cast<const float4*>(hrow + ks);
+            nw4[u].load(norm_w + ks);
+        }
+    };
+    auto take = [&](int m, int kb, float& ss) {
+        bf16* xrow = xs + static_cast<size_t>(m) * XS;
+#pragma unroll
+        for (int u = 0; u < PU; ++u) {
+            const int k = kb + u * 64 * 4;
+            if (k < K) {                                           // K % 8 == 0: whole groups of 4
+                float nw[4];
+                nw4[u].get(nw);
+                ss += hv[u].x * hv[u].x + hv[u].y * hv[u].y + hv[u].z * hv[u].z + hv[u].w * hv[u].w;
+                bf16x4 o;
+                o[0] = static_cast<__bf16>(nw[0] * hv[u].x);
+                o[1] = static_cast<__bf16>(nw[1] * hv[u].y);
+                o[2] = static_cast<__bf16>(nw[2] * hv[u].z);
+                o[3] = static_cast<__bf16>(nw[3] * hv[u].w);
+                *reinterpret_cast<bf16x4*>(xrow + k) = o;
+            }
+        }
+    };
+    if (wave < M) ask(wave, lane * 4);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int d = 0; d < GV_DEPTH; ++d) load_w(fw[d], unit_tile(d), unit_chunk(d));   // in flight during the prologue
+    __builtin_amdgcn_sched_barrier(0);
+    // (the first eight loads of the first row are taken apart from the loop: only straight-line
+    // code lets the compiler count that the weights' loads, asked for later, may stay in flight)
+    float ss_first = 0.f;
+    if (wave < M) take(wave, lane * 4, ss_first);
+    for (int m = wave; m < M; m += NW) {
+        const bool first = m == wave;
+        float ss = first ? ss_first : 0.f;
+        for (int kb = lane * 4 + (first ? 64 * 4 * PU : 0); kb < K; kb += 64 * 4 * PU) {
+            ask(m, kb);
+            take(m, kb, ss);
         }
         ss = wave_sum(ss);
         if (lane == 0) ssum[m] = ss;
     }
-    __syncthreads();
+    lds_barrier();                                      // (waits for LDS only: the weights stay in flight)
 
     const bf16* xlane = xs + static_cast<size_t>(r) * XS + q * 8;      // row m = r of the activation tile
     f32x4 acc[NT];
-    auto multiply = [&](const bf16x8 (&fw)[NT][GV_U], int chunk) {
+    auto multiply = [&](const bf16x8 (&f)[NT][GV_U], int chunk) {
         const int k0 = chunk * GV_CHUNK;
 #pragma unroll
         for (int u = 0; u < GV_U; ++u) {
@@ -158,29 +220,18 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
             const bf16x8 fx = ((kk + q * 8) < K) ? *reinterpret_cast<const bf16x8*>(xlane + kk) : gv_zero8();
 #pragma unroll
             for (int t = 0; t < NT; ++t)
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[t][u], fx, acc[t], 0, 0, 0);
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f[t][u], fx, acc[t], 0, 0, 0);
         }
     };
 
-    const int rounds = (items + gridDim.x - 1) / gridDim.x;
-    for (int round = 0; round < rounds; ++round) {
-        const int item = round * gridDim.x + blockIdx.x;
-        const int tile = tile_of(item);
-        if (round > 0 && kpart < n_chunks) load_w(fwa, tile, kpart);
 #pragma unroll
-        for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-        for (int chunk = kpart; chunk < n_chunks;) {
-            if (chunk + KS < n_chunks) load_w(fwb, tile, chunk + KS);
-            multiply(fwa, chunk);
-            chunk += KS;
-            if (chunk >= n_chunks) break;
-            if (chunk + KS < n_chunks) load_w(fwa, tile, chunk + KS);
-            multiply(fwb, chunk);
-            chunk += KS;
-        }
+    for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // the end of a round: the sums are added up, scaled and stored (further down)
+    auto finish_round = [&](int round) {
+        const int tile = tile_of(round * gridDim.x + blockIdx.x);
 #pragma unroll
         for (int t = 0; t < NT; ++t) red[(wave * NT + t) * 64 + lane] = acc[t];
-        __syncthreads();
+        lds_barrier();
         // the first wavefront of each tile adds up: lane l holds row m = l % 16, columns 4 (l / 16) + e
         f32x4 s[NT];
         const int m = lane & 15;
@@ -203,7 +254,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
 #pragma unroll
                 for (int e = 0; e < 4; ++e) ex[(slot * 16 + m) * 16 + (lane >> 4) * 4 + e] = s[0][e] * inv;
             }
-            __syncthreads();
+            lds_barrier();
             if (leader && m < M) {
                 const int hd = rope.hd, half = hd / 2;
                 const int head = tile / tiles_per_head;                 // among q heads, then k heads, then v heads
@@ -250,7 +301,19 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
                 }
             }
         }
-        __syncthreads();
+        lds_barrier();
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    };
+    for (int j = 0; j < units; j += GV_DEPTH) {
+#pragma unroll
+        for (int d = 0; d < GV_DEPTH; ++d) {
+            if (j + d < units) {                        // the same for the whole workgroup
+                multiply(fw[d], unit_chunk(j + d));
+                if ((j + d) % cpw == cpw - 1) finish_round((j + d) / cpw);
+            }
+            load_w(fw[d], unit_tile(j + d + GV_DEPTH), unit_chunk(j + d + GV_DEPTH));
+        }
     }
 }
 
@@ -303,6 +366,7 @@ extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_
     if (static_cast<size_t>(16) * (K + 8) * 2 > 132 * 1024) return kErrUnsupported;
     if (gated && N % 16 != 0) return kErrUnsupported;
     const int tiles = (N + 15) / 16;
+    if (static_cast<double>(gated ? 2 * N : N) * K * 2 >= 4294967296.0) return kErrUnsupported;   // 32-bit offsets
     if (tpr <= 0) {
         // few tiles: all 8 wavefronts on one tile, so that every tile has a workgroup of its own;
         // more tiles than compute units: 2 tiles at a time, 4 wavefronts each with several chunks of k
@@ -341,6 +405,7 @@ extern "C" int llme_gemv_norm_rope(const float* h, const void* norm_w, int norm_
         return kErrUnsupported;
     if (static_cast<size_t>(16) * (K + 8) * 2 > 132 * 1024) return kErrUnsupported;
     const int N = (n_q + 2 * n_kv) * hd;
+    if (static_cast<double>(N) * K * 2 >= 4294967296.0) return kErrUnsupported;   // 32-bit offsets into w
     const int pairs = N / 32;
     if (grid <= 0) grid = pairs > 512 ? 512 : pairs;
     const RopeTarget rope{positions, seq_idx, block_table, max_blocks, cos_t, sin_t, static_cast<bf16*>(q_out),
