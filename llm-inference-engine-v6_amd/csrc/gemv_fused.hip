@@ -305,16 +305,24 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
 #pragma unroll
         for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     };
-    for (int j = 0; j < units; j += GV_DEPTH) {
+    auto work = [&](int d, int j) {
+        multiply(fw[d], unit_chunk(j));
+        if (j % cpw == cpw - 1) finish_round(j / cpw);
+    };
+    // While more than GV_DEPTH units are left, every unit done is followed by the loads of the unit
+    // GV_DEPTH further on (without a condition: the compiler's count of loads in flight stays exact;
+    // a unit past the end reads zeros). The last GV_DEPTH units are only worked on.
+    int j = 0;
+    for (; j + GV_DEPTH < units; j += GV_DEPTH) {
 #pragma unroll
         for (int d = 0; d < GV_DEPTH; ++d) {
-            if (j + d < units) {                        // the same for the whole workgroup
-                multiply(fw[d], unit_chunk(j + d));
-                if ((j + d) % cpw == cpw - 1) finish_round((j + d) / cpw);
-            }
+            work(d, j + d);
             load_w(fw[d], unit_tile(j + d + GV_DEPTH), unit_chunk(j + d + GV_DEPTH));
         }
     }
+#pragma unroll
+    for (int d = 0; d < GV_DEPTH; ++d)
+        if (j + d < units) work(d, j + d);                  // (the same for the whole workgroup)
 }
 
 template <int NW, int TPR, int EPI, typename TNW>
