@@ -125,7 +125,10 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
 }
 
 // joins the splits of the decode kernel: grid (request, head); lanes over the splits for the
-// statistics, then over the head's dimensions for the weighted sum. nsplit <= 64.
+// statistics, then over the head's dimensions for the weighted sum. nsplit <= 64. The partial
+// outputs are asked for 16 splits at a time, the first 16 together with the statistics: asked
+// for one after the other, the trips to memory were most of this small kernel's time.
+constexpr int JOIN_AT_A_TIME = 16;
 __global__ __launch_bounds__(64) void attention_join_kernel(const float* __restrict__ part_o,
                                                             const float* __restrict__ part_ml, bf16* __restrict__ out,
                                                             const int* __restrict__ q_start, int n_q, int hd, int nsplit) {
@@ -134,6 +137,15 @@ __global__ __launch_bounds__(64) void attention_join_kernel(const float* __restr
     const int row0 = q_start[s];
     if (q_start[s + 1] - row0 != 1) return;
     const size_t base = (static_cast<size_t>(s) * n_q + h) * nsplit;
+    float part[JOIN_AT_A_TIME];
+    auto ask = [&](int first, int d) {                 // (splits past the last: the last again, with weight 0)
+#pragma unroll
+        for (int u = 0; u < JOIN_AT_A_TIME; ++u) {
+            const int i = first + u < nsplit ? first + u : nsplit - 1;
+            part[u] = part_o[(base + i) * hd + (d < hd ? d : 0)];
+        }
+    };
+    ask(0, lane);
     float mi = -INFINITY, li = 0.f;
     if (lane < nsplit) {
         mi = part_ml[(base + lane) * 2];
@@ -142,17 +154,16 @@ __global__ __launch_bounds__(64) void attention_join_kernel(const float* __restr
     const float mx = wave_max(mi);
     const float f = (mi <= kNoMax) ? 0.f : exp2f(mi - mx);
     const float total = wave_sum(f * li);
-    weight[lane] = f / total;
+    weight[lane] = f / total;                          // 0 for lanes past the last split
     __syncthreads();
     for (int d = lane; d < hd; d += 64) {
         float acc = 0.f;
-        int i = 0;
-        for (; i + 4 <= nsplit; i += 4) {
-            const float a0 = part_o[(base + i) * hd + d], a1 = part_o[(base + i + 1) * hd + d];
-            const float a2 = part_o[(base + i + 2) * hd + d], a3 = part_o[(base + i + 3) * hd + d];
-            acc += weight[i] * a0 + weight[i + 1] * a1 + weight[i + 2] * a2 + weight[i + 3] * a3;
+        for (int first = 0; first < nsplit; first += JOIN_AT_A_TIME) {
+            if (d != lane || first != 0) ask(first, d);            // (the first are on their way)
+#pragma unroll
+            for (int u = 0; u < JOIN_AT_A_TIME; ++u)
+                acc += (first + u < nsplit ? weight[first + u] : 0.f) * part[u];
         }
-        for (; i < nsplit; ++i) acc += weight[i] * part_o[(base + i) * hd + d];
         out[(static_cast<size_t>(row0) * n_q + h) * hd + d] = static_cast<bf16>(acc);
     }
 }
