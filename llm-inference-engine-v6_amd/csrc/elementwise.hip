@@ -19,6 +19,28 @@ __global__ void embed_gather_kernel(const TW* __restrict__ table, const int* __r
     float* o = out + static_cast<size_t>(t) * H;
     for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_float(row[i]);
 }
+// The same with eight elements per thread and load (H a multiple of 8, 16-byte aligned rows).
+template <typename TW>
+__global__ void embed_gather_vec_kernel(const TW* __restrict__ table, const int* __restrict__ tokens,
+                                        float* __restrict__ out, int H) {
+    const int t = blockIdx.x;
+    const TW* row = table + static_cast<size_t>(tokens[t]) * H;
+    float* o = out + static_cast<size_t>(t) * H;
+    for (int i = threadIdx.x * 8; i < H; i += blockDim.x * 8) {
+        float v[8];
+        if constexpr (sizeof(TW) == 2) {
+            typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+            const bf16x8 x = *reinterpret_cast<const bf16x8*>(row + i);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = static_cast<float>(x[j]);
+        } else {
+            const float4 a = *reinterpret_cast<const float4*>(row + i), b = *reinterpret_cast<const float4*>(row + i + 4);
+            v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+        }
+        *reinterpret_cast<float4*>(o + i) = float4{v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<float4*>(o + i + 4) = float4{v[4], v[5], v[6], v[7]};
+    }
+}
 
 // ---------------------------------------------------------------------------------
 // out[r, i] = w[i] * x[row(r), i] * rsqrt(mean_i x^2 + eps)   (src/kernels.cpp:18-24)
@@ -310,14 +332,20 @@ using namespace llme;
 extern "C" int llme_embed_gather(const void* table, int table_dtype, const int* tokens, float* out, int T,
                                  int H, hipStream_t stream) {
     if (T <= 0) return 0;
-    if (table_dtype == kF32)
-        hipLaunchKernelGGL(embed_gather_kernel<float>, dim3(T), dim3(256), 0, stream,
-                           static_cast<const float*>(table), tokens, out, H);
-    else if (table_dtype == kBF16)
-        hipLaunchKernelGGL(embed_gather_kernel<bf16>, dim3(T), dim3(256), 0, stream,
-                           static_cast<const bf16*>(table), tokens, out, H);
-    else
-        return kErrBadArgument;
+    const bool vec = H % 8 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+#define LLME_EMBED(TW)                                                                                     \
+    do {                                                                                                   \
+        if (vec)                                                                                           \
+            hipLaunchKernelGGL(embed_gather_vec_kernel<TW>, dim3(T), dim3(256), 0, stream,                 \
+                               static_cast<const TW*>(table), tokens, out, H);                             \
+        else                                                                                               \
+            hipLaunchKernelGGL(embed_gather_kernel<TW>, dim3(T), dim3(256), 0, stream,                     \
+                               static_cast<const TW*>(table), tokens, out, H);                             \
+    } while (0)
+    if (table_dtype == kF32) LLME_EMBED(float);
+    else if (table_dtype == kBF16) LLME_EMBED(bf16);
+    else return kErrBadArgument;
+#undef LLME_EMBED
     return launch_status();
 }
 

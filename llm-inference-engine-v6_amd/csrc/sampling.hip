@@ -45,7 +45,21 @@ __global__ __launch_bounds__(kSampleThreads) void argmax_part_kernel(const float
     const int end = (begin + chunk < V) ? begin + chunk : V;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = begin + threadIdx.x; i < end; i += kSampleThreads) argmax_combine(bv, bi, row[i], i);
+    // eight loads at a time (asked for one by one, each waits for its own trip to memory)
+    constexpr int U = 8;
+    for (int i0 = begin + threadIdx.x; i0 < end; i0 += kSampleThreads * U) {
+        float v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * kSampleThreads;
+            v[u] = row[i < end ? i : end - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * kSampleThreads;
+            if (i < end) argmax_combine(bv, bi, v[u], i);
+        }
+    }
     block_argmax(bv, bi, sv, si);
     if (threadIdx.x == 0) {
         part_val[blockIdx.x * gridDim.y + blockIdx.y] = bv;

@@ -29,7 +29,8 @@ def ops():
     return ops
 
 
-@pytest.mark.parametrize("V,H,dtype", [(37, 50, torch.float32), (129, 96, torch.bfloat16)])
+@pytest.mark.parametrize("V,H,dtype", [(37, 50, torch.float32), (129, 96, torch.bfloat16), (64, 72, torch.float32),
+                                       (300, 2048, torch.bfloat16), (41, 100, torch.bfloat16)])
 def test_embed_gather(ops, V, H, dtype):
     table = torch.randn(V, H, generator=_gen(0)).to(dtype)
     tokens = torch.tensor([0, 1, 7, V - 1, 3, 3], dtype=torch.int32)
