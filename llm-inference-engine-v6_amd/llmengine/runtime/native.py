@@ -113,6 +113,7 @@ _lib = None
 _lock = threading.Lock()
 
 _vp, _i, _l, _i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_int64
+_f, _d = ctypes.c_float, ctypes.c_double
 _pi, _pl, _pi64 = ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_long), ctypes.POINTER(ctypes.c_int64)
 
 _SIGNATURES = {
@@ -136,6 +137,17 @@ _SIGNATURES = {
     "llme_sched_complete": (_i, [_vp, _pi, _i, _pi, _i]), "llme_sched_num_results": (_i, [_vp]),
     "llme_sched_result_info": (_i, [_vp, _i, _pi64, _pl, _pl, _pi]), "llme_sched_result_tokens": (_i, [_vp, _i, _pi]),
     "llme_sched_clear_results": (None, [_vp]),
+    # plain C++ twins of the device kernels (csrc/host/plain_kernels.cpp), for tests
+    "llme_plain_embed": (_i, [_vp, _vp, _i, _i, _i, _vp]),
+    "llme_plain_rmsnorm": (_i, [_vp, _vp, _i, _i, _f, _vp]),
+    "llme_plain_linear": (_i, [_vp, _vp, _i, _i, _i, _vp, _i]),
+    "llme_plain_swiglu": (_i, [_vp, _vp, ctypes.c_size_t, _vp]),
+    "llme_plain_inv_freq": (_i, [_i, _d, _i, _d, _d, _d, _d, _vp]),
+    "llme_plain_rope_tables": (_i, [_vp, _vp, _i, _i, _vp, _vp]),
+    "llme_plain_rope_apply": (_i, [_vp, _vp, _vp, _i, _i, _i]),
+    "llme_plain_attention": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "llme_plain_argmax": (_i, [_vp, _i]),
+    "llme_plain_sample": (_i, [_vp, _i, _f, _f]),
 }
 
 # codes of csrc/host/host_api.h
