@@ -14,6 +14,10 @@ run at the configured context length. One JSON line goes to stdout.
 `--shape 3b` and `--shape 8b` take the layer sizes of Llama 3.2 3B and Llama 3.1 8B instead (for
 measurements at further sizes and context lengths; the default run is the 1B shape).
 
+`--phase serve` is another workload (with `--shape 3b`: 32 requests with prompts of 64 to 3,072
+tokens and 128 to 512 new tokens each, 2,048 prompt tokens a step at most) through the
+continuous-batching scheduler, prompt portions beside decoded tokens in every step.
+
 Beside the headline value the line holds: `prefill` (one 2,048-token prompt, logits at its last
 place), `roofline` (bytes the decode step has to read: every weight once plus the live
 requests' cache, over its time, against 8 TB/s), `points` (decode at batch 1 and 64).
@@ -84,6 +88,55 @@ def prefill_flops(c: dict, T: int) -> float:
     return gemm + attn + head
 
 
+def serve(args, engine, cfg: dict, gen, page: int) -> int:
+    """Requests of mixed lengths through the continuous-batching scheduler: every step is one
+    mixed batch (prompt portions under the token budget beside one token of every decoding
+    request). The rate counts generated tokens over the wall time from the first step to the
+    last, host work included."""
+    import torch
+    from llmengine import BlockManager, ContinuousBatchScheduler
+
+    lo, hi = (int(x) for x in args.prompt_range.split(","))
+    nlo, nhi = (int(x) for x in args.new_range.split(","))
+    V = cfg["vocab_size"]
+    prompts = [torch.randint(0, V, (int(torch.randint(lo, hi + 1, (1,), generator=gen)),), generator=gen).tolist()
+               for _ in range(args.requests)]
+    news = [int(torch.randint(nlo, nhi + 1, (1,), generator=gen)) for _ in range(args.requests)]
+    pages = sum((len(p) + n + page - 1) // page for p, n in zip(prompts, news))
+    runs = []
+    for rep in range(2):                                       # the first run warms up (and records the graphs)
+        manager = BlockManager(pages, page)
+        sched = ContinuousBatchScheduler(engine, manager, max_concurrent=args.max_concurrent,
+                                         max_prefill_tokens_per_step=args.prefill_budget)
+        for p, n in zip(prompts, news):
+            sched.enqueue(p, n)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        sched.run_until_idle()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        results = sched.results
+        generated = sum(len(r.token_ids) - r.prompt_len for r in results)
+        reasons = sorted({r.finish_reason for r in results})
+        runs.append((dt, generated, sched.steps))
+        log(f"serve run {rep}: {len(results)} requests, {sum(map(len, prompts))} prompt tokens, {generated} generated "
+            f"in {dt:.2f} s over {sched.steps} steps ({generated / dt:.0f} generated tok/s; finished: {reasons})")
+        assert manager.free_blocks == pages, "pages were lost"
+        del sched, manager
+    dt, generated, steps = runs[-1]
+    prompt_tokens = sum(map(len, prompts))
+    print(json.dumps({
+        "metric": "serve_generated_tokens_per_second", "value": round(generated / dt, 1), "unit": "tokens/s",
+        "n_gpus": 1, "dtype": args.dtype, "seconds": round(dt, 3), "steps": steps,
+        "all_tokens_per_second": round((generated + prompt_tokens) / dt, 1),
+        "config": {"model": args.shape, "layers": cfg["num_hidden_layers"], "requests": args.requests,
+                   "prompt_range": args.prompt_range, "new_range": args.new_range, "prompt_tokens": prompt_tokens,
+                   "generated_tokens": generated, "prefill_budget": args.prefill_budget,
+                   "max_concurrent": args.max_concurrent, "page_size": page},
+    }), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -97,8 +150,14 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode"],
-                    help="run only one part (for profiling); the JSON line then lacks the other")
+    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode", "serve"],
+                    help="run only one part (for profiling); the JSON line then lacks the other. 'serve' is another "
+                         "workload: requests of mixed lengths through the continuous-batching scheduler")
+    ap.add_argument("--requests", type=int, default=32, help="serve: number of requests")
+    ap.add_argument("--prompt-range", default="64,3072", help="serve: prompt lengths, uniform in [a, b]")
+    ap.add_argument("--new-range", default="128,512", help="serve: new tokens per request, uniform in [a, b]")
+    ap.add_argument("--prefill-budget", type=int, default=2048, help="serve: max_prefill_tokens_per_step")
+    ap.add_argument("--max-concurrent", type=int, default=32, help="serve: live requests at a time")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -122,6 +181,9 @@ def main() -> int:
 
     def sync():
         torch.cuda.synchronize()
+
+    if args.phase == "serve":
+        return serve(args, engine, cfg, gen, page)
 
     # ---- prefill: one prompt, logits at its last place ----
     T = args.prefill_tokens
