@@ -39,6 +39,8 @@ def main(argv=None) -> int:
     ap.add_argument("--num-blocks", type=int, default=0, help="pages in the pool (0: enough for all requests)")
     ap.add_argument("--max-concurrent", type=int, default=64)
     ap.add_argument("--prefill-budget", type=int, default=256, help="max_prefill_tokens_per_step")
+    ap.add_argument("--max-context", type=int, default=None,
+                    help="lower the model's position limit (max_position_embeddings) to this")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args(argv)
 
@@ -51,7 +53,8 @@ def main(argv=None) -> int:
     if not prompts:
         ap.error("no prompts given")
 
-    kw = dict(device=args.device, temperature=args.temperature, sampler_seed=args.sampler_seed, block_size=args.block_size)
+    kw = dict(device=args.device, temperature=args.temperature, sampler_seed=args.sampler_seed, block_size=args.block_size,
+              max_context=args.max_context)
     if args.model:
         engine = Engine(args.model, args.dtype, **kw)
     else:

@@ -74,13 +74,21 @@ class BlockManager:
 class Engine:
     def __init__(self, model_dir: str | None, dtype: str = "fp32", *, device: str = "cuda:0",
                  max_prefill_tokens_per_step: int = 8192, temperature: float = 0.0, sampler_seed: int = 0,
-                 block_size: int = 16, use_graphs: bool = True, _config: dict | None = None, _tensors=None):
+                 block_size: int = 16, use_graphs: bool = True, max_context: int | None = None,
+                 _config: dict | None = None, _tensors=None):
         self._dtype_name = {"float32": "fp32", "bfloat16": "bf16"}.get(dtype, dtype)
         self._torch_dtype = parse_dtype(dtype)
         if _config is None:
             cfg_dict, gen = read_model_json(model_dir)
         else:
             cfg_dict, gen = _config, None
+        if max_context is not None:
+            # the position limit may be lowered (never raised): the rotation table is built that far
+            if int(max_context) < 1:
+                raise ValueError("Engine: max_context must be >= 1")
+            have = cfg_dict.get("max_position_embeddings")
+            if isinstance(have, int) and have > int(max_context):
+                cfg_dict = dict(cfg_dict, max_position_embeddings=int(max_context))
         self.model_dir = model_dir
         self._cfg_dict = cfg_dict
         self._arch = resolve(architecture_name(cfg_dict))

@@ -87,3 +87,14 @@ def test_registering_another_architecture():
 def test_missing_config_file(tmp_path):
     with pytest.raises(ConfigError):
         load_config(str(tmp_path))
+
+
+def test_engine_max_context_lowers_the_position_limit_only():
+    from llmengine import Engine
+    assert Engine.from_random(TINY_A, 0, "fp32").max_pos == TINY_A["max_position_embeddings"]
+    assert Engine.from_random(TINY_A, 0, "fp32", max_context=40).max_pos == 40
+    assert Engine.from_random(TINY_A, 0, "fp32", max_context=10 ** 6).max_pos == TINY_A["max_position_embeddings"]
+    with pytest.raises(ValueError):
+        Engine.from_random(TINY_A, 0, "fp32", max_context=0)
+    with pytest.raises(RuntimeError, match="max_pos"):
+        Engine.from_random(TINY_A, 0, "fp32", max_context=8).generate([1, 2, 3, 4, 5], 8)
