@@ -42,6 +42,26 @@ __global__ void embed_gather_vec_kernel(const TW* __restrict__ table, const int*
     }
 }
 
+// The same from a bfloat16 table in the matrix kernels' blocked layout ([V / 16][H / 32] blocks of
+// [4][16][8], V a multiple of 16 and H of 32): the head that is tied to the embedding reads the
+// table as a weight matrix. A row's eight values of k = 8 j .. 8 j + 7 lie together.
+__global__ void embed_gather_blocked_kernel(const bf16* __restrict__ table, const int* __restrict__ tokens,
+                                            float* __restrict__ out, int H) {
+    typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+    const int t = blockIdx.x;
+    const int row = tokens[t];
+    const bf16* group = table + static_cast<size_t>(row / 16) * 16 * H + (row % 16) * 8;
+    float* o = out + static_cast<size_t>(t) * H;
+    for (int j = threadIdx.x; j < H / 8; j += blockDim.x) {
+        const bf16x8 x = *reinterpret_cast<const bf16x8*>(group + static_cast<size_t>(j / 4) * 512 + (j % 4) * 128);
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = static_cast<float>(x[e]);
+        *reinterpret_cast<float4*>(o + j * 8) = float4{v[0], v[1], v[2], v[3]};
+        *reinterpret_cast<float4*>(o + j * 8 + 4) = float4{v[4], v[5], v[6], v[7]};
+    }
+}
+
 // ---------------------------------------------------------------------------------
 // out[r, i] = w[i] * x[row(r), i] * rsqrt(mean_i x^2 + eps)   (src/kernels.cpp:18-24)
 // row(r) = rows ? rows[r] : r. The product is evaluated (w*x)*inv as the reference does.
@@ -330,8 +350,16 @@ __global__ __launch_bounds__(256) void rope_kv_write_group_kernel(
 using namespace llme;
 
 extern "C" int llme_embed_gather(const void* table, int table_dtype, const int* tokens, float* out, int T,
-                                 int H, hipStream_t stream) {
+                                 int H, int blocked, hipStream_t stream) {
     if (T <= 0) return 0;
+    if (blocked) {
+        if (table_dtype != kBF16 || H % 32 != 0 || reinterpret_cast<uintptr_t>(table) % 16 != 0 ||
+            reinterpret_cast<uintptr_t>(out) % 16 != 0)
+            return kErrUnsupported;
+        hipLaunchKernelGGL(embed_gather_blocked_kernel, dim3(T), dim3(256), 0, stream, static_cast<const bf16*>(table),
+                           tokens, out, H);
+        return launch_status();
+    }
     const bool vec = H % 8 == 0 && reinterpret_cast<uintptr_t>(table) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
 #define LLME_EMBED(TW)                                                                                     \
     do {                                                                                                   \

@@ -19,6 +19,12 @@
 //
 // K must be a multiple of 8 and all pointers 16-byte aligned (checked by the caller);
 // M and N are arbitrary: rows and columns past the edge are loaded as zeros and not stored.
+//
+// W comes row-major or blocked: [N / 16][K / 32] blocks of 1 KB, a block holding its 16 rows x
+// 32 k in the order of the instruction's operand, [4 q][16 r][8] (N a multiple of 16, K of 32).
+// A wavefront's load of an operand is then 1 KB of consecutive addresses, which is what lets
+// the skinny kernel stream weights a quarter faster; the tile kernel reads the same layout,
+// a slab of a tile being whole blocks, and puts it into LDS as rows as before.
 #include "common.h"
 
 namespace llme {
@@ -69,7 +75,7 @@ __device__ __forceinline__ void deal_between_products() {
 // kGatedBF16: w holds gate and up rows interleaved in groups of 16, so that even MFMA tile
 // columns are gates and odd ones the ups of the same 16 units; out [M, N / 2] bfloat16 gets
 // silu(gate) * up (src/engine.cpp:213-216).
-template <int WMT, int WNT, int MODE, bool KFULL>
+template <int WMT, int WNT, int MODE, bool KFULL, bool BLOCKED>
 __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w,
                                                         void* __restrict__ out, int M, int N, int K,
                                                         int tiles_m, int tiles_n, int ksplit) {
@@ -126,6 +132,18 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
     for (int i = 0; i < CA; ++i) aoff[i] = (static_cast<unsigned>(crow + 32 * i) * K + ckq) * 2;
 #pragma unroll
     for (int i = 0; i < CW; ++i) woff[i] = (static_cast<unsigned>(crow + 32 * i) * K + ckq) * 2;
+    // Blocked W: a slab of the tile is (BN / 16) row groups x 2 blocks of 1 KB; chunk c = 256 i + t of
+    // the slab is piece c % 64 of block (c % 128) / 64 of row group c / 128, so that a wavefront's
+    // load is one whole block. In LDS the piece goes to row 16 (c / 128) + c % 16, k 32 (block) + 8 (c % 64 / 16).
+    int w_lds[CW];                                    // elements from the slab's W buffer
+    if (BLOCKED) {
+#pragma unroll
+        for (int i = 0; i < CW; ++i) {
+            const int c = 256 * i + tid, group = c / 128, kb = (c % 128) / 64, piece = c % 64;
+            woff[i] = (static_cast<unsigned>(group) * (K / 32) + kb) * 1024u + piece * 16u;
+            w_lds[i] = (group * 16 + piece % 16) * TSTRIDE + kb * 32 + (piece / 16) * 8;
+        }
+    }
     struct Slab {
         u32x4 ra[CA], rw[CW];
     };
@@ -135,13 +153,17 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
 #pragma unroll
         for (int i = 0; i < CA; ++i) s.ra[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, aoff[i], k * 2, 0);
 #pragma unroll
-        for (int i = 0; i < CW; ++i) s.rw[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, woff[i], k * 2, 0);
+        for (int i = 0; i < CW; ++i)                  // (blocked: a slab is two blocks further in every row group)
+            s.rw[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, woff[i], BLOCKED ? kt * 2048 : k * 2, 0);
         if (!KFULL) {                                 // K is a multiple of 8: a chunk is in or out whole
             const bool ok = k + ckq < K;
 #pragma unroll
             for (int i = 0; i < CA; ++i) s.ra[i] = ok ? s.ra[i] : u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
-            for (int i = 0; i < CW; ++i) s.rw[i] = ok ? s.rw[i] : u32x4{0u, 0u, 0u, 0u};
+            for (int i = 0; i < CW; ++i) {
+                const bool w_ok = BLOCKED ? k + ((256 * i + tid) % 128) / 64 * 32 < K : ok;   // (a block is in or out whole)
+                s.rw[i] = w_ok ? s.rw[i] : u32x4{0u, 0u, 0u, 0u};
+            }
         }
     };
     auto store_lds = [&](int buf, const Slab& s) {
@@ -150,7 +172,8 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
 #pragma unroll
         for (int i = 0; i < CA; ++i) *reinterpret_cast<u32x4*>(sA + (crow + 32 * i) * TSTRIDE + ckq) = s.ra[i];
 #pragma unroll
-        for (int i = 0; i < CW; ++i) *reinterpret_cast<u32x4*>(sW + (crow + 32 * i) * TSTRIDE + ckq) = s.rw[i];
+        for (int i = 0; i < CW; ++i)
+            *reinterpret_cast<u32x4*>(sW + (BLOCKED ? w_lds[i] : (crow + 32 * i) * TSTRIDE + ckq)) = s.rw[i];
     };
 
     f32x4 acc[WMT][WNT];
@@ -348,26 +371,33 @@ static int launch_tile_kernel(int LDS, int BM, int BN, const bf16* A, const bf16
     return launch_status();
 }
 
-template <int WMT, int WNT, int MODE>
-static int launch_tile_mode(const bf16* A, const bf16* W, void* out, int M, int N, int K, int ksplit,
-                            hipStream_t stream) {
+template <int WMT, int WNT, int MODE, bool BLOCKED>
+static int launch_tile_layout(const bf16* A, const bf16* W, void* out, int M, int N, int K, int ksplit,
+                              hipStream_t stream) {
     constexpr int LDS = tile_lds_bytes<WMT, WNT>();
     if (K % TK != 0)
-        return launch_tile_kernel<gemm_tile_kernel<WMT, WNT, MODE, false>>(LDS, 32 * WMT, 32 * WNT, A, W, out, M, N, K,
-                                                                           ksplit, stream);
-    return launch_tile_kernel<gemm_tile_kernel<WMT, WNT, MODE, true>>(LDS, 32 * WMT, 32 * WNT, A, W, out, M, N, K,
-                                                                      ksplit, stream);
+        return launch_tile_kernel<gemm_tile_kernel<WMT, WNT, MODE, false, BLOCKED>>(LDS, 32 * WMT, 32 * WNT, A, W, out,
+                                                                                    M, N, K, ksplit, stream);
+    return launch_tile_kernel<gemm_tile_kernel<WMT, WNT, MODE, true, BLOCKED>>(LDS, 32 * WMT, 32 * WNT, A, W, out, M,
+                                                                               N, K, ksplit, stream);
+}
+
+template <int WMT, int WNT, int MODE>
+static int launch_tile_mode(const bf16* A, const bf16* W, void* out, int M, int N, int K, int ksplit, int blocked,
+                            hipStream_t stream) {
+    if (blocked) return launch_tile_layout<WMT, WNT, MODE, true>(A, W, out, M, N, K, ksplit, stream);
+    return launch_tile_layout<WMT, WNT, MODE, false>(A, W, out, M, N, K, ksplit, stream);
 }
 
 template <int WMT, int WNT>
 static int launch_tile(const bf16* A, const bf16* W, void* out, int M, int N, int K, int mode, int ksplit,
-                       hipStream_t stream) {
+                       int blocked, hipStream_t stream) {
     switch (mode) {
-        case kStoreF32: return launch_tile_mode<WMT, WNT, kStoreF32>(A, W, out, M, N, K, 1, stream);
-        case kAddF32: return launch_tile_mode<WMT, WNT, kAddF32>(A, W, out, M, N, K, 1, stream);
-        case kAtomicF32: return launch_tile_mode<WMT, WNT, kAtomicF32>(A, W, out, M, N, K, ksplit, stream);
-        case kGatedBF16: return launch_tile_mode<WMT, WNT, kGatedBF16>(A, W, out, M, N, K, 1, stream);
-        default: return launch_tile_mode<WMT, WNT, kStoreBF16>(A, W, out, M, N, K, 1, stream);
+        case kStoreF32: return launch_tile_mode<WMT, WNT, kStoreF32>(A, W, out, M, N, K, 1, blocked, stream);
+        case kAddF32: return launch_tile_mode<WMT, WNT, kAddF32>(A, W, out, M, N, K, 1, blocked, stream);
+        case kAtomicF32: return launch_tile_mode<WMT, WNT, kAtomicF32>(A, W, out, M, N, K, ksplit, blocked, stream);
+        case kGatedBF16: return launch_tile_mode<WMT, WNT, kGatedBF16>(A, W, out, M, N, K, 1, blocked, stream);
+        default: return launch_tile_mode<WMT, WNT, kStoreBF16>(A, W, out, M, N, K, 1, blocked, stream);
     }
 }
 
@@ -379,7 +409,7 @@ constexpr int SK_CHUNK = 32 * SK_U;      // 128 elements
 template <int MT, int NW, int MODE>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                               void* __restrict__ out, int M, int N, int K,
-                                                              int k_per_block) {
+                                                              int k_per_block, int blocked) {
     __shared__ f32x4 red[NW * MT * 64];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -388,8 +418,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     const int k_begin = blockIdx.y * k_per_block;
     const int k_end = (k_begin + k_per_block < K) ? k_begin + k_per_block : K;
 
+    // this lane's weights at k: row-major, row n0 + r from k + 8 q on; blocked, piece `lane` of block k / 32
+    // of row group n0 / 16 (K is a multiple of 32 then: a block is in or out whole)
     const bool wrow_ok = (n0 + r) < N;
-    const bf16* wrow = w + static_cast<size_t>(wrow_ok ? n0 + r : 0) * K + q * 8;
+    const bf16* wrow = blocked ? w + static_cast<size_t>(blockIdx.x) * 16 * K + lane * 8
+                               : w + static_cast<size_t>(wrow_ok ? n0 + r : 0) * K + q * 8;
+    const int wstep = blocked ? 16 : 1;                 // elements of w per element of k
     const bf16* xrow[MT];
     bool xrow_ok[MT];
 #pragma unroll
@@ -408,7 +442,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
         for (int u = 0; u < SK_U; ++u) {
             const int kk = k + u * 32;
             const bool k_ok = (kk + q * 8) < k_end;
-            fw[u] = load8(wrow + kk, wrow_ok && k_ok);
+            fw[u] = load8(wrow + static_cast<size_t>(kk) * wstep, wrow_ok && (blocked ? kk < k_end : k_ok));
 #pragma unroll
             for (int t = 0; t < MT; ++t) fx[t][u] = load8(xrow[t] + kk, xrow_ok[t] && k_ok);
         }
@@ -448,13 +482,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
 
 template <int MT, int NW>
 static void launch_skinny(const bf16* x, const bf16* w, void* out, int M, int N, int K, int mode, int ksplit,
-                          hipStream_t stream) {
+                          int blocked, hipStream_t stream) {
     const int tiles = (N + 15) / 16;
     int k_per_block = (K + ksplit - 1) / ksplit;
     k_per_block = ((k_per_block + SK_CHUNK - 1) / SK_CHUNK) * SK_CHUNK;
     const dim3 grid(tiles, (K + k_per_block - 1) / k_per_block), block(NW * 64);
 #define LLME_SK(MODE)                                                                            \
-    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NW, MODE>), grid, block, 0, stream, x, w, out, M, N, K, k_per_block)
+    hipLaunchKernelGGL((gemm_skinny_kernel<MT, NW, MODE>), grid, block, 0, stream, x, w, out, M, N, K, k_per_block, \
+                       blocked)
     if (mode == kStoreF32) LLME_SK(kStoreF32);
     else if (mode == kAddF32) LLME_SK(kAddF32);
     else if (mode == kAtomicF32) LLME_SK(kAtomicF32);
@@ -464,10 +499,10 @@ static void launch_skinny(const bf16* x, const bf16* w, void* out, int M, int N,
 
 template <int MT>
 static void launch_skinny_nw(const bf16* x, const bf16* w, void* out, int M, int N, int K, int mode, int nw,
-                             int ksplit, hipStream_t stream) {
-    if (nw >= 16 && MT <= 2) launch_skinny<MT, 16>(x, w, out, M, N, K, mode, ksplit, stream);
-    else if (nw >= 8) launch_skinny<MT, 8>(x, w, out, M, N, K, mode, ksplit, stream);
-    else launch_skinny<MT, 4>(x, w, out, M, N, K, mode, ksplit, stream);
+                             int ksplit, int blocked, hipStream_t stream) {
+    if (nw >= 16 && MT <= 2) launch_skinny<MT, 16>(x, w, out, M, N, K, mode, ksplit, blocked, stream);
+    else if (nw >= 8) launch_skinny<MT, 8>(x, w, out, M, N, K, mode, ksplit, blocked, stream);
+    else launch_skinny<MT, 4>(x, w, out, M, N, K, mode, ksplit, blocked, stream);
 }
 
 }  // namespace llme
@@ -479,10 +514,13 @@ using namespace llme;
 // groups of 16 and out is bfloat16 [M, N / 2] = silu(gate) * up (tile kernel only).
 // nw, ksplit: 0 lets the entry point choose the skinny kernel's wavefronts per workgroup and
 // the split over k; tile_shape: 0 chooses, 64 / 128 force the tile kernel with that tile
-// edge also for small M (for tests and measurements).
+// edge also for small M (for tests and measurements). blocked: w is stored in 1 KB blocks of
+// 16 rows x 32 k (see the head of this file; N a multiple of 16, K of 32).
 extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
-                              int accumulate, int gated, int nw, int ksplit, int tile_shape, hipStream_t stream) {
+                              int accumulate, int gated, int nw, int ksplit, int tile_shape, int blocked,
+                              hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
+    if (blocked && (N % 16 != 0 || K % 32 != 0)) return kErrUnsupported;
     if (K <= 0 || K % 8 != 0 || K >= (1 << 23)) return kErrUnsupported;   // 256 rows of K must stay below 2^32 bytes
     if (out_dtype != kF32 && out_dtype != kBF16) return kErrBadArgument;
     if (accumulate && out_dtype != kF32) return kErrBadArgument;
@@ -518,10 +556,10 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
         }
         const int mt = (M + 15) / 16;
         switch (mt) {
-            case 1: launch_skinny_nw<1>(A, W, out, M, N, K, mode, nw, ksplit, stream); break;
-            case 2: launch_skinny_nw<2>(A, W, out, M, N, K, mode, nw, ksplit, stream); break;
-            case 3: launch_skinny_nw<3>(A, W, out, M, N, K, mode, nw, ksplit, stream); break;
-            default: launch_skinny_nw<4>(A, W, out, M, N, K, mode, nw, ksplit, stream); break;
+            case 1: launch_skinny_nw<1>(A, W, out, M, N, K, mode, nw, ksplit, blocked, stream); break;
+            case 2: launch_skinny_nw<2>(A, W, out, M, N, K, mode, nw, ksplit, blocked, stream); break;
+            case 3: launch_skinny_nw<3>(A, W, out, M, N, K, mode, nw, ksplit, blocked, stream); break;
+            default: launch_skinny_nw<4>(A, W, out, M, N, K, mode, nw, ksplit, blocked, stream); break;
         }
         return launch_status();
     }
@@ -566,9 +604,9 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
         if (mode != kAddF32) return kErrBadArgument;
         mode = kAtomicF32;
     }
-    if (tile_shape == 128096) return launch_tile<4, 3>(A, W, out, M, N, K, mode, ksplit, stream);
-    if (tile_shape == 128064) return launch_tile<4, 2>(A, W, out, M, N, K, mode, ksplit, stream);
-    if (tile_shape == 128) return launch_tile<4, 4>(A, W, out, M, N, K, mode, ksplit, stream);
-    if (tile_shape == 64) return launch_tile<2, 2>(A, W, out, M, N, K, mode, ksplit, stream);
+    if (tile_shape == 128096) return launch_tile<4, 3>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
+    if (tile_shape == 128064) return launch_tile<4, 2>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
+    if (tile_shape == 128) return launch_tile<4, 4>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
+    if (tile_shape == 64) return launch_tile<2, 2>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
     return kErrBadArgument;
 }

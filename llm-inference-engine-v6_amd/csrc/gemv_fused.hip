@@ -24,7 +24,14 @@
 // nor a separate rotation kernel exist. A workgroup then takes the two tiles of 16 columns
 // that hold each other's rotation partners (the same head, hd/2 columns apart) at a time.
 //
-// Limits (checked by the caller): M <= 16, K a multiple of 8, 16 * (K + 8) * 2 bytes of LDS.
+// The weight matrix comes row-major ([rows, K]) or blocked: [rows / 16][K / 32] blocks of 1 KB,
+// a block holding its 16 rows x 32 k in the order of the matrix instruction's operand (lane
+// l = 16 q + r holds row r, k = 8 q .. 8 q + 7, so the block is [4 q][16 r][8]). A wavefront's
+// load is then 1 KB of consecutive addresses instead of 16 pieces of 64 bytes a row apart, which
+// streams a quarter faster from HBM (measured: 64 MB in 13.3 instead of 17.6 us).
+//
+// Limits (checked by the caller): M <= 16, K a multiple of 8, 16 * (K + 8) * 2 bytes of LDS;
+// blocked: K a multiple of 32 and the weight rows a multiple of 16.
 #include "common.h"
 #include <math.h>
 
@@ -82,7 +89,8 @@ template <int NW, int TPR, int EPI, typename TNW>
 __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restrict__ h, const int* __restrict__ rows,
                                                             const TNW* __restrict__ norm_w, float eps,
                                                             const bf16* __restrict__ w, void* __restrict__ out,
-                                                            int M, int N, int K, int tiles, RopeTarget rope) {
+                                                            int M, int N, int K, int tiles, int blocked,
+                                                            RopeTarget rope) {
     constexpr bool GATED = EPI == kGated;
     static_assert(EPI != kRope || TPR == 2, "the rotating epilogue works on pairs of tiles");
     constexpr int NT = GATED ? 2 : 1;                   // weight fragments per k step
@@ -112,19 +120,23 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
     bf16x8 fw[GV_DEPTH][NT][GV_U];
     auto load_w = [&](bf16x8 (&f)[NT][GV_U], int tile, int chunk) {
         // weight rows of this lane: plain: n = 16 tile + r; gated: gate row 32 tile + r, up row 16 further
+        // blocked: the 16-row group (NT t + tile's first), the 32-wide k block, 16 bytes per lane
         const int wr0 = GATED ? tile * 32 + r : tile * 16 + r;
         const int k0 = chunk * GV_CHUNK;
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
             const bool w_ok = tile < tiles && chunk < n_chunks && (wr0 + 16 * t) < n_rows_w;
-            const unsigned base = (static_cast<unsigned>(wr0 + 16 * t) * K + q * 8) * 2;
+            const unsigned base = blocked
+                ? (static_cast<unsigned>(tile * NT + t) * static_cast<unsigned>(K / 32)) * 1024u + lane * 16u
+                : (static_cast<unsigned>(wr0 + 16 * t) * K + q * 8) * 2;
 #pragma unroll
             for (int u = 0; u < GV_U; ++u) {
                 const int kk = k0 + u * 32;
                 // (all ones or zero, and the offset put together from both: written as a condition, the
                 // compiler made two loads under a branch out of it, with a wait for everything between)
-                const unsigned in = 0u - static_cast<unsigned>(w_ok && (kk + q * 8) < K);
-                const unsigned off = ((base + static_cast<unsigned>(kk) * 2) & in) | (kNowhere & ~in);
+                const unsigned in = 0u - static_cast<unsigned>(w_ok && (kk + (blocked ? 0 : q * 8)) < K);
+                const unsigned step = blocked ? static_cast<unsigned>(kk / 32) * 1024u : static_cast<unsigned>(kk) * 2;
+                const unsigned off = ((base + step) & in) | (kNowhere & ~in);
                 const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, off, 0, 0);
                 f[t][u] = __builtin_bit_cast(bf16x8, v);
             }
@@ -327,7 +339,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
 
 template <int NW, int TPR, int EPI, typename TNW>
 static int launch_gemv_norm(const float* h, const int* rows, const void* norm_w, float eps, const bf16* w, void* out,
-                            int M, int N, int K, int grid, const RopeTarget& rope, hipStream_t stream) {
+                            int M, int N, int K, int grid, int blocked, const RopeTarget& rope, hipStream_t stream) {
     const size_t lds = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(NW) * (EPI == kGated ? 2 : 1) * 64 * 16 +
                        64 + 2 * 16 * 16 * 4;
     if (lds > 160 * 1024) return kErrUnsupported;
@@ -341,20 +353,21 @@ static int launch_gemv_norm(const float* h, const int* rows, const void* norm_w,
     }
     const int tiles = (N + 15) / 16;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(NW * 64), lds, stream, h, rows, static_cast<const TNW*>(norm_w), eps,
-                       w, out, M, N, K, tiles, rope);
+                       w, out, M, N, K, tiles, blocked, rope);
     return launch_status();
 }
 
 template <int EPI, typename TNW>
 static int launch_gemv_norm_shape(int tpr, const float* h, const int* rows, const void* norm_w, float eps,
-                                  const bf16* w, void* out, int M, int N, int K, int grid, hipStream_t stream) {
+                                  const bf16* w, void* out, int M, int N, int K, int grid, int blocked,
+                                  hipStream_t stream) {
     const RopeTarget none{};
     // tpr: tiles at a time; 12 and 14: 2 and 4 tiles with 16 wavefronts instead of 8
-    if (tpr == 12) return launch_gemv_norm<16, 2, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
-    if (tpr == 14) return launch_gemv_norm<16, 4, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
-    if (tpr >= 4) return launch_gemv_norm<8, 4, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
-    if (tpr == 2) return launch_gemv_norm<8, 2, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
-    return launch_gemv_norm<8, 1, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, none, stream);
+    if (tpr == 12) return launch_gemv_norm<16, 2, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, blocked, none, stream);
+    if (tpr == 14) return launch_gemv_norm<16, 4, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, blocked, none, stream);
+    if (tpr >= 4) return launch_gemv_norm<8, 4, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, blocked, none, stream);
+    if (tpr == 2) return launch_gemv_norm<8, 2, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, blocked, none, stream);
+    return launch_gemv_norm<8, 1, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, blocked, none, stream);
 }
 
 }  // namespace llme
@@ -364,12 +377,14 @@ using namespace llme;
 // h [*, K] float32; rows: M indices into h or null; norm_w [K] (norm_dtype 0 float32, 1 bfloat16);
 // w bfloat16: plain [N, K], gated [2 N, K] with gate and up rows interleaved in groups of 16;
 // out: plain float32 [M, N], gated bfloat16 [M, N]. tpr (tiles a workgroup of 8 wavefronts works
-// on at a time: 1, 2 or 4) and grid (workgroups): 0 lets the entry point choose.
+// on at a time: 1, 2 or 4) and grid (workgroups): 0 lets the entry point choose. blocked: w is
+// stored in 1 KB blocks of 16 rows x 32 k (see the head of this file).
 extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_w, int norm_dtype, float eps,
                               const void* w, void* out, int M, int N, int K, int gated, int tpr, int grid,
-                              hipStream_t stream) {
+                              int blocked, hipStream_t stream) {
     if (M <= 0 || N <= 0) return 0;
     if (M > 16 || K <= 0 || K % 8 != 0) return kErrUnsupported;
+    if (blocked && (K % 32 != 0 || N % 16 != 0)) return kErrUnsupported;
     if (reinterpret_cast<uintptr_t>(norm_w) % 16 != 0 || reinterpret_cast<uintptr_t>(h) % 16 != 0) return kErrUnsupported;
     if (static_cast<size_t>(16) * (K + 8) * 2 > 132 * 1024) return kErrUnsupported;
     if (gated && N % 16 != 0) return kErrUnsupported;
@@ -388,12 +403,12 @@ extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_
     }
     const bf16* W = static_cast<const bf16*>(w);
     if (norm_dtype == kBF16) {
-        return gated ? launch_gemv_norm_shape<kGated, bf16>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream)
-                     : launch_gemv_norm_shape<kPlain, bf16>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream);
+        return gated ? launch_gemv_norm_shape<kGated, bf16>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, blocked, stream)
+                     : launch_gemv_norm_shape<kPlain, bf16>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, blocked, stream);
     }
     if (norm_dtype == kF32) {
-        return gated ? launch_gemv_norm_shape<kGated, float>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream)
-                     : launch_gemv_norm_shape<kPlain, float>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, stream);
+        return gated ? launch_gemv_norm_shape<kGated, float>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, blocked, stream)
+                     : launch_gemv_norm_shape<kPlain, float>(tpr, h, rows, norm_w, eps, W, out, M, N, K, grid, blocked, stream);
     }
     return kErrBadArgument;
 }
@@ -406,8 +421,10 @@ extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_
 extern "C" int llme_gemv_norm_rope(const float* h, const void* norm_w, int norm_dtype, float eps, const void* w,
                                    const int* positions, const int* seq_idx, const int* block_table, int max_blocks,
                                    const float* cos_t, const float* sin_t, void* q_out, void* k_cache, void* v_cache,
-                                   int M, int K, int n_q, int n_kv, int hd, int page, int grid, hipStream_t stream) {
+                                   int M, int K, int n_q, int n_kv, int hd, int page, int grid, int blocked,
+                                   hipStream_t stream) {
     if (M <= 0) return 0;
+    if (blocked && K % 32 != 0) return kErrUnsupported;
     if (reinterpret_cast<uintptr_t>(norm_w) % 16 != 0 || reinterpret_cast<uintptr_t>(h) % 16 != 0) return kErrUnsupported;
     if (M > 16 || K <= 0 || K % 8 != 0 || hd <= 0 || hd % 32 != 0 || n_q <= 0 || n_kv <= 0 || page <= 0)
         return kErrUnsupported;
@@ -420,8 +437,8 @@ extern "C" int llme_gemv_norm_rope(const float* h, const void* norm_w, int norm_
                           static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache), n_q, n_kv, hd, page};
     const bf16* W = static_cast<const bf16*>(w);
     if (norm_dtype == kBF16)
-        return launch_gemv_norm<16, 2, kRope, bf16>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, rope, stream);
+        return launch_gemv_norm<16, 2, kRope, bf16>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream);
     if (norm_dtype == kF32)
-        return launch_gemv_norm<16, 2, kRope, float>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, rope, stream);
+        return launch_gemv_norm<16, 2, kRope, float>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream);
     return kErrBadArgument;
 }

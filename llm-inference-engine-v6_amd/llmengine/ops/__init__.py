@@ -1,11 +1,13 @@
 """The HIP kernels of the engine, as Python functions over device tensors."""
 from .lib import KernelError, KernelLibraryError, library
-from .kernels import (argmax, argmax_into, attention, attention_generic, rope_q_only, embed_gather, gemm, gemm_generic, policy, rmsnorm,
-                      rope_kv_write, sample, swiglu)
+from .kernels import (argmax, argmax_into, attention, attention_generic, block_weight, can_block, embed_gather, gemm,
+                      gemm_generic, is_blocked, policy, rmsnorm, rope_kv_write, rope_q_only, sample, swiglu,
+                      unblock_weight, weight_shape)
 
 from . import mfma                                   # noqa: E402  (installs the MFMA kernels)
 from .mfma import (gemm_bf16, gemm_gated, gemv_norm, gemv_norm_rope, gemv_norm_rope_supported,
                    gemv_norm_supported)
 
-__all__ = ["gemm_bf16", "gemm_gated", "gemv_norm_rope", "gemv_norm_rope_supported", "gemv_norm", "gemv_norm_supported", "mfma", "KernelError", "KernelLibraryError", "library", "argmax", "argmax_into", "attention", "attention_generic", "rope_q_only", "embed_gather",
+__all__ = ["gemm_bf16", "gemm_gated", "gemv_norm_rope", "gemv_norm_rope_supported", "gemv_norm", "gemv_norm_supported", "mfma", "KernelError", "KernelLibraryError", "library", "argmax", "argmax_into", "attention", "attention_generic", "rope_q_only", "embed_gather", "block_weight", "can_block",
+           "is_blocked", "unblock_weight", "weight_shape",
            "gemm", "gemm_generic", "policy", "rmsnorm", "rope_kv_write", "sample", "swiglu"]

@@ -26,16 +26,64 @@ class Policy:
 policy = Policy()
 
 
+# --- weight layouts ------------------------------------------------------------------
+# A weight matrix [N, K] (y = x W^T) is a 2-d tensor, row-major, or a 5-d tensor
+# [N / 16, K / 32, 4, 16, 8] in the blocked layout of the matrix kernels: block (i, j) holds rows
+# 16 i .. 16 i + 15 and k = 32 j .. 32 j + 31 as [4 q][16 r][8], element (r, 8 q + e) of the block at
+# [q][r][e], which is the order in which a wavefront's 64 lanes hold a matrix-instruction operand.
+# A wavefront then loads an operand as 1 KB of consecutive addresses. The tensor's rank tells the
+# layout; row slices in steps of 16 rows are slices of the first dimension.
+def is_blocked(w: torch.Tensor) -> bool:
+    return w.dim() == 5
+
+
+def weight_shape(w: torch.Tensor) -> tuple[int, int]:
+    """(N, K) of a weight matrix in either layout."""
+    if w.dim() == 5:
+        if tuple(w.shape[2:]) != (4, 16, 8):
+            raise KernelError(f"a blocked weight has blocks of [4, 16, 8], not {tuple(w.shape[2:])}")
+        return w.shape[0] * 16, w.shape[1] * 32
+    if w.dim() != 2:
+        raise KernelError(f"a weight matrix is [N, K] or blocked [N / 16, K / 32, 4, 16, 8], not {tuple(w.shape)}")
+    return w.shape[0], w.shape[1]
+
+
+def can_block(w: torch.Tensor) -> bool:
+    return w.dim() == 2 and w.dtype == torch.bfloat16 and w.shape[0] % 16 == 0 and w.shape[1] % 32 == 0
+
+
+def block_weight(w: torch.Tensor) -> torch.Tensor:
+    """The blocked copy of a row-major bfloat16 matrix whose N is a multiple of 16 and K of 32."""
+    if not can_block(w):
+        raise KernelError(f"block_weight: needs bfloat16 [N, K] with N % 16 == 0 and K % 32 == 0, got "
+                          f"{w.dtype} {tuple(w.shape)}")
+    N, K = w.shape
+    return w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
+
+
+def unblock_weight(w: torch.Tensor) -> torch.Tensor:
+    """The row-major copy of a blocked matrix."""
+    N, K = weight_shape(w)
+    return w.permute(0, 3, 1, 2, 4).reshape(N, K).contiguous()
+
+
+def _require_weight(w: torch.Tensor, name: str, dtypes, K: int | None = None) -> tuple[int, int]:
+    require(w, name, dtypes)
+    N, Kw = weight_shape(w)
+    if K is not None and Kw != K:
+        raise KernelError(f"{name}: expected K = {K}, got a matrix of [{N}, {Kw}]")
+    return N, Kw
+
+
 # --- embedding ---------------------------------------------------------------------
 def embed_gather(table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
-    """out[t, :] = table[tokens[t], :] widened to 32-bit."""
-    require(table, "table", _FLOATS, (None, None))
-    V, H = table.shape
+    """out[t, :] = table[tokens[t], :] widened to 32-bit (the table row-major or blocked)."""
+    V, H = _require_weight(table, "table", _FLOATS)
     T = tokens.shape[0]
     require(tokens, "tokens", torch.int32, (T,))
     require(out, "out", torch.float32, (T, H))
-    check(entry("llme_embed_gather")(ptr(table), code(table.dtype), ptr(tokens), ptr(out), T, H, stream()),
-          "embed_gather")
+    check(entry("llme_embed_gather")(ptr(table), code(table.dtype), ptr(tokens), ptr(out), T, H,
+                                     1 if is_blocked(table) else 0, stream()), "embed_gather")
 
 
 # --- norm --------------------------------------------------------------------------
@@ -119,11 +167,11 @@ def rope_q_only(q32: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor |
 def gemm_generic(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
     require(a, "a", _FLOATS, (None, None))
     M, K = a.shape
-    require(w, "w", _FLOATS, (None, K))
-    N = w.shape[0]
+    N, _ = _require_weight(w, "w", _FLOATS, K)
     require(out, "out", _FLOATS, (M, N))
     check(entry("llme_gemm_generic")(ptr(a), code(a.dtype), ptr(w), code(w.dtype), ptr(out), code(out.dtype),
-                                     M, N, K, 1 if accumulate else 0, stream()), "gemm_generic")
+                                     M, N, K, 1 if accumulate else 0, 1 if is_blocked(w) else 0, stream()),
+          "gemm_generic")
 
 
 _fast_gemm = None       # set by ops/mfma.py when the MFMA kernels are present

@@ -30,12 +30,12 @@ _lock = threading.Lock()
 _vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 
 _SIGNATURES = {
-    "llme_embed_gather": [_vp, _i, _vp, _vp, _i, _i, _vp],
+    "llme_embed_gather": [_vp, _i, _vp, _vp, _i, _i, _i, _vp],
     "llme_rmsnorm": [_vp, _vp, _i, _vp, _i, _vp, _i, _i, _f, _vp],
     "llme_swiglu": [_vp, _i, _vp, _i, _i, _i, _i, _vp],
     "llme_rope_kv_write": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i,
                            _i, _i, _i, _i, _i, _i, _i, _vp],
-    "llme_gemm_generic": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
+    "llme_gemm_generic": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "llme_attention_generic": [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
                                _f, _i, _vp],
     "llme_argmax": [_vp, _vp, _vp, _vp, _i, _i, _vp],

@@ -12,14 +12,14 @@ from .lib import check, declare, entry, ptr, require, stream
 
 _vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 
-declare("llme_gemm_bf16", [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp])
+declare("llme_gemm_bf16", [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp])
 
 
 def gemm_bf16_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool) -> bool:
     return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
             and out.dtype in (torch.float32, torch.bfloat16)
             and not (accumulate and out.dtype != torch.float32)
-            and a.shape[1] % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and w.dim() in (2, 5) and a.shape[1] % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
             and out.data_ptr() % 16 == 0)
 
 
@@ -31,8 +31,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
     force_tile override the launch choices (tests and measurements)."""
     require(a, "a", torch.bfloat16, (None, None))
     M, K = a.shape
-    require(w, "w", torch.bfloat16, (None, K))
-    N = w.shape[0]
+    N, _ = kernels._require_weight(w, "w", torch.bfloat16, K)
     if gated:
         require(out, "out", torch.bfloat16, (M, N // 2))
         if N % 32 or accumulate:
@@ -45,7 +44,8 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
     if force_tile and not tile:
         tile = 128
     check(entry("llme_gemm_bf16")(ptr(a), ptr(w), ptr(out), 0 if out.dtype == torch.float32 else 1, M, N, K,
-                                  1 if accumulate else 0, 1 if gated else 0, waves, ksplit, tile, stream()),
+                                  1 if accumulate else 0, 1 if gated else 0, waves, ksplit, tile,
+                                  1 if kernels.is_blocked(w) else 0, stream()),
           "gemm_bf16")
 
 
@@ -65,7 +65,7 @@ def gemm_gated(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, grou
 
 
 def _fast_gemm(a, w, out, accumulate) -> bool:
-    if a.dim() != 2 or w.dim() != 2 or not gemm_bf16_supported(a, w, out, accumulate):
+    if a.dim() != 2 or w.dim() not in (2, 5) or not gemm_bf16_supported(a, w, out, accumulate):
         return False
     gemm_bf16(a, w, out, accumulate)
     return True
@@ -175,7 +175,7 @@ kernels._fast_attention = _fast_attention
 
 
 # --- projections fused with the norm in front of them (decoding) ---------------------------
-declare("llme_gemv_norm", [_vp, _vp, _vp, _i, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp])
+declare("llme_gemv_norm", [_vp, _vp, _vp, _i, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp])
 
 GEMV_NORM_MAX_ROWS = 16
 
@@ -183,10 +183,13 @@ GEMV_NORM_MAX_ROWS = 16
 def gemv_norm_supported(h: torch.Tensor, norm_weight: torch.Tensor, w: torch.Tensor, rows_out: int,
                         gated: bool) -> bool:
     K = h.shape[1]
-    n_out = w.shape[0] // 2 if gated else w.shape[0]
+    if w.dim() not in (2, 5):
+        return False
+    n_rows, k_w = kernels.weight_shape(w)
+    n_out = n_rows // 2 if gated else n_rows
     return (kernels.policy.fast_gemm and h.dtype == torch.float32 and w.dtype == torch.bfloat16
             and norm_weight.dtype in (torch.float32, torch.bfloat16) and 0 < rows_out <= GEMV_NORM_MAX_ROWS
-            and K % 8 == 0 and 16 * (K + 8) * 2 <= 132 * 1024 and w.shape[1] == K
+            and K % 8 == 0 and 16 * (K + 8) * 2 <= 132 * 1024 and k_w == K
             and (not gated or n_out % 16 == 0) and w.data_ptr() % 16 == 0 and h.data_ptr() % 16 == 0
             and norm_weight.data_ptr() % 16 == 0)
 
@@ -202,20 +205,20 @@ def gemv_norm(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.T
     if rows is not None:
         require(rows, "rows", torch.int32, (M,))
     require(norm_weight, "norm_weight", (torch.float32, torch.bfloat16), (K,))
-    require(w, "w", torch.bfloat16, (None, K))
-    N = w.shape[0] // 2 if gated else w.shape[0]
+    n_rows, _ = kernels._require_weight(w, "w", torch.bfloat16, K)
+    N = n_rows // 2 if gated else n_rows
     require(out, "out", torch.bfloat16 if gated else torch.float32, (M, N))
     if not gemv_norm_supported(h, norm_weight, w, M, gated):
         raise kernels.KernelError(f"gemv_norm: {M} rows (at most 16), K={K} (multiple of 8, 16 rows must fit "
                                   "into LDS) or the operand types are not supported")
     check(entry("llme_gemv_norm")(ptr(h), ptr(rows), ptr(norm_weight), 0 if norm_weight.dtype == torch.float32 else 1,
                                   float(eps), ptr(w), ptr(out), M, N, K, 1 if gated else 0, tiles_per_round, grid,
-                                  stream()),
+                                  1 if kernels.is_blocked(w) else 0, stream()),
           "gemv_norm")
 
 
 declare("llme_gemv_norm_rope", [_vp, _vp, _i, _f, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp,
-                                _i, _i, _i, _i, _i, _i, _i, _vp])
+                                _i, _i, _i, _i, _i, _i, _i, _i, _vp])
 
 
 def gemv_norm_rope_supported(h, norm_weight, w_qkv, k_cache, n_tokens: int, head_dim: int, rotary_dim: int) -> bool:
@@ -233,7 +236,9 @@ def gemv_norm_rope(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv
     require(h, "h", torch.float32, (None, None))
     M, K = h.shape
     require(norm_weight, "norm_weight", (torch.float32, torch.bfloat16), (K,))
-    require(w_qkv, "w_qkv", torch.bfloat16, ((n_q + 2 * n_kv) * head_dim, K))
+    n_rows, _ = kernels._require_weight(w_qkv, "w_qkv", torch.bfloat16, K)
+    if n_rows != (n_q + 2 * n_kv) * head_dim:
+        raise kernels.KernelError(f"gemv_norm_rope: w_qkv has {n_rows} rows, the heads need {(n_q + 2 * n_kv) * head_dim}")
     require(positions, "positions", torch.int32, (M,))
     require(seq_idx, "seq_idx", torch.int32, (M,))
     require(block_table, "block_table", torch.int32, (None, None))
@@ -249,4 +254,5 @@ def gemv_norm_rope(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv
     check(entry("llme_gemv_norm_rope")(
         ptr(h), ptr(norm_weight), 0 if norm_weight.dtype == torch.float32 else 1, float(eps), ptr(w_qkv),
         ptr(positions), ptr(seq_idx), ptr(block_table), block_table.shape[1], ptr(cos), ptr(sin), ptr(q_out),
-        ptr(k_cache), ptr(v_cache), M, K, n_q, n_kv, head_dim, page, grid, stream()), "gemv_norm_rope")
+        ptr(k_cache), ptr(v_cache), M, K, n_q, n_kv, head_dim, page, grid, 1 if kernels.is_blocked(w_qkv) else 0,
+        stream()), "gemv_norm_rope")

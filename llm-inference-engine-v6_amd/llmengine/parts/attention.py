@@ -53,8 +53,9 @@ class Attention(Mixer):
         for p in parts:
             fused[row:row + p.shape[0]].copy_(p)
             row += p.shape[0]
-        self.w_qkv = fused
-        self.w_o = placement.place(get("o_proj.weight"))
+        # (queries alone are sliced off for layers that read another layer's cache: whole row groups)
+        self.w_qkv = placement.matrix(fused) if self.q_dim % 16 == 0 else fused
+        self.w_o = placement.place_matrix(get("o_proj.weight"))
         if self.position is not None and hasattr(self.position, "materialize"):
             self.position.materialize(placement)
 
@@ -98,7 +99,7 @@ class Attention(Mixer):
         else:
             # A layer that reads another layer's cache projects queries only.
             q32 = step.buffer("attn.q32", (T, self.q_dim), torch.float32)
-            project(self.w_qkv[:self.q_dim], q32)
+            project(self.w_qkv[:self.q_dim // 16] if ops.is_blocked(self.w_qkv) else self.w_qkv[:self.q_dim], q32)
             ops.rope_q_only(q32, cos, sin, step.positions, q, n_q, hd, rot)
         o = step.buffer("attn.o", (T, self.q_dim), act)
         ops.attention(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, hd, self.scale, self.window)

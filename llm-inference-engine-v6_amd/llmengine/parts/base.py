@@ -58,6 +58,16 @@ class Placement:
         dtype = dtype or self.storage_dtype(t.dtype)
         return t.to(device=self.device, dtype=dtype).contiguous()
 
+    def matrix(self, w: torch.Tensor) -> torch.Tensor:
+        """A weight matrix [N, K] that is already on the device, in the layout the matrix kernels
+        stream fastest: blocked (a 5-d tensor, see ops.block_weight) where its type and sizes
+        allow, otherwise as it is."""
+        from .. import ops
+        return ops.block_weight(w) if ops.can_block(w) else w
+
+    def place_matrix(self, t: torch.Tensor, dtype: torch.dtype | None = None) -> torch.Tensor:
+        return self.matrix(self.place(t, dtype))
+
     def common_dtype(self, tensors: list[torch.Tensor]) -> torch.dtype:
         """The storage dtype of a buffer that fuses several checkpoint tensors."""
         kinds = {self.storage_dtype(t.dtype) for t in tensors}

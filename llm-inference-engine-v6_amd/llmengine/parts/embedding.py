@@ -23,7 +23,8 @@ class Embedding(Part):
         return {"weight": ParamSpec((self.vocab_size, self.hidden_size), "linear")}
 
     def load_params(self, get: Getter, placement: Placement) -> None:
-        self.weight = placement.place(get("weight"))
+        # (a tied head reads the table as a weight matrix: the gather takes either layout)
+        self.weight = placement.place_matrix(get("weight"))
 
     def forward(self, tokens: torch.Tensor, out: torch.Tensor) -> None:
         ops.embed_gather(self.weight, tokens, out)
@@ -48,7 +49,7 @@ class OutputHead(Part):
 
     def load_params(self, get: Getter, placement: Placement) -> None:
         if self.tied_to is None:
-            self._weight = placement.place(get("weight"))
+            self._weight = placement.place_matrix(get("weight"))
 
     @property
     def weight(self) -> torch.Tensor:

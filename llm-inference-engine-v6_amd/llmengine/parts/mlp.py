@@ -37,8 +37,8 @@ class GatedMLP(FeedForward):
         view = fused.view(FF // g, 2, g, H)
         view[:, 0].copy_(gate.view(FF // g, g, H))
         view[:, 1].copy_(up.view(FF // g, g, H))
-        self.w_gate_up = fused
-        self.w_down = placement.place(get("down_proj.weight"))
+        self.w_gate_up = placement.matrix(fused)
+        self.w_down = placement.place_matrix(get("down_proj.weight"))
 
     def fuses_norm(self, h, norm, step):
         # A few rows (decoding): one kernel applies the norm, both projections and the activation.

@@ -90,7 +90,9 @@ def test_storage_types(tmp_path):
     m32 = build_llama(parse_config(TINY_A))
     load_model_weights(m32, bf, CPU32)
     assert m32.embedding.weight.dtype == torch.float32
-    assert torch.equal(m32.embedding.weight, m.embedding.weight.float())     # widening is exact
+    from llmengine import ops
+    assert ops.is_blocked(m.embedding.weight) and not ops.is_blocked(m32.embedding.weight)   # bfloat16 matrices: blocked
+    assert torch.equal(m32.embedding.weight, ops.unblock_weight(m.embedding.weight).float())   # widening is exact
     # a tensor stored in 32-bit stays so in the bfloat16 model
     mixed = _state(TINY_A, 0, torch.bfloat16)
     mixed["model.norm.weight"] = mixed["model.norm.weight"].float()
