@@ -80,8 +80,8 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD,
                page_magic_of(page), static_cast<unsigned>(n_kv) * page * HD, static_cast<unsigned>(kvh) * page * HD};
     const int first = k_begin + __builtin_amdgcn_readfirstlane(wave) * 32;
-    attend_range<HD, 1>(kv, first, DEC_WAVES * 32, lo_all, k_end, qf, row_pos, row_lo, tile_free, scale * kLog2e,
-                        m, l, o);
+    attend_range<HD, 1, true>(kv, first, DEC_WAVES * 32, lo_all, k_end, qf, row_pos, row_lo, tile_free,
+                              scale * kLog2e, m, l, o);
 
     float lt = l[0];
     lt += __shfl_xor(lt, 16, 64);

@@ -102,7 +102,10 @@ __device__ __forceinline__ BlockPages lookup_pages(const PagedKV& kv, int t0, in
 // The full variant has no branch at all: the loop over full blocks then issues the same loads
 // on every turn, so the counter of loads in flight tells exactly which have arrived, and a
 // wait for this block's operand does not also wait for the next block's.
-template <int HD, bool FULL>
+// STREAM: the loads carry the hint that the data is read once (a decoding request's keys and
+// values are read by one workgroup per step): they then pass the L2 without displacing what is
+// used again, which streams measurably faster from HBM.
+template <int HD, bool FULL, bool STREAM = false>
 __device__ __forceinline__ void load_k(const PagedKV& kv, int t0, const BlockPages& pages, int key_lo, int key_end,
                                        KFrag<HD>& f) {
     constexpr int DC = (HD + 31) / 32;
@@ -121,7 +124,8 @@ __device__ __forceinline__ void load_k(const PagedKV& kv, int t0, const BlockPag
             if (HD % 32 != 0 && c == DC - 1) {       // the last 32 dims are half there: lanes of the upper half hold zeros
                 f.kf[hf][c] = (key_ok && g4 < 2) ? *reinterpret_cast<const bf16x8*>(base + lane_off + c * 32) : zero_frag();
             } else if (FULL) {
-                f.kf[hf][c] = *reinterpret_cast<const bf16x8*>(base + lane_off + c * 32);
+                const bf16x8* p = reinterpret_cast<const bf16x8*>(base + lane_off + c * 32);
+                f.kf[hf][c] = STREAM ? __builtin_nontemporal_load(p) : *p;
             } else {
                 f.kf[hf][c] = key_ok ? *reinterpret_cast<const bf16x8*>(base + lane_off + c * 32) : zero_frag();
             }
@@ -130,7 +134,7 @@ __device__ __forceinline__ void load_k(const PagedKV& kv, int t0, const BlockPag
 }
 
 // The same for the V operand, read 4 keys (8 bytes) at a time from the transposed pages.
-template <int HD, bool FULL>
+template <int HD, bool FULL, bool STREAM = false>
 __device__ __forceinline__ void load_v(const PagedKV& kv, int t0, const BlockPages& pages, int key_lo, int key_end,
                                        VFrag<HD>& f) {
     constexpr int DT = HD / 16;
@@ -152,8 +156,13 @@ __device__ __forceinline__ void load_v(const PagedKV& kv, int t0, const BlockPag
         bf16x4 lo4, hi4;
 #pragma unroll
         for (int e = 0; e < 4; ++e) lo4[e] = hi4[e] = static_cast<__bf16>(0.f);
-        if (FULL || ok[0]) lo4 = *reinterpret_cast<const bf16x4*>(base[0] + off);
-        if (FULL || ok[1]) hi4 = *reinterpret_cast<const bf16x4*>(base[1] + off);
+        if (FULL && STREAM) {
+            lo4 = __builtin_nontemporal_load(reinterpret_cast<const bf16x4*>(base[0] + off));
+            hi4 = __builtin_nontemporal_load(reinterpret_cast<const bf16x4*>(base[1] + off));
+        } else {
+            if (FULL || ok[0]) lo4 = *reinterpret_cast<const bf16x4*>(base[0] + off);
+            if (FULL || ok[1]) hi4 = *reinterpret_cast<const bf16x4*>(base[1] + off);
+        }
         f.vf[dt] = __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
     }
 }
@@ -276,7 +285,7 @@ __device__ __forceinline__ void attend_edge_block(const PagedKV& kv, int t0, int
 // arrive in; page ids are looked up one block further ahead, so that no load waits for a table
 // entry. The last turn asks for its own block once more instead of for nothing, and the lookups
 // ahead are clamped to the table's last entry in use: the same loads on every turn.
-template <int HD, int QT>
+template <int HD, int QT, bool STREAM = false>
 __device__ __forceinline__ void attend_range(const PagedKV& kv, int first, int stride, int key_lo, int key_end,
                                              const bf16x8 (&qf)[QT][(HD + 31) / 32], const int (&row_pos)[QT],
                                              const int (&row_lo)[QT], const int (&tile_free)[QT], float scale_log2,
@@ -300,8 +309,8 @@ __device__ __forceinline__ void attend_range(const PagedKV& kv, int first, int s
             const int h0 = min(t0 + stride + hf * 16, last_half);
             pg_next.pg[hf] = __builtin_amdgcn_readfirstlane(kv.table[page_of(kv, h0).block]);
         }
-        load_k<HD, true>(kv, t0, pg_cur, key_lo, key_end, kf);
-        load_v<HD, true>(kv, t0, pg_cur, key_lo, key_end, vf);
+        load_k<HD, true, STREAM>(kv, t0, pg_cur, key_lo, key_end, kf);
+        load_v<HD, true, STREAM>(kv, t0, pg_cur, key_lo, key_end, vf);
         for (; t0 < full_end; t0 += stride) {
             const bool more = t0 + stride < full_end;
             const int tn = more ? t0 + stride : t0;
@@ -313,7 +322,7 @@ __device__ __forceinline__ void attend_range(const PagedKV& kv, int first, int s
             }
             f32x4 s[QT][2];
             block_scores<HD, QT>(kf, qf, s);
-            load_k<HD, true>(kv, tn, pg_cur, key_lo, key_end, kf);
+            load_k<HD, true, STREAM>(kv, tn, pg_cur, key_lo, key_end, kf);
             bf16x8 pf[QT];
             block_weights<HD, QT>(s, t0, row_pos, row_lo, tile_free, scale_log2, m, l, o, pf);
 #pragma unroll
@@ -321,7 +330,7 @@ __device__ __forceinline__ void attend_range(const PagedKV& kv, int first, int s
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
                     o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[qt], vf.vf[dt], o[qt][dt], 0, 0, 0);
-            load_v<HD, true>(kv, tn, pg_cur, key_lo, key_end, vf);
+            load_v<HD, true, STREAM>(kv, tn, pg_cur, key_lo, key_end, vf);
         }
     }
     if (t0 < key_end)                                        // one block that ends behind key_end

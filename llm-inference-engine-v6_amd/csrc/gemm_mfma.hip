@@ -42,6 +42,10 @@ __device__ __forceinline__ bf16x8 zero8() {
 __device__ __forceinline__ bf16x8 load8(const bf16* p, bool ok) {
     return ok ? *reinterpret_cast<const bf16x8*>(p) : zero8();
 }
+// The same with the hint that the data is read once (the weights of a product with few rows).
+__device__ __forceinline__ bf16x8 load8_once(const bf16* p, bool ok) {
+    return ok ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p)) : zero8();
+}
 
 typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
 // The fourth word of a buffer descriptor for raw 32-bit data on this chip.
@@ -442,7 +446,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
         for (int u = 0; u < SK_U; ++u) {
             const int kk = k + u * 32;
             const bool k_ok = (kk + q * 8) < k_end;
-            fw[u] = load8(wrow + static_cast<size_t>(kk) * wstep, wrow_ok && (blocked ? kk < k_end : k_ok));
+            fw[u] = load8_once(wrow + static_cast<size_t>(kk) * wstep, wrow_ok && (blocked ? kk < k_end : k_ok));
 #pragma unroll
             for (int t = 0; t < MT; ++t) fx[t][u] = load8(xrow[t] + kk, xrow_ok[t] && k_ok);
         }
