@@ -397,7 +397,9 @@ extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_
         // few tiles: all 8 wavefronts on one tile, so that every tile has a workgroup of its own;
         // more tiles than compute units: 2 tiles at a time, 4 wavefronts each with several chunks of k
         tpr = tiles <= 256 ? 1 : 2;
-        if (gated && tiles > 256 && tiles <= 1024) tpr = 12;   // (measured: 16 wavefronts on 2 tiles, 14.2 against 14.8 us at 512 tiles)
+        // (measured: 16 wavefronts on 2 tiles, 14.2 against 14.8 us at 512 tiles; they need more LDS for their sums)
+        const size_t lds16 = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(16) * 2 * 64 * 16 + 64 + 2 * 16 * 16 * 4;
+        if (gated && tiles > 256 && tiles <= 1024 && lds16 <= 160 * 1024) tpr = 12;
     }
     if (tpr != 1 && tpr != 2 && tpr != 4 && tpr != 12 && tpr != 14) return kErrBadArgument;
     if (grid <= 0) {
