@@ -41,7 +41,7 @@ namespace llme {
 // 32-key block and add up through LDS.
 constexpr int DEC_WAVES = 4;
 
-template <int HD>
+template <int HD, bool STREAM>
 __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     bf16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD,
                page_magic_of(page), static_cast<unsigned>(n_kv) * page * HD, static_cast<unsigned>(kvh) * page * HD};
     const int first = k_begin + __builtin_amdgcn_readfirstlane(wave) * 32;
-    attend_range<HD, 1, true>(kv, first, DEC_WAVES * 32, lo_all, k_end, qf, row_pos, row_lo, tile_free,
+    attend_range<HD, 1, STREAM>(kv, first, DEC_WAVES * 32, lo_all, k_end, qf, row_pos, row_lo, tile_free,
                               scale * kLog2e, m, l, o);
 
     float lt = l[0];
@@ -246,6 +246,14 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     }
 }
 
+// Whether the decode kernel loads keys and values with the read-once hint. -1: the entry point
+// chooses; 0 / 1: never / always (llme_attention_bf16_set_stream, for measurements).
+static int g_stream_override = -1;
+static bool decode_reads_once(int n_decode) {
+    if (g_stream_override >= 0) return g_stream_override != 0;
+    return n_decode >= 0;
+}
+
 template <int HD>
 static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, float* part_o, float* part_ml,
                            const int* q_start, const int* ctx_len, const int* table, int max_blocks, int n_seq,
@@ -254,8 +262,14 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
     if (n_decode > 0) {
         const int G = n_q / n_kv;
         const dim3 grid(n_seq, n_kv * ((G + 15) / 16), nsplit);
-        hipLaunchKernelGGL((attention_decode_kernel<HD>), grid, dim3(DEC_WAVES * 64), 0, stream, q, kc, vc, out, part_o, part_ml,
-                           q_start, ctx_len, table, max_blocks, n_q, n_kv, page, scale, window, split_len, nsplit);
+        if (decode_reads_once(n_decode))
+            hipLaunchKernelGGL((attention_decode_kernel<HD, true>), grid, dim3(DEC_WAVES * 64), 0, stream, q, kc, vc, out,
+                               part_o, part_ml, q_start, ctx_len, table, max_blocks, n_q, n_kv, page, scale, window,
+                               split_len, nsplit);
+        else
+            hipLaunchKernelGGL((attention_decode_kernel<HD, false>), grid, dim3(DEC_WAVES * 64), 0, stream, q, kc, vc, out,
+                               part_o, part_ml, q_start, ctx_len, table, max_blocks, n_q, n_kv, page, scale, window,
+                               split_len, nsplit);
         if (nsplit > 1)
             hipLaunchKernelGGL(attention_join_kernel, dim3(n_seq, n_q), dim3(64), 0, stream, part_o, part_ml, out,
                                q_start, n_q, HD, nsplit);
@@ -294,6 +308,11 @@ extern "C" int llme_attention_bf16_set_rows(int rows, int shared) {
     g_rows_override = rows;
     g_shared_override = shared > 1 ? 1 : shared;
     prefill_shared_key_waves(shared > 1 ? shared - 1 : 0);
+    return 0;
+}
+extern "C" int llme_attention_bf16_set_stream(int mode) {
+    if (mode < -1 || mode > 1) return kErrBadArgument;
+    g_stream_override = mode;
     return 0;
 }
 static int direct_rows(int hd) {

@@ -77,6 +77,7 @@ kernels._fast_gemm = _fast_gemm
 # --- attention ---------------------------------------------------------------------------
 declare("llme_attention_bf16_rows", [_i, _i, _i])
 declare("llme_attention_bf16_set_rows", [_i, _i])
+declare("llme_attention_bf16_set_stream", [_i])
 declare("llme_attention_bf16", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i,
                                 _i, _i, _i, _i, _vp, _vp])
 
