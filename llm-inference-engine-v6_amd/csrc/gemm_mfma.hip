@@ -86,6 +86,9 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
     constexpr int BM = 32 * WMT, BN = 32 * WNT;
     constexpr int A_ELEMS = BM * TSTRIDE, W_ELEMS = BN * TSTRIDE;
     constexpr int CA = BM / 32, CW = BN / 32;        // 16-byte chunks per thread and slab
+    // The 64 x 64 tile serves products with up to 64 rows (decoding at large batches): one row of
+    // tiles, so every weight is read once, and the loads say so (the non-temporal bit).
+    constexpr int W_POLICY = (WMT == 2 && WNT == 2) ? 2 : 0;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     bf16* lds = reinterpret_cast<bf16*>(lds_raw);
     // buffers: sA[b] = lds + b * A_ELEMS, sW[b] = lds + 2 * A_ELEMS + b * W_ELEMS
@@ -158,7 +161,7 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
         for (int i = 0; i < CA; ++i) s.ra[i] = __builtin_amdgcn_raw_buffer_load_b128(a_rsrc, aoff[i], k * 2, 0);
 #pragma unroll
         for (int i = 0; i < CW; ++i)                  // (blocked: a slab is two blocks further in every row group)
-            s.rw[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, woff[i], BLOCKED ? kt * 2048 : k * 2, 0);
+            s.rw[i] = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, woff[i], BLOCKED ? kt * 2048 : k * 2, W_POLICY);
         if (!KFULL) {                                 // K is a multiple of 8: a chunk is in or out whole
             const bool ok = k + ckq < K;
 #pragma unroll
