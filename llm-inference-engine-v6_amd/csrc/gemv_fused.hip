@@ -21,8 +21,12 @@
 // A third form serves the attention's q/k/v projection: its epilogue rotates q and k heads at
 // the rows' positions (pairs (i, i + hd/2), src/kernels.cpp:189-203) and writes q to the query
 // buffer and k, v straight into the rows' cache pages, so that neither the 32-bit q/k/v rows
-// nor a separate rotation kernel exist. A workgroup then takes the two tiles of 16 columns
-// that hold each other's rotation partners (the same head, hd/2 columns apart) at a time.
+// nor a separate rotation kernel exist. For this form the weight rows of every q and k head
+// come in another order (the caller's copy of the matrix for this kernel alone): the j-th group
+// of 16 rows of a head holds dims 8 j .. 8 j + 7 and, behind them, their rotation partners
+// hd/2 + 8 j .. hd/2 + 8 j + 7. A tile of 16 output columns then has both values of 8 pairs,
+// a lane finds its partners in the lane 32 further on, and every tile is independent of the
+// others, so the matrix is spread over as many workgroups as the plain form's.
 //
 // The weight matrix comes row-major ([rows, K]) or blocked: [rows / 16][K / 32] blocks of 1 KB,
 // a block holding its 16 rows x 32 k in the order of the matrix instruction's operand (lane
@@ -93,7 +97,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
                                                             int M, int N, int K, int tiles, int blocked,
                                                             RopeTarget rope) {
     constexpr bool GATED = EPI == kGated;
-    static_assert(EPI != kRope || TPR == 2, "the rotating epilogue works on pairs of tiles");
     constexpr int NT = GATED ? 2 : 1;                   // weight fragments per k step
     constexpr int KS = NW / TPR;                        // wavefronts that share a tile, splitting k
     constexpr int GV_DEPTH = NW > 8 ? 1 : 2;             // chunks of weights a wavefront has in flight (registers: 128 or 256)
@@ -102,7 +105,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
     bf16* xs = reinterpret_cast<bf16*>(lds_raw);                                    // [16][XS]
     f32x4* red = reinterpret_cast<f32x4*>(lds_raw + static_cast<size_t>(16) * XS * 2);   // [NW][NT][64]
     float* ssum = reinterpret_cast<float*>(red + NW * NT * 64);                      // [16]
-    float* ex = ssum + 16;                                                           // [2][16][16] (rope)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
@@ -145,18 +147,10 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
             }
         }
     };
-    // Which tile this wavefront works on in a round. Rotating epilogue: work item p is a pair of
-    // tiles of one head, hd / 2 columns apart; slot 0 takes the first, slot 1 the second.
+    // Which tile this wavefront works on in a round.
     const int tiles_per_head = (EPI == kRope) ? rope.hd / 16 : 1;
-    auto tile_of = [&](int item) {
-        if (EPI == kRope) {
-            const int half_tiles = tiles_per_head / 2;
-            const int tile = (item / half_tiles) * tiles_per_head + item % half_tiles + slot * half_tiles;
-            return item < tiles / 2 ? tile : tiles;        // past the end: a tile that does not exist
-        }
-        return item * TPR + slot;
-    };
-    const int items = (EPI == kRope) ? tiles / 2 : (tiles + TPR - 1) / TPR;
+    auto tile_of = [&](int item) { return item * TPR + slot; };
+    const int items = (tiles + TPR - 1) / TPR;
     // A wavefront's work in order: unit j is chunk kpart + (j % cpw) KS of the tile of round j / cpw.
     // Every wavefront has the same number of units (chunks past the end of k are zeros that cost
     // nothing), GV_DEPTH of them in flight: a unit's loads are issued GV_DEPTH units ahead, also
@@ -264,18 +258,21 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
             inv = 1.0f / sqrtf(ssum[m] / static_cast<float>(K) + eps);
         }
         if (EPI == kRope) {
-            // both tiles of the pair show each other their values, then each rotates its half
-            if (leader) {
+            // A tile of a q or k head holds dims 8 j .. 8 j + 7 of the first half in its columns 0 .. 7
+            // and their partners in columns 8 .. 15: lanes 0 .. 31 hold first halves, and the lane 32
+            // further on the partners of the same row. A tile of a v head holds 16 dims as they are.
+            const int hd = rope.hd, half = hd / 2;
+            const int head = tile < tiles ? tile / tiles_per_head : 0;      // among q heads, then k heads, then v heads
+            const int j = tile % tiles_per_head, g = lane >> 4;
+            const bool is_q = head < rope.n_q, is_k = !is_q && head < rope.n_q + rope.n_kv;
+            float own[4], other[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) ex[(slot * 16 + m) * 16 + (lane >> 4) * 4 + e] = s[0][e] * inv;
+            for (int e = 0; e < 4; ++e) {
+                own[e] = leader ? s[0][e] * inv : 0.f;
+                other[e] = __shfl_xor(own[e], 32, 64);                       // (every lane of the wavefront takes part)
             }
-            lds_barrier();
             if (leader && m < M) {
-                const int hd = rope.hd, half = hd / 2;
-                const int head = tile / tiles_per_head;                 // among q heads, then k heads, then v heads
-                const int i0 = (tile % tiles_per_head) * 16 - slot * half + (lane >> 4) * 4;   // index within the half
                 const int pos = rope.positions[m];
-                const bool is_q = head < rope.n_q, is_k = !is_q && head < rope.n_q + rope.n_kv;
                 const int kvh = is_q ? 0 : (is_k ? head - rope.n_q : head - rope.n_q - rope.n_kv);
                 size_t page_off = 0;
                 int off = 0;
@@ -286,16 +283,15 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const int i = i0 + e;
-                    const float own = s[0][e] * inv;
-                    float v = own;
+                    float v = own[e];
+                    int d = j * 16 + g * 4 + e;                               // v heads: columns as they are
                     if (is_q || is_k) {
-                        const float other = ex[((slot ^ 1) * 16 + m) * 16 + (lane >> 4) * 4 + e];
+                        const int i = j * 8 + (g & 1) * 4 + e;                // index within the half
                         const float c = rope.cos_t[static_cast<size_t>(pos) * half + i];
                         const float sn = rope.sin_t[static_cast<size_t>(pos) * half + i];
-                        v = slot == 0 ? own * c - other * sn : own * c + other * sn;
+                        v = g < 2 ? own[e] * c - other[e] * sn : own[e] * c + other[e] * sn;
+                        d = g < 2 ? i : half + i;
                     }
-                    const int d = slot * half + i;
                     if (is_q) rope.q_out[(static_cast<size_t>(m) * rope.n_q + head) * hd + d] = static_cast<bf16>(v);
                     else if (is_k) rope.k_cache[page_off + static_cast<size_t>(off) * hd + d] = static_cast<bf16>(v);
                     else rope.v_cache[page_off + static_cast<size_t>(d) * rope.page + off] = static_cast<bf16>(v);
@@ -343,8 +339,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
 template <int NW, int TPR, int EPI, typename TNW>
 static int launch_gemv_norm(const float* h, const int* rows, const void* norm_w, float eps, const bf16* w, void* out,
                             int M, int N, int K, int grid, int blocked, const RopeTarget& rope, hipStream_t stream) {
-    const size_t lds = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(NW) * (EPI == kGated ? 2 : 1) * 64 * 16 +
-                       64 + 2 * 16 * 16 * 4;
+    const size_t lds = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(NW) * (EPI == kGated ? 2 : 1) * 64 * 16 + 64;
     if (lds > 160 * 1024) return kErrUnsupported;
     auto kernel = gemv_norm_kernel<NW, TPR, EPI, TNW>;
     static size_t granted = 0;                          // per instantiation
@@ -398,7 +393,7 @@ extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_
         // more tiles than compute units: 2 tiles at a time, 4 wavefronts each with several chunks of k
         tpr = tiles <= 256 ? 1 : 2;
         // (measured: 16 wavefronts on 2 tiles, 14.2 against 14.8 us at 512 tiles; they need more LDS for their sums)
-        const size_t lds16 = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(16) * 2 * 64 * 16 + 64 + 2 * 16 * 16 * 4;
+        const size_t lds16 = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(16) * 2 * 64 * 16 + 64;
         if (gated && tiles > 256 && tiles <= 1024 && lds16 <= 160 * 1024) tpr = 12;
     }
     if (tpr != 1 && tpr != 2 && tpr != 4 && tpr != 12 && tpr != 14) return kErrBadArgument;
@@ -421,9 +416,11 @@ extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_
 
 // The q/k/v projection of up to 16 rows with the norm in front and rotation plus cache write
 // behind: h [M, K] float32 (row m is batch row m), w [(n_q + 2 n_kv) hd, K] bfloat16 (q heads, k
-// heads, v heads), cos/sin [max_pos, hd / 2]; writes q_out [M, n_q hd] and the rows' k, v into
-// the pages that block_table[seq_idx[m]] names for positions[m]. Full rotation only (all hd
-// dimensions), hd a multiple of 32.
+// heads, v heads; within every q and k head the rows in the order dims 0 .. 7, hd/2 .. hd/2 + 7,
+// 8 .. 15, hd/2 + 8 .. hd/2 + 15, ..: see the head of this file), cos/sin [max_pos, hd / 2];
+// writes q_out [M, n_q hd] and the rows' k, v into the pages that block_table[seq_idx[m]] names
+// for positions[m], all in the usual order of dims. Full rotation only (all hd dimensions), hd a
+// multiple of 16.
 extern "C" int llme_gemv_norm_rope(const float* h, const void* norm_w, int norm_dtype, float eps, const void* w,
                                    const int* positions, const int* seq_idx, const int* block_table, int max_blocks,
                                    const float* cos_t, const float* sin_t, void* q_out, void* k_cache, void* v_cache,
@@ -432,19 +429,23 @@ extern "C" int llme_gemv_norm_rope(const float* h, const void* norm_w, int norm_
     if (M <= 0) return 0;
     if (blocked && K % 32 != 0) return kErrUnsupported;
     if (reinterpret_cast<uintptr_t>(norm_w) % 16 != 0 || reinterpret_cast<uintptr_t>(h) % 16 != 0) return kErrUnsupported;
-    if (M > 16 || K <= 0 || K % 8 != 0 || hd <= 0 || hd % 32 != 0 || n_q <= 0 || n_kv <= 0 || page <= 0)
+    if (M > 16 || K <= 0 || K % 8 != 0 || hd <= 0 || hd % 16 != 0 || n_q <= 0 || n_kv <= 0 || page <= 0)
         return kErrUnsupported;
     if (static_cast<size_t>(16) * (K + 8) * 2 > 132 * 1024) return kErrUnsupported;
     const int N = (n_q + 2 * n_kv) * hd;
     if (static_cast<double>(N) * K * 2 >= 4294967296.0) return kErrUnsupported;   // 32-bit offsets into w
-    const int pairs = N / 32;
-    if (grid <= 0) grid = pairs > 512 ? 512 : pairs;
+    const int tiles = N / 16;
+    const int tpr = tiles <= 256 ? 1 : 2;              // as the plain form
+    if (grid <= 0) grid = (tiles + tpr - 1) / tpr > 512 ? 512 : (tiles + tpr - 1) / tpr;
     const RopeTarget rope{positions, seq_idx, block_table, max_blocks, cos_t, sin_t, static_cast<bf16*>(q_out),
                           static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache), n_q, n_kv, hd, page};
     const bf16* W = static_cast<const bf16*>(w);
-    if (norm_dtype == kBF16)
-        return launch_gemv_norm<16, 2, kRope, bf16>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream);
-    if (norm_dtype == kF32)
-        return launch_gemv_norm<16, 2, kRope, float>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream);
-    return kErrBadArgument;
+    if (norm_dtype != kBF16 && norm_dtype != kF32) return kErrBadArgument;
+    if (tpr == 1)
+        return norm_dtype == kBF16
+            ? launch_gemv_norm<8, 1, kRope, bf16>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream)
+            : launch_gemv_norm<8, 1, kRope, float>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream);
+    return norm_dtype == kBF16
+        ? launch_gemv_norm<8, 2, kRope, bf16>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream)
+        : launch_gemv_norm<8, 2, kRope, float>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream);
 }

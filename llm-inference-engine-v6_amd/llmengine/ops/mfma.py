@@ -226,7 +226,22 @@ declare("llme_gemv_norm_rope", [_vp, _vp, _i, _f, _vp, _vp, _vp, _vp, _i, _vp, _
 
 def gemv_norm_rope_supported(h, norm_weight, w_qkv, k_cache, n_tokens: int, head_dim: int, rotary_dim: int) -> bool:
     return (gemv_norm_supported(h, norm_weight, w_qkv, n_tokens, gated=False) and rotary_dim == head_dim
-            and head_dim % 32 == 0 and k_cache.dtype == torch.bfloat16)
+            and head_dim % 16 == 0 and k_cache.dtype == torch.bfloat16)
+
+
+def pair_rows_for_rotation(w_qkv: torch.Tensor, n_rotated_heads: int, head_dim: int) -> torch.Tensor:
+    """The row order gemv_norm_rope wants of a row-major q/k/v matrix: within each of the first
+    n_rotated_heads heads (the q and k heads), dims 0 .. 7, then their rotation partners
+    hd/2 .. hd/2 + 7, then 8 .. 15, hd/2 + 8 .. hd/2 + 15 and so on; the other rows (v) as they
+    are. head_dim must be a multiple of 16."""
+    if w_qkv.dim() != 2 or head_dim % 16 or n_rotated_heads * head_dim > w_qkv.shape[0]:
+        raise kernels.KernelError(f"pair_rows_for_rotation: a row-major matrix of whole heads of a multiple of 16 dims, "
+                                  f"got {tuple(w_qkv.shape)} for {n_rotated_heads} heads of {head_dim}")
+    half = head_dim // 2
+    within = torch.arange(head_dim).view(2, half // 8, 8).permute(1, 0, 2).reshape(-1)     # [j][half][8]
+    order = (torch.arange(n_rotated_heads)[:, None] * head_dim + within[None, :]).reshape(-1)
+    rest = torch.arange(n_rotated_heads * head_dim, w_qkv.shape[0])
+    return w_qkv[torch.cat([order, rest]).to(w_qkv.device)].contiguous()
 
 
 def gemv_norm_rope(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv: torch.Tensor,
@@ -234,8 +249,9 @@ def gemv_norm_rope(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv
                    sin: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                    n_q: int, n_kv: int, head_dim: int, grid: int = 0) -> None:
     """For up to 16 rows: rmsnorm(h) @ w_qkv^T, q and k heads rotated at the rows' positions, q
-    written to q_out (bfloat16) and k, v into the rows' cache pages. Full rotation, head size a
-    multiple of 32."""
+    written to q_out (bfloat16) and k, v into the rows' cache pages. w_qkv is the q/k/v matrix with
+    the rows of its q and k heads in the order of pair_rows_for_rotation (row-major or blocked);
+    what is written has the usual order of dims. Full rotation, head size a multiple of 16."""
     require(h, "h", torch.float32, (None, None))
     M, K = h.shape
     require(norm_weight, "norm_weight", (torch.float32, torch.bfloat16), (K,))
@@ -252,7 +268,7 @@ def gemv_norm_rope(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv
     page = k_cache.shape[2]
     require(v_cache, "v_cache", torch.bfloat16, (k_cache.shape[0], n_kv, head_dim, page))
     if not gemv_norm_rope_supported(h, norm_weight, w_qkv, k_cache, M, head_dim, head_dim):
-        raise kernels.KernelError(f"gemv_norm_rope: {M} rows (at most 16), head size {head_dim} (multiple of 32) or "
+        raise kernels.KernelError(f"gemv_norm_rope: {M} rows (at most 16), head size {head_dim} (multiple of 16) or "
                                   "the operand types are not supported")
     check(entry("llme_gemv_norm_rope")(
         ptr(h), ptr(norm_weight), 0 if norm_weight.dtype == torch.float32 else 1, float(eps), ptr(w_qkv),

@@ -37,6 +37,7 @@ class Attention(Mixer):
         self.q_dim = self.num_heads * self.head_dim
         self.kv_dim = self.num_kv_heads * self.head_dim
         self.w_qkv: torch.Tensor | None = None
+        self.w_qkv_paired: torch.Tensor | None = None
         self.w_o: torch.Tensor | None = None
 
     def param_specs(self):
@@ -45,6 +46,8 @@ class Attention(Mixer):
                 "v_proj.weight": ParamSpec((self.kv_dim, H)), "o_proj.weight": ParamSpec((H, self.q_dim))}
 
     def load_params(self, get: Getter, placement: Placement) -> None:
+        if self.position is not None and hasattr(self.position, "materialize"):
+            self.position.materialize(placement)
         parts = [get("q_proj.weight"), get("k_proj.weight"), get("v_proj.weight")]
         dtype = placement.common_dtype(parts)
         fused = torch.empty((self.q_dim + 2 * self.kv_dim, self.hidden_size), dtype=dtype,
@@ -55,9 +58,16 @@ class Attention(Mixer):
             row += p.shape[0]
         # (queries alone are sliced off for layers that read another layer's cache: whole row groups)
         self.w_qkv = placement.matrix(fused) if self.q_dim % 16 == 0 else fused
+        # A second copy for decoding, where norm, projection, rotation and cache write are one kernel:
+        # that kernel wants each rotation pair inside one group of 16 rows (ops.pair_rows_for_rotation).
+        # It costs the matrix's memory once more and no traffic: a step reads one copy or the other.
+        self.w_qkv_paired = None
+        rotary = self.position.rotary_tables() if self.position is not None and hasattr(self.position, "rotary_tables") else None
+        if (fused.dtype == torch.bfloat16 and self.head_dim % 16 == 0 and rotary is not None
+                and rotary[2] == self.head_dim):
+            self.w_qkv_paired = placement.matrix(
+                ops.pair_rows_for_rotation(fused, self.num_heads + self.num_kv_heads, self.head_dim))
         self.w_o = placement.place_matrix(get("o_proj.weight"))
-        if self.position is not None and hasattr(self.position, "materialize"):
-            self.position.materialize(placement)
 
     def cache_spec(self) -> CacheSpec:
         return CacheSpec(kind="window" if self.window > 0 else "full", window=self.window,
@@ -86,10 +96,10 @@ class Attention(Mixer):
                 ops.gemv_norm(x, pre_norm.weight, pre_norm.eps, weight, dst)
             else:
                 ops.gemm(x, weight, dst)
-        if (write_cache and pre_norm is not None and cos is not None
-                and ops.gemv_norm_rope_supported(x, pre_norm.weight, self.w_qkv, k_cache, T, hd, rot)):
+        if (write_cache and pre_norm is not None and cos is not None and self.w_qkv_paired is not None
+                and ops.gemv_norm_rope_supported(x, pre_norm.weight, self.w_qkv_paired, k_cache, T, hd, rot)):
             # decoding: norm, projection, rotation and the cache write are one kernel
-            ops.gemv_norm_rope(x, pre_norm.weight, pre_norm.eps, self.w_qkv, step.positions, step.seq_idx,
+            ops.gemv_norm_rope(x, pre_norm.weight, pre_norm.eps, self.w_qkv_paired, step.positions, step.seq_idx,
                                block_table, cos, sin, q, k_cache, v_cache, n_q, n_kv, hd)
         elif write_cache:
             qkv = step.buffer("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)

@@ -489,7 +489,8 @@ def test_gemv_norm_refusals(ops):
 
 
 @pytest.mark.parametrize("M,n_q,n_kv,hd,K,page", [(1, 4, 2, 32, 64, 16), (8, 32, 8, 64, 2048, 16), (16, 3, 1, 96, 96, 32),
-                                                  (5, 6, 2, 128, 144, 16), (3, 40, 8, 64, 256, 64)])
+                                                  (5, 6, 2, 128, 144, 16), (3, 40, 8, 64, 256, 64), (4, 5, 1, 48, 72, 16),
+                                                  (2, 2, 2, 16, 40, 16), (7, 24, 8, 128, 512, 16)])
 @pytest.mark.parametrize("grid", [0, 3])
 def test_gemv_norm_rope(ops, M, n_q, n_kv, hd, K, page, grid):
     """The fused kernel against its parts: norm, projection, rotation, cache write."""
@@ -508,7 +509,8 @@ def test_gemv_norm_rope(ops, M, n_q, n_kv, hd, K, page, grid):
     k_cache = torch.zeros(M * 5, n_kv, page, hd, dtype=torch.bfloat16, device=DEV)
     v_cache = torch.zeros(M * 5, n_kv, hd, page, dtype=torch.bfloat16, device=DEV)
     q_out = torch.zeros(M, n_q * hd, dtype=torch.bfloat16, device=DEV)
-    ops.gemv_norm_rope(h.to(DEV), nw.to(DEV), 1e-5, w.to(DEV), positions.to(DEV), seq_idx.to(DEV), table.to(DEV),
+    paired = ops.pair_rows_for_rotation(w, n_q + n_kv, hd)          # the kernel's own order of the q and k rows
+    ops.gemv_norm_rope(h.to(DEV), nw.to(DEV), 1e-5, paired.to(DEV), positions.to(DEV), seq_idx.to(DEV), table.to(DEV),
                        cos.to(DEV), sin.to(DEV), q_out, k_cache, v_cache, n_q, n_kv, hd, grid=grid)
     x = plain_rmsnorm(h.double(), nw.double(), 1e-5)
     qkv = plain_linear(x, w.double())

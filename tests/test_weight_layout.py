@@ -49,6 +49,22 @@ def test_where_an_element_lies(ops):
             ops.block_weight(bad)
 
 
+def test_rows_paired_for_rotation(ops):
+    """Within a rotated head: dims 0 .. 7, their partners hd/2 .. hd/2 + 7, then 8 .. 15 and so on."""
+    n_q, n_kv, hd, K = 2, 1, 32, 8
+    w = torch.arange((n_q + 2 * n_kv) * hd, dtype=torch.float32)[:, None].repeat(1, K)     # row n holds n
+    got = ops.pair_rows_for_rotation(w, n_q + n_kv, hd)[:, 0].tolist()
+    head = list(range(0, 8)) + list(range(16, 24)) + list(range(8, 16)) + list(range(24, 32))
+    want = [h * hd + d for h in range(n_q + n_kv) for d in head] + list(range((n_q + n_kv) * hd, (n_q + 2 * n_kv) * hd))
+    assert got == want
+    same = ops.pair_rows_for_rotation(w[:, :8].contiguous(), 0, hd)
+    assert torch.equal(same, w[:, :8])
+    assert torch.equal(ops.pair_rows_for_rotation(torch.arange(64.)[:, None].repeat(1, 8), 4, 16)[:, 0], torch.arange(64.))
+    from llmengine.ops import KernelError
+    with pytest.raises(KernelError):
+        ops.pair_rows_for_rotation(w, 3, 24)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 2048), (8, 3072, 2048), (16, 48, 96), (33, 96, 96), (64, 2048, 8192),
                                    (50, 128, 992), (3, 16, 32)])
@@ -188,7 +204,8 @@ def test_norm_product_rotation_and_cache_write(ops, M, n_q, n_kv, hd, K, page, g
     ang = torch.arange(5 * page, dtype=torch.float64)[:, None] * inv[None, :]
     cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
     got = []
-    for weight in (w, ops.block_weight(w)):
+    paired = ops.pair_rows_for_rotation(w, n_q + n_kv, hd)
+    for weight in (paired, ops.block_weight(paired)):
         k_cache = torch.zeros(M * 5, n_kv, page, hd, dtype=torch.bfloat16, device=DEV)
         v_cache = torch.zeros(M * 5, n_kv, hd, page, dtype=torch.bfloat16, device=DEV)
         q_out = torch.zeros(M, n_q * hd, dtype=torch.bfloat16, device=DEV)
