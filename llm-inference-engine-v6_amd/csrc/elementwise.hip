@@ -422,7 +422,9 @@ extern "C" int llme_rope_kv_write(const float* qkv, const float* cos_t, const fl
                      reinterpret_cast<uintptr_t>(k_cache) % 16 == 0 && reinterpret_cast<uintptr_t>(cos_t) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(sin_t) % 16 == 0;
     // many tokens: 16 per workgroup, v written in pieces of 16 positions where they lie together
-    const bool grouped = vec && T >= 4 * ROPE_GROUP && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
+    // (up to 256 tokens, which may be as many decoding requests with a page each, a workgroup per
+    // token is faster: 5.2 against 9.5 us for 64 single tokens)
+    const bool grouped = vec && T > 16 * ROPE_GROUP && reinterpret_cast<uintptr_t>(v_cache) % 16 == 0;
 #define LLME_ROPE(TQ, TC)                                                                                   \
     do {                                                                                                    \
         if (grouped)                                                                                        \

@@ -532,13 +532,13 @@ def test_gemv_norm_rope(ops, M, n_q, n_kv, hd, K, page, grid):
 
 @pytest.mark.parametrize("n_q,n_kv,hd,page", [(4, 2, 64, 16), (3, 1, 128, 48), (6, 3, 80, 32), (2, 2, 16, 16)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_rope_write_of_many_tokens(ops, n_q, n_kv, hd, page, dtype):
+@pytest.mark.parametrize("new", [[40, 50, 3, 16, 33], [104, 114, 3, 48, 65]])     # a workgroup per token; 16 tokens per workgroup
+def test_rope_write_of_many_tokens(ops, n_q, n_kv, hd, page, dtype, new):
     """Rotation and cache write for a step of many tokens (16 tokens per workgroup, v written in
     pieces of 16 positions where they lie together in a page): portions that start at multiples
     of 16, portions that do not, a request shorter than a group, and groups that span two
     requests. Every written place of both caches is compared, and no other place is touched."""
     ctx = [32, 5, 0, 48, 16]                      # tokens already cached
-    new = [40, 50, 3, 16, 33]                     # tokens of this step
     T, S = sum(new), len(new)
     g = _gen(71)
     qkv = torch.randn(T, (n_q + 2 * n_kv) * hd, generator=g)
