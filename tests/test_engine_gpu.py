@@ -307,10 +307,11 @@ def _random_configuration(case: int):
     n_kv, group = r.choice([1, 2, 3, 5]), r.choice([1, 2, 3, 4, 7])
     cfg = {"architectures": ["LlamaForCausalLM"], "model_type": "llama",
            "head_dim": r.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 256]),
-           "hidden_size": r.choice([34, 50, 72, 100, 136, 200, 264]),
-           "intermediate_size": r.choice([50, 98, 176, 264, 400]), "num_hidden_layers": r.choice([1, 2, 3]),
+           # (widths that are multiples of 32 put the matrices into the blocked layout, the others do not)
+           "hidden_size": r.choice([34, 50, 64, 72, 96, 100, 136, 160, 200, 264, 288]),
+           "intermediate_size": r.choice([50, 98, 128, 176, 264, 352, 400]), "num_hidden_layers": r.choice([1, 2, 3]),
            "num_attention_heads": n_kv * group, "num_key_value_heads": n_kv,
-           "vocab_size": r.choice([50, 257, 384, 701]), "max_position_embeddings": 512,
+           "vocab_size": r.choice([50, 257, 384, 512, 701]), "max_position_embeddings": 512,
            "rms_norm_eps": r.choice([1e-5, 1e-6]), "rope_theta": r.choice([1e4, 5e5]),
            "tie_word_embeddings": r.random() < 0.5}
     if r.random() < 0.5:
@@ -319,7 +320,7 @@ def _random_configuration(case: int):
     return cfg, r.choice([4, 8, 16, 16, 32, 48, 64]), [r.randint(1, 220) for _ in range(4)]
 
 
-@pytest.mark.parametrize("case", range(10))
+@pytest.mark.parametrize("case", range(14))
 def test_random_configurations(case):
     """Sizes drawn at random from what a configuration allows: head sizes in steps of 16 up to 256,
     odd numbers of heads and groups, widths that are no multiple of 8, any page size. 32-bit against
