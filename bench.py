@@ -104,8 +104,8 @@ def serve(args, engine, cfg: dict, gen, page: int) -> int:
     news = [int(torch.randint(nlo, nhi + 1, (1,), generator=gen)) for _ in range(args.requests)]
     pages = sum((len(p) + n + page - 1) // page for p, n in zip(prompts, news))
     runs = []
-    for rep in range(2):                                       # the first run warms up (and records the graphs)
-        manager = BlockManager(pages, page)
+    manager = BlockManager(pages, page)                        # one pool for both runs: the second finds the decode
+    for rep in range(2):                                       # steps' HIP graphs that the first recorded over it
         sched = ContinuousBatchScheduler(engine, manager, max_concurrent=args.max_concurrent,
                                          max_prefill_tokens_per_step=args.prefill_budget)
         for p, n in zip(prompts, news):
@@ -122,7 +122,7 @@ def serve(args, engine, cfg: dict, gen, page: int) -> int:
         log(f"serve run {rep}: {len(results)} requests, {sum(map(len, prompts))} prompt tokens, {generated} generated "
             f"in {dt:.2f} s over {sched.steps} steps ({generated / dt:.0f} generated tok/s; finished: {reasons})")
         assert manager.free_blocks == pages, "pages were lost"
-        del sched, manager
+        del sched
     dt, generated, steps = runs[-1]
     prompt_tokens = sum(map(len, prompts))
     print(json.dumps({
