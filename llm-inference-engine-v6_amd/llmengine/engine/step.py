@@ -200,6 +200,7 @@ class ModelRunner:
     """A loaded model on a device plus the scratch memory its steps use."""
 
     GRAPH_BLOCK_BUCKET = 64         # block-table widths of recorded steps are multiples of this
+    GRAPH_LIMIT = 192               # recorded steps kept per page pool; the least recently used one goes first
 
     def __init__(self, model: DecoderModel, dtype: torch.dtype, device: torch.device, use_graphs: bool = True):
         self.model = model
@@ -283,8 +284,12 @@ class ModelRunner:
         bucket = self.GRAPH_BLOCK_BUCKET
         width = (need + bucket - 1) // bucket * bucket
         key = (S, width, greedy)
-        rec = cache.graphs.get(key)
+        rec = cache.graphs.pop(key, None)
+        if rec is not None:
+            cache.graphs[key] = rec                      # (most recently used last)
         if rec is None:
+            while len(cache.graphs) >= self.GRAPH_LIMIT:
+                del cache.graphs[next(iter(cache.graphs))]
             # First time: run it plainly (this also sizes the scratch buffers), then record.
             # The recorded step reads its integer arrays from a buffer of its own.
             groups = len(mgr.groups)

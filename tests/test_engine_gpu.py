@@ -167,20 +167,23 @@ def model_c(tmp_path_factory):
     return d
 
 
-@pytest.mark.parametrize("graphs", ["recorded", "recorded-narrow", "plain"])
+@pytest.mark.parametrize("graphs", ["recorded", "recorded-narrow", "recorded-few", "plain"])
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
 def test_long_decoding(model_c, dtype, graphs, monkeypatch):
     """A 40-token prompt, then 400 tokens decoded one by one: positions far beyond the rope
     scaling's original length, many pages, logits compared at every position. Decode steps are
     replayed from a recorded HIP graph ("recorded"; "recorded-narrow" records a new one every 32
-    tokens, so that replays, new recordings and plain steps alternate) or launched plainly."""
+    tokens, so that replays, new recordings and plain steps alternate; "recorded-few" also keeps
+    three recordings at most, so that old ones are dropped on the way) or launched plainly."""
     from llmengine import Engine
     from llmengine.engine.step import ModelRunner
     ids = random_tokens(440, TINY_C["vocab_size"], 7)
     pcfg, pw = load_plain_model(model_c)
     ref = plain_forward(pcfg, pw, ids, rounder=bf16_round if dtype == "bf16" else None).numpy()
-    if graphs == "recorded-narrow":
+    if graphs in ("recorded-narrow", "recorded-few"):
         monkeypatch.setattr(ModelRunner, "GRAPH_BLOCK_BUCKET", 2)
+    if graphs == "recorded-few":
+        monkeypatch.setattr(ModelRunner, "GRAPH_LIMIT", 3)
     engine = Engine(model_c, dtype, use_graphs=graphs != "plain")
     steps = replay.tail_one_by_one({"long": ids}, tail=400)
     cache = engine.new_cache(28, 16, max_requests=1)
@@ -189,7 +192,7 @@ def test_long_decoding(model_c, dtype, graphs, monkeypatch):
         err = np.abs(got[pos] - ref[pos]).max() / np.abs(ref[pos]).max()
         assert err < TOL[dtype], f"position {pos}: {err:.3e}"
     assert (engine.runner.graph_replays > 300) == (graphs != "plain")
-    assert len(cache.graphs) == {"recorded": 1, "recorded-narrow": 13, "plain": 0}[graphs]
+    assert len(cache.graphs) == {"recorded": 1, "recorded-narrow": 13, "recorded-few": 3, "plain": 0}[graphs]
 
 
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
