@@ -14,7 +14,7 @@
 // through tiles of 16 output columns (gated: the 16 gate and the 16 up rows of 16 units, which
 // lie next to each other in the interleaved weight matrix), TPR tiles at a time: NW / TPR
 // wavefronts share a tile, each streaming every (NW / TPR)-th 128-element chunk of k of the
-// tile's weight rows from HBM straight into MFMA operand registers, four chunks ahead (two with 16
+// tile's weight rows from HBM straight into MFMA operand registers, two chunks ahead (one with 16
 // wavefronts), also across tiles; the partial sums are added through LDS, scaled by inv_m and stored. The grid
 // is sized so that the prologue is paid once per several tiles.
 //
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
     constexpr bool GATED = EPI == kGated;
     constexpr int NT = GATED ? 2 : 1;                   // weight fragments per k step
     constexpr int KS = NW / TPR;                        // wavefronts that share a tile, splitting k
-    constexpr int GV_DEPTH = NW > 8 ? 1 : 2;             // chunks of weights a wavefront has in flight (registers: 128 or 256)
+    constexpr int GV_DEPTH = NW > 8 ? 1 : 2;             // chunks of weights a wavefront has in flight (measured: more stream more slowly)
     extern __shared__ __align__(16) unsigned char lds_raw[];
     const int XS = K + 8;                               // padded row of the activation tile (elements)
     bf16* xs = reinterpret_cast<bf16*>(lds_raw);                                    // [16][XS]

@@ -49,7 +49,8 @@ def weight_shape(w: torch.Tensor) -> tuple[int, int]:
 
 
 def can_block(w: torch.Tensor) -> bool:
-    return w.dim() == 2 and w.dtype == torch.bfloat16 and w.shape[0] % 16 == 0 and w.shape[1] % 32 == 0
+    return (w.dim() == 2 and w.dtype == torch.bfloat16 and w.shape[0] % 16 == 0 and w.shape[1] % 32 == 0
+            and w.is_contiguous())
 
 
 def block_weight(w: torch.Tensor) -> torch.Tensor:
