@@ -235,9 +235,25 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
 
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // Rotating epilogue: where this lane's row goes (its position, its page) is asked for now, and a
+    // round's table values before its sums are added up: each is a trip to memory that the
+    // epilogue would otherwise wait for one after the other at the kernel's very end.
+    int row_pos = 0, row_page = 0;
+    if (EPI == kRope && kpart == 0 && (lane & 15) < M) {
+        row_pos = rope.positions[lane & 15];
+        row_page = rope.block_table[static_cast<size_t>(rope.seq_idx[lane & 15]) * rope.max_blocks + row_pos / rope.page];
+    }
     // the end of a round: the sums are added up, scaled and stored (further down)
     auto finish_round = [&](int round) {
         const int tile = tile_of(round * gridDim.x + blockIdx.x);
+        float4 cs4 = float4{1.f, 1.f, 1.f, 1.f}, sn4 = float4{0.f, 0.f, 0.f, 0.f};
+        if (EPI == kRope && kpart == 0 && tile < tiles && (lane & 15) < M &&
+            tile / tiles_per_head < rope.n_q + rope.n_kv) {
+            // (four neighbouring values, 16-byte aligned: hd / 2 and the index are multiples of 4)
+            const size_t at = static_cast<size_t>(row_pos) * (rope.hd / 2) + (tile % tiles_per_head) * 8 + ((lane >> 4) & 1) * 4;
+            cs4 = *reinterpret_cast<const float4*>(rope.cos_t + at);
+            sn4 = *reinterpret_cast<const float4*>(rope.sin_t + at);
+        }
 #pragma unroll
         for (int t = 0; t < NT; ++t) red[(wave * NT + t) * 64 + lane] = acc[t];
         lds_barrier();
@@ -272,23 +288,17 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
                 other[e] = __shfl_xor(own[e], 32, 64);                       // (every lane of the wavefront takes part)
             }
             if (leader && m < M) {
-                const int pos = rope.positions[m];
                 const int kvh = is_q ? 0 : (is_k ? head - rope.n_q : head - rope.n_q - rope.n_kv);
-                size_t page_off = 0;
-                int off = 0;
-                if (!is_q) {
-                    const int pg = rope.block_table[static_cast<size_t>(rope.seq_idx[m]) * rope.max_blocks + pos / rope.page];
-                    off = pos % rope.page;
-                    page_off = (static_cast<size_t>(pg) * rope.n_kv + kvh) * rope.page * hd;
-                }
+                const int off = row_pos % rope.page;
+                const size_t page_off = (static_cast<size_t>(row_page) * rope.n_kv + kvh) * rope.page * hd;
+                const float cs[4] = {cs4.x, cs4.y, cs4.z, cs4.w}, sns[4] = {sn4.x, sn4.y, sn4.z, sn4.w};
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     float v = own[e];
                     int d = j * 16 + g * 4 + e;                               // v heads: columns as they are
                     if (is_q || is_k) {
                         const int i = j * 8 + (g & 1) * 4 + e;                // index within the half
-                        const float c = rope.cos_t[static_cast<size_t>(pos) * half + i];
-                        const float sn = rope.sin_t[static_cast<size_t>(pos) * half + i];
+                        const float c = cs[e], sn = sns[e];
                         v = g < 2 ? own[e] * c - other[e] * sn : own[e] * c + other[e] * sn;
                         d = g < 2 ? i : half + i;
                     }
@@ -431,6 +441,8 @@ extern "C" int llme_gemv_norm_rope(const float* h, const void* norm_w, int norm_
     if (reinterpret_cast<uintptr_t>(norm_w) % 16 != 0 || reinterpret_cast<uintptr_t>(h) % 16 != 0) return kErrUnsupported;
     if (M > 16 || K <= 0 || K % 8 != 0 || hd <= 0 || hd % 16 != 0 || n_q <= 0 || n_kv <= 0 || page <= 0)
         return kErrUnsupported;
+    if (reinterpret_cast<uintptr_t>(cos_t) % 16 != 0 || reinterpret_cast<uintptr_t>(sin_t) % 16 != 0)
+        return kErrUnsupported;                        // the tables are read four values at a time
     if (static_cast<size_t>(16) * (K + 8) * 2 > 132 * 1024) return kErrUnsupported;
     const int N = (n_q + 2 * n_kv) * hd;
     if (static_cast<double>(N) * K * 2 >= 4294967296.0) return kErrUnsupported;   // 32-bit offsets into w

@@ -263,6 +263,8 @@ def gemv_norm_rope(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv
     require(block_table, "block_table", torch.int32, (None, None))
     require(cos, "cos", torch.float32, (None, head_dim // 2))
     require(sin, "sin", torch.float32, tuple(cos.shape))
+    if cos.data_ptr() % 16 or sin.data_ptr() % 16:
+        raise kernels.KernelError("gemv_norm_rope: the rotation tables must be 16-byte aligned")
     require(q_out, "q_out", torch.bfloat16, (M, n_q * head_dim))
     require(k_cache, "k_cache", torch.bfloat16, (None, n_kv, None, head_dim))
     page = k_cache.shape[2]
