@@ -51,15 +51,23 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     __shared__ float sh_o[DEC_WAVES][16][HD];
     __shared__ float sh_m[DEC_WAVES][16], sh_l[DEC_WAVES][16];
     const int s = blockIdx.x;
-    const int row0 = q_start[s];
-    if (q_start[s + 1] - row0 != 1) return;            // not a decoding request (whole workgroup)
+    // What the walk over the keys needs first is asked for together, before anything depends on
+    // it: the request's rows, its length, and the line of its block table that this split's first
+    // page ids lie in (the walk's own lookups then find it in the cache). One after the other
+    // these were three trips to memory in front of the first key.
+    const int row0 = q_start[s], row1 = q_start[s + 1];
+    const int pos = ctx_len[s];                         // the token's position; it sees keys lo..pos
+    const long first_block = static_cast<long>(blockIdx.z) * split_len / page;
+    const int table_line = block_table[static_cast<size_t>(s) * max_blocks +
+                                       (first_block < max_blocks ? first_block : max_blocks - 1)];
+    if (row1 - row0 != 1) return;                       // not a decoding request (whole workgroup)
+    asm volatile("" ::"v"(table_line));                 // (the load is wanted for its effect on the cache)
     const int G = n_q / n_kv;
     const int gtiles = (G + 15) / 16;
     const int kvh = blockIdx.y / gtiles, gt = blockIdx.y % gtiles;
     const int split = blockIdx.z;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g4 = lane >> 4;
 
-    const int pos = ctx_len[s];                         // the token's position; it sees keys lo..pos
     const int lo_all = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
     int k_begin = split * split_len, k_end = k_begin + split_len;
     if (k_end > pos + 1) k_end = pos + 1;
