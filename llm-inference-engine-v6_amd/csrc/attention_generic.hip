@@ -1,5 +1,7 @@
 // Attention over cache pages, plain-precision kernel: one wavefront per (token, query
-// head), scores, softmax statistics and the weighted sum all in 32-bit. It serves the
+// head), or, when a step has few tokens (decoding), several that take every NW-th chunk of the
+// keys and join their results through LDS; scores, softmax statistics and the weighted sum all
+// in 32-bit. It serves the
 // 32-bit model, and the bfloat16 model for head sizes or page sizes that the MFMA
 // kernels refuse. Any head size up to 256, any page size, any head counts.
 //
@@ -22,17 +24,19 @@ namespace llme {
 
 constexpr int kMaxHead = 256;
 
-template <typename TQ, typename TC>
-__global__ __launch_bounds__(64) void attention_generic_kernel(
+template <typename TQ, typename TC, int NW>
+__global__ __launch_bounds__(NW * 64) void attention_generic_kernel(
     const TQ* __restrict__ q, const TC* __restrict__ k_cache, const TC* __restrict__ v_cache,
     TQ* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ seq_idx,
     const int* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int hd, int page, float scale,
     int window) {
+    constexpr int PER_LANE = kMaxHead / kWave;
     __shared__ float qs[kMaxHead];
-    __shared__ float ps[kWave];
+    __shared__ float join_m[NW], join_l[NW];
+    __shared__ float join_acc[NW > 1 ? NW : 1][NW > 1 ? kMaxHead : 1];
     const int t = blockIdx.x;
     const int h = blockIdx.y;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int kvh = h / (n_q / n_kv);
     const int pos = positions[t];
     const int* table = block_table + static_cast<size_t>(seq_idx[t]) * max_blocks;
@@ -40,13 +44,14 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
 
     const TQ* qrow = q + (static_cast<size_t>(t) * n_q + h) * hd;
-    for (int d = lane; d < hd; d += kWave) qs[d] = to_float(qrow[d]);
+    for (int d = threadIdx.x; d < hd; d += NW * kWave) qs[d] = to_float(qrow[d]);
     __syncthreads();
 
     float m = -INFINITY, l = 0.f;
-    float acc[kMaxHead / kWave] = {0.f, 0.f, 0.f, 0.f};
+    float acc[PER_LANE] = {0.f, 0.f, 0.f, 0.f};
 
-    for (int t0 = lo; t0 < hi; t0 += kWave) {
+    // this wavefront's chunks of 64 keys (no barrier inside: the wavefronts take different numbers of turns)
+    for (int t0 = lo + wave * kWave; t0 < hi; t0 += NW * kWave) {
         const int key = t0 + lane;
         float sc = -INFINITY;
         if (key < hi) {
@@ -61,28 +66,48 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
         const float p = (key < hi) ? expf(sc - m_new) : 0.f;
         l = l * alpha + wave_sum(p);
         m = m_new;
-        ps[lane] = p;
-        __syncthreads();
 #pragma unroll
-        for (int i = 0; i < kMaxHead / kWave; ++i) acc[i] *= alpha;
+        for (int i = 0; i < PER_LANE; ++i) acc[i] *= alpha;
         const int n = (hi - t0 < kWave) ? hi - t0 : kWave;
         for (int j = 0; j < n; ++j) {
             const int kj = t0 + j;
             const int pg = table[kj / page];
             const TC* vb = v_cache + (static_cast<size_t>(pg) * n_kv + kvh) * hd * page + kj % page;
-            const float pj = ps[j];
+            const float pj = __shfl(p, j, kWave);
 #pragma unroll
-            for (int i = 0; i < kMaxHead / kWave; ++i) {
+            for (int i = 0; i < PER_LANE; ++i) {
                 const int d = lane + i * kWave;
                 if (d < hd) acc[i] = fmaf(pj, to_float(vb[static_cast<size_t>(d) * page]), acc[i]);
             }
         }
+    }
+    if (NW > 1) {
+        // join the wavefronts' parts: each is scaled to the common maximum (a wavefront that saw no
+        // key has m = -inf and l = 0: its weight is 0; the first wavefront always saw key lo)
+        if (lane == 0) {
+            join_m[wave] = m;
+            join_l[wave] = l;
+        }
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i) join_acc[wave][lane + i * kWave] = acc[i];
         __syncthreads();
+        if (wave != 0) return;
+        float mx = -INFINITY;
+        for (int w = 0; w < NW; ++w) mx = fmaxf(mx, join_m[w]);
+        l = 0.f;
+#pragma unroll
+        for (int i = 0; i < PER_LANE; ++i) acc[i] = 0.f;
+        for (int w = 0; w < NW; ++w) {
+            const float f = expf(join_m[w] - mx);
+            l += f * join_l[w];
+#pragma unroll
+            for (int i = 0; i < PER_LANE; ++i) acc[i] += f * join_acc[w][lane + i * kWave];
+        }
     }
     const float inv = 1.0f / l;
     TQ* orow = out + (static_cast<size_t>(t) * n_q + h) * hd;
 #pragma unroll
-    for (int i = 0; i < kMaxHead / kWave; ++i) {
+    for (int i = 0; i < PER_LANE; ++i) {
         const int d = lane + i * kWave;
         if (d < hd) orow[d] = from_float<TQ>(acc[i] * inv);
     }
@@ -99,11 +124,21 @@ extern "C" int llme_attention_generic(const void* q, int q_dtype, const void* k_
     if (T <= 0) return 0;
     if (hd <= 0 || hd > kMaxHead || n_kv <= 0 || n_q % n_kv != 0 || page <= 0) return kErrBadArgument;
     const dim3 grid(T, n_q);
-#define LLME_ATTN(TQ, TC)                                                                           \
-    hipLaunchKernelGGL((attention_generic_kernel<TQ, TC>), grid, dim3(64), 0, stream,               \
-                       static_cast<const TQ*>(q), static_cast<const TC*>(k_cache),                  \
-                       static_cast<const TC*>(v_cache), static_cast<TQ*>(out), positions, seq_idx,  \
-                       block_table, max_blocks, n_q, n_kv, hd, page, scale, window)
+    // few (token, head) pairs, as in decoding: 16 wavefronts each, so that the chip has work
+    const bool few = static_cast<long>(T) * n_q < 4096;
+#define LLME_ATTN(TQ, TC)                                                                              \
+    do {                                                                                               \
+        if (few)                                                                                       \
+            hipLaunchKernelGGL((attention_generic_kernel<TQ, TC, 16>), grid, dim3(16 * 64), 0, stream, \
+                               static_cast<const TQ*>(q), static_cast<const TC*>(k_cache),             \
+                               static_cast<const TC*>(v_cache), static_cast<TQ*>(out), positions,      \
+                               seq_idx, block_table, max_blocks, n_q, n_kv, hd, page, scale, window);  \
+        else                                                                                           \
+            hipLaunchKernelGGL((attention_generic_kernel<TQ, TC, 1>), grid, dim3(64), 0, stream,       \
+                               static_cast<const TQ*>(q), static_cast<const TC*>(k_cache),             \
+                               static_cast<const TC*>(v_cache), static_cast<TQ*>(out), positions,      \
+                               seq_idx, block_table, max_blocks, n_q, n_kv, hd, page, scale, window);  \
+    } while (0)
     if (q_dtype == kF32 && cache_dtype == kF32) LLME_ATTN(float, float);
     else if (q_dtype == kBF16 && cache_dtype == kBF16) LLME_ATTN(bf16, bf16);
     else if (q_dtype == kF32 && cache_dtype == kBF16) LLME_ATTN(float, bf16);

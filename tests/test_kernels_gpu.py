@@ -149,7 +149,8 @@ def _paged_setup(ops, lens, n_q, n_kv, hd, page, dtype, seed, rotate=True, scram
 
 @pytest.mark.parametrize("n_q,n_kv,hd,page,lens", [
     (4, 2, 32, 4, [1]), (4, 2, 32, 4, [7]), (8, 2, 16, 8, [13, 5]), (3, 1, 48, 16, [33, 2, 17]),
-    (6, 3, 80, 16, [70]), (4, 4, 128, 32, [65, 40]), (2, 1, 256, 16, [20])])
+    (6, 3, 80, 16, [70]), (4, 4, 128, 32, [65, 40]), (2, 1, 256, 16, [20]),
+    (8, 2, 32, 16, [300, 230])])        # (4,096 (token, head) pairs and more: one wavefront each; fewer: 16 that join)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rope_write_and_attention_generic(ops, n_q, n_kv, hd, page, lens, dtype):
     s = _paged_setup(ops, lens, n_q, n_kv, hd, page, dtype, seed=11)
