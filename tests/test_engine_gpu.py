@@ -286,7 +286,7 @@ def test_real_layer_sizes_match_plain(wide, dtype):
     from llmengine import Engine
     cfg, tensors, reqs, rows, plain = wide
     engine = Engine(None, dtype, _config=cfg, _tensors=dict(tensors), block_size=16)
-    for name in ("whole", "tail", "mixed3"):
+    for name in ("whole", "tail", "portions", "mixed3"):
         steps = replay.want_only(SCHEDULES[name](reqs), rows)
         pages = replay.trace_peak_tokens(steps, round_to=16) // 16
         cache = engine.new_cache(pages, 16, max_requests=4)
