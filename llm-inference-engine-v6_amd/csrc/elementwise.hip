@@ -65,25 +65,64 @@ __global__ void embed_gather_blocked_kernel(const bf16* __restrict__ table, cons
 // ---------------------------------------------------------------------------------
 // out[r, i] = w[i] * x[row(r), i] * rsqrt(mean_i x^2 + eps)   (src/kernels.cpp:18-24)
 // row(r) = rows ? rows[r] : r. The product is evaluated (w*x)*inv as the reference does.
-template <typename TW, typename TO>
+// Four neighbouring values of a weight vector or of an output row in one load or store.
+template <typename T>
+__device__ __forceinline__ void norm_load4(const T* p, float (&v)[4]);
+template <>
+__device__ __forceinline__ void norm_load4<float>(const float* p, float (&v)[4]) {
+    const float4 x = *reinterpret_cast<const float4*>(p);
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+}
+template <>
+__device__ __forceinline__ void norm_load4<bf16>(const bf16* p, float (&v)[4]) {
+    typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+    const bf16x4 x = *reinterpret_cast<const bf16x4*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = static_cast<float>(x[i]);
+}
+template <typename T>
+__device__ __forceinline__ void norm_store4(T* p, const float (&v)[4]);
+template <>
+__device__ __forceinline__ void norm_store4<float>(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = float4{v[0], v[1], v[2], v[3]};
+}
+template <>
+__device__ __forceinline__ void norm_store4<bf16>(bf16* p, const float (&v)[4]) {
+    typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+    bf16x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = static_cast<__bf16>(v[i]);
+    *reinterpret_cast<bf16x4*>(p) = o;
+}
+
+// VEC: the row's length is a multiple of 4, at most 32 * blockDim, and x, w and out are aligned
+// for 16-byte (bfloat16: 8-byte) accesses: a thread then keeps its up to 8 groups of four values
+// and their weights in registers between the two passes, all asked for at once, and stores four
+// values at a time. Otherwise the row is read twice, value by value.
+template <typename TW, typename TO, bool VEC>
 __global__ void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ w,
                                TO* __restrict__ out, const int* __restrict__ rows, int H, float eps) {
     __shared__ float scratch[16];
+    constexpr int NV = 8;
     const int r = blockIdx.x;
     const int src = rows ? rows[r] : r;
     const float* xr = x + static_cast<size_t>(src) * H;
     TO* o = out + static_cast<size_t>(r) * H;
-    // Rows of up to 8 * blockDim values whose length is a multiple of 4 stay in registers
-    // between the two passes (two 16-byte loads per thread); others are read twice.
-    const bool in_regs = (H % 4 == 0) && (H <= 8 * static_cast<int>(blockDim.x));
-    float4 v[2];
+    float v[NV][4], wv[NV][4];
     float ss = 0.f;
-    if (in_regs) {
+    if (VEC) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < NV; ++j) {
             const int i = (threadIdx.x + j * blockDim.x) * 4;
-            v[j] = (i < H) ? *reinterpret_cast<const float4*>(xr + i) : float4{0.f, 0.f, 0.f, 0.f};
-            ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+            if (i < H) {
+                norm_load4<float>(xr + i, v[j]);
+                norm_load4<TW>(w + i, wv[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int i = (threadIdx.x + j * blockDim.x) * 4;
+            if (i < H) ss += v[j][0] * v[j][0] + v[j][1] * v[j][1] + v[j][2] * v[j][2] + v[j][3] * v[j][3];
         }
     } else {
         for (int i = threadIdx.x; i < H; i += blockDim.x) {
@@ -93,15 +132,15 @@ __global__ void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict
     }
     ss = block_sum(ss, scratch, blockDim.x / kWave);
     const float inv = 1.0f / sqrtf(ss / static_cast<float>(H) + eps);
-    if (in_regs) {
+    if (VEC) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < NV; ++j) {
             const int i = (threadIdx.x + j * blockDim.x) * 4;
             if (i >= H) continue;
-            o[i] = from_float<TO>((to_float(w[i]) * v[j].x) * inv);
-            o[i + 1] = from_float<TO>((to_float(w[i + 1]) * v[j].y) * inv);
-            o[i + 2] = from_float<TO>((to_float(w[i + 2]) * v[j].z) * inv);
-            o[i + 3] = from_float<TO>((to_float(w[i + 3]) * v[j].w) * inv);
+            float y[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) y[e] = (wv[j][e] * v[j][e]) * inv;
+            norm_store4<TO>(o + i, y);
         }
     } else {
         for (int i = threadIdx.x; i < H; i += blockDim.x)
@@ -380,9 +419,17 @@ extern "C" int llme_embed_gather(const void* table, int table_dtype, const int* 
 extern "C" int llme_rmsnorm(const float* x, const void* w, int w_dtype, void* out, int out_dtype,
                             const int* rows, int R, int H, float eps, hipStream_t stream) {
     if (R <= 0) return 0;
-#define LLME_NORM(TW, TO)                                                                        \
-    hipLaunchKernelGGL((rmsnorm_kernel<TW, TO>), dim3(R), dim3(256), 0, stream, x,               \
-                       static_cast<const TW*>(w), static_cast<TO*>(out), rows, H, eps)
+    const bool vec = H % 4 == 0 && H <= 32 * 256 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+#define LLME_NORM(TW, TO)                                                                             \
+    do {                                                                                              \
+        if (vec)                                                                                      \
+            hipLaunchKernelGGL((rmsnorm_kernel<TW, TO, true>), dim3(R), dim3(256), 0, stream, x,      \
+                               static_cast<const TW*>(w), static_cast<TO*>(out), rows, H, eps);       \
+        else                                                                                          \
+            hipLaunchKernelGGL((rmsnorm_kernel<TW, TO, false>), dim3(R), dim3(256), 0, stream, x,     \
+                               static_cast<const TW*>(w), static_cast<TO*>(out), rows, H, eps);       \
+    } while (0)
     if (w_dtype == kF32 && out_dtype == kF32) LLME_NORM(float, float);
     else if (w_dtype == kF32 && out_dtype == kBF16) LLME_NORM(float, bf16);
     else if (w_dtype == kBF16 && out_dtype == kF32) LLME_NORM(bf16, float);
