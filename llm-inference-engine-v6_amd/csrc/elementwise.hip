@@ -10,6 +10,13 @@
 namespace llme {
 
 // ---------------------------------------------------------------------------------
+// Zeros for a buffer that a product cut over k adds its parts into. n4 groups of four floats.
+__global__ __launch_bounds__(256) void clear_kernel(float4* __restrict__ p, size_t n4) {
+    for (size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x; i < n4; i += static_cast<size_t>(gridDim.x) * 256)
+        p[i] = float4{0.f, 0.f, 0.f, 0.f};
+}
+
+// ---------------------------------------------------------------------------------
 // out[t, :] = table[tokens[t], :]        (src/kernels.cpp:59-66; no scaling)
 template <typename TW>
 __global__ void embed_gather_kernel(const TW* __restrict__ table, const int* __restrict__ tokens,
@@ -387,6 +394,16 @@ __global__ __launch_bounds__(256) void rope_kv_write_group_kernel(
 }  // namespace llme
 
 using namespace llme;
+
+// n floats, a multiple of 4, at a 16-byte aligned address.
+extern "C" int llme_clear_f32(float* p, size_t n, hipStream_t stream) {
+    if (n == 0) return 0;
+    if (n % 4 != 0 || reinterpret_cast<uintptr_t>(p) % 16 != 0) return kErrUnsupported;
+    const size_t n4 = n / 4;
+    const unsigned grid = static_cast<unsigned>(n4 / 256 + 1 < 1024 ? n4 / 256 + 1 : 1024);
+    hipLaunchKernelGGL(clear_kernel, dim3(grid), dim3(256), 0, stream, reinterpret_cast<float4*>(p), n4);
+    return launch_status();
+}
 
 extern "C" int llme_embed_gather(const void* table, int table_dtype, const int* tokens, float* out, int T,
                                  int H, int blocked, hipStream_t stream) {

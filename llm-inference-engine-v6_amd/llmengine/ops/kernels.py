@@ -175,6 +175,14 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate
           "gemm_generic")
 
 
+def clear(t: torch.Tensor) -> None:
+    """Zeros a 32-bit buffer (for a product cut over k, whose parts add into it)."""
+    require(t, "buffer", torch.float32)
+    if t.numel() % 4 or t.data_ptr() % 16:
+        raise KernelError("clear: a multiple of 4 values at a 16-byte aligned address")
+    check(entry("llme_clear_f32")(ptr(t), t.numel(), stream()), "clear")
+
+
 _fast_gemm = None       # set by ops/mfma.py when the MFMA kernels are present
 
 

@@ -31,6 +31,7 @@ _vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 
 _SIGNATURES = {
     "llme_embed_gather": [_vp, _i, _vp, _vp, _i, _i, _i, _vp],
+    "llme_clear_f32": [_vp, ctypes.c_size_t, _vp],
     "llme_rmsnorm": [_vp, _vp, _i, _vp, _i, _vp, _i, _i, _f, _vp],
     "llme_swiglu": [_vp, _i, _vp, _i, _i, _i, _i, _vp],
     "llme_rope_kv_write": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i,

@@ -103,7 +103,15 @@ class Attention(Mixer):
                                block_table, cos, sin, q, k_cache, v_cache, n_q, n_kv, hd)
         elif write_cache:
             qkv = step.buffer("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
-            project(self.w_qkv, qkv)
+            if (pre_norm is None and 16 < T <= 64 and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16
+                    and qkv.numel() % 4 == 0):
+                # a few dozen rows (decoding at larger batches): q/k/v has too few output tiles for the
+                # chip, so the product is cut over k and adds its parts into a cleared buffer
+                # (measured at 32 rows of the 3B sizes: 10.7 + clearing against 19.5 us)
+                ops.clear(qkv)
+                ops.gemm(x, self.w_qkv, qkv, accumulate=True)
+            else:
+                project(self.w_qkv, qkv)
             ops.rope_kv_write(qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
                               n_q, n_kv, hd, rot, write_cache=True)
         else:
