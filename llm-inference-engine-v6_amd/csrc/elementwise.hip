@@ -102,15 +102,16 @@ __device__ __forceinline__ void norm_store4<bf16>(bf16* p, const float (&v)[4]) 
     *reinterpret_cast<bf16x4*>(p) = o;
 }
 
-// VEC: the row's length is a multiple of 4, at most 32 * blockDim, and x, w and out are aligned
-// for 16-byte (bfloat16: 8-byte) accesses: a thread then keeps its up to 8 groups of four values
+// NV > 0: the row's length is a multiple of 4, at most 4 NV blockDim, and x, w and out are aligned
+// for 16-byte (bfloat16: 8-byte) accesses: a thread then keeps its up to NV groups of four values
 // and their weights in registers between the two passes, all asked for at once, and stores four
-// values at a time. Otherwise the row is read twice, value by value.
-template <typename TW, typename TO, bool VEC>
+// values at a time. NV = 0: the row is read twice, value by value.
+template <typename TW, typename TO, int NVEC>
 __global__ void rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ w,
                                TO* __restrict__ out, const int* __restrict__ rows, int H, float eps) {
     __shared__ float scratch[16];
-    constexpr int NV = 8;
+    constexpr bool VEC = NVEC > 0;
+    constexpr int NV = VEC ? NVEC : 1;
     const int r = blockIdx.x;
     const int src = rows ? rows[r] : r;
     const float* xr = x + static_cast<size_t>(src) * H;
@@ -438,14 +439,16 @@ extern "C" int llme_rmsnorm(const float* x, const void* w, int w_dtype, void* ou
     if (R <= 0) return 0;
     const bool vec = H % 4 == 0 && H <= 32 * 256 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
                      reinterpret_cast<uintptr_t>(w) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
-#define LLME_NORM(TW, TO)                                                                             \
-    do {                                                                                              \
-        if (vec)                                                                                      \
-            hipLaunchKernelGGL((rmsnorm_kernel<TW, TO, true>), dim3(R), dim3(256), 0, stream, x,      \
-                               static_cast<const TW*>(w), static_cast<TO*>(out), rows, H, eps);       \
-        else                                                                                          \
-            hipLaunchKernelGGL((rmsnorm_kernel<TW, TO, false>), dim3(R), dim3(256), 0, stream, x,     \
-                               static_cast<const TW*>(w), static_cast<TO*>(out), rows, H, eps);       \
+    const int nv = !vec ? 0 : H <= 8 * 256 ? 2 : H <= 16 * 256 ? 4 : 8;      // groups of four per thread
+#define LLME_NORM_NV(TW, TO, NV)                                                                  \
+    hipLaunchKernelGGL((rmsnorm_kernel<TW, TO, NV>), dim3(R), dim3(256), 0, stream, x,            \
+                       static_cast<const TW*>(w), static_cast<TO*>(out), rows, H, eps)
+#define LLME_NORM(TW, TO)                                                                         \
+    do {                                                                                          \
+        if (nv == 2) LLME_NORM_NV(TW, TO, 2);                                                     \
+        else if (nv == 4) LLME_NORM_NV(TW, TO, 4);                                                \
+        else if (nv == 8) LLME_NORM_NV(TW, TO, 8);                                                \
+        else LLME_NORM_NV(TW, TO, 0);                                                             \
     } while (0)
     if (w_dtype == kF32 && out_dtype == kF32) LLME_NORM(float, float);
     else if (w_dtype == kF32 && out_dtype == kBF16) LLME_NORM(float, bf16);
@@ -453,6 +456,7 @@ extern "C" int llme_rmsnorm(const float* x, const void* w, int w_dtype, void* ou
     else if (w_dtype == kBF16 && out_dtype == kBF16) LLME_NORM(bf16, bf16);
     else return kErrBadArgument;
 #undef LLME_NORM
+#undef LLME_NORM_NV
     return launch_status();
 }
 
