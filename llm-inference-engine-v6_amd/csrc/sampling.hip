@@ -1,4 +1,5 @@
-// Token choice on the device, one workgroup per row of logits [R, V].
+// Token choice on the device for rows of logits [R, V]; a row is cut into parts so that a few
+// rows of a large vocabulary still fill the chip.
 //
 // Greedy: the first index of the maximum (ties go to the lowest id), as the
 // reference's argmax (src/engine.cpp:52-58, src/scheduler.cpp:10-16).
@@ -83,57 +84,113 @@ __global__ __launch_bounds__(kWave) void argmax_join_kernel(const float* __restr
     if (threadIdx.x == 0) out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
 }
 
-// Rows with temperature <= 0 are greedy.
-__global__ __launch_bounds__(kSampleThreads) void sample_kernel(const float* __restrict__ logits,
-                                                                const float* __restrict__ temperature,
-                                                                const float* __restrict__ uniform,
-                                                                int* __restrict__ out, int V) {
-    __shared__ float sv[kSampleThreads / kWave];
-    __shared__ int si[kSampleThreads / kWave];
-    __shared__ float seg_sum[kSampleThreads];
-    __shared__ float scratch[16];
-    const int r = blockIdx.x;
-    const float* row = logits + static_cast<size_t>(r) * V;
-    const float temp = temperature[r];
+// Temperature sampling in three stages over the same parts as the greedy choice. The first is
+// argmax_part_kernel: the row's maximum is the maximum of its parts. The second sums
+// exp(x / T - max / T) over each part. The third adds the parts' sums in ascending order, finds
+// the part in which the cumulative sum passes u * total, and walks that part alone: every thread
+// owns a run of consecutive ids there, the runs' sums are scanned in thread order, and the
+// lowest id whose cumulative sum exceeds the target wins. Rows with temperature <= 0 are greedy.
+__device__ __forceinline__ float row_maximum(const float* __restrict__ part_val, int parts) {
+    float m = -INFINITY;
+    for (int p = 0; p < parts; ++p) m = fmaxf(m, part_val[p]);
+    return m;
+}
 
-    float bv = -INFINITY;
-    int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += kSampleThreads) argmax_combine(bv, bi, row[i], i);
-    block_argmax(bv, bi, sv, si);
-    if (bi == 0x7fffffff) bi = 0;
+__global__ __launch_bounds__(kSampleThreads) void sample_sum_kernel(const float* __restrict__ logits,
+                                                                    const float* __restrict__ temperature,
+                                                                    const float* __restrict__ part_val,
+                                                                    float* __restrict__ part_sum, int V, int chunk) {
+    __shared__ float scratch[kSampleThreads / kWave];
+    const int r = blockIdx.x, parts = gridDim.y;
+    const float temp = temperature[r];
+    if (!(temp > 0.f)) return;
+    const float inv_t = 1.0f / temp;
+    const float mx = row_maximum(part_val + r * parts, parts) * inv_t;
+    const float* row = logits + static_cast<size_t>(r) * V;
+    const int begin = blockIdx.y * chunk;
+    const int end = (begin + chunk < V) ? begin + chunk : V;
+    float mine = 0.f;
+    constexpr int U = 8;
+    for (int i0 = begin + threadIdx.x; i0 < end; i0 += kSampleThreads * U) {
+        float v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * kSampleThreads;
+            v[u] = row[i < end ? i : end - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (i0 + u * kSampleThreads < end) mine += expf(v[u] * inv_t - mx);
+    }
+    const float total = block_sum(mine, scratch, kSampleThreads / kWave);
+    if (threadIdx.x == 0) part_sum[r * parts + blockIdx.y] = total;
+}
+
+__global__ __launch_bounds__(kSampleThreads) void sample_pick_kernel(const float* __restrict__ logits,
+                                                                     const float* __restrict__ temperature,
+                                                                     const float* __restrict__ uniform,
+                                                                     const float* __restrict__ part_val,
+                                                                     const int* __restrict__ part_idx,
+                                                                     const float* __restrict__ part_sum,
+                                                                     int* __restrict__ out, int V, int chunk,
+                                                                     int parts) {
+    __shared__ float wave_total[kSampleThreads / kWave];
+    __shared__ int pick;
+    const int r = blockIdx.x;
+    const float temp = temperature[r];
     if (!(temp > 0.f)) {
-        if (threadIdx.x == 0) out[r] = bi;
+        if (threadIdx.x == 0) {
+            float bv = -INFINITY;
+            int bi = 0x7fffffff;
+            for (int p = 0; p < parts; ++p) argmax_combine(bv, bi, part_val[r * parts + p], part_idx[r * parts + p]);
+            out[r] = (bi == 0x7fffffff) ? 0 : bi;
+        }
         return;
     }
-    // Each thread owns a run of consecutive ids, so that segment sums added in
-    // thread order are the cumulative sums in ascending id order.
-    const float inv_t = 1.0f / temp;
-    const float mx = bv * inv_t;
-    const int seg = (V + kSampleThreads - 1) / kSampleThreads;
-    const int begin = threadIdx.x * seg;
-    const int end = (begin + seg < V) ? begin + seg : V;
-    float mine = 0.f;
-    for (int i = begin; i < end; ++i) mine += expf(row[i] * inv_t - mx);
-    seg_sum[threadIdx.x] = mine;
-    const float total = block_sum(mine, scratch, kSampleThreads / kWave);
-    if (threadIdx.x == 0) {
-        const float target = uniform[r] * total;
-        float cum = 0.f;
-        int s = 0;
-        while (s < kSampleThreads - 1 && cum + seg_sum[s] <= target) { cum += seg_sum[s]; ++s; }
-        const int b = s * seg;
-        const int e = (b + seg < V) ? b + seg : V;
-        int pick = -1;
-        for (int i = b; i < e; ++i) {
-            cum += expf(row[i] * inv_t - mx);
-            if (cum > target) { pick = i; break; }
-        }
-        if (pick < 0) {
-            // Rounding left the target beyond the last partial sum: take the last id with mass.
-            pick = (e > b) ? e - 1 : bi;
-        }
-        out[r] = pick;
+    // every thread walks the parts' sums alike: the part in which the cumulative sum passes
+    // the target (the last one if rounding leaves none), and the sum before it
+    float total = 0.f;
+    for (int p = 0; p < parts; ++p) total += part_sum[r * parts + p];
+    const float target = uniform[r] * total;
+    float before = 0.f;
+    int part = 0;
+    while (part < parts - 1 && before + part_sum[r * parts + part] <= target) {
+        before += part_sum[r * parts + part];
+        ++part;
     }
+    const float inv_t = 1.0f / temp;
+    const float mx = row_maximum(part_val + r * parts, parts) * inv_t;
+    const float* row = logits + static_cast<size_t>(r) * V;
+    const int begin = part * chunk;
+    const int end = (begin + chunk < V) ? begin + chunk : V;
+    const int run = (end - begin + kSampleThreads - 1) / kSampleThreads;
+    const int mine_begin = begin + threadIdx.x * run;
+    const int mine_end = (mine_begin + run < end) ? mine_begin + run : end;
+    float mine = 0.f;
+    for (int i = mine_begin; i < mine_end; ++i) mine += expf(row[i] * inv_t - mx);
+    // sums of the runs before this thread's: within the wave, then over the waves before it
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    float inclusive = mine;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const float other = __shfl_up(inclusive, off, kWave);
+        if (lane >= off) inclusive += other;
+    }
+    if (threadIdx.x == 0) pick = 0x7fffffff;
+    if (lane == kWave - 1) wave_total[wave] = inclusive;
+    __syncthreads();
+    float cum = before + (inclusive - mine);
+    for (int w = 0; w < wave; ++w) cum += wave_total[w];
+    for (int i = mine_begin; i < mine_end; ++i) {
+        cum += expf(row[i] * inv_t - mx);
+        if (cum > target) {
+            atomicMin(&pick, i);
+            break;
+        }
+    }
+    __syncthreads();
+    // Rounding left the target beyond the last cumulative sum: the last id of the part.
+    if (threadIdx.x == 0) out[r] = (pick == 0x7fffffff) ? end - 1 : pick;
 }
 
 }  // namespace llme
@@ -159,11 +216,18 @@ extern "C" int llme_argmax(const float* logits, int* out, float* part_val, int* 
     return launch_status();
 }
 
+// part_val, part_idx and part_sum: scratch for R * llme_argmax_parts(V) values each.
 extern "C" int llme_sample(const float* logits, const float* temperature, const float* uniform, int* out,
-                           int R, int V, hipStream_t stream) {
+                           float* part_val, int* part_idx, float* part_sum, int R, int V, hipStream_t stream) {
     if (R <= 0) return 0;
     if (V <= 0) return kErrBadArgument;
-    hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(kSampleThreads), 0, stream, logits, temperature, uniform,
-                       out, V);
+    const int parts = llme_argmax_parts(V);
+    const int chunk = (V + parts - 1) / parts;
+    hipLaunchKernelGGL(argmax_part_kernel, dim3(R, parts), dim3(kSampleThreads), 0, stream, logits, part_val,
+                       part_idx, V, chunk);
+    hipLaunchKernelGGL(sample_sum_kernel, dim3(R, parts), dim3(kSampleThreads), 0, stream, logits, temperature,
+                       part_val, part_sum, V, chunk);
+    hipLaunchKernelGGL(sample_pick_kernel, dim3(R), dim3(kSampleThreads), 0, stream, logits, temperature, uniform,
+                       part_val, part_idx, part_sum, out, V, chunk, parts);
     return launch_status();
 }

@@ -243,18 +243,23 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     argmax_into(logits, ptr(out))
 
 
+def _parts_scratch(device, need: int):
+    scratch = _argmax_scratch.get(device)
+    if scratch is None or scratch[0].numel() < need:
+        n = max(need, 4096)
+        scratch = (torch.empty(n, dtype=torch.float32, device=device), torch.empty(n, dtype=torch.int32, device=device),
+                   torch.empty(n, dtype=torch.float32, device=device))
+        _argmax_scratch[device] = scratch
+    return scratch
+
+
 def argmax_into(logits: torch.Tensor, out_ptr: int) -> None:
     """argmax with the result (one int32 per row) written to an address the device can reach:
     device memory, or pinned host memory, which the device sees at the same address."""
     require(logits, "logits", torch.float32, (None, None))
     R, V = logits.shape
-    need = R * entry("llme_argmax_parts")(V)
-    scratch = _argmax_scratch.get(logits.device)
-    if scratch is None or scratch[0].numel() < need:
-        scratch = (torch.empty(max(need, 4096), dtype=torch.float32, device=logits.device),
-                   torch.empty(max(need, 4096), dtype=torch.int32, device=logits.device))
-        _argmax_scratch[logits.device] = scratch
-    check(entry("llme_argmax")(ptr(logits), out_ptr, ptr(scratch[0]), ptr(scratch[1]), R, V, stream()), "argmax")
+    val, idx, _ = _parts_scratch(logits.device, R * entry("llme_argmax_parts")(V))
+    check(entry("llme_argmax")(ptr(logits), out_ptr, ptr(val), ptr(idx), R, V, stream()), "argmax")
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor) -> None:
@@ -263,4 +268,6 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tenso
     require(temperature, "temperature", torch.float32, (R,))
     require(uniform, "uniform", torch.float32, (R,))
     require(out, "out", torch.int32, (R,))
-    check(entry("llme_sample")(ptr(logits), ptr(temperature), ptr(uniform), ptr(out), R, V, stream()), "sample")
+    val, idx, sums = _parts_scratch(logits.device, R * entry("llme_argmax_parts")(V))
+    check(entry("llme_sample")(ptr(logits), ptr(temperature), ptr(uniform), ptr(out), ptr(val), ptr(idx), ptr(sums),
+                               R, V, stream()), "sample")

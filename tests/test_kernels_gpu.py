@@ -201,9 +201,8 @@ def test_argmax_first_maximum(ops, V):
     assert out.tolist()[1] == V // 2
 
 
-@pytest.mark.parametrize("V", [7, 300, 5000])
-def test_temperature_sampling_interval(ops, V):
-    R = 64
+@pytest.mark.parametrize("V,R", [(7, 64), (300, 64), (5000, 64), (2049, 3), (128256, 8)])
+def test_temperature_sampling_interval(ops, V, R):
     logits = 2 * torch.randn(R, V, generator=_gen(10))
     u = torch.rand(R, generator=_gen(11))
     temp = torch.full((R,), 0.8)
