@@ -132,19 +132,15 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     }
 }
 
-// joins the splits of the decode kernel: grid (request, head); lanes over the splits for the
-// statistics, then over the head's dimensions for the weighted sum. nsplit <= 64. The partial
-// outputs are asked for 16 splits at a time, the first 16 together with the statistics: asked
-// for one after the other, the trips to memory were most of this small kernel's time.
+// Joins the splits of one (row, head): one wavefront, lanes over the splits for the statistics,
+// then over the head's dimensions for the weighted sum. nsplit <= 64. `base` is the first of the
+// nsplit parts. The partial outputs are asked for 16 splits at a time, the first 16 together with
+// the statistics: asked for one after the other, the trips to memory were most of the time.
 constexpr int JOIN_AT_A_TIME = 16;
-__global__ __launch_bounds__(64) void attention_join_kernel(const float* __restrict__ part_o,
-                                                            const float* __restrict__ part_ml, bf16* __restrict__ out,
-                                                            const int* __restrict__ q_start, int n_q, int hd, int nsplit) {
-    __shared__ float weight[64];
-    const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    const int row0 = q_start[s];
-    if (q_start[s + 1] - row0 != 1) return;
-    const size_t base = (static_cast<size_t>(s) * n_q + h) * nsplit;
+__device__ __forceinline__ void join_splits(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                            bf16* __restrict__ out_row, size_t base, int hd, int nsplit,
+                                            float* weight) {
+    const int lane = threadIdx.x;
     float part[JOIN_AT_A_TIME];
     auto ask = [&](int first, int d) {                 // (splits past the last: the last again, with weight 0)
 #pragma unroll
@@ -172,8 +168,43 @@ __global__ __launch_bounds__(64) void attention_join_kernel(const float* __restr
             for (int u = 0; u < JOIN_AT_A_TIME; ++u)
                 acc += (first + u < nsplit ? weight[first + u] : 0.f) * part[u];
         }
-        out[(static_cast<size_t>(row0) * n_q + h) * hd + d] = static_cast<bf16>(acc);
+        out_row[d] = static_cast<bf16>(acc);
     }
+}
+
+// The decode kernel's splits: grid (request, head); parts indexed by request.
+__global__ __launch_bounds__(64) void attention_join_kernel(const float* __restrict__ part_o,
+                                                            const float* __restrict__ part_ml, bf16* __restrict__ out,
+                                                            const int* __restrict__ q_start, int n_q, int hd, int nsplit) {
+    __shared__ float weight[64];
+    const int s = blockIdx.x, h = blockIdx.y;
+    const int row0 = q_start[s];
+    if (q_start[s + 1] - row0 != 1) return;
+    join_splits(part_o, part_ml, out + (static_cast<size_t>(row0) * n_q + h) * hd,
+                (static_cast<size_t>(s) * n_q + h) * nsplit, hd, nsplit, weight);
+}
+
+// The prefill kernel's key runs: grid (batch row, head); parts indexed by batch row. Rows of
+// requests that bring one token belong to the decode kernel and are left alone.
+__global__ __launch_bounds__(64) void attention_join_rows_kernel(const float* __restrict__ part_o,
+                                                                 const float* __restrict__ part_ml,
+                                                                 bf16* __restrict__ out, const int* __restrict__ q_start,
+                                                                 int n_seq, int n_q, int hd, int nsplit) {
+    __shared__ float weight[64];
+    const int row = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    bool mine = false;                                  // (the same in every lane)
+    for (int first = 0; first < n_seq; first += 64) {
+        const int i = first + lane;
+        bool hit = false;
+        if (i < n_seq) {
+            const int a = q_start[i], b = q_start[i + 1];
+            hit = a <= row && row < b && b - a >= 2;
+        }
+        mine = mine || __any(hit);
+    }
+    if (!mine) return;
+    join_splits(part_o, part_ml, out + (static_cast<size_t>(row) * n_q + h) * hd,
+                (static_cast<size_t>(row) * n_q + h) * nsplit, hd, nsplit, weight);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -266,7 +297,8 @@ template <int HD>
 static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, float* part_o, float* part_ml,
                            const int* q_start, const int* ctx_len, const int* table, int max_blocks, int n_seq,
                            int n_q, int n_kv, int page, float scale, int window, int n_decode, int split_len,
-                           int nsplit, int prefill_groups, int qt, int shared_rows, int* queue, hipStream_t stream) {
+                           int nsplit, int prefill_groups, int qt, int shared_rows, int* queue, int n_rows,
+                           int prefill_splits, float* pre_part_o, float* pre_part_ml, hipStream_t stream) {
     if (n_decode > 0) {
         const int G = n_q / n_kv;
         const dim3 grid(n_seq, n_kv * ((G + 15) / 16), nsplit);
@@ -283,9 +315,15 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
                                q_start, n_q, HD, nsplit);
     }
     if (prefill_groups > 0) {
-        if (shared_rows > 0)
-            return launch_prefill_shared(q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, HD,
-                                         page, scale, window, prefill_groups, shared_rows, queue, stream);
+        if (shared_rows > 0) {
+            const int status = launch_prefill_shared(q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q,
+                                                     n_kv, HD, page, scale, window, prefill_groups, shared_rows, queue,
+                                                     prefill_splits, pre_part_o, pre_part_ml, stream);
+            if (status != 0 || prefill_splits <= 1) return status;
+            hipLaunchKernelGGL(attention_join_rows_kernel, dim3(n_rows, n_q), dim3(64), 0, stream, pre_part_o,
+                               pre_part_ml, out, q_start, n_seq, n_q, HD, prefill_splits);
+            return launch_status();
+        }
         const dim3 grid(prefill_groups, (n_q + 3) / 4);
 #define LLME_PREFILL(QT)                                                                                       \
     hipLaunchKernelGGL((attention_prefill_kernel<HD, QT>), grid, dim3(256), 0, stream, q, kc, vc, out, q_start, \
@@ -343,12 +381,24 @@ extern "C" int llme_attention_bf16_rows(int hd, int n_q, int n_kv) {
 // row groups of llme_attention_bf16_rows(hd, n_q, n_kv) rows over the requests with two or more tokens.
 // queue: two integers, zero, for the prefill kernel's work counter (needed when prefill_groups > 0;
 // the kernel leaves them zero; launches that may overlap need separate ones).
+// prefill_splits > 1 (only where llme_attention_bf16_splits_prefill says so): the keys of every
+// prefill work item are cut into that many runs, joined by a second kernel over the batch's n_rows
+// rows; pre_part_o [n_rows, n_q, prefill_splits, hd] and pre_part_ml [n_rows, n_q, prefill_splits, 2]
+// floats are their scratch.
+extern "C" int llme_attention_bf16_splits_prefill(int hd, int n_q, int n_kv) {
+    return shared_rows_for(hd, n_q, n_kv) > 0 ? 1 : 0;
+}
+
 extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const void* v_cache, void* out, float* part_o,
                                    float* part_ml, const int* q_start, const int* ctx_len, const int* block_table,
                                    int max_blocks, int n_seq, int n_q, int n_kv, int hd, int page, float scale,
                                    int window, int n_decode, int split_len, int nsplit, int prefill_groups,
-                                   int* queue, hipStream_t stream) {
+                                   int* queue, int n_rows, int prefill_splits, float* pre_part_o, float* pre_part_ml,
+                                   hipStream_t stream) {
     if (n_seq <= 0) return 0;
+    if (prefill_splits < 1 || prefill_splits > 64 || n_rows < 0) return kErrBadArgument;
+    if (prefill_splits > 1 && (shared_rows_for(hd, n_q, n_kv) <= 0 || pre_part_o == nullptr || pre_part_ml == nullptr))
+        return kErrBadArgument;
     if (hd % 16 != 0 || hd > 128 || hd <= 0 || page % 16 != 0 || n_kv <= 0 || n_q % n_kv != 0) return kErrUnsupported;
     if (!(scale > 0.f)) return kErrBadArgument;      // the lazy maximum compares scaled scores
     // page lookups divide by multiplication, exact while (keys / 16) * (page / 16) < 2^32
@@ -362,7 +412,8 @@ extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const voi
         return launch_for_head<HD>(static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache),              \
                                    static_cast<const bf16*>(v_cache), static_cast<bf16*>(out), part_o, part_ml, \
                                    q_start, ctx_len, block_table, max_blocks, n_seq, n_q, n_kv, page, scale,    \
-                                   window, n_decode, split_len, nsplit, prefill_groups, qt, shared_rows, queue, stream)
+                                   window, n_decode, split_len, nsplit, prefill_groups, qt, shared_rows, queue, n_rows, \
+                                   prefill_splits, pre_part_o, pre_part_ml, stream)
     switch (hd) {
         LLME_HEAD(16); LLME_HEAD(32); LLME_HEAD(48); LLME_HEAD(64);
         LLME_HEAD(80); LLME_HEAD(96); LLME_HEAD(112); LLME_HEAD(128);

@@ -22,6 +22,11 @@
 //
 // Takes head sizes 64 and 128 and pages that are multiples of 16; other sizes go to the kernel
 // without LDS.
+//
+// Few rows over a long context (a portion of a prompt far into it) are few work items that each
+// walk many keys. Then an item's keys are cut into `nsplit` runs of whole stretches, one work item
+// each, which leave their rows' maxima, sums and unscaled outputs in 32-bit scratch indexed by
+// batch row; a second kernel joins them, as it joins the splits of the decode kernel.
 #include "attention_tiles.h"
 
 namespace llme {
@@ -156,9 +161,10 @@ __device__ __forceinline__ void read_block(const bf16* stage, int sb, KFrag<HD>&
 }
 
 // One work item: span `bx` (counted over the requests with two or more tokens, the last spans of
-// a request first) for head group `by`.
-template <int HD, int QT, int HPW, int KW>
-__device__ __forceinline__ void prefill_item(int bx, int by, bf16* lds, const bf16* __restrict__ q,
+// a request first) for head group `by`, run `z` of the `nsplit` runs of its keys (SPLIT; else all).
+template <int HD, int QT, int HPW, int KW, bool SPLIT>
+__device__ __forceinline__ void prefill_item(int bx, int by, int z, int nsplit, float* __restrict__ part_o,
+                                             float* __restrict__ part_ml, bf16* lds, const bf16* __restrict__ q,
                                              const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
                                              bf16* __restrict__ out, const int* __restrict__ q_start,
                                              const int* __restrict__ ctx_len, const int* __restrict__ block_table,
@@ -221,9 +227,16 @@ __device__ __forceinline__ void prefill_item(int bx, int by, bf16* lds, const bf
     const int my_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
 
     // the workgroup's keys
-    const int key_end = pos_span + n_span;
+    int key_end = pos_span + n_span;
     const int key_lo = (window > 0 && pos_span - window + 1 > 0) ? pos_span - window + 1 : 0;
-    const int k_begin = key_lo & ~(KB - 1);
+    int k_begin = key_lo & ~(KB - 1);
+    if (SPLIT) {
+        // run z of the stretches; a run past the last key is empty and leaves sums of zero
+        const int stretches = (key_end - k_begin + KB - 1) / KB;
+        const int per_run = (stretches + nsplit - 1) / nsplit;
+        k_begin += z * per_run * KB;
+        if (key_end > k_begin + per_run * KB) key_end = k_begin + per_run * KB;
+    }
     PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD,
                page_magic_of(page), static_cast<unsigned>(n_kv) * page * HD, static_cast<unsigned>(kvh) * page * HD};
     const float scale_log2 = scale * kLog2e;
@@ -314,6 +327,24 @@ __device__ __forceinline__ void prefill_item(int bx, int by, bf16* lds, const bf
         float lt = l[qt];
         lt += __shfl_xor(lt, 16, 64);
         lt += __shfl_xor(lt, 32, 64);
+        if (SPLIT) {
+            // this run's part of row `row`, head `head`: statistics from the lanes of the row's
+            // first quarter, outputs unscaled (the join divides)
+            if (g4 == 0 && qt * 16 + r < n_rows) {
+                const size_t pidx = (static_cast<size_t>(first_w + qt * 16 + r) * n_q + head) * nsplit + z;
+                part_ml[pidx * 2] = m[qt];
+                part_ml[pidx * 2 + 1] = lt;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int row = qt * 16 + g4 * 4 + e;
+                if (row >= n_rows) continue;
+                const size_t pidx = (static_cast<size_t>(first_w + row) * n_q + head) * nsplit + z;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) part_o[pidx * HD + dt * 16 + r] = o[qt][dt][e];
+            }
+            continue;
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int rr = g4 * 4 + e;
@@ -336,25 +367,28 @@ __device__ __forceinline__ void prefill_item(int bx, int by, bf16* lds, const bf
 // workgroup to leave clears them), so the same two integers serve every launch on a stream.
 // KW = 2: eight wavefronts, two per tile, each taking every other 32-key block: half the time
 // for a work item, for batches with too few items to fill the chip.
-template <int HD, int QT, int HPW, int KW>
+template <int HD, int QT, int HPW, int KW, bool SPLIT>
 __global__ __launch_bounds__(256 * KW) void attention_prefill_shared_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     bf16* __restrict__ out, const int* __restrict__ q_start, const int* __restrict__ ctx_len,
     const int* __restrict__ block_table, int max_blocks, int n_seq, int n_q, int n_kv, int page, float scale,
-    int window, int spans, int* __restrict__ queue) {
+    int window, int spans, int* __restrict__ queue, int nsplit, float* __restrict__ part_o,
+    float* __restrict__ part_ml) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     __shared__ int next_item;
     bf16* lds = reinterpret_cast<bf16*>(lds_raw);
     const int head_groups = n_q / HPW;
-    const int n_items = spans * head_groups;
+    const int n_items = spans * head_groups * (SPLIT ? nsplit : 1);
     for (;;) {
         __syncthreads();                                   // everybody is done with the last item's LDS
         if (threadIdx.x == 0) next_item = atomicAdd(queue, 1);
         __syncthreads();
         const int item = __builtin_amdgcn_readfirstlane(next_item);
         if (item >= n_items) break;                        // the counter only grows: every workgroup gets here
-        prefill_item<HD, QT, HPW, KW>(item / head_groups, item % head_groups, lds, q, k_cache, v_cache, out, q_start,
-                                  ctx_len, block_table, max_blocks, n_seq, n_q, n_kv, page, scale, window);
+        const int whole = SPLIT ? item / nsplit : item;     // (an item's runs are neighbours in the queue)
+        prefill_item<HD, QT, HPW, KW, SPLIT>(whole / head_groups, whole % head_groups, SPLIT ? item % nsplit : 0, nsplit,
+                                             part_o, part_ml, lds, q, k_cache, v_cache, out, q_start, ctx_len,
+                                             block_table, max_blocks, n_seq, n_q, n_kv, page, scale, window);
     }
     if (threadIdx.x == 0) {
         // whoever leaves last has seen every other workgroup take its final number: nobody touches
@@ -381,12 +415,13 @@ int prefill_shared_rows(int hd, int n_q, int n_kv) {
     return 32 * (4 / heads_per_workgroup(n_q, n_kv));
 }
 
-template <int HD, int QT, int HPW, int KW>
+template <int HD, int QT, int HPW, int KW, bool SPLIT>
 static int launch_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, const int* q_start,
                          const int* ctx_len, const int* table, int max_blocks, int n_seq, int n_q, int n_kv, int page,
-                         float scale, int window, int items, int* queue, hipStream_t stream) {
+                         float scale, int window, int items, int* queue, int nsplit, float* part_o, float* part_ml,
+                         hipStream_t stream) {
     constexpr int LDS = StageLayout<HD>::BYTES;
-    auto kernel = attention_prefill_shared_kernel<HD, QT, HPW, KW>;
+    auto kernel = attention_prefill_shared_kernel<HD, QT, HPW, KW, SPLIT>;
     static bool attr_set = false;                      // per instantiation
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -405,32 +440,39 @@ static int launch_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* ou
         if (e != hipSuccess) return static_cast<int>(e);
         resident = cus * (per_cu > 0 ? per_cu : 1);
     }
-    const int n_items = items * (n_q / HPW);
+    const int n_items = items * (n_q / HPW) * (SPLIT ? nsplit : 1);
     hipLaunchKernelGGL(kernel, dim3(n_items < resident ? n_items : resident), dim3(256 * KW), LDS, stream, q, kc, vc, out,
-                       q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, page, scale, window, items, queue);
+                       q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, page, scale, window, items, queue, nsplit,
+                       part_o, part_ml);
     return launch_status();
 }
 
 int launch_prefill_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, const int* q_start,
                           const int* ctx_len, const int* table, int max_blocks, int n_seq, int n_q, int n_kv, int hd,
-                          int page, float scale, int window, int items, int rows_per_item, int* queue,
-                          hipStream_t stream) {
+                          int page, float scale, int window, int items, int rows_per_item, int* queue, int nsplit,
+                          float* part_o, float* part_ml, hipStream_t stream) {
     if (queue == nullptr) return kErrBadArgument;
+    if (nsplit < 1 || (nsplit > 1 && (part_o == nullptr || part_ml == nullptr))) return kErrBadArgument;
     const int hpw = heads_per_workgroup(n_q, n_kv);
     const int rows = rows_per_item / (4 / hpw);            // per row group
     // Two wavefronts per tile while the items are too few to keep three workgroups of four
     // wavefronts on every compute unit: then an item's length, not the chip, sets the time.
-    int kw = static_cast<long>(items) * (n_q / hpw) <= kSplitBelowItems ? 2 : 1;
+    int kw = static_cast<long>(items) * (n_q / hpw) * nsplit <= kSplitBelowItems ? 2 : 1;
     if (g_key_waves == 1 || g_key_waves == 2) kw = g_key_waves;
-#define LLME_SHARED(HD, QT, HPW)                                                                                   \
-    if (hd == HD && rows == 16 * QT && hpw == HPW)                                                                 \
-        return kw == 2 ? launch_shared<HD, QT, HPW, 2>(q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, \
-                                                       n_q, n_kv, page, scale, window, items, queue, stream)       \
-                       : launch_shared<HD, QT, HPW, 1>(q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, \
-                                                       n_q, n_kv, page, scale, window, items, queue, stream)
-    LLME_SHARED(64, 2, 4); LLME_SHARED(64, 2, 2); LLME_SHARED(64, 2, 1);
-    LLME_SHARED(128, 2, 4); LLME_SHARED(128, 2, 2); LLME_SHARED(128, 2, 1);
+#define LLME_SHARED_ARGS q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, page, scale, window, \
+                         items, queue, nsplit, part_o, part_ml, stream
+#define LLME_SHARED(HD, QT, HPW)                                                       \
+    if (hd == HD && rows == 16 * QT && hpw == HPW) {                                   \
+        if (nsplit > 1)                                                                \
+            return kw == 2 ? launch_shared<HD, QT, HPW, 2, true>(LLME_SHARED_ARGS)     \
+                           : launch_shared<HD, QT, HPW, 1, true>(LLME_SHARED_ARGS);    \
+        return kw == 2 ? launch_shared<HD, QT, HPW, 2, false>(LLME_SHARED_ARGS)        \
+                       : launch_shared<HD, QT, HPW, 1, false>(LLME_SHARED_ARGS);       \
+    }
+    LLME_SHARED(64, 2, 4) LLME_SHARED(64, 2, 2) LLME_SHARED(64, 2, 1)
+    LLME_SHARED(128, 2, 4) LLME_SHARED(128, 2, 2) LLME_SHARED(128, 2, 1)
 #undef LLME_SHARED
+#undef LLME_SHARED_ARGS
     return kErrUnsupported;
 }
 

@@ -351,11 +351,13 @@ __device__ __forceinline__ void load_q(const bf16* qrow, bool ok, bf16x8 (&qf)[(
 
 // The prefill kernel that shares K and V blocks among a workgroup's wavefronts through LDS
 // (attention_prefill.hip). rows_per_item: rows of one work item, see prefill_shared_rows; queue:
-// two integers that are zero and that no other launch in flight uses.
+// two integers that are zero and that no other launch in flight uses. nsplit > 1: every item's
+// keys are cut into nsplit runs whose results go to part_o [rows, n_q, nsplit, hd] and part_ml
+// [rows, n_q, nsplit, 2] (by batch row) instead of out; the caller joins them.
 int launch_prefill_shared(const bf16* q, const bf16* k_cache, const bf16* v_cache, bf16* out, const int* q_start,
                           const int* ctx_len, const int* block_table, int max_blocks, int n_seq, int n_q, int n_kv,
                           int hd, int page, float scale, int window, int items, int rows_per_item, int* queue,
-                          hipStream_t stream);
+                          int nsplit, float* part_o, float* part_ml, hipStream_t stream);
 // Rows per work item of the shared kernel for these sizes, or 0 if it does not take them.
 int prefill_shared_rows(int hd, int n_q, int n_kv);
 // Wavefronts that share a tile's keys: 0 lets the launcher choose by the number of items, 1 or 2 forces it.

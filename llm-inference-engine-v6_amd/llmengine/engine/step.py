@@ -43,8 +43,14 @@ class Workspace:
         self._buffers: dict[tuple[str, torch.dtype], torch.Tensor] = {}
         self.keep_replaced = False      # set once a recorded graph holds addresses of these buffers
         self._replaced: list[torch.Tensor] = []
+        # the shaped views handed out, by (name, dtype, shape): a step asks for the same ones layer after layer
+        self._views: dict[tuple, torch.Tensor] = {}
 
     def get(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        shape = tuple(shape)
+        view = self._views.get((name, dtype, shape))
+        if view is not None:
+            return view
         n = 1
         for d in shape:
             n *= int(d)
@@ -55,7 +61,11 @@ class Workspace:
                 self._replaced.append(buf)          # a recorded graph may still read and write it
             buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._buffers[key] = buf
-        return buf[:n].view(shape)
+            self._views = {k: v for k, v in self._views.items() if k[:2] != key}
+        if len(self._views) >= 4096:
+            self._views.clear()
+        view = self._views[(name, dtype, shape)] = buf[:n].view(shape)
+        return view
 
 
 @dataclass

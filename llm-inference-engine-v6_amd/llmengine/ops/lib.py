@@ -94,7 +94,14 @@ def code(dtype: torch.dtype) -> int:
         raise KernelError(f"kernels take float32 or bfloat16 tensors, not {dtype}") from None
 
 
+# The current stream's handle without the Stream object around it: asked for before every launch.
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_current_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def stream() -> int:
+    if _raw_stream is not None and _current_device is not None:
+        return _raw_stream(_current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -113,6 +120,18 @@ def check(status: int, what: str) -> None:
 
 def require(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
     """Host-side check of an operand before a launch: device, layout, type, shape."""
+    # (called several times per launch: the passing case takes the short way)
+    if type(t) is torch.Tensor and t.is_cuda and t.is_contiguous():
+        if dtype is None or t.dtype is dtype or (type(dtype) is not torch.dtype and t.dtype in dtype):
+            if shape is None:
+                return
+            have = t.shape
+            if len(shape) == len(have):
+                for s, d in zip(shape, have):
+                    if s is not None and s != d:
+                        break
+                else:
+                    return
     if not isinstance(t, torch.Tensor):
         raise KernelError(f"{name}: expected a tensor, got {type(t).__name__}")
     if t.device.type != "cuda":

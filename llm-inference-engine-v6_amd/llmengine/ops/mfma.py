@@ -78,8 +78,9 @@ kernels._fast_gemm = _fast_gemm
 declare("llme_attention_bf16_rows", [_i, _i, _i])
 declare("llme_attention_bf16_set_rows", [_i, _i])
 declare("llme_attention_bf16_set_stream", [_i])
+declare("llme_attention_bf16_splits_prefill", [_i, _i, _i])
 declare("llme_attention_bf16", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i,
-                                _i, _i, _i, _i, _vp, _vp])
+                                _i, _i, _i, _i, _vp, _i, _i, _vp, _vp, _vp])
 
 _work_queues: dict = {}
 
@@ -100,6 +101,11 @@ def work_queue(device: torch.device) -> torch.Tensor:
 DECODE_BLOCKS_WANTED = 256
 MIN_SPLIT = 128                     # keys per split at least: one 32-key block per wavefront
 MAX_SPLITS = 64                     # the join kernel's limit
+# Portions of prompts: work items (a span of rows x a group of heads) the prefill kernel should
+# have at least; with fewer, every item's keys are cut into runs of at least PREFILL_MIN_RUN keys.
+PREFILL_ITEMS_WANTED = 512
+PREFILL_MIN_RUN = 512
+PREFILL_MAX_SPLITS = 16
 
 
 def attention_bf16_supported(q, k_cache, head_dim: int) -> bool:
@@ -115,7 +121,13 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
     rows = entry("llme_attention_bf16_rows")(head_dim, n_q, n_kv)
     decode = [c + 1 for n, c in zip(new_lens, ctx_lens) if n == 1]
     groups = sum((n + rows - 1) // rows for n in new_lens if n >= 2)
-    plan = {"n_decode": len(decode), "groups": groups, "split_len": 32, "nsplit": 1}
+    plan = {"n_decode": len(decode), "groups": groups, "split_len": 32, "nsplit": 1, "prefill_splits": 1}
+    if groups and entry("llme_attention_bf16_splits_prefill")(head_dim, n_q, n_kv):
+        # few rows over long contexts: too few work items for the chip, each with many keys
+        group = n_q // n_kv
+        items = groups * (n_q // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
+        keys = max(c + n for n, c in zip(new_lens, ctx_lens) if n >= 2)
+        plan["prefill_splits"] = max(1, min(PREFILL_ITEMS_WANTED // items, keys // PREFILL_MIN_RUN, PREFILL_MAX_SPLITS))
     if decode:
         longest = max(decode) if plan_len is None else max(plan_len, max(decode))
         pairs = len(decode) * n_kv * ((n_q // n_kv + 15) // 16)
@@ -127,9 +139,11 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
 
 
 def attention_bf16(q, k_cache, v_cache, out, q_start, ctx_len, block_table, n_q: int, n_kv: int, head_dim: int,
-                   scale: float, window: int, plan: dict, part_o=None, part_ml=None) -> None:
+                   scale: float, window: int, plan: dict, part_o=None, part_ml=None, pre_part_o=None,
+                   pre_part_ml=None) -> None:
     """Attention of a step's tokens over bfloat16 pages. q_start [S + 1], ctx_len [S] int32 on
-    the device; plan from plan_attention; part_o / part_ml: float32 scratch for split decoding."""
+    the device; plan from plan_attention; part_o / part_ml: float32 scratch for split decoding,
+    pre_part_o / pre_part_ml: for prompt portions whose keys are cut (plan["prefill_splits"] > 1)."""
     T = q.shape[0]
     S = ctx_len.shape[0]
     require(q, "q", torch.bfloat16, (T, n_q * head_dim))
@@ -150,11 +164,19 @@ def attention_bf16(q, k_cache, v_cache, out, q_start, ctx_len, block_table, n_q:
         require(part_ml, "part_ml", torch.float32)
         if part_o.numel() < S * n_q * plan["nsplit"] * head_dim or part_ml.numel() < S * n_q * plan["nsplit"] * 2:
             raise kernels.KernelError("attention_bf16: the scratch for split decoding is too small")
+    pre_splits = plan.get("prefill_splits", 1) if plan["groups"] else 1
+    if pre_splits > 1:
+        require(pre_part_o, "pre_part_o", torch.float32)
+        require(pre_part_ml, "pre_part_ml", torch.float32)
+        if pre_part_o.numel() < T * n_q * pre_splits * head_dim or pre_part_ml.numel() < T * n_q * pre_splits * 2:
+            raise kernels.KernelError("attention_bf16: the scratch for prompt portions with cut keys is too small")
     check(entry("llme_attention_bf16")(
         ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), ptr(part_o), ptr(part_ml), ptr(q_start), ptr(ctx_len),
         ptr(block_table), block_table.shape[1], S, n_q, n_kv, head_dim, page, float(scale), int(window),
         plan["n_decode"], plan["split_len"], plan["nsplit"], plan["groups"],
-        ptr(work_queue(q.device)) if plan["groups"] else None, stream()), "attention_bf16")
+        ptr(work_queue(q.device)) if plan["groups"] else None, T, pre_splits,
+        ptr(pre_part_o) if pre_splits > 1 else None, ptr(pre_part_ml) if pre_splits > 1 else None, stream()),
+        "attention_bf16")
 
 
 def _fast_attention(q, k_cache, v_cache, out, step, block_table, n_q, n_kv, head_dim, scale, window) -> bool:
@@ -169,8 +191,13 @@ def _fast_attention(q, k_cache, v_cache, out, step, block_table, n_q, n_kv, head
         S = step.num_seqs
         part_o = step.buffer("attn.part_o", (S * n_q * plan["nsplit"] * head_dim,), torch.float32)
         part_ml = step.buffer("attn.part_ml", (S * n_q * plan["nsplit"] * 2,), torch.float32)
+    pre_part_o = pre_part_ml = None
+    if plan["groups"] and plan["prefill_splits"] > 1:
+        T = q.shape[0]
+        pre_part_o = step.buffer("attn.pre_part_o", (T * n_q * plan["prefill_splits"] * head_dim,), torch.float32)
+        pre_part_ml = step.buffer("attn.pre_part_ml", (T * n_q * plan["prefill_splits"] * 2,), torch.float32)
     attention_bf16(q, k_cache, v_cache, out, step.q_start, step.ctx_len, block_table, n_q, n_kv, head_dim, scale,
-                   window, plan, part_o, part_ml)
+                   window, plan, part_o, part_ml, pre_part_o, pre_part_ml)
     return True
 
 

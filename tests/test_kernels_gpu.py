@@ -308,8 +308,9 @@ def test_gemm_dispatch_and_refusals(ops):
 
 
 # --- MFMA attention ----------------------------------------------------------------------
-def _attn_case(ops, lens, news, n_q, n_kv, hd, page, window=0, seed=50):
-    """Requests with lens[i] tokens in the cache, of which the last news[i] are this step's."""
+def _attn_case(ops, lens, news, n_q, n_kv, hd, page, window=0, seed=50, prefill_splits=None):
+    """Requests with lens[i] tokens in the cache, of which the last news[i] are this step's.
+    prefill_splits: cut the keys of the prompt portions into that many runs, whatever the plan says."""
     s = _paged_setup(ops, lens, n_q, n_kv, hd, page, torch.bfloat16, seed=seed)
     rows, q_start, ctx = [], [0], []
     base = 0
@@ -325,8 +326,13 @@ def _attn_case(ops, lens, news, n_q, n_kv, hd, page, window=0, seed=50):
     S = len(lens)
     part_o = torch.empty(S * n_q * plan["nsplit"] * hd, device=DEV)
     part_ml = torch.empty(S * n_q * plan["nsplit"] * 2, device=DEV)
+    if prefill_splits is not None:
+        plan["prefill_splits"] = prefill_splits
+    # (the scratch starts as NaN: a part that is joined without having been written shows)
+    pre_o = torch.full((len(rows) * n_q * plan["prefill_splits"] * hd,), float("nan"), device=DEV)
+    pre_ml = torch.full((len(rows) * n_q * plan["prefill_splits"] * 2,), float("nan"), device=DEV)
     ops.mfma.attention_bf16(q, s["k_cache"], s["v_cache"], out, torch.tensor(q_start, **i32), torch.tensor(ctx, **i32),
-                            s["table"], n_q, n_kv, hd, 1.0 / math.sqrt(hd), window, plan, part_o, part_ml)
+                            s["table"], n_q, n_kv, hd, 1.0 / math.sqrt(hd), window, plan, part_o, part_ml, pre_o, pre_ml)
     ref = torch.cat([plain_attention(qq, kk, vv, window)[n - new:].reshape(new, n_q * hd)
                      for (qq, kk, vv), n, new in zip(s["plain"], lens, news)])
     return out.cpu().double(), ref, plan
@@ -388,6 +394,51 @@ def test_attention_prefill_shared_window(ops, window, n_q, n_kv):
     news = [140, 70, 2]
     out, ref, _ = _attn_case(ops, lens, news, n_q, n_kv, 64, 16, window=window, seed=62)
     assert _rel(out, ref) < 8e-3
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,page", [(8, 2, 64, 16), (6, 2, 64, 32), (3, 3, 64, 16), (8, 2, 128, 16),
+                                              (5, 5, 128, 48)])
+@pytest.mark.parametrize("splits,key_waves", [(2, -1), (3, 2), (7, 3), (16, -1)])
+def test_attention_prefill_cut_keys(ops, n_q, n_kv, hd, page, splits, key_waves):
+    """Prompt portions whose keys are cut into runs that a second kernel joins: runs that end
+    inside a span's own rows, runs with no key at all (more runs than 64-key stretches), whole
+    prompts and decoded tokens beside them, with one and two wavefronts per tile."""
+    set_rows = ops.lib.entry("llme_attention_bf16_set_rows")
+    assert set_rows(0, key_waves) == 0
+    try:
+        lens = [700, 2, 131, 64, 517, 65, 9]
+        news = [40, 2, 67, 64, 130, 3, 1]
+        out, ref, plan = _attn_case(ops, lens, news, n_q, n_kv, hd, page, seed=63, prefill_splits=splits)
+        assert plan["n_decode"] == 1 and plan["prefill_splits"] == splits
+        assert not out.isnan().any()
+        assert _rel(out, ref) < 8e-3
+    finally:
+        set_rows(0, -1)
+
+
+@pytest.mark.parametrize("window", [1, 64, 65, 200])
+def test_attention_prefill_cut_keys_window(ops, window):
+    out, ref, _ = _attn_case(ops, [600, 70, 190], [140, 70, 2], 8, 2, 64, 16, window=window, seed=64, prefill_splits=4)
+    assert not out.isnan().any()
+    assert _rel(out, ref) < 8e-3
+
+
+def test_attention_prefill_cut_keys_by_plan(ops):
+    """A short portion far into a prompt: the plan cuts its keys by itself."""
+    n_q, n_kv, hd, page = 8, 2, 64, 16
+    lens, news = [2100], [48]
+    out, ref, plan = _attn_case(ops, lens, news, n_q, n_kv, hd, page, seed=65)
+    assert plan["prefill_splits"] > 1                    # the plan cuts this one by itself
+    assert _rel(out, ref) < 8e-3
+
+
+def test_attention_plan_cuts_only_few_rows_over_many_keys(ops):
+    plan = ops.mfma.plan_attention([256], [16128], 32, 8, 64)
+    assert plan["prefill_splits"] == 8
+    assert ops.mfma.plan_attention([2048], [0], 32, 8, 64)["prefill_splits"] == 1       # many items
+    assert ops.mfma.plan_attention([64], [300], 32, 8, 64)["prefill_splits"] == 1       # few keys
+    assert ops.mfma.plan_attention([64], [3000], 6, 2, 48)["prefill_splits"] == 1       # a head size without the kernel
+    assert ops.mfma.plan_attention([1, 1], [5000, 9000], 32, 8, 64)["prefill_splits"] == 1
 
 
 @pytest.mark.parametrize("window", [1, 5, 16, 33, 100])
