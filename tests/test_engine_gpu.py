@@ -95,6 +95,34 @@ def test_schedules_match_plain(zoo, name, page_override, schedule, dtype):
     assert all(cache.manager.free_pages(g) == cache.manager.num_pages(g) for g in cache.manager.groups)
 
 
+@pytest.mark.parametrize("schedule", ["portions", "mixed"])
+@pytest.mark.parametrize("name", ["C", "F"])
+@pytest.mark.parametrize("min_run,max_splits", [(32, 16), (32, 3)])
+def test_prompt_portions_with_cut_keys_match_plain(zoo, name, schedule, min_run, max_splits, monkeypatch):
+    """Serving cuts the keys of a short prompt portion only far into a long prompt; here the
+    thresholds are lowered so that every portion that ends behind 64 keys has its keys cut into runs that
+    are joined, beside decoded tokens of other requests and on pages that are used again."""
+    from llmengine.ops import mfma
+    monkeypatch.setattr(mfma, "PREFILL_MIN_RUN", min_run)
+    monkeypatch.setattr(mfma, "PREFILL_MAX_SPLITS", max_splits)
+    cut = []
+    plan_attention = mfma.plan_attention
+
+    def noting(*args, **kw):
+        plan = plan_attention(*args, **kw)
+        cut.append(plan["prefill_splits"])
+        return plan
+    monkeypatch.setattr(mfma, "plan_attention", noting)
+    model_dir, reqs, plain, page = zoo[name]
+    engine = engine_for(model_dir, "bf16")
+    steps = SCHEDULES[schedule](reqs)
+    pages = replay.trace_peak_tokens(steps, round_to=page) // page
+    cache = engine.new_cache(pages, page, max_requests=4)
+    got = replay.run_trace(engine, cache, steps)
+    assert max(cut) > 1, "no step cut its keys"
+    check_against_plain(got, plain["bf16"], reqs, "bf16")
+
+
 @pytest.mark.parametrize("schedule", ["whole", "mixed"])
 def test_weights_stored_in_32_bit_stay_so_in_the_bfloat16_model(tmp_path, schedule):
     """A checkpoint in float32 run with dtype bf16: activations and cache are bfloat16, the
