@@ -102,8 +102,11 @@ DECODE_BLOCKS_WANTED = 256
 MIN_SPLIT = 128                     # keys per split at least: one 32-key block per wavefront
 MAX_SPLITS = 64                     # the join kernel's limit
 # Portions of prompts: work items (a span of rows x a group of heads) the prefill kernel should
-# have at least; with fewer, every item's keys are cut into runs of at least PREFILL_MIN_RUN keys.
+# have at least; with PREFILL_CUT_ITEMS or fewer (half a workgroup per compute unit; measured: 256
+# items cut in two were 3 % slower than whole), every item's keys are cut into runs of at least
+# PREFILL_MIN_RUN keys.
 PREFILL_ITEMS_WANTED = 512
+PREFILL_CUT_ITEMS = 128
 PREFILL_MIN_RUN = 512
 PREFILL_MAX_SPLITS = 16
 
@@ -127,7 +130,9 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
         group = n_q // n_kv
         items = groups * (n_q // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
         keys = max(c + n for n, c in zip(new_lens, ctx_lens) if n >= 2)
-        plan["prefill_splits"] = max(1, min(PREFILL_ITEMS_WANTED // items, keys // PREFILL_MIN_RUN, PREFILL_MAX_SPLITS))
+        if items <= PREFILL_CUT_ITEMS:
+            plan["prefill_splits"] = max(1, min(PREFILL_ITEMS_WANTED // items, keys // PREFILL_MIN_RUN,
+                                                PREFILL_MAX_SPLITS))
     if decode:
         longest = max(decode) if plan_len is None else max(plan_len, max(decode))
         pairs = len(decode) * n_kv * ((n_q // n_kv + 15) // 16)

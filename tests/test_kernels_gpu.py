@@ -436,6 +436,8 @@ def test_attention_plan_cuts_only_few_rows_over_many_keys(ops):
     plan = ops.mfma.plan_attention([256], [16128], 32, 8, 64)
     assert plan["prefill_splits"] == 8
     assert ops.mfma.plan_attention([2048], [0], 32, 8, 64)["prefill_splits"] == 1       # many items
+    assert ops.mfma.plan_attention([1024], [15360], 32, 8, 128)["prefill_splits"] == 1  # one item per compute unit
+    assert ops.mfma.plan_attention([512], [15872], 32, 8, 128)["prefill_splits"] == 4
     assert ops.mfma.plan_attention([64], [300], 32, 8, 64)["prefill_splits"] == 1       # few keys
     assert ops.mfma.plan_attention([64], [3000], 6, 2, 48)["prefill_splits"] == 1       # a head size without the kernel
     assert ops.mfma.plan_attention([1, 1], [5000, 9000], 32, 8, 64)["prefill_splits"] == 1
