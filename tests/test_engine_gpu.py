@@ -278,6 +278,35 @@ def test_a_far_key_is_found(tmp_path):
             assert err < 1e-5, (pos, err)
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_short_portions_far_into_a_long_prompt(zoo, dtype, monkeypatch):
+    """A prompt of 1,900 tokens: most of it in one step, then portions of 2 to 64 tokens and single
+    tokens. In bfloat16 the short portions behind 1,024 keys have their keys cut into runs by the
+    plan's own thresholds; the logits must not depend on that."""
+    from llmengine.ops import mfma
+    cut = []
+    plan_attention = mfma.plan_attention
+
+    def noting(*args, **kw):
+        plan = plan_attention(*args, **kw)
+        cut.append(plan["prefill_splits"])
+        return plan
+    monkeypatch.setattr(mfma, "plan_attention", noting)
+    model_dir, _, _, page = zoo["C"]
+    ids = random_tokens(1900, TINY_C["vocab_size"], 77)
+    pcfg, pw = load_plain_model(model_dir)
+    ref = plain_forward(pcfg, pw, ids, rounder=bf16_round if dtype == "bf16" else None).numpy()
+    engine = engine_for(model_dir, dtype)
+    steps = replay.portions({"s": ids}, sizes=(1100, 48, 2, 64, 1, 31, 300, 1, 17))
+    cache = engine.new_cache((1900 + page - 1) // page, page, max_requests=1)
+    got = replay.run_trace(engine, cache, steps)["s"]
+    if dtype == "bf16":
+        assert max(cut) > 1, "no step cut its keys"
+    for pos in range(len(ids)):
+        err = np.abs(got[pos].astype(np.float64) - ref[pos]).max() / np.abs(ref[pos]).max()
+        assert err < TOL[dtype], (pos, err)
+
+
 # A layer or two with the sizes of Llama 3.2 1B, 3.2 3B and 3.1 8B: the kernels that serving picks at
 # real widths (tiled products over several row tiles, the prefill attention with many work items, the
 # fused decode kernels at widths 2048, 3072 and 4096, the output head over the whole vocabulary).
