@@ -185,26 +185,44 @@ __global__ __launch_bounds__(64) void attention_join_kernel(const float* __restr
 }
 
 // The prefill kernel's key runs: grid (batch row, head); parts indexed by batch row. Rows of
-// requests that bring one token belong to the decode kernel and are left alone.
+// requests that bring one token belong to the decode kernel and are left alone, and so are rows
+// of work items with a single run, which wrote their output themselves. span_rows: rows of one
+// work item; the row's item and its number of runs are found as the prefill kernel finds them.
 __global__ __launch_bounds__(64) void attention_join_rows_kernel(const float* __restrict__ part_o,
                                                                  const float* __restrict__ part_ml,
                                                                  bf16* __restrict__ out, const int* __restrict__ q_start,
-                                                                 int n_seq, int n_q, int hd, int nsplit) {
+                                                                 const int* __restrict__ ctx_len, int n_seq, int n_q,
+                                                                 int hd, int nsplit, int run, int span_rows, int window) {
     __shared__ float weight[64];
     const int row = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-    bool mine = false;                                  // (the same in every lane)
+    int first_row = -1, n_new = 0, ctx = 0;             // the row's request (the same in every lane)
     for (int first = 0; first < n_seq; first += 64) {
         const int i = first + lane;
+        int a = 0, b = 0, c = 0;
         bool hit = false;
         if (i < n_seq) {
-            const int a = q_start[i], b = q_start[i + 1];
+            a = q_start[i];
+            b = q_start[i + 1];
             hit = a <= row && row < b && b - a >= 2;
+            if (hit) c = ctx_len[i];
         }
-        mine = mine || __any(hit);
+        const unsigned long long votes = __ballot(hit);
+        if (votes != 0) {
+            const int src = __ffsll(static_cast<long long>(votes)) - 1;
+            first_row = __shfl(a, src, 64);
+            n_new = __shfl(b, src, 64) - first_row;
+            ctx = __shfl(c, src, 64);
+        }
     }
-    if (!mine) return;
+    if (first_row < 0) return;
+    const int span = (row - first_row) / span_rows;
+    const int pos_span = ctx + span * span_rows;
+    const int n_span = n_new - span * span_rows < span_rows ? n_new - span * span_rows : span_rows;
+    const int key_lo = (window > 0 && pos_span - window + 1 > 0) ? pos_span - window + 1 : 0;
+    const int runs = key_runs(key_lo & ~63, pos_span + n_span, run, nsplit);
+    if (runs == 1) return;
     join_splits(part_o, part_ml, out + (static_cast<size_t>(row) * n_q + h) * hd,
-                (static_cast<size_t>(row) * n_q + h) * nsplit, hd, nsplit, weight);
+                (static_cast<size_t>(row) * n_q + h) * nsplit, hd, runs, weight);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -298,7 +316,8 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
                            const int* q_start, const int* ctx_len, const int* table, int max_blocks, int n_seq,
                            int n_q, int n_kv, int page, float scale, int window, int n_decode, int split_len,
                            int nsplit, int prefill_groups, int qt, int shared_rows, int* queue, int n_rows,
-                           int prefill_splits, float* pre_part_o, float* pre_part_ml, hipStream_t stream) {
+                           int prefill_splits, int prefill_run, float* pre_part_o, float* pre_part_ml,
+                           hipStream_t stream) {
     if (n_decode > 0) {
         const int G = n_q / n_kv;
         const dim3 grid(n_seq, n_kv * ((G + 15) / 16), nsplit);
@@ -318,10 +337,11 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
         if (shared_rows > 0) {
             const int status = launch_prefill_shared(q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q,
                                                      n_kv, HD, page, scale, window, prefill_groups, shared_rows, queue,
-                                                     prefill_splits, pre_part_o, pre_part_ml, stream);
+                                                     prefill_splits, prefill_run, pre_part_o, pre_part_ml, stream);
             if (status != 0 || prefill_splits <= 1) return status;
             hipLaunchKernelGGL(attention_join_rows_kernel, dim3(n_rows, n_q), dim3(64), 0, stream, pre_part_o,
-                               pre_part_ml, out, q_start, n_seq, n_q, HD, prefill_splits);
+                               pre_part_ml, out, q_start, ctx_len, n_seq, n_q, HD, prefill_splits, prefill_run,
+                               shared_rows, window);
             return launch_status();
         }
         const dim3 grid(prefill_groups, (n_q + 3) / 4);
@@ -381,10 +401,11 @@ extern "C" int llme_attention_bf16_rows(int hd, int n_q, int n_kv) {
 // row groups of llme_attention_bf16_rows(hd, n_q, n_kv) rows over the requests with two or more tokens.
 // queue: two integers, zero, for the prefill kernel's work counter (needed when prefill_groups > 0;
 // the kernel leaves them zero; launches that may overlap need separate ones).
-// prefill_splits > 1 (only where llme_attention_bf16_splits_prefill says so): the keys of every
-// prefill work item are cut into that many runs, joined by a second kernel over the batch's n_rows
-// rows; pre_part_o [n_rows, n_q, prefill_splits, hd] and pre_part_ml [n_rows, n_q, prefill_splits, 2]
-// floats are their scratch.
+// prefill_splits > 1 (only where llme_attention_bf16_splits_prefill says so): the keys of a prefill
+// work item are cut into runs of prefill_run stretches of 64 keys, at most prefill_splits (the
+// last run takes the rest), joined by a second kernel over the batch's n_rows rows; pre_part_o
+// [n_rows, n_q, prefill_splits, hd] and pre_part_ml [n_rows, n_q, prefill_splits, 2] floats are
+// their scratch.
 extern "C" int llme_attention_bf16_splits_prefill(int hd, int n_q, int n_kv) {
     return shared_rows_for(hd, n_q, n_kv) > 0 ? 1 : 0;
 }
@@ -393,11 +414,12 @@ extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const voi
                                    float* part_ml, const int* q_start, const int* ctx_len, const int* block_table,
                                    int max_blocks, int n_seq, int n_q, int n_kv, int hd, int page, float scale,
                                    int window, int n_decode, int split_len, int nsplit, int prefill_groups,
-                                   int* queue, int n_rows, int prefill_splits, float* pre_part_o, float* pre_part_ml,
-                                   hipStream_t stream) {
+                                   int* queue, int n_rows, int prefill_splits, int prefill_run, float* pre_part_o,
+                                   float* pre_part_ml, hipStream_t stream) {
     if (n_seq <= 0) return 0;
     if (prefill_splits < 1 || prefill_splits > 64 || n_rows < 0) return kErrBadArgument;
-    if (prefill_splits > 1 && (shared_rows_for(hd, n_q, n_kv) <= 0 || pre_part_o == nullptr || pre_part_ml == nullptr))
+    if (prefill_splits > 1 && (shared_rows_for(hd, n_q, n_kv) <= 0 || prefill_run < 1 || pre_part_o == nullptr ||
+                               pre_part_ml == nullptr))
         return kErrBadArgument;
     if (hd % 16 != 0 || hd > 128 || hd <= 0 || page % 16 != 0 || n_kv <= 0 || n_q % n_kv != 0) return kErrUnsupported;
     if (!(scale > 0.f)) return kErrBadArgument;      // the lazy maximum compares scaled scores
@@ -413,7 +435,7 @@ extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const voi
                                    static_cast<const bf16*>(v_cache), static_cast<bf16*>(out), part_o, part_ml, \
                                    q_start, ctx_len, block_table, max_blocks, n_seq, n_q, n_kv, page, scale,    \
                                    window, n_decode, split_len, nsplit, prefill_groups, qt, shared_rows, queue, n_rows, \
-                                   prefill_splits, pre_part_o, pre_part_ml, stream)
+                                   prefill_splits, prefill_run, pre_part_o, pre_part_ml, stream)
     switch (hd) {
         LLME_HEAD(16); LLME_HEAD(32); LLME_HEAD(48); LLME_HEAD(64);
         LLME_HEAD(80); LLME_HEAD(96); LLME_HEAD(112); LLME_HEAD(128);

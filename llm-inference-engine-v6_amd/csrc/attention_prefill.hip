@@ -24,9 +24,11 @@
 // without LDS.
 //
 // Few rows over a long context (a portion of a prompt far into it) are few work items that each
-// walk many keys. Then an item's keys are cut into `nsplit` runs of whole stretches, one work item
-// each, which leave their rows' maxima, sums and unscaled outputs in 32-bit scratch indexed by
-// batch row; a second kernel joins them, as it joins the splits of the decode kernel.
+// walk many keys, and in a prompt of a few thousand tokens the items of the last rows take twice
+// the average while the chip has room left. Then an item's keys are cut into up to `nsplit` runs of
+// `run` stretches, one work item each, which leave their rows' maxima, sums and unscaled outputs
+// in 32-bit scratch indexed by batch row; a second kernel joins them, as it joins the splits of
+// the decode kernel. Items with few keys have one run and write their output themselves.
 #include "attention_tiles.h"
 
 namespace llme {
@@ -161,9 +163,9 @@ __device__ __forceinline__ void read_block(const bf16* stage, int sb, KFrag<HD>&
 }
 
 // One work item: span `bx` (counted over the requests with two or more tokens, the last spans of
-// a request first) for head group `by`, run `z` of the `nsplit` runs of its keys (SPLIT; else all).
+// a request first) for head group `by`, run `z` of its keys (SPLIT; else all keys).
 template <int HD, int QT, int HPW, int KW, bool SPLIT>
-__device__ __forceinline__ void prefill_item(int bx, int by, int z, int nsplit, float* __restrict__ part_o,
+__device__ __forceinline__ void prefill_item(int bx, int by, int z, int nsplit, int run, float* __restrict__ part_o,
                                              float* __restrict__ part_ml, bf16* lds, const bf16* __restrict__ q,
                                              const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
                                              bf16* __restrict__ out, const int* __restrict__ q_start,
@@ -230,12 +232,12 @@ __device__ __forceinline__ void prefill_item(int bx, int by, int z, int nsplit, 
     int key_end = pos_span + n_span;
     const int key_lo = (window > 0 && pos_span - window + 1 > 0) ? pos_span - window + 1 : 0;
     int k_begin = key_lo & ~(KB - 1);
+    int runs = 1;
     if (SPLIT) {
-        // run z of the stretches; a run past the last key is empty and leaves sums of zero
-        const int stretches = (key_end - k_begin + KB - 1) / KB;
-        const int per_run = (stretches + nsplit - 1) / nsplit;
-        k_begin += z * per_run * KB;
-        if (key_end > k_begin + per_run * KB) key_end = k_begin + per_run * KB;
+        runs = key_runs(k_begin, key_end, run, nsplit);
+        if (z >= runs) return;                             // (the whole workgroup: no such run)
+        k_begin += z * run * KB;
+        if (z < runs - 1) key_end = k_begin + run * KB;    // (the last run takes the rest)
     }
     PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD,
                page_magic_of(page), static_cast<unsigned>(n_kv) * page * HD, static_cast<unsigned>(kvh) * page * HD};
@@ -327,7 +329,7 @@ __device__ __forceinline__ void prefill_item(int bx, int by, int z, int nsplit, 
         float lt = l[qt];
         lt += __shfl_xor(lt, 16, 64);
         lt += __shfl_xor(lt, 32, 64);
-        if (SPLIT) {
+        if (SPLIT && runs > 1) {
             // this run's part of row `row`, head `head`: statistics from the lanes of the row's
             // first quarter, outputs unscaled (the join divides)
             if (g4 == 0 && qt * 16 + r < n_rows) {
@@ -372,7 +374,7 @@ __global__ __launch_bounds__(256 * KW) void attention_prefill_shared_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     bf16* __restrict__ out, const int* __restrict__ q_start, const int* __restrict__ ctx_len,
     const int* __restrict__ block_table, int max_blocks, int n_seq, int n_q, int n_kv, int page, float scale,
-    int window, int spans, int* __restrict__ queue, int nsplit, float* __restrict__ part_o,
+    int window, int spans, int* __restrict__ queue, int nsplit, int run, float* __restrict__ part_o,
     float* __restrict__ part_ml) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     __shared__ int next_item;
@@ -387,7 +389,7 @@ __global__ __launch_bounds__(256 * KW) void attention_prefill_shared_kernel(
         if (item >= n_items) break;                        // the counter only grows: every workgroup gets here
         const int whole = SPLIT ? item / nsplit : item;     // (an item's runs are neighbours in the queue)
         prefill_item<HD, QT, HPW, KW, SPLIT>(whole / head_groups, whole % head_groups, SPLIT ? item % nsplit : 0, nsplit,
-                                             part_o, part_ml, lds, q, k_cache, v_cache, out, q_start, ctx_len,
+                                             run, part_o, part_ml, lds, q, k_cache, v_cache, out, q_start, ctx_len,
                                              block_table, max_blocks, n_seq, n_q, n_kv, page, scale, window);
     }
     if (threadIdx.x == 0) {
@@ -418,8 +420,8 @@ int prefill_shared_rows(int hd, int n_q, int n_kv) {
 template <int HD, int QT, int HPW, int KW, bool SPLIT>
 static int launch_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, const int* q_start,
                          const int* ctx_len, const int* table, int max_blocks, int n_seq, int n_q, int n_kv, int page,
-                         float scale, int window, int items, int* queue, int nsplit, float* part_o, float* part_ml,
-                         hipStream_t stream) {
+                         float scale, int window, int items, int* queue, int nsplit, int run, float* part_o,
+                         float* part_ml, hipStream_t stream) {
     constexpr int LDS = StageLayout<HD>::BYTES;
     auto kernel = attention_prefill_shared_kernel<HD, QT, HPW, KW, SPLIT>;
     static bool attr_set = false;                      // per instantiation
@@ -443,24 +445,24 @@ static int launch_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* ou
     const int n_items = items * (n_q / HPW) * (SPLIT ? nsplit : 1);
     hipLaunchKernelGGL(kernel, dim3(n_items < resident ? n_items : resident), dim3(256 * KW), LDS, stream, q, kc, vc, out,
                        q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, page, scale, window, items, queue, nsplit,
-                       part_o, part_ml);
+                       run, part_o, part_ml);
     return launch_status();
 }
 
 int launch_prefill_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, const int* q_start,
                           const int* ctx_len, const int* table, int max_blocks, int n_seq, int n_q, int n_kv, int hd,
                           int page, float scale, int window, int items, int rows_per_item, int* queue, int nsplit,
-                          float* part_o, float* part_ml, hipStream_t stream) {
+                          int run, float* part_o, float* part_ml, hipStream_t stream) {
     if (queue == nullptr) return kErrBadArgument;
-    if (nsplit < 1 || (nsplit > 1 && (part_o == nullptr || part_ml == nullptr))) return kErrBadArgument;
+    if (nsplit < 1 || (nsplit > 1 && (run < 1 || part_o == nullptr || part_ml == nullptr))) return kErrBadArgument;
     const int hpw = heads_per_workgroup(n_q, n_kv);
     const int rows = rows_per_item / (4 / hpw);            // per row group
     // Two wavefronts per tile while the items are too few to keep three workgroups of four
     // wavefronts on every compute unit: then an item's length, not the chip, sets the time.
-    int kw = static_cast<long>(items) * (n_q / hpw) * nsplit <= kSplitBelowItems ? 2 : 1;
+    int kw = static_cast<long>(items) * (n_q / hpw) <= kSplitBelowItems ? 2 : 1;
     if (g_key_waves == 1 || g_key_waves == 2) kw = g_key_waves;
 #define LLME_SHARED_ARGS q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, page, scale, window, \
-                         items, queue, nsplit, part_o, part_ml, stream
+                         items, queue, nsplit, run, part_o, part_ml, stream
 #define LLME_SHARED(HD, QT, HPW)                                                       \
     if (hd == HD && rows == 16 * QT && hpw == HPW) {                                   \
         if (nsplit > 1)                                                                \

@@ -351,13 +351,22 @@ __device__ __forceinline__ void load_q(const bf16* qrow, bool ok, bf16x8 (&qf)[(
 
 // The prefill kernel that shares K and V blocks among a workgroup's wavefronts through LDS
 // (attention_prefill.hip). rows_per_item: rows of one work item, see prefill_shared_rows; queue:
-// two integers that are zero and that no other launch in flight uses. nsplit > 1: every item's
-// keys are cut into nsplit runs whose results go to part_o [rows, n_q, nsplit, hd] and part_ml
-// [rows, n_q, nsplit, 2] (by batch row) instead of out; the caller joins them.
+// two integers that are zero and that no other launch in flight uses. nsplit > 1: an item's keys
+// are cut into key_runs(...) runs of `run` stretches; items with one run write out, the runs of
+// the others go to part_o [rows, n_q, nsplit, hd] and part_ml [rows, n_q, nsplit, 2] (by batch
+// row) and the caller joins them.
 int launch_prefill_shared(const bf16* q, const bf16* k_cache, const bf16* v_cache, bf16* out, const int* q_start,
                           const int* ctx_len, const int* block_table, int max_blocks, int n_seq, int n_q, int n_kv,
                           int hd, int page, float scale, int window, int items, int rows_per_item, int* queue,
-                          int nsplit, float* part_o, float* part_ml, hipStream_t stream);
+                          int nsplit, int run, float* part_o, float* part_ml, hipStream_t stream);
+
+// Runs that the keys [k_begin, key_end) of a prefill work item are cut into: `run` stretches of 64
+// keys each, at most max_runs (the last run then takes the rest).
+__host__ __device__ __forceinline__ int key_runs(int k_begin, int key_end, int run, int max_runs) {
+    const int stretches = (key_end - k_begin + 63) / 64;
+    const int runs = (stretches + run - 1) / run;
+    return runs < 1 ? 1 : (runs > max_runs ? max_runs : runs);
+}
 // Rows per work item of the shared kernel for these sizes, or 0 if it does not take them.
 int prefill_shared_rows(int hd, int n_q, int n_kv);
 // Wavefronts that share a tile's keys: 0 lets the launcher choose by the number of items, 1 or 2 forces it.

@@ -80,7 +80,7 @@ declare("llme_attention_bf16_set_rows", [_i, _i])
 declare("llme_attention_bf16_set_stream", [_i])
 declare("llme_attention_bf16_splits_prefill", [_i, _i, _i])
 declare("llme_attention_bf16", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i,
-                                _i, _i, _i, _i, _vp, _i, _i, _vp, _vp, _vp])
+                                _i, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp, _vp])
 
 _work_queues: dict = {}
 
@@ -103,10 +103,13 @@ MIN_SPLIT = 128                     # keys per split at least: one 32-key block 
 MAX_SPLITS = 64                     # the join kernel's limit
 # Portions of prompts: work items (a span of rows x a group of heads) the prefill kernel should
 # have at least; with PREFILL_CUT_ITEMS or fewer (half a workgroup per compute unit; measured: 256
-# items cut in two were 3 % slower than whole), every item's keys are cut into runs of at least
-# PREFILL_MIN_RUN keys.
+# items cut in two were 3 % slower than whole), the longest item's keys are cut into that many
+# runs of at least PREFILL_MIN_RUN keys, and the others' into runs of the same length.
 PREFILL_ITEMS_WANTED = 512
 PREFILL_CUT_ITEMS = 128
+# (A whole prompt of 2,048 tokens, whose last rows' items walk twice the average, was also tried with
+# the items behind 1,024 keys cut in two: 6.5 to 6.6 ms against 5.95 whole; the partial outputs and
+# the join cost more than the evener load wins.)
 PREFILL_MIN_RUN = 512
 PREFILL_MAX_SPLITS = 16
 
@@ -124,15 +127,20 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
     rows = entry("llme_attention_bf16_rows")(head_dim, n_q, n_kv)
     decode = [c + 1 for n, c in zip(new_lens, ctx_lens) if n == 1]
     groups = sum((n + rows - 1) // rows for n in new_lens if n >= 2)
-    plan = {"n_decode": len(decode), "groups": groups, "split_len": 32, "nsplit": 1, "prefill_splits": 1}
+    plan = {"n_decode": len(decode), "groups": groups, "split_len": 32, "nsplit": 1, "prefill_splits": 1,
+            "prefill_run": 1}
     if groups and entry("llme_attention_bf16_splits_prefill")(head_dim, n_q, n_kv):
         # few rows over long contexts: too few work items for the chip, each with many keys
         group = n_q // n_kv
         items = groups * (n_q // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
         keys = max(c + n for n, c in zip(new_lens, ctx_lens) if n >= 2)
+        splits = 1
         if items <= PREFILL_CUT_ITEMS:
-            plan["prefill_splits"] = max(1, min(PREFILL_ITEMS_WANTED // items, keys // PREFILL_MIN_RUN,
-                                                PREFILL_MAX_SPLITS))
+            splits = max(1, min(PREFILL_ITEMS_WANTED // items, keys // PREFILL_MIN_RUN, PREFILL_MAX_SPLITS))
+            stretches = (keys + 63) // 64
+            run = (stretches + splits - 1) // splits       # stretches of 64 keys per run
+        if splits > 1:
+            plan["prefill_splits"], plan["prefill_run"] = splits, run
     if decode:
         longest = max(decode) if plan_len is None else max(plan_len, max(decode))
         pairs = len(decode) * n_kv * ((n_q // n_kv + 15) // 16)
@@ -179,7 +187,7 @@ def attention_bf16(q, k_cache, v_cache, out, q_start, ctx_len, block_table, n_q:
         ptr(q), ptr(k_cache), ptr(v_cache), ptr(out), ptr(part_o), ptr(part_ml), ptr(q_start), ptr(ctx_len),
         ptr(block_table), block_table.shape[1], S, n_q, n_kv, head_dim, page, float(scale), int(window),
         plan["n_decode"], plan["split_len"], plan["nsplit"], plan["groups"],
-        ptr(work_queue(q.device)) if plan["groups"] else None, T, pre_splits,
+        ptr(work_queue(q.device)) if plan["groups"] else None, T, pre_splits, max(1, int(plan.get("prefill_run", 1))),
         ptr(pre_part_o) if pre_splits > 1 else None, ptr(pre_part_ml) if pre_splits > 1 else None, stream()),
         "attention_bf16")
 

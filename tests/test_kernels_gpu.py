@@ -308,9 +308,10 @@ def test_gemm_dispatch_and_refusals(ops):
 
 
 # --- MFMA attention ----------------------------------------------------------------------
-def _attn_case(ops, lens, news, n_q, n_kv, hd, page, window=0, seed=50, prefill_splits=None):
+def _attn_case(ops, lens, news, n_q, n_kv, hd, page, window=0, seed=50, prefill_splits=None, prefill_run=1):
     """Requests with lens[i] tokens in the cache, of which the last news[i] are this step's.
-    prefill_splits: cut the keys of the prompt portions into that many runs, whatever the plan says."""
+    prefill_splits, prefill_run: cut the keys of the prompt portions into at most that many runs of that
+    many 64-key stretches, whatever the plan says."""
     s = _paged_setup(ops, lens, n_q, n_kv, hd, page, torch.bfloat16, seed=seed)
     rows, q_start, ctx = [], [0], []
     base = 0
@@ -327,7 +328,7 @@ def _attn_case(ops, lens, news, n_q, n_kv, hd, page, window=0, seed=50, prefill_
     part_o = torch.empty(S * n_q * plan["nsplit"] * hd, device=DEV)
     part_ml = torch.empty(S * n_q * plan["nsplit"] * 2, device=DEV)
     if prefill_splits is not None:
-        plan["prefill_splits"] = prefill_splits
+        plan["prefill_splits"], plan["prefill_run"] = prefill_splits, prefill_run
     # (the scratch starts as NaN: a part that is joined without having been written shows)
     pre_o = torch.full((len(rows) * n_q * plan["prefill_splits"] * hd,), float("nan"), device=DEV)
     pre_ml = torch.full((len(rows) * n_q * plan["prefill_splits"] * 2,), float("nan"), device=DEV)
@@ -398,17 +399,18 @@ def test_attention_prefill_shared_window(ops, window, n_q, n_kv):
 
 @pytest.mark.parametrize("n_q,n_kv,hd,page", [(8, 2, 64, 16), (6, 2, 64, 32), (3, 3, 64, 16), (8, 2, 128, 16),
                                               (5, 5, 128, 48)])
-@pytest.mark.parametrize("splits,key_waves", [(2, -1), (3, 2), (7, 3), (16, -1)])
-def test_attention_prefill_cut_keys(ops, n_q, n_kv, hd, page, splits, key_waves):
+@pytest.mark.parametrize("splits,key_waves,run", [(2, -1, 1), (3, 2, 2), (7, 3, 1), (16, -1, 3), (4, -1, 5), (4, 3, 100)])
+def test_attention_prefill_cut_keys(ops, n_q, n_kv, hd, page, splits, key_waves, run):
     """Prompt portions whose keys are cut into runs that a second kernel joins: runs that end
-    inside a span's own rows, runs with no key at all (more runs than 64-key stretches), whole
-    prompts and decoded tokens beside them, with one and two wavefronts per tile."""
+    inside a span's own rows, a last run that takes the rest, items with a single run beside items
+    with several (and all of them single), whole prompts and decoded tokens beside them, with one
+    and two wavefronts per tile."""
     set_rows = ops.lib.entry("llme_attention_bf16_set_rows")
     assert set_rows(0, key_waves) == 0
     try:
         lens = [700, 2, 131, 64, 517, 65, 9]
         news = [40, 2, 67, 64, 130, 3, 1]
-        out, ref, plan = _attn_case(ops, lens, news, n_q, n_kv, hd, page, seed=63, prefill_splits=splits)
+        out, ref, plan = _attn_case(ops, lens, news, n_q, n_kv, hd, page, seed=63, prefill_splits=splits, prefill_run=run)
         assert plan["n_decode"] == 1 and plan["prefill_splits"] == splits
         assert not out.isnan().any()
         assert _rel(out, ref) < 8e-3
@@ -418,7 +420,8 @@ def test_attention_prefill_cut_keys(ops, n_q, n_kv, hd, page, splits, key_waves)
 
 @pytest.mark.parametrize("window", [1, 64, 65, 200])
 def test_attention_prefill_cut_keys_window(ops, window):
-    out, ref, _ = _attn_case(ops, [600, 70, 190], [140, 70, 2], 8, 2, 64, 16, window=window, seed=64, prefill_splits=4)
+    out, ref, _ = _attn_case(ops, [600, 70, 190], [140, 70, 2], 8, 2, 64, 16, window=window, seed=64, prefill_splits=4,
+                             prefill_run=2)
     assert not out.isnan().any()
     assert _rel(out, ref) < 8e-3
 
@@ -435,9 +438,10 @@ def test_attention_prefill_cut_keys_by_plan(ops):
 def test_attention_plan_cuts_only_few_rows_over_many_keys(ops):
     plan = ops.mfma.plan_attention([256], [16128], 32, 8, 64)
     assert plan["prefill_splits"] == 8
-    assert ops.mfma.plan_attention([2048], [0], 32, 8, 64)["prefill_splits"] == 1       # many items
     assert ops.mfma.plan_attention([1024], [15360], 32, 8, 128)["prefill_splits"] == 1  # one item per compute unit
-    assert ops.mfma.plan_attention([512], [15872], 32, 8, 128)["prefill_splits"] == 4
+    plan = ops.mfma.plan_attention([512], [15872], 32, 8, 128)
+    assert (plan["prefill_splits"], plan["prefill_run"]) == (4, 64)
+    assert ops.mfma.plan_attention([2048], [0], 32, 8, 64)["prefill_splits"] == 1       # many items
     assert ops.mfma.plan_attention([64], [300], 32, 8, 64)["prefill_splits"] == 1       # few keys
     assert ops.mfma.plan_attention([64], [3000], 6, 2, 48)["prefill_splits"] == 1       # a head size without the kernel
     assert ops.mfma.plan_attention([1, 1], [5000, 9000], 32, 8, 64)["prefill_splits"] == 1
