@@ -483,13 +483,37 @@ def test_attention_mfma_finds_one_far_key(ops):
     plan = ops.mfma.plan_attention([1, 10], [399, 390], n_q, n_kv, hd)
     part_o = torch.empty(2 * n_q * plan["nsplit"] * hd, device=DEV)
     part_ml = torch.empty(2 * n_q * plan["nsplit"] * 2, device=DEV)
-    ops.mfma.attention_bf16(q, k_cache, v_cache, out, torch.tensor([0, 1, 11], **i32),
-                            torch.tensor([399, 390], **i32), table.to(DEV), n_q, n_kv, hd, 1.0, 0, plan, part_o, part_ml)
     v = qkv[:, (n_q + n_kv) * hd:].to(torch.bfloat16).double().view(T, n_kv, hd)
-    for row, base in ((0, 0), (10, 400)):
-        for h in range(n_q):
-            got = out[row].cpu().double().view(n_q, hd)[h]
-            assert (got - v[base + far, h // 2]).abs().max() < 2e-2, (row, h)
+    # whole, and with the portion's keys cut into runs of 128: the far key lies in the first run,
+    # the rows' own keys in the last
+    for splits, run in ((1, 1), (4, 2)):
+        plan["prefill_splits"], plan["prefill_run"] = splits, run
+        pre_o = torch.full((len(rows) * n_q * splits * hd,), float("nan"), device=DEV)
+        pre_ml = torch.full((len(rows) * n_q * splits * 2,), float("nan"), device=DEV)
+        out.zero_()
+        ops.mfma.attention_bf16(q, k_cache, v_cache, out, torch.tensor([0, 1, 11], **i32),
+                                torch.tensor([399, 390], **i32), table.to(DEV), n_q, n_kv, hd, 1.0, 0, plan, part_o,
+                                part_ml, pre_o, pre_ml)
+        for row, base in ((0, 0), (10, 400)):
+            for h in range(n_q):
+                got = out[row].cpu().double().view(n_q, hd)[h]
+                assert (got - v[base + far, h // 2]).abs().max() < 2e-2, (splits, row, h)
+    # cut keys need their scratch, and a head size that the kernel with LDS takes
+    from llmengine.ops import KernelError
+    with pytest.raises(KernelError):
+        ops.mfma.attention_bf16(q, k_cache, v_cache, out, torch.tensor([0, 1, 11], **i32),
+                                torch.tensor([399, 390], **i32), table.to(DEV), n_q, n_kv, hd, 1.0, 0, plan, part_o,
+                                part_ml, pre_o[:100], pre_ml)
+    with pytest.raises(KernelError):
+        ops.mfma.attention_bf16(q, k_cache, v_cache, out, torch.tensor([0, 1, 11], **i32),
+                                torch.tensor([399, 390], **i32), table.to(DEV), n_q, n_kv, hd, 1.0, 0, plan, part_o,
+                                part_ml)
+    q32 = q.view(len(rows), 2 * n_q, 32).contiguous().view(len(rows), -1)      # the same bytes as heads of 32
+    k32, v32 = k_cache.view(2 * nblk, 2 * n_kv, page, 32), v_cache.view(2 * nblk, 2 * n_kv, 32, page)
+    with pytest.raises(KernelError):
+        ops.mfma.attention_bf16(q32, k32, v32, out, torch.tensor([0, 1, 11], **i32), torch.tensor([399, 390], **i32),
+                                table.to(DEV), 2 * n_q, 2 * n_kv, 32, 1.0, 0, plan, part_o, part_ml,
+                                torch.empty(len(rows) * 2 * n_q * 4 * 32, device=DEV), pre_ml.repeat(2))
 
 
 # --- projections fused with the norm in front of them -----------------------------------
