@@ -39,6 +39,7 @@ class Sampler:
             raise ValueError("temperature must be >= 0")
         self.temperature = float(temperature)
         self.seed = int(seed)
+        self._device_rows: dict = {}            # (device, rows) -> [2, rows]: temperatures, draws
 
     def choose(self, logits: torch.Tensor, draws: Sequence[tuple[int, int]] | None = None) -> list[int]:
         """One token per row of logits [R, V] (32-bit, on the device). `draws` gives
@@ -50,7 +51,12 @@ class Sampler:
         else:
             if draws is None or len(draws) != R:
                 raise ValueError("temperature sampling needs a (request, index) pair per row")
-            u = torch.tensor([uniform_draw(self.seed, r, i) for r, i in draws], dtype=torch.float32)
-            t = torch.full((R,), self.temperature, dtype=torch.float32)
-            ops.sample(logits, t.to(logits.device), u.to(logits.device), out)
+            # the temperatures stay on the device from one step to the next; only the draws go up
+            key = (logits.device, R)
+            held = self._device_rows.get(key)
+            if held is None:
+                held = self._device_rows[key] = torch.empty(2, R, dtype=torch.float32, device=logits.device)
+                held[0].fill_(self.temperature)
+            held[1].copy_(torch.tensor([uniform_draw(self.seed, r, i) for r, i in draws], dtype=torch.float32))
+            ops.sample(logits, held[0], held[1], out)
         return out.tolist()
