@@ -107,11 +107,11 @@ MAX_SPLITS = 64                     # the join kernel's limit
 # runs of at least PREFILL_MIN_RUN keys, and the others' into runs of the same length.
 PREFILL_ITEMS_WANTED = 512
 PREFILL_CUT_ITEMS = 128
+PREFILL_MIN_RUN = 512
+PREFILL_MAX_SPLITS = 16
 # (A whole prompt of 2,048 tokens, whose last rows' items walk twice the average, was also tried with
 # the items behind 1,024 keys cut in two: 6.5 to 6.6 ms against 5.95 whole; the partial outputs and
 # the join cost more than the evener load wins.)
-PREFILL_MIN_RUN = 512
-PREFILL_MAX_SPLITS = 16
 
 
 def attention_bf16_supported(q, k_cache, head_dim: int) -> bool:
