@@ -137,6 +137,33 @@ def serve(args, engine, cfg: dict, gen, page: int) -> int:
     return 0
 
 
+def portion(args, engine, cfg: dict, gen, page: int) -> int:
+    """A long prompt that arrives in portions (a prefill budget per step): the steps of --portion
+    tokens once --context tokens are cached. Few rows over many keys."""
+    import torch
+    from llmengine import StepEntry
+    V, n, ctx = cfg["vocab_size"], args.portion, args.context
+    steps = max(4, min(args.steps, 16))
+    cache = engine.new_cache((ctx + (steps + 2) * n) // page + 2, page, 1)
+    cache.admit("p")
+    for at in range(0, ctx, 2048):
+        engine.step(cache, [StepEntry("p", torch.randint(0, V, (min(2048, ctx - at),), generator=gen).tolist(), [])])
+    tokens = torch.randint(0, V, (n,), generator=gen).tolist()
+    engine.step(cache, [StepEntry("p", tokens, [n - 1])])
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    for _ in range(steps):
+        engine.step(cache, [StepEntry("p", tokens, [n - 1])])
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t) / steps * 1e3
+    log(f"portions of {n} tokens behind {ctx}: {ms:.2f} ms a step")
+    print(json.dumps({"metric": "portion_tokens_per_second", "value": round(n / (ms / 1e3), 1), "unit": "tokens/s",
+                      "n_gpus": 1, "dtype": args.dtype, "ms_per_step": round(ms, 3), "steps": steps,
+                      "config": {"model": args.shape, "layers": args.layers, "context": ctx, "portion": n,
+                                 "page_size": page}}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -150,9 +177,11 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode", "serve"],
+    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode", "serve", "portion"],
                     help="run only one part (for profiling); the JSON line then lacks the other. 'serve' is another "
-                         "workload: requests of mixed lengths through the continuous-batching scheduler")
+                         "workload: requests of mixed lengths through the continuous-batching scheduler; 'portion': "
+                         "steps of --portion prompt tokens of one request behind --context tokens")
+    ap.add_argument("--portion", type=int, default=256, help="portion: prompt tokens a step")
     ap.add_argument("--requests", type=int, default=32, help="serve: number of requests")
     ap.add_argument("--prompt-range", default="64,3072", help="serve: prompt lengths, uniform in [a, b]")
     ap.add_argument("--new-range", default="128,512", help="serve: new tokens per request, uniform in [a, b]")
@@ -184,6 +213,8 @@ def main() -> int:
 
     if args.phase == "serve":
         return serve(args, engine, cfg, gen, page)
+    if args.phase == "portion":
+        return portion(args, engine, cfg, gen, page)
 
     # ---- prefill: one prompt, logits at its last place ----
     T = args.prefill_tokens
