@@ -103,6 +103,7 @@ class Engine:
         self._runner: ModelRunner | None = None
         self._lock = threading.RLock()
         self.sampler = Sampler(temperature, sampler_seed)
+        self._samplers = {(self.sampler.temperature, self.sampler.seed): self.sampler}   # kept: they hold device rows
         self.block_size = int(block_size)
         self.prefill_chunk = int(max_prefill_tokens_per_step)
         self._own_cache: CacheContext | None = None
@@ -199,8 +200,11 @@ class Engine:
             logits = self.runner.step(cache, entries, max_position=self.max_pos)
             if logits is None:
                 return []
-            sampler = self.sampler if (temperature == self.sampler.temperature and seed == self.sampler.seed) \
-                else Sampler(temperature, seed)
+            sampler = self._samplers.get((float(temperature), int(seed)))
+            if sampler is None:
+                if len(self._samplers) >= 64:
+                    self._samplers = {(self.sampler.temperature, self.sampler.seed): self.sampler}
+                sampler = self._samplers[(float(temperature), int(seed))] = Sampler(temperature, seed)
             return sampler.choose(logits, draws)
 
     # ---- whole-sequence logits (src/engine.cpp:694-716) ----

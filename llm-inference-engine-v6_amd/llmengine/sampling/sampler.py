@@ -39,7 +39,7 @@ class Sampler:
             raise ValueError("temperature must be >= 0")
         self.temperature = float(temperature)
         self.seed = int(seed)
-        self._device_rows: dict = {}            # (device, rows) -> [2, rows]: temperatures, draws
+        self._device_rows: dict = {}            # (device, rows) -> ([2, rows] temperatures and draws, pinned draws)
 
     def choose(self, logits: torch.Tensor, draws: Sequence[tuple[int, int]] | None = None) -> list[int]:
         """One token per row of logits [R, V] (32-bit, on the device). `draws` gives
@@ -52,11 +52,16 @@ class Sampler:
             if draws is None or len(draws) != R:
                 raise ValueError("temperature sampling needs a (request, index) pair per row")
             # the temperatures stay on the device from one step to the next; only the draws go up
+            # (from pinned memory, so the copy does not wait; the tokens' read-back below ends
+            # the step before the next one writes the pinned row again)
             key = (logits.device, R)
             held = self._device_rows.get(key)
             if held is None:
-                held = self._device_rows[key] = torch.empty(2, R, dtype=torch.float32, device=logits.device)
-                held[0].fill_(self.temperature)
-            held[1].copy_(torch.tensor([uniform_draw(self.seed, r, i) for r, i in draws], dtype=torch.float32))
-            ops.sample(logits, held[0], held[1], out)
+                rows = torch.empty(2, R, dtype=torch.float32, device=logits.device)
+                rows[0].fill_(self.temperature)
+                held = self._device_rows[key] = (rows, torch.empty(R, dtype=torch.float32, pin_memory=True))
+            rows, pinned = held
+            pinned.copy_(torch.tensor([uniform_draw(self.seed, r, i) for r, i in draws], dtype=torch.float32))
+            rows[1].copy_(pinned, non_blocking=True)
+            ops.sample(logits, rows[0], rows[1], out)
         return out.tolist()
