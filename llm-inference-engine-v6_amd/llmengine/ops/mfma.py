@@ -24,7 +24,8 @@ def gemm_bf16_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, acc
 
 
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, *,
-              gated: bool = False, waves: int = 0, ksplit: int = 0, tile: int = 0, force_tile: bool = False) -> None:
+              gated: bool = False, waves: int = 0, ksplit: int = 0, tile: int = 0, force_tile: bool = False,
+              _supported: bool = False) -> None:
     """bfloat16 a [M, K] and w [N, K] -> out [M, N] (float32 or bfloat16), 32-bit accumulation.
     K must be a multiple of 8. gated: w holds gate and up rows interleaved in groups of 16 and
     out is bfloat16 [M, N / 2] = silu(gate) * up. waves / ksplit / tile (64, 128, 128096, 128064) /
@@ -38,7 +39,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
             raise kernels.KernelError("gemm_bf16: a gated product needs a multiple of 32 weight rows and no accumulation")
     else:
         require(out, "out", (torch.float32, torch.bfloat16), (M, N))
-    if not gemm_bf16_supported(a, w, out, accumulate):
+    if not _supported and not gemm_bf16_supported(a, w, out, accumulate):     # (the dispatcher has asked already)
         raise kernels.KernelError(f"gemm_bf16: K={K} must be a multiple of 8, pointers 16-byte aligned, and "
                                   "accumulation needs a float32 output")
     if force_tile and not tile:
@@ -57,7 +58,7 @@ def gemm_gated(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, grou
     T, FF = out.shape
     if (kernels.policy.fast_gemm and group == 16 and out.dtype == torch.bfloat16 and (2 * FF) % 32 == 0
             and x.dtype == torch.bfloat16 and gemm_bf16_supported(x, w_gate_up, out, False)):
-        gemm_bf16(x, w_gate_up, out, gated=True)
+        gemm_bf16(x, w_gate_up, out, gated=True, _supported=True)
         return
     gu = scratch((T, 2 * FF), torch.float32)
     kernels.gemm(x, w_gate_up, gu)
@@ -67,7 +68,7 @@ def gemm_gated(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, grou
 def _fast_gemm(a, w, out, accumulate) -> bool:
     if a.dim() != 2 or w.dim() not in (2, 5) or not gemm_bf16_supported(a, w, out, accumulate):
         return False
-    gemm_bf16(a, w, out, accumulate)
+    gemm_bf16(a, w, out, accumulate, _supported=True)
     return True
 
 
