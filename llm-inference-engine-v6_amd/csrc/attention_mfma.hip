@@ -31,7 +31,10 @@
 //
 // Limits (the caller checks them and otherwise uses the plain-precision kernel): head size a
 // multiple of 16 up to 128; page size a multiple of 16.
+#include <mutex>
+
 #include "attention_tiles.h"
+#include "llmengine_noalloc.h"
 
 namespace llme {
 
@@ -442,4 +445,74 @@ extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const voi
         default: return kErrUnsupported;
     }
 #undef LLME_HEAD
+}
+
+// ------------------------------------------------------------------------------------------
+// Decode attention for callers that cannot allocate (declared in llmengine_noalloc.h). The split
+// decode kernel and its join are the ones above; the splits' partial results go into a fixed
+// array in device memory instead of a workspace that the caller brings. Every device the library
+// runs on holds its own copy of the array, at its own address, until the process ends; the address
+// is asked for once per device, with that device current, and kept.
+static __device__ __align__(256) float scratch[LLME_NOALLOC_SCRATCH_FLOATS];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+// The array's address on the current device (host code must never use the array's name as one).
+int scratch_of_current_device(float** ptr) {
+    int device = -1;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return static_cast<int>(err);
+    if (device < 0 || device >= kMaxDevices) return kErrUnsupported;
+    std::lock_guard<std::mutex> guard(g_scratch_mutex);
+    if (g_scratch_ptr[device] == nullptr) {
+        void* address = nullptr;
+        err = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return static_cast<int>(err);
+        if (address == nullptr) return kErrUnsupported;
+        g_scratch_ptr[device] = static_cast<float*>(address);
+    }
+    *ptr = g_scratch_ptr[device];
+    return 0;
+}
+}  // namespace
+
+extern "C" int llme_noalloc_init(void) {
+    float* ptr = nullptr;
+    return scratch_of_current_device(&ptr);
+}
+
+extern "C" long llme_attention_decode_noalloc_scratch_floats(int n_seq, int n_q, int hd, int nsplit) {
+    return static_cast<long>(n_seq) * n_q * nsplit * (hd + 2);
+}
+
+extern "C" int llme_attention_decode_noalloc(const void* q, const void* k_cache, const void* v_cache, void* out,
+                                             const int* q_start, const int* ctx_len, const int* block_table,
+                                             int max_blocks, int n_seq, int n_q, int n_kv, int hd, int page,
+                                             float scale, int window, int split_len, int nsplit,
+                                             hipStream_t stream) {
+    if (n_seq <= 0) return 0;
+    if (q == nullptr || k_cache == nullptr || v_cache == nullptr || out == nullptr || q_start == nullptr ||
+        ctx_len == nullptr || block_table == nullptr || max_blocks <= 0)
+        return kErrBadArgument;
+    if (n_q <= 0 || n_kv <= 0 || hd <= 0 || split_len <= 0 || split_len % 32 != 0 || nsplit <= 0 || nsplit > 64)
+        return kErrBadArgument;
+    // the partial results of all splits must fit into the fixed array
+    const double need = static_cast<double>(n_seq) * n_q * nsplit * (hd + 2);
+    if (nsplit > 1 && need > static_cast<double>(LLME_NOALLOC_SCRATCH_FLOATS)) return kErrUnsupported;
+    float* base = nullptr;
+    const int status = scratch_of_current_device(&base);
+    if (status != 0) return status;
+    // Layout: part_o [n_seq, n_q, nsplit, hd], then part_ml [n_seq, n_q, nsplit, 2] (hd is a multiple
+    // of 16, so part_ml starts on a 64-byte boundary). Every part the join reads has been written by
+    // the decode kernel of the same call (a split past a request's last key writes an empty part),
+    // so nothing has to be cleared between calls.
+    float* part_o = base;
+    float* part_ml = base + static_cast<size_t>(n_seq) * n_q * nsplit * hd;
+    return llme_attention_bf16(q, k_cache, v_cache, out, part_o, part_ml, q_start, ctx_len, block_table, max_blocks,
+                               n_seq, n_q, n_kv, hd, page, scale, window, /*n_decode=*/n_seq, split_len, nsplit,
+                               /*prefill_groups=*/0, /*queue=*/nullptr, /*n_rows=*/n_seq, /*prefill_splits=*/1,
+                               /*prefill_run=*/1, nullptr, nullptr, stream);
 }
