@@ -1,21 +1,25 @@
 // Decode-time projections fused with the RMSNorm in front of them (and, for the gated
 // feed-forward, with the activation behind them), for up to 16 rows:
 //
-//   plain:  out[m, n]  = inv_m * sum_k bf16(w_norm[k] * h[row(m), k]) * W[n, k]
+//   plain:  out[m, n]  = sum_k bf16((w_norm[k] * h[row(m), k]) * inv_m) * W[n, k]
 //   gated:  out[m, j]  = silu(g) * u,  g, u = the same sums over the gate and the up row of unit j
 //   inv_m = 1 / sqrt(mean_k h[row(m), k]^2 + eps)          (src/kernels.cpp:18-24, 26-31, 33-57)
 //
-// The norm's scale is a factor per row, so it is applied to the 32-bit sums after the product;
-// the activations enter the product as bf16(w_norm * h). h is the 32-bit residual stream,
-// row(m) = rows ? rows[m] : m (the output head reads the wanted rows only).
+// The activations enter the product as the norm kernel would have stored them: the normed value
+// rounded to bfloat16, scale included. (Rounding bf16(w_norm * h) and scaling the 32-bit sums
+// afterwards saves a pass over the row and is as accurate, but rounds other values than the norm
+// kernel does: a token then gets other logits, within rounding, when it is decoded than when it
+// is part of a prompt, and measured against one rounded reference the difference doubles.)
+// h is the 32-bit residual stream, row(m) = rows ? rows[m] : m (the output head reads the wanted
+// rows only).
 //
-// A workgroup first puts bf16(w_norm * h) of all rows into LDS, each wavefront summing the
-// squares of its rows, while its first weight loads are already in flight. It then works
+// A workgroup first puts the normed rows into LDS, each wavefront taking its rows: sum of squares,
+// scale, rounded values, while its first weight loads are already in flight. It then works
 // through tiles of 16 output columns (gated: the 16 gate and the 16 up rows of 16 units, which
 // lie next to each other in the interleaved weight matrix), TPR tiles at a time: NW / TPR
 // wavefronts share a tile, each streaming every (NW / TPR)-th 128-element chunk of k of the
 // tile's weight rows from HBM straight into MFMA operand registers, two chunks ahead (one with 16
-// wavefronts), also across tiles; the partial sums are added through LDS, scaled by inv_m and stored. The grid
+// wavefronts), also across tiles; the partial sums are added through LDS and stored. The grid
 // is sized so that the prologue is paid once per several tiles.
 //
 // A third form serves the attention's q/k/v projection: its epilogue rotates q and k heads at
@@ -90,7 +94,7 @@ struct RopeTarget {
     int n_q, n_kv, hd, page;
 };
 
-template <int NW, int TPR, int EPI, typename TNW>
+template <int NW, int TPR, int EPI, typename TNW, int PU = 8>
 __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restrict__ h, const int* __restrict__ rows,
                                                             const TNW* __restrict__ norm_w, float eps,
                                                             const bf16* __restrict__ w, void* __restrict__ out,
@@ -104,7 +108,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
     const int XS = K + 8;                               // padded row of the activation tile (elements)
     bf16* xs = reinterpret_cast<bf16*>(lds_raw);                                    // [16][XS]
     f32x4* red = reinterpret_cast<f32x4*>(lds_raw + static_cast<size_t>(16) * XS * 2);   // [NW][NT][64]
-    float* ssum = reinterpret_cast<float*>(red + NW * NT * 64);                      // [16]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, q = lane >> 4;
@@ -161,61 +164,95 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
     const int units = rounds * cpw;
     auto unit_tile = [&](int j) { return j < units ? tile_of((j / cpw) * gridDim.x + blockIdx.x) : tiles; };
     auto unit_chunk = [&](int j) { return kpart + (j % cpw) * KS; };
-    // ---- prologue: xs[m][k] = bf16(w_norm[k] * h[row(m)][k]); ssum[m] = sum_k h^2 ----
+    // ---- prologue: xs[m][k] = bf16((w_norm[k] * h[row(m)][k]) * inv_m) ----
     // Rows m >= M stay as they are: a product's row m depends on activation row m alone, and
     // the results of the rows that do not exist are never stored.
     // A row's loads are asked for eight at a time (one after the other, each trip to memory took
     // as long as the row's whole share of the products), and the first row's before the first
     // weights: loads come back in the order they were asked for, and the weights' come from far.
-    constexpr int PU = 8;
+    // The rows are dealt out over the wavefronts: with fewer rows than wavefronts, several
+    // wavefronts share a row (each takes every wpr-th group of 256 values) and add their sums of
+    // squares through LDS. A wavefront's share of its row stays in registers from the sum of squares
+    // to the rounding where it fits (PU loads of four values per lane); a longer share, or a second
+    // row, is read again for the second pass, from the cache.
+    // A row that fits one wavefront's registers is not shared: its sum of squares then needs no
+    // trip through LDS and no barrier (measured at one row of 2,048: 0.9 us a kernel).
+    const int Mp = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
+    int wpr = 1;                                        // wavefronts that share a row
+    while (K > 64 * 4 * PU * wpr && 2 * wpr * Mp <= NW) wpr *= 2;
+    const int row_step = NW / wpr;                      // rows that the workgroup covers at a time
+    const int seg = wave % wpr, m0 = wave / wpr;
+    const int stride = 64 * 4 * wpr;                    // between a lane's neighbouring loads
+    const int span = stride * PU;                       // values of a row that its wavefronts' registers hold
+    const int kb0 = (seg * 64 + lane) * 4;
+    float* ssq = reinterpret_cast<float*>(red);         // [16 rows][16 shares]; the area is free until the first round ends
     float4 hv[PU];
     Norm4<TNW> nw4[PU];
     auto ask = [&](int m, int kb) {
         const float* hrow = h + static_cast<size_t>(rows ? rows[m] : m) * K;
 #pragma unroll
         for (int u = 0; u < PU; ++u) {
-            const int k = kb + u * 64 * 4;
+            const int k = kb + u * stride;
             const int ks = k < K ? k : 0;                          // past the row: a place that exists
             hv[u] = *reinterpret_cast<const float4*>(hrow + ks);
             nw4[u].load(norm_w + ks);
         }
     };
-    auto take = [&](int m, int kb, float& ss) {
+    auto squares = [&](int kb, float& ss) {
+#pragma unroll
+        for (int u = 0; u < PU; ++u) {
+            const float4 v = hv[u];
+            if (kb + u * stride < K) ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+    };
+    // xs = bf16((w_norm * h) * inv): the product and the order of its factors are the norm kernel's
+    // (elementwise.hip), so a row is rounded to the same values whichever kernel norms it.
+    auto take = [&](int m, int kb, float inv) {
         bf16* xrow = xs + static_cast<size_t>(m) * XS;
 #pragma unroll
         for (int u = 0; u < PU; ++u) {
-            const int k = kb + u * 64 * 4;
+            const int k = kb + u * stride;
             if (k < K) {                                           // K % 8 == 0: whole groups of 4
                 float nw[4];
                 nw4[u].get(nw);
-                ss += hv[u].x * hv[u].x + hv[u].y * hv[u].y + hv[u].z * hv[u].z + hv[u].w * hv[u].w;
+                const float4 v = hv[u];
                 bf16x4 o;
-                o[0] = static_cast<__bf16>(nw[0] * hv[u].x);
-                o[1] = static_cast<__bf16>(nw[1] * hv[u].y);
-                o[2] = static_cast<__bf16>(nw[2] * hv[u].z);
-                o[3] = static_cast<__bf16>(nw[3] * hv[u].w);
+                o[0] = static_cast<__bf16>((nw[0] * v.x) * inv);
+                o[1] = static_cast<__bf16>((nw[1] * v.y) * inv);
+                o[2] = static_cast<__bf16>((nw[2] * v.z) * inv);
+                o[3] = static_cast<__bf16>((nw[3] * v.w) * inv);
                 *reinterpret_cast<bf16x4*>(xrow + k) = o;
             }
         }
     };
-    if (wave < M) ask(wave, lane * 4);
+    if (m0 < M) ask(m0, kb0);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int d = 0; d < GV_DEPTH; ++d) load_w(fw[d], unit_tile(d), unit_chunk(d));   // in flight during the prologue
     __builtin_amdgcn_sched_barrier(0);
-    // (the first eight loads of the first row are taken apart from the loop: only straight-line
-    // code lets the compiler count that the weights' loads, asked for later, may stay in flight)
+    // (the first loads of the first row are taken apart from the loop: only straight-line code lets
+    // the compiler count that the weights' loads, asked for later, may stay in flight)
     float ss_first = 0.f;
-    if (wave < M) take(wave, lane * 4, ss_first);
-    for (int m = wave; m < M; m += NW) {
-        const bool first = m == wave;
-        float ss = first ? ss_first : 0.f;
-        for (int kb = lane * 4 + (first ? 64 * 4 * PU : 0); kb < K; kb += 64 * 4 * PU) {
+    if (m0 < M) squares(kb0, ss_first);
+    const bool held = K <= span && m0 + row_step >= M;  // one row, and this wavefront's share of it is in its registers
+    for (int m = m0; m < M; m += row_step) {
+        float ss = m == m0 ? ss_first : 0.f;
+        for (int kb = kb0 + (m == m0 ? span : 0); kb < K; kb += span) {
             ask(m, kb);
-            take(m, kb, ss);
+            squares(kb, ss);
         }
         ss = wave_sum(ss);
-        if (lane == 0) ssum[m] = ss;
+        if (lane == 0) ssq[m * 16 + seg] = ss;
+    }
+    if (wpr > 1) lds_barrier();                         // (the same for the whole workgroup; alone, a wavefront reads what it wrote)
+    for (int m = m0; m < M; m += row_step) {
+        float ss = 0.f;
+        for (int i = 0; i < wpr; ++i) ss += ssq[m * 16 + i];        // (the same order in every wavefront of the row)
+        const float inv = 1.0f / sqrtf(ss / static_cast<float>(K) + eps);
+        for (int kb = kb0; kb < K; kb += span) {
+            if (!held) ask(m, kb);
+            take(m, kb, inv);
+        }
     }
     lds_barrier();                                      // (waits for LDS only: the weights stay in flight)
 
@@ -261,7 +298,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
         f32x4 s[NT];
         const int m = lane & 15;
         const bool leader = kpart == 0 && tile < tiles;
-        float inv = 0.f;
         if (leader) {
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
@@ -271,7 +307,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
                     s[t][0] += p[0]; s[t][1] += p[1]; s[t][2] += p[2]; s[t][3] += p[3];
                 }
             }
-            inv = 1.0f / sqrtf(ssum[m] / static_cast<float>(K) + eps);
         }
         if (EPI == kRope) {
             // A tile of a q or k head holds dims 8 j .. 8 j + 7 of the first half in its columns 0 .. 7
@@ -284,7 +319,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
             float own[4], other[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                own[e] = leader ? s[0][e] * inv : 0.f;
+                own[e] = leader ? s[0][e] : 0.f;
                 other[e] = __shfl_xor(own[e], 32, 64);                       // (every lane of the wavefront takes part)
             }
             if (leader && m < M) {
@@ -314,11 +349,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
                 const int c = c0 + e;
                 if (c >= N) continue;
                 if (GATED) {
-                    const float g = s[0][e] * inv, u = s[NT - 1][e] * inv;
+                    const float g = s[0][e], u = s[NT - 1][e];
                     static_cast<bf16*>(out)[static_cast<size_t>(m) * N + c] =
                         static_cast<bf16>((g / (1.0f + expf(-g))) * u);
                 } else {
-                    static_cast<float*>(out)[static_cast<size_t>(m) * N + c] = s[0][e] * inv;
+                    static_cast<float*>(out)[static_cast<size_t>(m) * N + c] = s[0][e];
                 }
             }
         }
@@ -346,12 +381,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_norm_kernel(const float* __restr
         if (j + d < units) work(d, j + d);                  // (the same for the whole workgroup)
 }
 
-template <int NW, int TPR, int EPI, typename TNW>
-static int launch_gemv_norm(const float* h, const int* rows, const void* norm_w, float eps, const bf16* w, void* out,
-                            int M, int N, int K, int grid, int blocked, const RopeTarget& rope, hipStream_t stream) {
+template <int NW, int TPR, int EPI, typename TNW, int PU>
+static int launch_gemv_norm_held(const float* h, const int* rows, const void* norm_w, float eps, const bf16* w, void* out,
+                                 int M, int N, int K, int grid, int blocked, const RopeTarget& rope, hipStream_t stream) {
     const size_t lds = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(NW) * (EPI == kGated ? 2 : 1) * 64 * 16 + 64;
     if (lds > 160 * 1024) return kErrUnsupported;
-    auto kernel = gemv_norm_kernel<NW, TPR, EPI, TNW>;
+    auto kernel = gemv_norm_kernel<NW, TPR, EPI, TNW, PU>;
     static size_t granted = 0;                          // per instantiation
     if (lds > granted) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -363,6 +398,18 @@ static int launch_gemv_norm(const float* h, const int* rows, const void* norm_w,
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(NW * 64), lds, stream, h, rows, static_cast<const TNW*>(norm_w), eps,
                        w, out, M, N, K, tiles, blocked, rope);
     return launch_status();
+}
+
+template <int NW, int TPR, int EPI, typename TNW>
+static int launch_gemv_norm(const float* h, const int* rows, const void* norm_w, float eps, const bf16* w, void* out,
+                            int M, int N, int K, int grid, int blocked, const RopeTarget& rope, hipStream_t stream) {
+    // Rows wider than 2,048 leave room for one workgroup per compute unit anyway (their LDS): eight
+    // wavefronts then have the registers to hold twice as much of a row between the two passes of
+    // the norm, and rows up to 4,096 wide are still read once.
+    if (NW == 8 && K > 2048)
+        return launch_gemv_norm_held<NW, TPR, EPI, TNW, NW == 8 ? 16 : 8>(h, rows, norm_w, eps, w, out, M, N, K, grid,
+                                                                          blocked, rope, stream);
+    return launch_gemv_norm_held<NW, TPR, EPI, TNW, 8>(h, rows, norm_w, eps, w, out, M, N, K, grid, blocked, rope, stream);
 }
 
 template <int EPI, typename TNW>

@@ -75,7 +75,7 @@ class Engine:
     def __init__(self, model_dir: str | None, dtype: str = "fp32", *, device: str = "cuda:0",
                  max_prefill_tokens_per_step: int = 8192, temperature: float = 0.0, sampler_seed: int = 0,
                  block_size: int = 16, use_graphs: bool = True, max_context: int | None = None,
-                 _config: dict | None = None, _tensors=None):
+                 deterministic: bool = False, _config: dict | None = None, _tensors=None):
         self._dtype_name = {"float32": "fp32", "bfloat16": "bf16"}.get(dtype, dtype)
         self._torch_dtype = parse_dtype(dtype)
         if _config is None:
@@ -108,6 +108,10 @@ class Engine:
         self.prefill_chunk = int(max_prefill_tokens_per_step)
         self._own_cache: CacheContext | None = None
         self.use_graphs = bool(use_graphs)
+        # deterministic: every sum in one fixed order, so that the same steps give the same bits in
+        # every run (bfloat16 products into the residual stream are otherwise cut over k and joined
+        # with atomics in the order the workgroups happen to finish).
+        self.deterministic = bool(deterministic)
 
     # ---- construction from random weights ----
     @classmethod
@@ -161,7 +165,8 @@ class Engine:
                         self._tensors = {k: None for k in self._tensors}    # keep the names only
                     else:
                         load_model_weights(model, self.model_dir, placement)
-                self._runner = ModelRunner(model, self._torch_dtype, device, use_graphs=self.use_graphs)
+                self._runner = ModelRunner(model, self._torch_dtype, device, use_graphs=self.use_graphs,
+                                           deterministic=self.deterministic)
             return self._runner
 
     @property

@@ -91,6 +91,10 @@ class StepContext:
     # launch sizes must not follow the momentary lengths: kernels plan for requests of up to
     # `plan_len` tokens instead (None: plan from ctx_lens / new_lens).
     plan_len: int | None = None
+    # Sums into the residual stream may be cut over k and added with atomics in whatever order the
+    # workgroups finish (faster at few rows; the last bits then differ from run to run). True: every
+    # sum has one fixed order, and a step gives the same bits every time it runs.
+    fixed_order: bool = False
     extra: dict = field(default_factory=dict)          # per-step notes of kernels (launch plans)
 
     def buffer(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
@@ -212,8 +216,10 @@ class ModelRunner:
     GRAPH_BLOCK_BUCKET = 64         # block-table widths of recorded steps are multiples of this
     GRAPH_LIMIT = 192               # recorded steps kept per page pool; the least recently used one goes first
 
-    def __init__(self, model: DecoderModel, dtype: torch.dtype, device: torch.device, use_graphs: bool = True):
+    def __init__(self, model: DecoderModel, dtype: torch.dtype, device: torch.device, use_graphs: bool = True,
+                 deterministic: bool = False):
         self.model = model
+        self.deterministic = bool(deterministic)
         self.dtype = dtype
         self.device = device
         self.workspace = Workspace(device)
@@ -436,6 +442,6 @@ class ModelRunner:
             block_tables={g: view(6 + gi, (S, max_blocks)) for gi, g in enumerate(groups)},
             act_dtype=self.dtype, workspace=self.workspace, new_lens=new_lens, ctx_lens=ctx_lens,
             slot_list=slot_list, max_position=max(c + n for c, n in zip(ctx_lens, new_lens)) - 1,
-            plan_len=plan_len)
+            plan_len=plan_len, fixed_order=self.deterministic)
         logit_rows = view(len(sizes) - 1) if R else None
         return ctx, logit_rows

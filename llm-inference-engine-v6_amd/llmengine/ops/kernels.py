@@ -186,9 +186,13 @@ def clear(t: torch.Tensor) -> None:
 _fast_gemm = None       # set by ops/mfma.py when the MFMA kernels are present
 
 
-def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
-    """out[m, n] (+)= sum_k a[m, k] w[n, k]; 32-bit accumulation whatever the types."""
-    if policy.fast_gemm and _fast_gemm is not None and _fast_gemm(a, w, out, accumulate):
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
+         fixed_order: bool = False) -> None:
+    """out[m, n] (+)= sum_k a[m, k] w[n, k]; 32-bit accumulation whatever the types. A sum that
+    adds into `out` may be cut over k into parts that several workgroups add with atomics, in
+    whatever order they finish: the result then differs from run to run in its last bits.
+    fixed_order forbids that cut (every output element is summed by one workgroup in one order)."""
+    if policy.fast_gemm and _fast_gemm is not None and _fast_gemm(a, w, out, accumulate, fixed_order):
         return
     gemm_generic(a, w, out, accumulate)
 

@@ -65,10 +65,11 @@ def gemm_gated(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, grou
     kernels.swiglu(gu, out, group)
 
 
-def _fast_gemm(a, w, out, accumulate) -> bool:
+def _fast_gemm(a, w, out, accumulate, fixed_order=False) -> bool:
     if a.dim() != 2 or w.dim() not in (2, 5) or not gemm_bf16_supported(a, w, out, accumulate):
         return False
-    gemm_bf16(a, w, out, accumulate, _supported=True)
+    # (ksplit 1: the entry point cuts nothing over k, so no partial sums meet in atomics)
+    gemm_bf16(a, w, out, accumulate, ksplit=1 if fixed_order and accumulate else 0, _supported=True)
     return True
 
 

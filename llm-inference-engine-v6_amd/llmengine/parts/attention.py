@@ -109,7 +109,7 @@ class Attention(Mixer):
                 # chip, so the product is cut over k and adds its parts into a cleared buffer
                 # (measured at 32 rows of the 3B sizes: 10.7 + clearing against 19.5 us)
                 ops.clear(qkv)
-                ops.gemm(x, self.w_qkv, qkv, accumulate=True)
+                ops.gemm(x, self.w_qkv, qkv, accumulate=True, fixed_order=step.fixed_order)
             else:
                 project(self.w_qkv, qkv)
             ops.rope_kv_write(qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
@@ -121,7 +121,7 @@ class Attention(Mixer):
             ops.rope_q_only(q32, cos, sin, step.positions, q, n_q, hd, rot)
         o = step.buffer("attn.o", (T, self.q_dim), act)
         ops.attention(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, hd, self.scale, self.window)
-        ops.gemm(o, self.w_o, out, accumulate)
+        ops.gemm(o, self.w_o, out, accumulate, fixed_order=step.fixed_order)
 
 
 register_part("mixer", "attention", Attention)

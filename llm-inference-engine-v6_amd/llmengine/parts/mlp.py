@@ -55,7 +55,7 @@ class GatedMLP(FeedForward):
             act = step.buffer("mlp.act", (T, FF), x.dtype)
             ops.gemm_gated(x, self.w_gate_up, act, self.group,
                            lambda shape, dtype: step.buffer("mlp.gate_up", shape, dtype))
-        ops.gemm(act, self.w_down, out, accumulate)
+        ops.gemm(act, self.w_down, out, accumulate, fixed_order=step.fixed_order)
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

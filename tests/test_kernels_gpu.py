@@ -557,6 +557,43 @@ def test_gemv_norm_gated(ops, M, FF, K):
         assert _rel(out.cpu().double(), ref) < 1e-2, (tpr, grid)
 
 
+@pytest.mark.parametrize("M,K", [(1, 64), (3, 2048), (8, 2048), (16, 2048), (1, 3072), (8, 3072), (8, 4096), (16, 4096),
+                                 (2, 4104), (13, 1000)])
+@pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
+def test_gemv_norm_rounds_what_the_norm_kernel_rounds(ops, M, K, wdtype):
+    """A token's normed activations are rounded to the same bfloat16 values whether the norm is
+    its own kernel (prompts) or part of the projection (decoding): the two ways then differ by the
+    order of 32-bit sums only. (Scaling after the product instead of before the rounding is as
+    accurate but differs from the norm kernel's result by a bfloat16 rounding, a thousand times more.)
+    Rows are shared by several wavefronts, held in registers or read twice, depending on M and K."""
+    h = 3 * torch.randn(M, K, generator=_gen(80))
+    nw = (1 + 0.2 * torch.randn(K, generator=_gen(81))).to(wdtype)
+    hd, nwd = h.to(DEV), nw.to(DEV)
+    x = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
+    ops.rmsnorm(hd, nwd, 1e-5, x)
+    # plain epilogue: few tiles (a workgroup of 8 wavefronts each)
+    w = (0.05 * torch.randn(272, K, generator=_gen(82))).to(torch.bfloat16).to(DEV)
+    fused, apart = torch.empty(M, 272, device=DEV), torch.empty(M, 272, device=DEV)
+    ops.gemv_norm(hd, nwd, 1e-5, w, fused)
+    ops.gemm(x, w, apart)
+    # (the two kernels add the squares in another order: a scale that differs in its last bit moves
+    # one value in some ten thousand across a rounding boundary, which is 1e-5 of a sum; rounding
+    # before the scale would be 4e-3)
+    assert _rel(fused.cpu().double(), apart.cpu().double()) < 1e-4
+    # gated epilogue with more than 256 tiles: workgroups of 16 wavefronts
+    FF = 4352
+    wgu = (0.05 * torch.randn(2 * FF, K, generator=_gen(83))).to(torch.bfloat16).to(DEV)
+    fused_g = torch.empty(M, FF, dtype=torch.bfloat16, device=DEV)
+    apart_g = torch.empty(M, FF, dtype=torch.bfloat16, device=DEV)
+    ops.gemv_norm(hd, nwd, 1e-5, wgu, fused_g, gated=True)
+    ops.gemm_gated(x, wgu, apart_g, 16, lambda shape, dtype: torch.empty(shape, dtype=dtype, device=DEV))
+    differ = (fused_g != apart_g).float().mean().item()
+    # (sums that differ by 1e-5 put up to one output in a hundred on the other side of a rounding
+    # boundary; with the activations rounded before the scale, every second output differs)
+    assert differ < 0.05, differ
+    assert _rel(fused_g.cpu().double(), apart_g.cpu().double()) < 8e-3
+
+
 def test_gemv_norm_refusals(ops):
     from llmengine.ops import KernelError
     h = torch.randn(17, 64, device=DEV)
