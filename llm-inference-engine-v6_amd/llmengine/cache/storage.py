@@ -44,9 +44,9 @@ class CacheStorage:
                 continue
             group = group_name(spec) if spec.paged else None
             paged = {}
-            for name, shape in spec.paged.items():
+            for name, (shape, page_dtype) in spec.paged_tensors(dtype).items():
                 full = (pages[group],) + tuple(page_size if d == PAGE else d for d in shape)
-                paged[name] = torch.zeros(full, dtype=dtype, device=device)
+                paged[name] = torch.zeros(full, dtype=page_dtype, device=device)
                 self.bytes += paged[name].numel() * paged[name].element_size()
             state = {}
             for name, (shape, sdtype) in spec.state.items():

@@ -94,6 +94,7 @@ class Engine:
         self._arch = resolve(architecture_name(cfg_dict))
         self.cfg = self._arch.parse_config(cfg_dict, gen, architecture=self._arch.name)
         self._index_names: list[str] | None = None
+        self._aliases: dict[str, str] | None = None
         if model_dir is not None and _tensors is None:
             index = TensorIndex(model_dir)          # parse headers now: malformed files fail here
             self._index_names = index.names()
@@ -140,9 +141,14 @@ class Engine:
         return self.cfg.eos_token_ids
 
     def weight_names(self) -> list[str]:
+        """The checkpoint's tensor names, plus the second names under which the model knows some
+        of them (a tied head answers to the embedding's name and to its own)."""
         names = set(self._index_names if self._index_names is not None else self._tensors)
-        if getattr(self.cfg, "tie_word_embeddings", False) and "model.embed_tokens.weight" in names:
-            names.add("lm_head.weight")         # the tied head answers to both names
+        if self._aliases is None:
+            self._aliases = self._arch.build_model(self.cfg).named_aliases()     # (the tree alone: no tensors)
+        for alias, target in self._aliases.items():
+            if target in names:
+                names.add(alias)
         return sorted(names)
 
     def has_weight(self, name: str) -> bool:

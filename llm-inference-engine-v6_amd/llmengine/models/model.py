@@ -54,6 +54,13 @@ class DecoderModel(Part):
         out[n["head"]] = self.head
         return out
 
+    def aliases(self):
+        # A tied head is the embedding table under a second name (src/weights.cpp:244-267): a
+        # checkpoint may store it under both, and then both must agree in shape and type.
+        if self.head.tied_to is self.embedding:
+            return {f"{self.names['head']}.weight": f"{self.names['embedding']}.weight"}
+        return {}
+
     # ---- caches ----
     def cache_specs(self) -> dict[int, CacheSpec | None]:
         """cache id -> what is kept there: the spec of the first call that writes it."""

@@ -18,7 +18,6 @@ import torch
 
 from .. import ops
 from .base import PAGE, CacheSpec, Getter, Mixer, ParamSpec, Placement, PositionEncoding
-from .norm import RMSNorm
 from .registry import register_part
 
 
@@ -69,6 +68,10 @@ class Attention(Mixer):
                 ops.pair_rows_for_rotation(fused, self.num_heads + self.num_kv_heads, self.head_dim))
         self.w_o = placement.place_matrix(get("o_proj.weight"))
 
+    def tree_graph_safe(self) -> bool:
+        # (the position encoding is no child with tensors of its own, but it runs inside forward)
+        return super().tree_graph_safe() and (self.position is None or self.position.tree_graph_safe())
+
     def cache_spec(self) -> CacheSpec:
         return CacheSpec(kind="window" if self.window > 0 else "full", window=self.window,
                          paged={"k": (self.num_kv_heads, PAGE, self.head_dim),
@@ -76,34 +79,40 @@ class Attention(Mixer):
 
     def fuses_norm(self, h, norm, step):
         # A few rows (decoding): the q/k/v projection applies the norm itself.
-        return (isinstance(norm, RMSNorm) and step.act_dtype == torch.bfloat16
-                and ops.gemv_norm_supported(h, norm.weight, self.w_qkv, h.shape[0], gated=False))
+        rms = norm.fused_rms()
+        return (rms is not None and step.act_dtype == torch.bfloat16
+                and ops.gemv_norm_supported(h, rms[0], self.w_qkv, h.shape[0], gated=False))
 
     def forward(self, x, step, cache, out, accumulate, write_cache=True, pre_norm=None):
+        """pre_norm: the norm in front of this mixer when `fuses_norm` said yes; x is then the
+        un-normed 32-bit stream and the projection applies pre_norm.fused_rms() itself."""
         T = x.shape[0]
         n_q, n_kv, hd = self.num_heads, self.num_kv_heads, self.head_dim
         tables = self.position.rotary_tables() if self.position is not None else None
         cos, sin, rot = tables if tables is not None else (None, None, 0)
+        # an encoding that is no rotation by a table of angles transforms q and k itself
+        applies = self.position is not None and tables is None
         if cos is not None and step.max_position >= cos.shape[0]:
             raise ValueError(f"position {step.max_position} is beyond the position table ({cos.shape[0]} rows)")
         block_table = step.block_tables[cache.group]
         k_cache, v_cache = cache.paged["k"], cache.paged["v"]
         act = step.act_dtype
         q = step.buffer("attn.q", (T, self.q_dim), act)
+        rms = pre_norm.fused_rms() if pre_norm is not None else None
 
         def project(weight, dst):
-            if pre_norm is not None:
-                ops.gemv_norm(x, pre_norm.weight, pre_norm.eps, weight, dst)
+            if rms is not None:
+                ops.gemv_norm(x, rms[0], rms[1], weight, dst)
             else:
                 ops.gemm(x, weight, dst)
-        if (write_cache and pre_norm is not None and cos is not None and self.w_qkv_paired is not None
-                and ops.gemv_norm_rope_supported(x, pre_norm.weight, self.w_qkv_paired, k_cache, T, hd, rot)):
+        if (write_cache and rms is not None and cos is not None and self.w_qkv_paired is not None
+                and ops.gemv_norm_rope_supported(x, rms[0], self.w_qkv_paired, k_cache, T, hd, rot)):
             # decoding: norm, projection, rotation and the cache write are one kernel
-            ops.gemv_norm_rope(x, pre_norm.weight, pre_norm.eps, self.w_qkv_paired, step.positions, step.seq_idx,
+            ops.gemv_norm_rope(x, rms[0], rms[1], self.w_qkv_paired, step.positions, step.seq_idx,
                                block_table, cos, sin, q, k_cache, v_cache, n_q, n_kv, hd)
         elif write_cache:
             qkv = step.buffer("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
-            if (pre_norm is None and 16 < T <= 64 and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16
+            if (rms is None and 16 < T <= 64 and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16
                     and qkv.numel() % 4 == 0):
                 # a few dozen rows (decoding at larger batches): q/k/v has too few output tiles for the
                 # chip, so the product is cut over k and adds its parts into a cleared buffer
@@ -112,12 +121,17 @@ class Attention(Mixer):
                 ops.gemm(x, self.w_qkv, qkv, accumulate=True, fixed_order=step.fixed_order)
             else:
                 project(self.w_qkv, qkv)
+            if applies:
+                self.position.apply(qkv[:, :self.q_dim].view(T, n_q, hd),
+                                    qkv[:, self.q_dim:self.q_dim + self.kv_dim].view(T, n_kv, hd), step.positions)
             ops.rope_kv_write(qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
                               n_q, n_kv, hd, rot, write_cache=True)
         else:
             # A layer that reads another layer's cache projects queries only.
             q32 = step.buffer("attn.q32", (T, self.q_dim), torch.float32)
             project(self.w_qkv[:self.q_dim // 16] if ops.is_blocked(self.w_qkv) else self.w_qkv[:self.q_dim], q32)
+            if applies:
+                self.position.apply(q32.view(T, n_q, hd), None, step.positions)
             ops.rope_q_only(q32, cos, sin, step.positions, q, n_q, hd, rot)
         o = step.buffer("attn.o", (T, self.q_dim), act)
         ops.attention(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, hd, self.scale, self.window)

@@ -95,6 +95,12 @@ class Part:
         """Tensor names that a checkpoint may hold for this part and that are not read."""
         return set()
 
+    def aliases(self) -> dict[str, str]:
+        """Second names of tensors of this part: alias -> the name whose tensor it is (both
+        relative to this part). A checkpoint may store an alias too; it is then not read, but its
+        shape and type must agree with the tensor it stands for."""
+        return {}
+
     def load_params(self, get: Getter, placement: Placement) -> None:
         """Reads the part's own tensors (children are loaded by the walker)."""
 
@@ -109,6 +115,12 @@ class Part:
         out = {prefix + k for k in self.ignored_names()}
         for name, child in self.children().items():
             out |= child.named_ignored(f"{prefix}{name}.")
+        return out
+
+    def named_aliases(self, prefix: str = "") -> dict[str, str]:
+        out = {prefix + a: prefix + t for a, t in self.aliases().items()}
+        for name, child in self.children().items():
+            out.update(child.named_aliases(f"{prefix}{name}."))
         return out
 
     def tree_graph_safe(self) -> bool:
@@ -129,7 +141,8 @@ class CacheSpec:
     """What one mixer keeps for a request.
 
     paged: tensors kept per token, in pages: name -> shape of one page, with `PAGE`
-           where the page size goes. Layers with the same (kind, window) share a
+           where the page size goes, or (shape, dtype) for a tensor that is not kept in
+           the model's activation type. Layers with the same (kind, window) share a
            page pool and a block table (one page id covers all of them).
     kind:  "full": every token of the request stays; "window": only the last
            `window` tokens are ever read, pages behind them are given back.
@@ -138,7 +151,7 @@ class CacheSpec:
     """
     kind: str = "full"
     window: int = 0
-    paged: Mapping[str, tuple[int, ...]] = field(default_factory=dict)
+    paged: Mapping[str, tuple] = field(default_factory=dict)
     state: Mapping[str, tuple[tuple[int, ...], torch.dtype]] = field(default_factory=dict)
 
     def __post_init__(self):
@@ -146,6 +159,16 @@ class CacheSpec:
             raise ValueError(f"cache kind {self.kind!r} is not 'full' or 'window'")
         if self.kind == "window" and self.window <= 0:
             raise ValueError("a window cache needs window > 0")
+
+    def paged_tensors(self, default_dtype: torch.dtype) -> dict[str, tuple[tuple[int, ...], torch.dtype]]:
+        """name -> (shape of one page, dtype), the model's activation type where none is given."""
+        out = {}
+        for name, value in self.paged.items():
+            if len(value) == 2 and isinstance(value[1], torch.dtype):
+                out[name] = (tuple(value[0]), value[1])
+            else:
+                out[name] = (tuple(value), default_dtype)
+        return out
 
     @property
     def group_key(self) -> tuple:
@@ -165,11 +188,27 @@ class Norm(Part):
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: torch.Tensor | None = None) -> None:
         raise NotImplementedError
 
+    def fused_rms(self) -> tuple[torch.Tensor, float] | None:
+        """(weight, eps) if this norm is exactly y = weight * x / sqrt(mean(x^2) + eps), so that a
+        kernel which applies that formula in front of a projection may stand in for `forward`;
+        None (the default) for every other formula: the norm then always runs as its own step."""
+        return None
+
 
 class PositionEncoding(Part):
     def rotary_tables(self):
-        """(cos [P, r/2], sin [P, r/2], r) for rotate-half pairs (i, i + r/2), or None."""
+        """(cos [P, r/2], sin [P, r/2], r) for rotate-half pairs (i, i + r/2): the mixer's kernels
+        rotate q and k by them. None: the encoding is something else and transforms q and k itself
+        in `apply`."""
         return None
+
+    def apply(self, q: torch.Tensor, k: torch.Tensor | None, positions: torch.Tensor) -> None:
+        """For encodings without rotary tables: transforms, in place, the step's projected queries
+        q [T, n_q, hd] and keys k [T, n_kv, hd] (32-bit views, rows in batch order; k is None for a
+        layer that reads another layer's keys) for the tokens at `positions` [T] (int32, on the
+        device). Keys are cached as this leaves them. A part that computes on the host here must
+        leave `graph_safe` False."""
+        raise NotImplementedError(f"{type(self).__name__} has neither rotary tables nor apply()")
 
     @property
     def max_position(self) -> int:

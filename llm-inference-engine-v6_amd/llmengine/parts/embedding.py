@@ -43,10 +43,6 @@ class OutputHead(Part):
             return {}
         return {"weight": ParamSpec((self.vocab_size, self.hidden_size), "linear")}
 
-    def ignored_names(self):
-        # A tied checkpoint may still store the head; the embedding is used either way.
-        return {"weight"} if self.tied_to is not None else set()
-
     def load_params(self, get: Getter, placement: Placement) -> None:
         if self.tied_to is None:
             self._weight = placement.place_matrix(get("weight"))
@@ -56,13 +52,14 @@ class OutputHead(Part):
         return self.tied_to.weight if self.tied_to is not None else self._weight
 
     def fuses_norm(self, h: torch.Tensor, norm, n_rows: int, act_dtype) -> bool:
-        from .norm import RMSNorm
-        return (isinstance(norm, RMSNorm) and act_dtype == torch.bfloat16
-                and ops.gemv_norm_supported(h, norm.weight, self.weight, n_rows, gated=False))
+        rms = norm.fused_rms()
+        return (rms is not None and act_dtype == torch.bfloat16
+                and ops.gemv_norm_supported(h, rms[0], self.weight, n_rows, gated=False))
 
     def forward(self, x: torch.Tensor, out: torch.Tensor) -> None:
         ops.gemm(x, self.weight, out)
 
     def forward_normed_rows(self, h: torch.Tensor, rows: torch.Tensor, norm, out: torch.Tensor) -> None:
         """Logits of the chosen rows of the 32-bit stream, the final norm applied inside the product."""
-        ops.gemv_norm(h, norm.weight, norm.eps, self.weight, out, rows=rows)
+        weight, eps = norm.fused_rms()
+        ops.gemv_norm(h, weight, eps, self.weight, out, rows=rows)

@@ -11,7 +11,6 @@ import torch
 
 from .. import ops
 from .base import FeedForward, Getter, ParamSpec, Placement
-from .norm import RMSNorm
 from .registry import register_part
 
 
@@ -42,15 +41,17 @@ class GatedMLP(FeedForward):
 
     def fuses_norm(self, h, norm, step):
         # A few rows (decoding): one kernel applies the norm, both projections and the activation.
-        return (isinstance(norm, RMSNorm) and self.group == 16 and step.act_dtype == torch.bfloat16
-                and ops.gemv_norm_supported(h, norm.weight, self.w_gate_up, h.shape[0], gated=True))
+        rms = norm.fused_rms()
+        return (rms is not None and self.group == 16 and step.act_dtype == torch.bfloat16
+                and ops.gemv_norm_supported(h, rms[0], self.w_gate_up, h.shape[0], gated=True))
 
     def forward(self, x, step, out, accumulate, pre_norm=None):
         T = x.shape[0]
         FF = self.intermediate_size
         if pre_norm is not None:
             act = step.buffer("mlp.act", (T, FF), torch.bfloat16)
-            ops.gemv_norm(x, pre_norm.weight, pre_norm.eps, self.w_gate_up, act, gated=True)
+            weight, eps = pre_norm.fused_rms()
+            ops.gemv_norm(x, weight, eps, self.w_gate_up, act, gated=True)
         else:
             act = step.buffer("mlp.act", (T, FF), x.dtype)
             ops.gemm_gated(x, self.w_gate_up, act, self.group,

@@ -27,31 +27,42 @@ def _fmt(shape) -> str:
     return "[" + ",".join(str(int(d)) for d in shape) + "]"
 
 
-def check_names(model: Part, available: dict[str, tuple[int, ...]], where: str) -> None:
-    """Raises one WeightError that lists every missing, unexpected and wrongly shaped tensor."""
+def check_names(model: Part, available: dict[str, tuple[int, ...]], where: str, dtypes: dict | None = None) -> None:
+    """Raises one WeightError that lists every missing, unexpected and wrongly shaped tensor.
+    A tensor stored under a second name of another (a tied output head, src/weights.cpp:259-264)
+    must agree with that tensor in shape and, where `dtypes` (name -> stored type) is given, type."""
     expected = model.named_specs()
     ignored = model.named_ignored()
+    aliases = model.named_aliases()
     missing = sorted(n for n in expected if n not in available)
-    unexpected = sorted(n for n in available if n not in expected and n not in ignored)
+    unexpected = sorted(n for n in available if n not in expected and n not in ignored and n not in aliases)
     wrong = sorted((n, expected[n].shape, available[n]) for n in expected
                    if n in available and tuple(available[n]) != tuple(expected[n].shape))
-    if not (missing or unexpected or wrong):
+    disagree = sorted((a, t) for a, t in aliases.items() if a in available and t in available and (
+        tuple(available[a]) != tuple(available[t]) or (dtypes is not None and dtypes.get(a) != dtypes.get(t))))
+    if not (missing or unexpected or wrong or disagree):
         return
     lines = [f"weights in {where} do not fit the model:"]
+    for a, t in disagree:
+        what = "tie_word_embeddings=true but " if a.endswith("lm_head.weight") else ""
+        lines.append(f"  {what}{a} shape/dtype disagrees with {t} ({_fmt(available[a])}"
+                     f"{' ' + str(dtypes[a]) if dtypes else ''} against {_fmt(available[t])}"
+                     f"{' ' + str(dtypes[t]) if dtypes else ''})")
     for n in missing:
         lines.append(f"  missing weight: {n} (expected shape {_fmt(expected[n].shape)})")
     for n, want, got in wrong:
         lines.append(f"  shape mismatch for {n}: expected {_fmt(want)}, got {_fmt(got)}")
     for n in unexpected:
         lines.append(f"  unexpected tensor: {n} {_fmt(available[n])}")
-    raise WeightError("\n".join(lines), missing, unexpected, [w[0] for w in wrong])
+    raise WeightError("\n".join(lines), missing, unexpected, [w[0] for w in wrong] + [a for a, _ in disagree])
 
 
 def load_model_weights(model: Part, model_dir: str, placement: Placement) -> list[str]:
     """Fills the model's parts from the folder's tensors; returns the tensor names read."""
     index = TensorIndex(model_dir)
     try:
-        check_names(model, {n: index.entry(n).shape for n in index.names()}, model_dir)
+        check_names(model, {n: index.entry(n).shape for n in index.names()}, model_dir,
+                    {n: index.entry(n).dtype for n in index.names()})
         read: list[str] = []
 
         def get(name: str) -> torch.Tensor:
@@ -68,5 +79,6 @@ def load_model_weights(model: Part, model_dir: str, placement: Placement) -> lis
 
 def load_state_dict(model: Part, tensors: dict[str, torch.Tensor], placement: Placement) -> None:
     """The same from tensors in memory (random weights that are never written out)."""
-    check_names(model, {n: tuple(t.shape) for n, t in tensors.items()}, "the given tensors")
+    check_names(model, {n: tuple(t.shape) for n, t in tensors.items()}, "the given tensors",
+                {n: t.dtype for n, t in tensors.items()})
     model.load_tree(lambda name: tensors[name], placement)

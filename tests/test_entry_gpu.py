@@ -41,6 +41,29 @@ def test_greedy_generate_equals_plain(dir_a):
     assert engine.dtype == "fp32" and engine.max_pos == 128 and engine.cfg.hidden_size == 64
 
 
+@pytest.mark.parametrize("chunk", [2, 7, 16])
+def test_prompts_longer_than_a_prefill_step(dir_a, chunk):
+    """max_prefill_tokens_per_step below the prompt's length: `generate` and `forward_logits` feed
+    the prompt in portions of that many tokens (the last one shorter), and nothing changes."""
+    from llmengine import Engine
+    cfg, w = load_plain_model(dir_a)
+    engine = Engine(dir_a, "fp32", block_size=4, max_prefill_tokens_per_step=chunk)
+    steps = []
+    step = engine.step
+    engine.step = lambda cache, entries: (steps.append([len(e.tokens) for e in entries]), step(cache, entries))[1]
+    for i, n in enumerate((5, 33, 40)):
+        prompt = random_tokens(n, 256, 60 + i)
+        steps.clear()
+        assert engine.generate(prompt, 6) == plain_generate(cfg, w, prompt, 6)
+        assert steps[:-5] == [[chunk]] * (n // chunk) + ([[n % chunk]] if n % chunk else [])
+    ids = random_tokens(41, 256, 70)
+    steps.clear()
+    got = engine.forward_logits(ids)
+    assert steps == [[chunk]] * (41 // chunk) + ([[41 % chunk]] if 41 % chunk else [])
+    ref = plain_forward(cfg, w, ids).numpy()
+    assert got.shape == ref.shape and np.abs(got - ref).max() / np.abs(ref).max() < 1e-5
+
+
 def test_bf16_generate_is_greedy_under_its_own_rounding(dir_b):
     """In bfloat16 a near-tie may fall the other way; every chosen token must still be a
     maximum of the plain logits up to the bfloat16 tolerance."""
@@ -289,3 +312,58 @@ def test_trace_run_program(dir_b, tmp_path, dtype):
                 assert np.abs(rows[r] - ref).max() / np.abs(ref).max() < tol, (s["step"], e["id"], wnt)
                 r += 1
             pos[e["id"]] += len(e["tokens"])
+
+
+def test_trace_run_random_config_index_and_repeatability(tmp_path):
+    """bin/trace_run over a model made from a configuration and a seed, with pages that do not
+    divide 64 and the index of (request, position) per row; run twice in bfloat16, the files are
+    the same bits (the model is wide enough that serving would cut its sums over k)."""
+    cfg = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": 1024,
+           "intermediate_size": 2048, "num_hidden_layers": 2, "num_attention_heads": 16, "num_key_value_heads": 4,
+           "head_dim": 64, "vocab_size": 320, "max_position_embeddings": 512, "rms_norm_eps": 1e-5,
+           "rope_theta": 10000.0, "tie_word_embeddings": True}
+    cfgf = tmp_path / "config.json"
+    cfgf.write_text(json.dumps(cfg))
+    reqs = {f"q{i}": random_tokens(n, 320, 700 + i) for i, n in enumerate((70, 40, 3, 55, 64))}
+    steps = replay.mixed(reqs, max_live=4, seed=4)
+    peak = replay.trace_peak_tokens(steps, 64)
+    text = "\n".join(json.dumps(s) for s in steps) + "\n"
+    outs = []
+    for run in range(2):
+        out_dir = tmp_path / f"out{run}"
+        p = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--random-config", str(cfgf), "--seed", "9",
+                            "--dtype", "bfloat16", "--out", str(out_dir), "--max-tokens", str(peak), "--block-size",
+                            "48", "--index"], input=text, capture_output=True, text=True, timeout=600)
+        assert p.returncode == 0, p.stderr[-3000:]
+        outs.append(out_dir)
+    # the index names every row
+    index = [json.loads(line) for line in (outs[0] / "index.jsonl").read_text().splitlines()]
+    pos = {rid: 0 for rid in reqs}
+    expected = []
+    for s in steps:
+        rows = [[e["id"], pos[e["id"]] + w] for e in s["entries"] for w in e["want"]]
+        for e in s["entries"]:
+            pos[e["id"]] += len(e["tokens"])
+        if rows:
+            expected.append({"step": s["step"], "rows": rows})
+    assert index == expected
+    for s in steps:
+        a = np.fromfile(outs[0] / f"{s['step']}.f32", dtype="<f4")
+        b = np.fromfile(outs[1] / f"{s['step']}.f32", dtype="<f4")
+        assert a.size == 320 * sum(len(e["want"]) for e in s["entries"]) and np.array_equal(a, b), s["step"]
+    # and the logits are the model's: the same weights through the plain implementation
+    from llmengine.weights import random_state
+    wide = {k: v.double() for k, v in random_state(cfg, 9, torch.bfloat16)}
+    rid, ids = "q1", reqs["q1"]
+    ref = plain_forward(cfg, wide, ids, rounder=bf16_round).numpy()
+    pos = 0
+    for s in steps:
+        r = 0
+        for e in s["entries"]:
+            if e["id"] == rid:
+                rows = np.fromfile(outs[0] / f"{s['step']}.f32", dtype="<f4").reshape(-1, 320)
+                for w in e["want"]:
+                    got = rows[r + e["want"].index(w)]
+                    assert np.abs(got - ref[pos + w]).max() / np.abs(ref[pos + w]).max() < 2e-2
+                pos += len(e["tokens"])
+            r += len(e["want"])

@@ -500,3 +500,127 @@ def test_toy_routed_feed_forward_position_encoding_and_arrangement():
         for rid, ids in reqs.items():
             for pos in range(len(ids)):
                 assert _rel(got[rid][pos], plain[rid][pos]) < 1e-5, (rid, pos)
+
+
+# --- an encoding that is no table of angles, a norm with another formula, pages of another type ---
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_toy_interleaved_encoding_shifted_norm_and_wide_pages(dtype):
+    """Three parts that the Llama kernels' shortcuts must not swallow, defined here and registered:
+    a rotation of neighbouring pairs (2i, 2i + 1) that transforms q and k itself (`apply`, no rotary
+    tables); a norm y = (1 + w) x / sqrt(mean(x^2) + eps) that subclasses RMSNorm, which the decode
+    kernels must not fuse with the Llama formula; an attention that keeps its keys and values in
+    32-bit pages inside a bfloat16 model."""
+    from llmengine import Engine
+    from llmengine.config import register_architecture
+    from llmengine.models.model import DecoderModel
+    from llmengine.parts import (Attention, CacheSpec, Embedding, LayerSpec, OutputHead, PartChoice, PositionEncoding,
+                                 RMSNorm, build_layer, register_part)
+    from llmengine.parts.base import PAGE
+    from llmengine.weights import random_state
+
+    class InterleavedRotary(PositionEncoding):
+        def __init__(self, head_dim, theta, max_position):
+            self.hd, self.theta, self._max = head_dim, theta, max_position
+            self.freq = None
+
+        @property
+        def max_position(self):
+            return self._max
+
+        def materialize(self, placement):
+            i = torch.arange(self.hd // 2, dtype=torch.float64)
+            self.freq = (self.theta ** (-2.0 * i / self.hd)).float().to(placement.device)
+
+        def apply(self, q, k, positions):
+            angle = positions.float()[:, None] * self.freq[None, :]                # [T, hd / 2]
+            cos, sin = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
+            for x in (q, k):
+                if x is None:
+                    continue
+                a, b = x[..., 0::2].clone(), x[..., 1::2].clone()
+                x[..., 0::2] = a * cos - b * sin
+                x[..., 1::2] = b * cos + a * sin
+
+    class ShiftedRMSNorm(RMSNorm):
+        def forward(self, x, out, rows=None):
+            src = x if rows is None else x[rows.long()]
+            y = (1.0 + self.weight.float()) * src / torch.sqrt((src * src).mean(-1, keepdim=True) + self.eps)
+            out.copy_(y)
+
+    class WidePagesAttention(Attention):
+        def cache_spec(self):
+            return CacheSpec(paged={"k": ((self.num_kv_heads, PAGE, self.head_dim), torch.float32),
+                                    "v": ((self.num_kv_heads, self.head_dim, PAGE), torch.float32)})
+
+    register_part("position", "interleaved_rotary", InterleavedRotary, replace=True)
+    register_part("norm", "shifted_rmsnorm", ShiftedRMSNorm, replace=True)
+    register_part("mixer", "wide_pages_attention", WidePagesAttention, replace=True)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        max_pos: int
+        eos_token_ids: tuple = ()
+
+    H, V, FF, HD, NQ, NKV, THETA, EPS = 64, 90, 96, 16, 4, 2, 50.0, 1e-5
+
+    def build(c):
+        norm = PartChoice("shifted_rmsnorm", {"size": H, "eps": EPS})
+        layer = LayerSpec(PartChoice("prenorm"),
+                          PartChoice("wide_pages_attention", {"hidden_size": H, "num_heads": NQ, "num_kv_heads": NKV,
+                                                              "head_dim": HD}),
+                          PartChoice("gated_mlp", {"hidden_size": H, "intermediate_size": FF}), norm, norm,
+                          PartChoice("interleaved_rotary", {"head_dim": HD, "theta": THETA, "max_position": c.max_pos}))
+        emb = Embedding(V, H)
+        return DecoderModel(c, emb, [build_layer(layer), build_layer(layer)], ShiftedRMSNorm(H, EPS),
+                            OutputHead(V, H, tied_to=emb))
+
+    register_architecture("ToyInterleavedForCausalLM", lambda cfg, gen=None, architecture="":
+                          ToyConfig(cfg["max_position_embeddings"]), build, replace=True)
+    cfg = {"architectures": ["ToyInterleavedForCausalLM"], "max_position_embeddings": 128}
+    store = torch.float32 if dtype == "fp32" else torch.bfloat16
+    tensors = dict(random_state(cfg, 31, store, 0.1, 0.0, 0.3))                    # norm weights around 0: 1 + w matters
+    engine = Engine(None, dtype, _config=cfg, _tensors=dict(tensors), block_size=16)
+    model = engine.model
+    assert model.layers[0].mixer_norm.fused_rms() is None and RMSNorm(H, EPS).fused_rms() is not None
+    assert not engine.runner.use_graphs                                            # the encoding computes in `apply`
+
+    rnd = (lambda t: t.float().bfloat16().double()) if dtype == "bf16" else (lambda t: t)
+
+    def norm(x, w):
+        return rnd((1.0 + w) * x / torch.sqrt((x * x).mean(-1, keepdim=True) + EPS))
+
+    def rotate(x, n):
+        angle = torch.arange(n, dtype=torch.float64)[:, None] * (THETA ** (-2.0 * torch.arange(HD // 2, dtype=torch.float64) / HD))
+        cos, sin = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
+        out = torch.empty_like(x)
+        out[..., 0::2] = x[..., 0::2] * cos - x[..., 1::2] * sin
+        out[..., 1::2] = x[..., 1::2] * cos + x[..., 0::2] * sin
+        return out
+
+    def plain_toy(ids):
+        w = {k: v.double() for k, v in tensors.items()}
+        n = len(ids)
+        h = w["model.embed_tokens.weight"][ids]
+        for layer in range(2):
+            p = f"model.layers.{layer}."
+            x = norm(h, w[p + "input_layernorm.weight"])
+            q = rnd(rotate(plain_linear(x, w[p + "self_attn.q_proj.weight"]).view(n, NQ, HD), n))
+            k = rotate(plain_linear(x, w[p + "self_attn.k_proj.weight"]).view(n, NKV, HD), n)     # 32-bit pages: not rounded
+            v = plain_linear(x, w[p + "self_attn.v_proj.weight"]).view(n, NKV, HD)
+            h = h + plain_linear(rnd(plain_attention(q, k, v)).reshape(n, -1), w[p + "self_attn.o_proj.weight"])
+            h = h + plain_mlp(norm(h, w[p + "post_attention_layernorm.weight"]), w[p + "mlp.gate_proj.weight"],
+                              w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"],
+                              rnd if dtype == "bf16" else None)
+        return plain_linear(norm(h, w["model.norm.weight"]), w["model.embed_tokens.weight"]).numpy()
+
+    reqs = {f"i{i}": random_tokens(n, V, 120 + i) for i, n in enumerate((40, 7, 66, 21))}
+    plain = {k: plain_toy(v) for k, v in reqs.items()}
+    tol = 1e-5 if dtype == "fp32" else 2e-2
+    for steps in (replay.whole(reqs), replay.tail_one_by_one(reqs, 32), replay.portions(reqs),
+                  replay.mixed(reqs, max_live=3, seed=2)):
+        cache = engine.new_cache(replay.trace_peak_tokens(steps, 16) // 16, 16, 3)
+        assert cache.storage.layers[0].paged["k"].dtype == torch.float32
+        got = replay.run_trace(engine, cache, steps)
+        for rid, ids in reqs.items():
+            for pos in range(len(ids)):
+                assert _rel(got[rid][pos], plain[rid][pos]) < tol, (rid, pos)

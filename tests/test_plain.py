@@ -80,18 +80,51 @@ def test_inv_freq_bands():
     assert all(x > y for x, y in zip(got, got[1:]))         # still decreasing
 
 
-def test_inv_freq_is_continuous_at_the_band_edges():
-    # a frequency whose wavelength sits exactly at an edge gets the neighbouring band's value
-    factor, low, high, orig = 8.0, 1.0, 4.0, 8192
+# theta 16 and 32 dims give inverse frequencies 2^(-i/4); with an original length of 16 pi the
+# ratio original / wavelength is 8 * 2^(-i/4): 8, 6.7, 5.7, 4.8, 4 (the high edge), 3.4, 2.8, 2.4, 2,
+# 1.7, 1.4, 1.2, 1 (the low edge), 0.84, 0.71, 0.59. Entries 5 to 11 lie inside the band, entry 8
+# at smooth = (2 - 1) / (4 - 1) = 1/3: 0.25 * (1/3 + (2/3) / 8) = 0.104166..; with high = 5 the
+# band starts at entry 3 and entry 8 has smooth 1/4: 0.25 * (1/4 + (3/4) / 8) = 0.0859375.
+# Worked by hand from src/kernels.cpp:134-155 (new = (1 - smooth) * f / factor + smooth * f with
+# smooth = (original / wavelength - low) / (high - low)). The reference's own tests hold this
+# formula against the transformers package (tests/test_kernels.py:88-110); library model code is
+# not a source here, so parity with that package is unpinned and these numbers stand in.
+_MID_BAND = {
+    (1.0, 4.0): [1.0, 0.840896415, 0.707106781, 0.594603558, 0.5, 0.342404254, 0.232741102, 0.156689181,
+                 0.104166667, 0.0680823883, 0.0434538841, 0.0267847212, 0.015625, 0.0131390065, 0.0110485435,
+                 0.00929068059],
+    (1.0, 5.0): [1.0, 0.840896415, 0.707106781, 0.56297435, 0.390625, 0.269942197, 0.18560437, 0.126807567,
+                 0.0859375, 0.0576312945, 0.0381146848, 0.0247338812, 0.015625, 0.0131390065, 0.0110485435,
+                 0.00929068059],
+}
 
-    def blend(wavelen):
-        fr = 2 * math.pi / wavelen
-        smooth = (orig / wavelen - low) / (high - low)
-        return (1 - smooth) * fr / factor + smooth * fr, fr
-    v, fr = blend(orig / low)
-    assert abs(v - fr / factor) < 1e-15
-    v, fr = blend(orig / high)
-    assert abs(v - fr) < 1e-15
+
+@pytest.mark.parametrize("low,high", list(_MID_BAND))
+def test_inv_freq_mid_band_values(low, high):
+    """Seven (nine) entries inside the band at known blend weights. A blend with its weights
+    swapped, a squared weight, the wavelength in place of its inverse, or a constant weight all
+    give other numbers (entry 8 alone: 0.177, 0.0556, 0.0703, 0.141 instead of 0.104)."""
+    got = plain_inv_freq(32, 16.0, (8.0, low, high, 16.0 * math.pi))
+    want = _MID_BAND[(low, high)]
+    for i, (g, w) in enumerate(zip(got, want)):
+        assert abs(g - w) <= 2e-7 * w, (i, g, w)
+    assert abs(got[8] - (0.25 * (1 / 3 + (2 / 3) / 8) if high == 4.0 else 0.0859375)) < 1e-8
+
+
+def test_inv_freq_blend_is_affine_in_the_frequency_and_continuous():
+    """new / old = 1/factor + smooth (1 - 1/factor) with smooth affine in the frequency itself:
+    inside the band the points (old, new / old) lie on one line, which runs from 1/factor at the
+    low edge to 1 at the high edge (so the bands meet without a jump)."""
+    factor, low, high, orig = 32.0, 1.0, 4.0, 8192
+    base = plain_inv_freq(128, 500000.0, None)                       # the sizes of the real models
+    got = plain_inv_freq(128, 500000.0, (factor, low, high, orig))
+    mid = [(b, g / b) for b, g in zip(base, got) if orig / high <= 2 * math.pi / b <= orig / low]
+    assert len(mid) >= 5
+    edge_lo, edge_hi = 2 * math.pi * low / orig, 2 * math.pi * high / orig     # the band's frequencies
+    for b, ratio in mid:
+        smooth = (b - edge_lo) / (edge_hi - edge_lo)
+        assert abs(ratio - (1 / factor + smooth * (1 - 1 / factor))) < 1e-6, (b, ratio)
+    assert all(r1 > r2 for (_, r1), (_, r2) in zip(mid, mid[1:]))    # higher frequencies keep more
 
 
 def test_rope_tables_values():
@@ -205,8 +238,28 @@ def test_mlp_is_gated():
 
 # --- whole model ---------------------------------------------------------------------
 def _random_weights(cfg, seed):
-    from llmengine.weights import random_state
-    return dict(random_state(cfg, seed, torch.float32, 0.05, 1.0, 0.1))
+    """A checkpoint's tensors by the names and shapes of src/model.cpp:179-287, drawn here (nothing
+    of the engine is imported)."""
+    c = plain_config(cfg)
+    g = _gen(seed)
+    H, FF, q_dim, kv_dim = c["H"], c["FF"], c["n_q"] * c["hd"], c["n_kv"] * c["hd"]
+
+    def lin(*shape):
+        return 0.05 * torch.randn(*shape, generator=g)
+
+    def norm():
+        return 1.0 + 0.1 * torch.randn(H, generator=g)
+    w = {"model.embed_tokens.weight": lin(c["V"], H), "model.norm.weight": norm()}
+    if not c["tie"]:
+        w["lm_head.weight"] = lin(c["V"], H)
+    for layer in range(c["L"]):
+        p = f"model.layers.{layer}."
+        w.update({p + "input_layernorm.weight": norm(), p + "post_attention_layernorm.weight": norm(),
+                  p + "self_attn.q_proj.weight": lin(q_dim, H), p + "self_attn.k_proj.weight": lin(kv_dim, H),
+                  p + "self_attn.v_proj.weight": lin(kv_dim, H), p + "self_attn.o_proj.weight": lin(H, q_dim),
+                  p + "mlp.gate_proj.weight": lin(FF, H), p + "mlp.up_proj.weight": lin(FF, H),
+                  p + "mlp.down_proj.weight": lin(H, FF)})
+    return w
 
 
 def test_config_defaults():

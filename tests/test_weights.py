@@ -111,6 +111,16 @@ def test_tied_head_is_the_embedding(tmp_path):
     t2 = build_llama(parse_config(TINY_A))
     load_model_weights(t2, _write(tmp_path / "a2", TINY_A, both), CPU32)
     assert t2.head.weight.data_ptr() == t2.embedding.weight.data_ptr()
+    # .. unless it disagrees with the embedding in shape or type (src/weights.cpp:259-264)
+    for bad, what in ((torch.zeros(64, 256), "[64,256]"), (torch.zeros(255, 64), "[255,64]"),
+                      (torch.zeros(256, 64, dtype=torch.bfloat16), "bfloat16")):
+        state = _state(TINY_A)
+        state["lm_head.weight"] = bad
+        with pytest.raises(WeightError) as e:
+            load_model_weights(build_llama(parse_config(TINY_A)), _write(tmp_path / f"bad{what}", TINY_A, state), CPU32)
+        assert ("tie_word_embeddings=true but lm_head.weight shape/dtype disagrees with model.embed_tokens.weight"
+                in str(e.value)) and what in str(e.value)
+        assert e.value.wrong_shape == ["lm_head.weight"] and not e.value.missing and not e.value.unexpected
     untied = build_llama(parse_config(TINY_B))
     load_model_weights(untied, _write(tmp_path / "b", TINY_B, _state(TINY_B)), CPU32)
     assert untied.head.weight.data_ptr() != untied.embedding.weight.data_ptr()
