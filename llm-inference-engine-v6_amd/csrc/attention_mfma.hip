@@ -306,13 +306,25 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     }
 }
 
-// Whether the decode kernel loads keys and values with the read-once hint. -1: the entry point
-// chooses; 0 / 1: never / always (llme_attention_bf16_set_stream, for measurements).
-static int g_stream_override = -1;
-static bool decode_reads_once(int n_decode) {
-    if (g_stream_override >= 0) return g_stream_override != 0;
-    return n_decode >= 0;
+// What a caller may override of the launch choices, for tests and measurements, packed into
+// the entry points' `tuning` argument (0: every choice is the entry point's):
+//   bits 0-7   rows per work item of the prefill kernel without LDS: 16, 32 or 64 (0: by head size)
+//   bits 8-11  1 + shared: -1 the kernel that shares K and V through LDS where it takes the sizes
+//              (the default), 0 never, 1 wherever it can, 2 / 3 the same with one / two wavefronts
+//              per tile whatever the number of work items
+//   bits 12-13 1 + read_once: whether the decode kernel loads keys and values with the read-once
+//              hint: -1 the entry point chooses, 0 never, 1 always
+struct Tuning {
+    int rows, shared, key_waves, read_once;
+};
+static bool parse_tuning(int packed, Tuning* t) {
+    if (packed < 0 || packed >= (1 << 14)) return false;
+    const int rows = packed & 0xFF, shared = ((packed >> 8) & 0xF) - 1, read_once = ((packed >> 12) & 0x3) - 1;
+    if (rows % 16 != 0 || rows > 64 || shared > 3 || read_once > 1) return false;
+    *t = Tuning{rows, shared > 1 ? 1 : shared, shared > 1 ? shared - 1 : 0, read_once};
+    return true;
 }
+static bool decode_reads_once(const Tuning& t) { return t.read_once != 0; }
 
 template <int HD>
 static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, float* part_o, float* part_ml,
@@ -320,11 +332,11 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
                            int n_q, int n_kv, int page, float scale, int window, int n_decode, int split_len,
                            int nsplit, int prefill_groups, int qt, int shared_rows, int* queue, int n_rows,
                            int prefill_splits, int prefill_run, float* pre_part_o, float* pre_part_ml,
-                           hipStream_t stream) {
+                           const Tuning& tuning, hipStream_t stream) {
     if (n_decode > 0) {
         const int G = n_q / n_kv;
         const dim3 grid(n_seq, n_kv * ((G + 15) / 16), nsplit);
-        if (decode_reads_once(n_decode))
+        if (decode_reads_once(tuning))
             hipLaunchKernelGGL((attention_decode_kernel<HD, true>), grid, dim3(DEC_WAVES * 64), 0, stream, q, kc, vc, out,
                                part_o, part_ml, q_start, ctx_len, table, max_blocks, n_q, n_kv, page, scale, window,
                                split_len, nsplit);
@@ -340,7 +352,8 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
         if (shared_rows > 0) {
             const int status = launch_prefill_shared(q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q,
                                                      n_kv, HD, page, scale, window, prefill_groups, shared_rows, queue,
-                                                     prefill_splits, prefill_run, pre_part_o, pre_part_ml, stream);
+                                                     prefill_splits, prefill_run, pre_part_o, pre_part_ml,
+                                                     tuning.key_waves, stream);
             if (status != 0 || prefill_splits <= 1) return status;
             hipLaunchKernelGGL(attention_join_rows_kernel, dim3(n_rows, n_q), dim3(64), 0, stream, pre_part_o,
                                pre_part_ml, out, q_start, ctx_len, n_seq, n_q, HD, prefill_splits, prefill_run,
@@ -366,42 +379,27 @@ using namespace llme;
 // Rows per prefill work item for a model's head sizes: the caller sizes the grid with it. More
 // rows reuse every K and V load more often; fewer rows give more wavefronts to hide latencies
 // and to even out the causal triangle. The kernel that shares K and V through LDS is used
-// where it takes the sizes. llme_attention_bf16_set_rows overrides the choice for
-// measurements: rows per item of the kernel without LDS (0: the default), shared -1: as by
-// default, 0: never, 1: if it can.
-static int g_rows_override = 0;
-static int g_shared_override = -1;
-extern "C" int llme_attention_bf16_set_rows(int rows, int shared) {
-    // shared 2 and 3: the kernel with LDS with one or two wavefronts per tile, whatever the batch
-    if (rows < 0 || rows % 16 != 0 || rows > 256 || shared < -1 || shared > 3) return kErrBadArgument;
-    g_rows_override = rows;
-    g_shared_override = shared > 1 ? 1 : shared;
-    prefill_shared_key_waves(shared > 1 ? shared - 1 : 0);
-    return 0;
-}
-extern "C" int llme_attention_bf16_set_stream(int mode) {
-    if (mode < -1 || mode > 1) return kErrBadArgument;
-    g_stream_override = mode;
-    return 0;
-}
-static int direct_rows(int hd) {
+// where it takes the sizes.
+static int direct_rows(int hd, const Tuning& t) {
     int rows = hd <= 64 ? 64 : 32;
-    if (g_rows_override == 16 || g_rows_override == 32 || g_rows_override == 64) rows = g_rows_override;
+    if (t.rows == 16 || t.rows == 32 || t.rows == 64) rows = t.rows;
     if (hd > 64 && rows > 32) rows = 32;
     return rows;
 }
-static int shared_rows_for(int hd, int n_q, int n_kv) {
-    return g_shared_override == 0 ? 0 : prefill_shared_rows(hd, n_q, n_kv);
+static int shared_rows_for(int hd, int n_q, int n_kv, const Tuning& t) {
+    return t.shared == 0 ? 0 : prefill_shared_rows(hd, n_q, n_kv);
 }
-extern "C" int llme_attention_bf16_rows(int hd, int n_q, int n_kv) {
-    const int shared = shared_rows_for(hd, n_q, n_kv);
-    return shared > 0 ? shared : direct_rows(hd);
+extern "C" int llme_attention_bf16_rows(int hd, int n_q, int n_kv, int tuning) {
+    Tuning t;
+    if (!parse_tuning(tuning, &t)) return -1;
+    const int shared = shared_rows_for(hd, n_q, n_kv, t);
+    return shared > 0 ? shared : direct_rows(hd, t);
 }
 
 // n_decode: requests with one token (0: none, skip the decode kernels); split_len (multiple of
 // 32) and nsplit: how the decode kernel cuts the keys; part_o [n_seq, n_q, nsplit, hd] and
 // part_ml [n_seq, n_q, nsplit, 2] floats (needed when nsplit > 1). prefill_groups: number of
-// row groups of llme_attention_bf16_rows(hd, n_q, n_kv) rows over the requests with two or more tokens.
+// row groups of llme_attention_bf16_rows(hd, n_q, n_kv, tuning) rows over the requests with two or more tokens.
 // queue: two integers, zero, for the prefill kernel's work counter (needed when prefill_groups > 0;
 // the kernel leaves them zero; launches that may overlap need separate ones).
 // prefill_splits > 1 (only where llme_attention_bf16_splits_prefill says so): the keys of a prefill
@@ -409,8 +407,10 @@ extern "C" int llme_attention_bf16_rows(int hd, int n_q, int n_kv) {
 // last run takes the rest), joined by a second kernel over the batch's n_rows rows; pre_part_o
 // [n_rows, n_q, prefill_splits, hd] and pre_part_ml [n_rows, n_q, prefill_splits, 2] floats are
 // their scratch.
-extern "C" int llme_attention_bf16_splits_prefill(int hd, int n_q, int n_kv) {
-    return shared_rows_for(hd, n_q, n_kv) > 0 ? 1 : 0;
+extern "C" int llme_attention_bf16_splits_prefill(int hd, int n_q, int n_kv, int tuning) {
+    Tuning t;
+    if (!parse_tuning(tuning, &t)) return 0;
+    return shared_rows_for(hd, n_q, n_kv, t) > 0 ? 1 : 0;
 }
 
 extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const void* v_cache, void* out, float* part_o,
@@ -418,10 +418,12 @@ extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const voi
                                    int max_blocks, int n_seq, int n_q, int n_kv, int hd, int page, float scale,
                                    int window, int n_decode, int split_len, int nsplit, int prefill_groups,
                                    int* queue, int n_rows, int prefill_splits, int prefill_run, float* pre_part_o,
-                                   float* pre_part_ml, hipStream_t stream) {
+                                   float* pre_part_ml, int tuning, hipStream_t stream) {
     if (n_seq <= 0) return 0;
+    Tuning tune;
+    if (!parse_tuning(tuning, &tune)) return kErrBadArgument;
     if (prefill_splits < 1 || prefill_splits > 64 || n_rows < 0) return kErrBadArgument;
-    if (prefill_splits > 1 && (shared_rows_for(hd, n_q, n_kv) <= 0 || prefill_run < 1 || pre_part_o == nullptr ||
+    if (prefill_splits > 1 && (shared_rows_for(hd, n_q, n_kv, tune) <= 0 || prefill_run < 1 || pre_part_o == nullptr ||
                                pre_part_ml == nullptr))
         return kErrBadArgument;
     if (hd % 16 != 0 || hd > 128 || hd <= 0 || page % 16 != 0 || n_kv <= 0 || n_q % n_kv != 0) return kErrUnsupported;
@@ -430,15 +432,15 @@ extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const voi
     if (static_cast<double>(max_blocks) * (page / 16) * (page / 16) >= 4294967296.0) return kErrUnsupported;
     if (static_cast<double>(n_kv) * page * hd >= 4294967296.0) return kErrUnsupported;   // a page's elements: 32 bits
     if (n_decode > 0 && (split_len <= 0 || split_len % 32 != 0 || nsplit <= 0 || nsplit > 64)) return kErrBadArgument;
-    const int qt = direct_rows(hd) / 16;
-    const int shared_rows = shared_rows_for(hd, n_q, n_kv);
+    const int qt = direct_rows(hd, tune) / 16;
+    const int shared_rows = shared_rows_for(hd, n_q, n_kv, tune);
 #define LLME_HEAD(HD)                                                                                           \
     case HD:                                                                                                    \
         return launch_for_head<HD>(static_cast<const bf16*>(q), static_cast<const bf16*>(k_cache),              \
                                    static_cast<const bf16*>(v_cache), static_cast<bf16*>(out), part_o, part_ml, \
                                    q_start, ctx_len, block_table, max_blocks, n_seq, n_q, n_kv, page, scale,    \
                                    window, n_decode, split_len, nsplit, prefill_groups, qt, shared_rows, queue, n_rows, \
-                                   prefill_splits, prefill_run, pre_part_o, pre_part_ml, stream)
+                                   prefill_splits, prefill_run, pre_part_o, pre_part_ml, tune, stream)
     switch (hd) {
         LLME_HEAD(16); LLME_HEAD(32); LLME_HEAD(48); LLME_HEAD(64);
         LLME_HEAD(80); LLME_HEAD(96); LLME_HEAD(112); LLME_HEAD(128);
@@ -514,5 +516,5 @@ extern "C" int llme_attention_decode_noalloc(const void* q, const void* k_cache,
     return llme_attention_bf16(q, k_cache, v_cache, out, part_o, part_ml, q_start, ctx_len, block_table, max_blocks,
                                n_seq, n_q, n_kv, hd, page, scale, window, /*n_decode=*/n_seq, split_len, nsplit,
                                /*prefill_groups=*/0, /*queue=*/nullptr, /*n_rows=*/n_seq, /*prefill_splits=*/1,
-                               /*prefill_run=*/1, nullptr, nullptr, stream);
+                               /*prefill_run=*/1, nullptr, nullptr, /*tuning=*/0, stream);
 }

@@ -403,7 +403,6 @@ __global__ __launch_bounds__(256 * KW) void attention_prefill_shared_kernel(
 }
 
 constexpr long kSplitBelowItems = 768;
-static int g_key_waves = 0;                 // 0: by the number of items; 1, 2: forced (measurements, tests)
 
 static int heads_per_workgroup(int n_q, int n_kv) {
     const int G = n_q / n_kv;
@@ -452,7 +451,7 @@ static int launch_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* ou
 int launch_prefill_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, const int* q_start,
                           const int* ctx_len, const int* table, int max_blocks, int n_seq, int n_q, int n_kv, int hd,
                           int page, float scale, int window, int items, int rows_per_item, int* queue, int nsplit,
-                          int run, float* part_o, float* part_ml, hipStream_t stream) {
+                          int run, float* part_o, float* part_ml, int key_waves, hipStream_t stream) {
     if (queue == nullptr) return kErrBadArgument;
     if (nsplit < 1 || (nsplit > 1 && (run < 1 || part_o == nullptr || part_ml == nullptr))) return kErrBadArgument;
     const int hpw = heads_per_workgroup(n_q, n_kv);
@@ -460,7 +459,7 @@ int launch_prefill_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* o
     // Two wavefronts per tile while the items are too few to keep three workgroups of four
     // wavefronts on every compute unit: then an item's length, not the chip, sets the time.
     int kw = static_cast<long>(items) * (n_q / hpw) <= kSplitBelowItems ? 2 : 1;
-    if (g_key_waves == 1 || g_key_waves == 2) kw = g_key_waves;
+    if (key_waves == 1 || key_waves == 2) kw = key_waves;  // (forced by the caller: tests, measurements)
 #define LLME_SHARED_ARGS q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, page, scale, window, \
                          items, queue, nsplit, run, part_o, part_ml, stream
 #define LLME_SHARED(HD, QT, HPW)                                                       \
@@ -477,7 +476,5 @@ int launch_prefill_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* o
 #undef LLME_SHARED_ARGS
     return kErrUnsupported;
 }
-
-void prefill_shared_key_waves(int kw) { g_key_waves = kw; }
 
 }  // namespace llme

@@ -358,7 +358,7 @@ __device__ __forceinline__ void load_q(const bf16* qrow, bool ok, bf16x8 (&qf)[(
 int launch_prefill_shared(const bf16* q, const bf16* k_cache, const bf16* v_cache, bf16* out, const int* q_start,
                           const int* ctx_len, const int* block_table, int max_blocks, int n_seq, int n_q, int n_kv,
                           int hd, int page, float scale, int window, int items, int rows_per_item, int* queue,
-                          int nsplit, int run, float* part_o, float* part_ml, hipStream_t stream);
+                          int nsplit, int run, float* part_o, float* part_ml, int key_waves, hipStream_t stream);
 
 // Runs that the keys [k_begin, key_end) of a prefill work item are cut into: `run` stretches of 64
 // keys each, at most max_runs (the last run then takes the rest).
@@ -369,7 +369,5 @@ __host__ __device__ __forceinline__ int key_runs(int k_begin, int key_end, int r
 }
 // Rows per work item of the shared kernel for these sizes, or 0 if it does not take them.
 int prefill_shared_rows(int hd, int n_q, int n_kv);
-// Wavefronts that share a tile's keys: 0 lets the launcher choose by the number of items, 1 or 2 forces it.
-void prefill_shared_key_waves(int kw);
 
 }  // namespace llme

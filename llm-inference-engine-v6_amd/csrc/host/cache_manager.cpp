@@ -348,16 +348,20 @@ int llme_cm_num_pages(void* h, int group) {
 int llme_cm_check(void* h) { return static_cast<CacheManager*>(h)->check(); }
 
 // A step of one new token per request, in one call: the requests' lengths, and a page for each
-// new token where it starts a page (all or none). Returns 1, 0 (pools short, nothing changed) or
-// an error code.
-int llme_cm_decode_begin(void* h, int S, const int64_t* keys, int* lengths) {
+// new token where it starts a page (all or none). max_length > 0: no request may become longer
+// than that; if one would, nothing is reserved and the call returns 2 (the lengths are filled in).
+// Returns 1, 0 (pools short, nothing changed), 2 or an error code.
+int llme_cm_decode_begin(void* h, int S, const int64_t* keys, int* lengths, long max_length) {
     auto* m = static_cast<CacheManager*>(h);
     std::vector<long> ones(static_cast<size_t>(S), 1);
+    bool too_long = false;
     for (int i = 0; i < S; ++i) {
         auto* r = m->find(keys[i]);
         if (!r) return LLME_HOST_NOT_LIVE;
         lengths[i] = static_cast<int>(r->length);
+        if (max_length > 0 && r->length + 1 > max_length) too_long = true;
     }
+    if (too_long) return 2;
     return m->reserve_batch(S, keys, ones.data());
 }
 // commit for several requests: n_new tokens each

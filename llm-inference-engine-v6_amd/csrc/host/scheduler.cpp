@@ -19,7 +19,10 @@
 //
 // This file decides; it runs nothing. A step is plan() (admission, the batch), then the caller
 // runs the batch through the model and samples, then complete() (the sampled tokens arrive,
-// sequences move on or finish, pages go back). The cache manager is the one the step function
+// prompts move on by the portions that ran, sequences move on or finish, pages go back). If the
+// model run fails, the caller calls abort() instead of complete(): the planned portions have not
+// run, the prompts stay where they were, and the next plan() offers them again. (What plan()
+// decided apart from the batch stands: admissions, and requests ended for want of pages.) The cache manager is the one the step function
 // reserves and commits in; sequence ids are its request keys.
 #include "host_api.h"
 
@@ -27,6 +30,7 @@
 #include <cstdint>
 #include <deque>
 #include <memory>
+#include <utility>
 #include <vector>
 
 extern "C" {
@@ -82,8 +86,10 @@ public:
     // Admission, then the step's batch. Returns the number of entries, or an error code.
     int plan(int* n_admitted, int* admitted_slots, int64_t* entry_seq, int* entry_count, int* entry_want,
              long* entry_gen, int* tokens, long tokens_cap) {
+        if (planned_) return LLME_HOST_BAD_ARGUMENT;  // the last step was neither completed nor aborted
         owners_.clear();
         prompt_ends_.clear();
+        portions_.clear();
         *n_admitted = 0;
         // admission: no page check, as in the reference
         while (!waiting_.empty() && static_cast<int>(prefilling_.size() + running_.size()) < max_concurrent_) {
@@ -131,7 +137,7 @@ public:
             const bool ends = s.cursor + n == s.prompt_len;
             if (!add_entry(s, s.cursor, n, ends && s.max_new > 0, 0)) return LLME_HOST_BAD_ARGUMENT;
             if (ends) prompt_ends_.push_back(&s);
-            s.cursor += n;
+            portions_.push_back({&s, n});             // (the prompt moves on in complete(), once the portion has run)
             budget -= n;
         }
         // one token for every decoding request
@@ -152,6 +158,8 @@ public:
     int complete(const int* sampled, int n, const int* eos, int n_eos) {
         if (!planned_ || n != static_cast<int>(owners_.size())) return LLME_HOST_BAD_ARGUMENT;
         planned_ = false;
+        for (const auto& portion : portions_) portion.first->cursor += portion.second;
+        portions_.clear();
         for (int i = 0; i < n; ++i) {
             Seq& s = *owners_[static_cast<size_t>(i)];
             // a sampled token arrives for a sequence (src/scheduler.cpp:208-227, 271-282)
@@ -197,6 +205,14 @@ public:
         return finished;
     }
 
+    // The planned step did not run: forget the batch, keep every prompt where it was.
+    void abort() {
+        planned_ = false;
+        owners_.clear();
+        prompt_ends_.clear();
+        portions_.clear();
+    }
+
     int num_results() const { return static_cast<int>(results_.size()); }
     const Seq* result(int i) const {
         return i >= 0 && i < num_results() ? results_[static_cast<size_t>(i)].get() : nullptr;
@@ -216,6 +232,7 @@ private:
     std::deque<std::unique_ptr<Seq>> waiting_;
     std::vector<std::unique_ptr<Seq>> prefilling_, running_, results_;
     std::vector<Seq*> owners_, prompt_ends_;       // between plan() and complete()
+    std::vector<std::pair<Seq*, long>> portions_;  // prompt tokens that the planned step carries
 };
 
 }  // namespace llme_host
@@ -248,6 +265,7 @@ int llme_sched_plan(void* h, int* n_admitted, int* admitted_slots, int64_t* entr
 int llme_sched_complete(void* h, const int* sampled, int n, const int* eos, int n_eos) {
     return static_cast<Scheduler*>(h)->complete(sampled, n, eos, n_eos);
 }
+void llme_sched_abort(void* h) { static_cast<Scheduler*>(h)->abort(); }
 int llme_sched_num_results(void* h) { return static_cast<Scheduler*>(h)->num_results(); }
 // reason: 1 "stop", 2 "length", 3 "capacity"
 int llme_sched_result_info(void* h, int i, int64_t* seq_id, long* prompt_len, long* n_tokens, int* reason) {

@@ -21,6 +21,7 @@ when the reference's next step would find them.
 from __future__ import annotations
 
 import ctypes
+import weakref
 from dataclasses import dataclass
 from typing import Protocol, Sequence
 
@@ -74,7 +75,19 @@ class ContinuousBatchScheduler:
         self._budget = int(max_prefill_tokens_per_step)
         self.temperature = float(temperature)
         self.seed = int(seed)
+        # Sequence ids are the requests' keys in the cache manager, and every scheduler counts from
+        # 0: two schedulers over one block manager would take each other's keys, and a second one
+        # that asks for more slots would have the pool replaced under the first.
+        other = getattr(block_manager, "_scheduler", None)
+        other = other() if other is not None else None
+        if other is not None and not other.idle:
+            raise ValueError("ContinuousBatchScheduler: this block manager already serves a scheduler with "
+                             "requests in flight; give every scheduler a BlockManager of its own")
         self._cache = engine.open_cache(block_manager, self.max_concurrent)
+        try:
+            block_manager._scheduler = weakref.ref(self)
+        except AttributeError:
+            pass                                        # (a stand-in manager without attributes)
         self._lib = native.library()
         self._h = self._lib.llme_sched_create(self._cache.manager.handle, self.max_concurrent, self._budget)
         if not self._h:
@@ -154,8 +167,11 @@ class ContinuousBatchScheduler:
                                       self._entry_count, self._entry_want, self._entry_gen, self._tokens,
                                       self._tokens_cap)
         if E < 0:
-            raise RuntimeError(f"the scheduler could not plan a step (code {E}): the cache it was given has fewer "
-                               f"slots than max_concurrent = {self.max_concurrent}")
+            why = {-1: "a sequence id of this scheduler is already live in the cache (another user of the same "
+                       "block manager holds that key)",
+                   -2: f"the cache it was given has fewer slots than max_concurrent = {self.max_concurrent}",
+                   -6: "the step before was neither completed nor aborted, or the batch does not fit its buffers"}
+            raise RuntimeError(f"the scheduler could not plan a step (code {E}): {why.get(E, 'host runtime error')}")
         told = getattr(self._cache, "slot_admitted", None)
         if told is not None:
             for i in range(n_admitted.value):
@@ -172,9 +188,15 @@ class ContinuousBatchScheduler:
             pos += n
         sampled: list[int] = []
         if entries:
-            sampled = self.engine.run_step(self._cache, entries, draws, self.temperature, self.seed)
-            if len(sampled) != len(draws):
-                raise RuntimeError(f"the step returned {len(sampled)} tokens for {len(draws)} wanted rows")
+            try:
+                sampled = self.engine.run_step(self._cache, entries, draws, self.temperature, self.seed)
+                if len(sampled) != len(draws):
+                    raise RuntimeError(f"the step returned {len(sampled)} tokens for {len(draws)} wanted rows")
+            except BaseException:
+                # the batch did not run: the prompts stay where they were and the next step offers
+                # the same portions again (the step function changes nothing when it fails)
+                self._lib.llme_sched_abort(self._h)
+                raise
             self.steps += 1
         eos = [int(t) for t in self.engine.eos_token_ids]
         rc = self._lib.llme_sched_complete(self._h, (ctypes.c_int * max(len(sampled), 1))(*[int(t) for t in sampled]),

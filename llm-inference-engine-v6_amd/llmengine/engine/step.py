@@ -183,6 +183,7 @@ class _DecodeRecord:
         self.done = (ctypes.c_int * max(G * S, 1))()        # per group and request: table entries written so far
         self.serials = (ctypes.c_int64 * S)()               # which admission of its key sits in each place
         self.event: torch.cuda.Event | None = None
+        self.scratch = None
 
     def refresh(self, mgr: CacheManager, entries: Sequence[StepEntry], keys=None) -> None:
         if self.event is not None:
@@ -238,7 +239,10 @@ class ModelRunner:
         all entries are reserved first (CapacityError, with nothing changed, if the
         pools are short); then the tokens run as one batch; then the requests are
         that much longer. Returns logits [sum(len(want)), vocab] on the device, in
-        the order of the entries and of their `want` lists, or None."""
+        the order of the entries and of their `want` lists, or None. The tensor is scratch
+        memory of this runner (or of the recorded step that was replayed): it holds these
+        logits until the runner's next step, which writes its own into the same place; a
+        caller that needs them longer copies them."""
         mgr = cache.manager
         if not entries:
             return None
@@ -312,20 +316,23 @@ class ModelRunner:
             meta = torch.empty(7 * S + 1 + groups * S * width + 64, dtype=torch.int32, device=self.device)
             ctx, logit_rows = self._build_context(cache, entries, max_blocks=width, plan_len=width * page, dev=meta)
             logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
-            tok_host = None
+            tok_host = scratch = None
             if greedy:
                 # pinned host memory is mapped into the device's address space: the kernel writes
-                # the tokens where the host reads them, without a copy of its own
+                # the tokens where the host reads them, without a copy of its own; the argmax's
+                # scratch belongs to the recording (the one that plain calls share may be replaced)
                 tok_host = torch.zeros(S, dtype=torch.int32, pin_memory=True)
-                ops.argmax_into(logits, tok_host.data_ptr())
+                scratch = ops.sampling_scratch(self.device, S, self.model.vocab_size)
+                ops.argmax_into(logits, tok_host.data_ptr(), scratch)
             torch.cuda.synchronize(self.device)
             self.workspace.keep_replaced = True
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
                 if greedy:
-                    ops.argmax_into(logits, tok_host.data_ptr())
+                    ops.argmax_into(logits, tok_host.data_ptr(), scratch)
             cache.graphs[key] = rec = _DecodeRecord(graph, logits, meta, S, width, list(mgr.groups), tok_host)
+            rec.scratch = scratch                       # (kept alive: the graph holds its addresses)
         return rec
 
     def step_greedy(self, cache: CacheContext, entries: Sequence[StepEntry], max_position: int | None = None
@@ -350,16 +357,17 @@ class ModelRunner:
         mgr = cache.manager
         keys = (ctypes.c_int64 * S)(*[mgr.key_of(r) for r in ids])
         lengths = (ctypes.c_int * S)()
-        rc = mgr._lib.llme_cm_decode_begin(mgr.handle, S, keys, lengths)
+        # lengths, the position limit and the pages in one call; a call that fails has changed nothing
+        rc = mgr._lib.llme_cm_decode_begin(mgr.handle, S, keys, lengths, int(max_position or 0))
         if rc < 0:
             raise RuntimeError(f"a request of the step is not live (code {rc})")
         longest = max(lengths)
+        if rc == 2:
+            raise ValueError(f"{longest + 1} tokens exceed the position limit {max_position}")
         if rc == 0:
             need = {g: sum(mgr.pages_needed(r, 1)[g] for r in ids) for g in mgr.groups}
             raise CapacityError(f"the step needs {need} more pages, free are "
                                 f"{({g: mgr.free_pages(g) for g in mgr.groups})}")
-        if max_position is not None and longest + 1 > max_position:
-            raise ValueError(f"{longest + 1} tokens exceed the position limit {max_position}")
         rec = self._decode_record(cache, entries, longest, greedy=True)
         rec.refresh(mgr, entries, keys)
         rec.graph.replay()

@@ -1,7 +1,7 @@
 """The HIP kernels of the engine, as Python functions over device tensors."""
 from .lib import KernelError, KernelLibraryError, library
 from .kernels import (argmax, argmax_into, attention, attention_generic, block_weight, can_block, clear, embed_gather, gemm,
-                      gemm_generic, is_blocked, policy, rmsnorm, rope_kv_write, rope_q_only, sample, swiglu,
+                      gemm_generic, is_blocked, policy, rmsnorm, rope_kv_write, rope_q_only, sample, sampling_scratch, swiglu,
                       unblock_weight, weight_shape)
 
 from . import mfma                                   # noqa: E402  (installs the MFMA kernels)
@@ -10,4 +10,4 @@ from .mfma import (gemm_bf16, gemm_gated, gemv_norm, gemv_norm_rope, gemv_norm_r
 
 __all__ = ["gemm_bf16", "gemm_gated", "gemv_norm_rope", "gemv_norm_rope_supported", "pair_rows_for_rotation", "gemv_norm", "gemv_norm_supported", "mfma", "KernelError", "KernelLibraryError", "library", "argmax", "argmax_into", "attention", "attention_generic", "rope_q_only", "embed_gather", "block_weight", "can_block", "clear",
            "is_blocked", "unblock_weight", "weight_shape",
-           "gemm", "gemm_generic", "policy", "rmsnorm", "rope_kv_write", "sample", "swiglu"]
+           "gemm", "gemm_generic", "policy", "rmsnorm", "rope_kv_write", "sample", "sampling_scratch", "swiglu"]

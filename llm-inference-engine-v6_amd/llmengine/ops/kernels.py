@@ -236,42 +236,63 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out
 
 
 # --- sampling ------------------------------------------------------------------------
-_argmax_scratch: dict = {}
+# The two-stage argmax and the sampler keep per-part results in scratch memory. Calls on one
+# stream run one after the other and share a scratch per (device, stream); a caller whose launches
+# are recorded into a graph brings a scratch of its own (`sampling_scratch`), which then lives as
+# long as the recording does: the shared one is replaced when a later call needs a larger one.
+_shared_scratch: dict = {}
 
 
-def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+def sampling_scratch(device, rows: int, vocab: int):
+    """Scratch for argmax / sample calls of up to `rows` rows of `vocab` columns."""
+    n = max(1, rows * entry("llme_argmax_parts")(vocab))
+    return (torch.empty(n, dtype=torch.float32, device=device), torch.empty(n, dtype=torch.int32, device=device),
+            torch.empty(n, dtype=torch.float32, device=device))
+
+
+def _scratch_for(logits: torch.Tensor, scratch):
+    R, V = logits.shape
+    need = R * entry("llme_argmax_parts")(V)
+    if scratch is not None:
+        if len(scratch) != 3 or any(t.numel() < need or t.device != logits.device for t in scratch):
+            raise KernelError(f"the sampling scratch is too small for {R} rows of {V} columns")
+        return scratch
+    key = (logits.device, stream())
+    have = _shared_scratch.get(key)
+    if have is None or have[0].numel() < need:
+        if len(_shared_scratch) >= 64:
+            _shared_scratch.clear()
+        n = max(need, 4096)
+        have = _shared_scratch[key] = (torch.empty(n, dtype=torch.float32, device=logits.device),
+                                       torch.empty(n, dtype=torch.int32, device=logits.device),
+                                       torch.empty(n, dtype=torch.float32, device=logits.device))
+    return have
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor, scratch=None) -> None:
     """out[r] = first index of the maximum of logits[r, :]."""
     require(logits, "logits", torch.float32, (None, None))
     R, V = logits.shape
     require(out, "out", torch.int32, (R,))
-    argmax_into(logits, ptr(out))
+    argmax_into(logits, ptr(out), scratch)
 
 
-def _parts_scratch(device, need: int):
-    scratch = _argmax_scratch.get(device)
-    if scratch is None or scratch[0].numel() < need:
-        n = max(need, 4096)
-        scratch = (torch.empty(n, dtype=torch.float32, device=device), torch.empty(n, dtype=torch.int32, device=device),
-                   torch.empty(n, dtype=torch.float32, device=device))
-        _argmax_scratch[device] = scratch
-    return scratch
-
-
-def argmax_into(logits: torch.Tensor, out_ptr: int) -> None:
+def argmax_into(logits: torch.Tensor, out_ptr: int, scratch=None) -> None:
     """argmax with the result (one int32 per row) written to an address the device can reach:
     device memory, or pinned host memory, which the device sees at the same address."""
     require(logits, "logits", torch.float32, (None, None))
     R, V = logits.shape
-    val, idx, _ = _parts_scratch(logits.device, R * entry("llme_argmax_parts")(V))
+    val, idx, _ = _scratch_for(logits, scratch)
     check(entry("llme_argmax")(ptr(logits), out_ptr, ptr(val), ptr(idx), R, V, stream()), "argmax")
 
 
-def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor) -> None:
+def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor,
+           scratch=None) -> None:
     require(logits, "logits", torch.float32, (None, None))
     R, V = logits.shape
     require(temperature, "temperature", torch.float32, (R,))
     require(uniform, "uniform", torch.float32, (R,))
     require(out, "out", torch.int32, (R,))
-    val, idx, sums = _parts_scratch(logits.device, R * entry("llme_argmax_parts")(V))
+    val, idx, sums = _scratch_for(logits, scratch)
     check(entry("llme_sample")(ptr(logits), ptr(temperature), ptr(uniform), ptr(out), ptr(val), ptr(idx), ptr(sums),
                                R, V, stream()), "sample")

@@ -77,12 +77,22 @@ kernels._fast_gemm = _fast_gemm
 
 
 # --- attention ---------------------------------------------------------------------------
-declare("llme_attention_bf16_rows", [_i, _i, _i])
-declare("llme_attention_bf16_set_rows", [_i, _i])
-declare("llme_attention_bf16_set_stream", [_i])
-declare("llme_attention_bf16_splits_prefill", [_i, _i, _i])
+declare("llme_attention_bf16_rows", [_i, _i, _i, _i])
+declare("llme_attention_bf16_splits_prefill", [_i, _i, _i, _i])
 declare("llme_attention_bf16", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i,
-                                _i, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp, _vp])
+                                _i, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp, _i, _vp])
+
+
+def attention_tuning(rows: int = 0, shared: int = -1, read_once: int = -1) -> int:
+    """Overrides of the attention kernels' launch choices for one call (tests, measurements), as
+    the entry points take them; 0 leaves every choice to the entry point. rows: rows per work item
+    of the prefill kernel without LDS (16, 32, 64; 0: by head size). shared: the prefill kernel that
+    shares K and V through LDS: -1 where it takes the sizes, 0 never, 1 wherever it can, 2 / 3 with
+    one / two wavefronts per tile whatever the number of items. read_once: the decode kernel's
+    cache hint on keys and values: -1 the entry point chooses, 0 off, 1 on."""
+    if rows not in (0, 16, 32, 64) or not -1 <= shared <= 3 or not -1 <= read_once <= 1:
+        raise kernels.KernelError(f"attention_tuning: rows {rows}, shared {shared}, read_once {read_once}")
+    return rows | (shared + 1) << 8 | (read_once + 1) << 12
 
 _work_queues: dict = {}
 
@@ -122,16 +132,19 @@ def attention_bf16_supported(q, k_cache, head_dim: int) -> bool:
             and k_cache.data_ptr() % 16 == 0)
 
 
-def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_len: int | None = None) -> dict:
+def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_len: int | None = None,
+                   tuning: int = 0) -> dict:
     """Launch sizes for a step, from how its batch is cut (host-side numbers only). plan_len:
     plan the decode splits for requests of up to this many tokens, whatever their length now
-    (a recorded step is replayed while the requests grow)."""
-    rows = entry("llme_attention_bf16_rows")(head_dim, n_q, n_kv)
+    (a recorded step is replayed while the requests grow). tuning: see attention_tuning."""
+    rows = entry("llme_attention_bf16_rows")(head_dim, n_q, n_kv, tuning)
+    if rows <= 0:
+        raise kernels.KernelError(f"plan_attention: tuning {tuning} is not one that attention_tuning makes")
     decode = [c + 1 for n, c in zip(new_lens, ctx_lens) if n == 1]
     groups = sum((n + rows - 1) // rows for n in new_lens if n >= 2)
     plan = {"n_decode": len(decode), "groups": groups, "split_len": 32, "nsplit": 1, "prefill_splits": 1,
-            "prefill_run": 1}
-    if groups and entry("llme_attention_bf16_splits_prefill")(head_dim, n_q, n_kv):
+            "prefill_run": 1, "tuning": tuning}
+    if groups and entry("llme_attention_bf16_splits_prefill")(head_dim, n_q, n_kv, tuning):
         # few rows over long contexts: too few work items for the chip, each with many keys
         group = n_q // n_kv
         items = groups * (n_q // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
@@ -190,7 +203,8 @@ def attention_bf16(q, k_cache, v_cache, out, q_start, ctx_len, block_table, n_q:
         ptr(block_table), block_table.shape[1], S, n_q, n_kv, head_dim, page, float(scale), int(window),
         plan["n_decode"], plan["split_len"], plan["nsplit"], plan["groups"],
         ptr(work_queue(q.device)) if plan["groups"] else None, T, pre_splits, max(1, int(plan.get("prefill_run", 1))),
-        ptr(pre_part_o) if pre_splits > 1 else None, ptr(pre_part_ml) if pre_splits > 1 else None, stream()),
+        ptr(pre_part_o) if pre_splits > 1 else None, ptr(pre_part_ml) if pre_splits > 1 else None,
+        int(plan.get("tuning", 0)), stream()),
         "attention_bf16")
 
 

@@ -128,7 +128,7 @@ _SIGNATURES = {
     "llme_cm_commit": (_i, [_vp, _i64, _l]), "llme_cm_release": (_i, [_vp, _i64]),
     "llme_cm_table_len": (_i, [_vp, _i64, _i]), "llme_cm_table_copy": (_i, [_vp, _i64, _i, _i, _i, _pi]),
     "llme_cm_free_pages": (_i, [_vp, _i]), "llme_cm_num_pages": (_i, [_vp, _i]), "llme_cm_check": (_i, [_vp]),
-    "llme_cm_decode_begin": (_i, [_vp, _i, _pi64, _pi]), "llme_cm_commit_batch": (_i, [_vp, _i, _pi64, _l]),
+    "llme_cm_decode_begin": (_i, [_vp, _i, _pi64, _pi, _l]), "llme_cm_commit_batch": (_i, [_vp, _i, _pi64, _l]),
     "llme_cm_fill_decode": (_i, [_vp, _i, _pi64, _i, _vp, _vp, _vp, _pi, _pi64]),
     "llme_sched_create": (_vp, [_vp, _i, _l]), "llme_sched_destroy": (None, [_vp]),
     "llme_sched_set_budget": (_i, [_vp, _l]), "llme_sched_enqueue": (_l, [_vp, _pi, _l, _l]),
@@ -136,7 +136,7 @@ _SIGNATURES = {
     "llme_sched_plan": (_i, [_vp, _pi, _pi, _pi64, _pi, _pi, _pl, _pi, _l]),
     "llme_sched_complete": (_i, [_vp, _pi, _i, _pi, _i]), "llme_sched_num_results": (_i, [_vp]),
     "llme_sched_result_info": (_i, [_vp, _i, _pi64, _pl, _pl, _pi]), "llme_sched_result_tokens": (_i, [_vp, _i, _pi]),
-    "llme_sched_clear_results": (None, [_vp]),
+    "llme_sched_clear_results": (None, [_vp]), "llme_sched_abort": (None, [_vp]),
     # plain C++ twins of the device kernels (csrc/host/plain_kernels.cpp), for tests
     "llme_plain_embed": (_i, [_vp, _vp, _i, _i, _i, _vp]),
     "llme_plain_rmsnorm": (_i, [_vp, _vp, _i, _i, _f, _vp]),

@@ -218,3 +218,25 @@ def test_native_manager_agrees_with_the_plain_one(seed):
             assert (a.slot(rid), a.length(rid)) == (b.slot(rid), b.length(rid))
             for g in a.groups:
                 assert a.block_table(rid, g) == b.block_table(rid, g)
+
+
+def test_decode_begin_checks_the_position_limit_before_it_reserves():
+    """The decode step's one call for lengths, limit and pages: a request that would pass the
+    position limit stops the call before any page is reserved for any request of the batch."""
+    import ctypes
+    m = CacheManager([GroupSpec("full", "full", 0, 8)], 4, 3)
+    for rid, n in ((0, 4), (1, 8), (2, 3)):             # requests 0 and 1 need a new page for their next token
+        m.admit(rid)
+        assert m.reserve(rid, n)
+        m.commit(rid, n)
+    free = m.free_pages()
+    keys = (ctypes.c_int64 * 3)(*[m.key_of(r) for r in (0, 1, 2)])
+    lengths = (ctypes.c_int * 3)()
+    assert m._lib.llme_cm_decode_begin(m.handle, 3, keys, lengths, 8) == 2       # request 1 would be 9 long
+    assert list(lengths) == [4, 8, 3] and m.free_pages() == free
+    m.check()
+    assert m._lib.llme_cm_decode_begin(m.handle, 3, keys, lengths, 9) == 1
+    assert m.free_pages() == free - 2
+    assert m._lib.llme_cm_commit_batch(m.handle, 3, keys, 1) == 0
+    m.check()
+    assert m._lib.llme_cm_decode_begin(m.handle, 3, keys, lengths, 0) == 1       # 0: no limit

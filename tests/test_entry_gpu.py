@@ -218,6 +218,14 @@ def test_greedy_step_with_the_argmax_in_the_recording(dir_b):
             for c in caches:
                 c.release("y")
             del last["y"]
+        if turn == 7:
+            # a large argmax elsewhere replaces the scratch that plain calls share, and new tensors
+            # take the freed memory: the recordings keep a scratch of their own and must not notice
+            from llmengine import ops
+            big = torch.randn(72, 128256, device="cuda:0")
+            ops.argmax(big, torch.empty(72, dtype=torch.int32, device="cuda:0"))
+            torch.cuda.synchronize()
+            filler = [torch.full((4096,), float("nan"), device="cuda:0") for _ in range(64)]
     assert engine.runner.graph_replays >= 10
     with pytest.raises(CapacityError):                       # 12 pages of 8: the three requests outgrow them
         for _ in range(40):
@@ -227,6 +235,18 @@ def test_greedy_step_with_the_argmax_in_the_recording(dir_b):
     with pytest.raises(CapacityError):
         engine.run_step(caches[0], [StepEntry(r, [last[r]], [0]) for r in last], None)
     assert before == {r: caches[0].manager.length(r) for r in last}      # a refused step changes nothing
+    # .. and so does one that would pass the position limit (256 here): nothing is reserved for anyone
+    roomy = engine.new_cache(40, 8, 2)
+    for rid, n in (("p", 255), ("q", 40)):
+        roomy.admit(rid)
+        engine.step(roomy, [StepEntry(rid, random_tokens(n, 384, n), [])])
+    free = roomy.manager.free_pages("full")
+    engine.run_step(roomy, [StepEntry("p", [1], [0]), StepEntry("q", [2], [0])], None)       # p is 256 long now
+    assert roomy.manager.free_pages("full") == free - 1                  # (q began a page)
+    with pytest.raises(ValueError, match="position limit"):
+        engine.run_step(roomy, [StepEntry("p", [1], [0]), StepEntry("q", [2], [0])], None)
+    assert roomy.manager.free_pages("full") == free - 1 and roomy.manager.length("q") == 41
+    roomy.manager.check()
 
 
 def test_scheduler_capacity_on_the_gpu(dir_a):

@@ -308,7 +308,7 @@ def test_gemm_dispatch_and_refusals(ops):
 
 
 # --- MFMA attention ----------------------------------------------------------------------
-def _attn_case(ops, lens, news, n_q, n_kv, hd, page, window=0, seed=50, prefill_splits=None, prefill_run=1):
+def _attn_case(ops, lens, news, n_q, n_kv, hd, page, window=0, seed=50, prefill_splits=None, prefill_run=1, tuning=0):
     """Requests with lens[i] tokens in the cache, of which the last news[i] are this step's.
     prefill_splits, prefill_run: cut the keys of the prompt portions into at most that many runs of that
     many 64-key stretches, whatever the plan says."""
@@ -323,7 +323,7 @@ def _attn_case(ops, lens, news, n_q, n_kv, hd, page, window=0, seed=50, prefill_
     q = s["q"][torch.tensor(rows, device=DEV)].contiguous()
     out = torch.zeros_like(q)
     i32 = dict(dtype=torch.int32, device=DEV)
-    plan = ops.mfma.plan_attention(news, ctx, n_q, n_kv, hd)
+    plan = ops.mfma.plan_attention(news, ctx, n_q, n_kv, hd, tuning=tuning)
     S = len(lens)
     part_o = torch.empty(S * n_q * plan["nsplit"] * hd, device=DEV)
     part_ml = torch.empty(S * n_q * plan["nsplit"] * 2, device=DEV)
@@ -376,16 +376,12 @@ def test_attention_prefill_shared_and_direct(ops, n_q, n_kv, hd, page, rows, sha
     """The prefill kernel that shares K and V through LDS, for 4, 2 and 1 heads of a kv head per
     workgroup, spans that end inside a 64-key stretch, portions that start deep in a context,
     and the kernel without LDS at the same sizes."""
-    set_rows = ops.lib.entry("llme_attention_bf16_set_rows")
-    assert set_rows(rows, shared) == 0
-    try:
-        lens = [330, 2, 131, 64, 517, 65, 9]
-        news = [330, 2, 67, 64, 130, 3, 1]
-        out, ref, plan = _attn_case(ops, lens, news, n_q, n_kv, hd, page, seed=61)
-        assert plan["n_decode"] == 1 and plan["groups"] >= 6
-        assert _rel(out, ref) < 8e-3
-    finally:
-        set_rows(0, -1)
+    lens = [330, 2, 131, 64, 517, 65, 9]
+    news = [330, 2, 67, 64, 130, 3, 1]
+    out, ref, plan = _attn_case(ops, lens, news, n_q, n_kv, hd, page, seed=61,
+                                tuning=ops.mfma.attention_tuning(rows=rows, shared=shared))
+    assert plan["n_decode"] == 1 and plan["groups"] >= 6
+    assert _rel(out, ref) < 8e-3
 
 
 @pytest.mark.parametrize("window", [1, 7, 64, 65, 200])
@@ -405,17 +401,13 @@ def test_attention_prefill_cut_keys(ops, n_q, n_kv, hd, page, splits, key_waves,
     inside a span's own rows, a last run that takes the rest, items with a single run beside items
     with several (and all of them single), whole prompts and decoded tokens beside them, with one
     and two wavefronts per tile."""
-    set_rows = ops.lib.entry("llme_attention_bf16_set_rows")
-    assert set_rows(0, key_waves) == 0
-    try:
-        lens = [700, 2, 131, 64, 517, 65, 9]
-        news = [40, 2, 67, 64, 130, 3, 1]
-        out, ref, plan = _attn_case(ops, lens, news, n_q, n_kv, hd, page, seed=63, prefill_splits=splits, prefill_run=run)
-        assert plan["n_decode"] == 1 and plan["prefill_splits"] == splits
-        assert not out.isnan().any()
-        assert _rel(out, ref) < 8e-3
-    finally:
-        set_rows(0, -1)
+    lens = [700, 2, 131, 64, 517, 65, 9]
+    news = [40, 2, 67, 64, 130, 3, 1]
+    out, ref, plan = _attn_case(ops, lens, news, n_q, n_kv, hd, page, seed=63, prefill_splits=splits, prefill_run=run,
+                                tuning=ops.mfma.attention_tuning(shared=key_waves))
+    assert plan["n_decode"] == 1 and plan["prefill_splits"] == splits
+    assert not out.isnan().any()
+    assert _rel(out, ref) < 8e-3
 
 
 @pytest.mark.parametrize("window", [1, 64, 65, 200])

@@ -182,3 +182,55 @@ def test_invalid_knobs_and_requests():
     assert len(s.results[0].token_ids) == 16
     s.clear_results()
     assert s.results == []
+
+
+def test_a_failing_step_changes_nothing():
+    """The model run raises once, in a step that carries prompt portions and decoded tokens: the
+    scheduler forgets the batch, the prompts stay where they were, and the streams that come out
+    afterwards are those of an undisturbed run (a prompt that had moved on would skip tokens)."""
+    prompts = [[1, 2, 3], list(range(20, 50)), list(range(5, 25)), [9]]
+
+    class Failing(FakeEngine):
+        def __init__(self, fail_at):
+            super().__init__()
+            self.fail_at, self.calls = fail_at, 0
+
+        def run_step(self, cache, entries, draws, temperature, seed):
+            self.calls += 1
+            if self.calls == self.fail_at:
+                raise RuntimeError("the step failed")
+            return super().run_step(cache, entries, draws, temperature, seed)
+
+    for fail_at in (1, 2, 3, 5):
+        eng, bm = Failing(fail_at), FakeBlocks(64, 4)
+        s = ContinuousBatchScheduler(eng, bm, max_concurrent=3, max_prefill_tokens_per_step=8)
+        for p in prompts:
+            s.enqueue(p, 7)
+        failures = 0
+        while True:
+            try:
+                if not s.step():
+                    break
+            except RuntimeError as e:
+                assert "the step failed" in str(e)
+                failures += 1
+        assert failures == 1
+        for r, p in zip(s.results, prompts):
+            assert (r.token_ids, r.finish_reason) == single_generate(p, 7), (fail_at, r.seq_id)
+        assert bm.free_blocks == bm.num_blocks and s.idle
+        bm.cache.manager.check()
+
+
+def test_one_scheduler_per_block_manager():
+    eng, bm = FakeEngine(), FakeBlocks(64, 4)
+    first = ContinuousBatchScheduler(eng, bm, max_concurrent=2)
+    first.enqueue([1, 2, 3], 4)
+    first.step()
+    with pytest.raises(ValueError, match="BlockManager of its own"):
+        ContinuousBatchScheduler(eng, bm, max_concurrent=4)
+    first.run_until_idle()
+    eng.history.clear()                                               # (the stand-in keys its histories by sequence id)
+    second = ContinuousBatchScheduler(eng, bm, max_concurrent=4)      # the first is idle: the manager is free again
+    second.enqueue([4, 5], 3)
+    second.run_until_idle()
+    assert second.results[0].token_ids[:2] == [4, 5]

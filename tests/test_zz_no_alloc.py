@@ -30,7 +30,7 @@ def lib():
                                                   _i, _i, _vp]
     lib.llme_attention_decode_noalloc.restype = _i
     lib.llme_attention_bf16.argtypes = [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i,
-                                        _i, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp, _vp]
+                                        _i, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp, _i, _vp]
     lib.llme_attention_bf16.restype = _i
     return lib
 
@@ -65,7 +65,7 @@ def _run_both(lib, lens, n_q, n_kv, hd, page, split_len, nsplit, seed):
     rc = lib.llme_attention_bf16(q.data_ptr(), s["k_cache"].data_ptr(), s["v_cache"].data_ptr(), out_ws.data_ptr(),
                                  part_o.data_ptr(), part_ml.data_ptr(), q_start.data_ptr(), ctx_len.data_ptr(),
                                  table.data_ptr(), table.shape[1], S, n_q, n_kv, hd, page, scale, 0, S, split_len,
-                                 nsplit, 0, None, S, 1, 1, None, None, stream)
+                                 nsplit, 0, None, S, 1, 1, None, None, 0, stream)
     assert rc == 0
     out_na = torch.zeros_like(q)
     torch.cuda.synchronize()
