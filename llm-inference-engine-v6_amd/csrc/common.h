@@ -59,6 +59,20 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Compute units of the current device, asked once per process: launch heuristics are sized by
+// it (how many workgroups fill the chip once, when a sum is worth cutting over k). 256 on the
+// MI355X that the measurements quoted beside those heuristics were taken on.
+inline int compute_units() {
+    static int cached = 0;
+    if (cached > 0) return cached;
+    int device = 0, cus = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || cus <= 0)
+        cus = 256;
+    cached = cus;
+    return cus;
+}
+
 // Every entry point returns hipGetLastError() after its launches: 0 on success.
 inline int launch_status() { return static_cast<int>(hipGetLastError()); }
 

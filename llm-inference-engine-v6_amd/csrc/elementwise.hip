@@ -434,6 +434,8 @@ extern "C" int llme_embed_gather(const void* table, int table_dtype, const int* 
     return launch_status();
 }
 
+extern "C" int llme_compute_units(void) { return compute_units(); }
+
 extern "C" int llme_rmsnorm(const float* x, const void* w, int w_dtype, void* out, int out_dtype,
                             const int* rows, int R, int H, float eps, hipStream_t stream) {
     if (R <= 0) return 0;

@@ -541,16 +541,17 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     // (measured at 64 rows: 3,072 columns 12.7 us skinny against 13.8 with tiles, 5,120 columns 31.9
     // against 20.7, 6,144 columns of k = 4,096 40.5 against 27.2)
     const bool skinny = M <= 16 || (M <= 64 && !accumulate && N < 4096);
+    const int cus = compute_units();
     if (skinny && tile_shape <= 0 && !gated) {
         const int tiles = (N + 15) / 16;
-        if (nw <= 0 && ksplit <= 0 && accumulate && out_dtype == kF32 && tiles < 512) {
+        if (nw <= 0 && ksplit <= 0 && accumulate && out_dtype == kF32 && tiles < 2 * cus) {
             // Few output columns and a sum to join anyway (the residual stream): cut k over
             // several workgroups that add their parts with atomics, so that the whole chip
             // streams the matrix. (The order of these additions is not fixed.)
             // (measured at 128 tiles: k = 2,048: 512 workgroups of 4 wavefronts 4.0 us, 256 of 8 4.1 us;
             // k = 8,192: 8.9 against 8.3 us)
-            const bool long_k = K >= 4096 && tiles <= 256;
-            ksplit = (long_k ? 256 : 512) / tiles;
+            const bool long_k = K >= 4096 && tiles <= cus;
+            ksplit = (long_k ? cus : 2 * cus) / tiles;
             if (ksplit > K / 512) ksplit = K / 512;
             if (ksplit < 1) ksplit = 1;
             nw = long_k ? 8 : 4;
@@ -582,9 +583,9 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     if (tile_shape <= 0) {
         const long wg128 = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
         tile_shape = (M > 64 && wg128 >= 64) ? 128 : 64;
-        if (tile_shape == 128 && wg128 < 1024 && !(mode == kAddF32 && wg128 <= 256 && K >= 4096)) {
-            // Medium outputs: narrower tiles can fill the 256 compute units (two workgroups
-            // each) more evenly. Estimated time: rounds of 256 workgroups x tile area / measured
+        if (tile_shape == 128 && wg128 < 4 * cus && !(mode == kAddF32 && wg128 <= cus && K >= 4096)) {
+            // Medium outputs: narrower tiles can fill the compute units (two workgroups
+            // each) more evenly. Estimated time: rounds of one workgroup per compute unit x tile area / measured
             // efficiency of the shape; a workgroup alone on its compute unit overlaps nothing.
             const long tm = (M + 127) / 128;
             const int shapes[3] = {128, 128096, 128064};
@@ -593,11 +594,11 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
             float best = 0.f;
             for (int c = 0; c < 3; ++c) {
                 const long wgs = tm * ((N + widths[c] - 1) / widths[c]);
-                const long rounds = (wgs + 255) / 256;
+                const long rounds = (wgs + cus - 1) / cus;
                 float cost = static_cast<float>(rounds) * 128.f * widths[c] / eff[c];
                 // (less so for the gated product, whose epilogue is long: measured at 129 to 256 rows,
                 // 128 x 128 tiles 26.5 against 31 us at the 1B sizes, 36.6 against 43.7 at the 3B sizes)
-                if (wgs <= 256) cost *= (mode == kGatedBF16 ? 1.1f : 1.25f);
+                if (wgs <= cus) cost *= (mode == kGatedBF16 ? 1.1f : 1.25f);
                 if (c == 0 || cost < best) {
                     best = cost;
                     tile_shape = shapes[c];
@@ -612,8 +613,8 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
             const int bm = tile_shape == 64 ? 64 : 128;
             const int bn = tile_shape == 64 ? 64 : tile_shape == 128 ? 128 : tile_shape == 128096 ? 96 : 64;
             const long wgs = static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-            long ks = (tile_shape == 64 ? 512 : 256) / wgs;
-            if (tile_shape == 128 && wg128 <= 256 && K >= 4096 && ks < 2) ks = 2;
+            long ks = (tile_shape == 64 ? 2 * cus : cus) / wgs;
+            if (tile_shape == 128 && wg128 <= cus && K >= 4096 && ks < 2) ks = 2;
             if (ks > K / 512) ks = K / 512;
             if (ks > 8) ks = 8;
             ksplit = ks < 1 ? 1 : static_cast<int>(ks);

@@ -448,16 +448,16 @@ extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_
     if (tpr <= 0) {
         // few tiles: all 8 wavefronts on one tile, so that every tile has a workgroup of its own;
         // more tiles than compute units: 2 tiles at a time, 4 wavefronts each with several chunks of k
-        tpr = tiles <= 256 ? 1 : 2;
+        tpr = tiles <= compute_units() ? 1 : 2;
         // (measured: 16 wavefronts on 2 tiles, 14.2 against 14.8 us at 512 tiles; they need more LDS for their sums)
         const size_t lds16 = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(16) * 2 * 64 * 16 + 64;
-        if (gated && tiles > 256 && tiles <= 1024 && lds16 <= 160 * 1024) tpr = 12;
+        if (gated && tiles > compute_units() && tiles <= 4 * compute_units() && lds16 <= 160 * 1024) tpr = 12;
     }
     if (tpr != 1 && tpr != 2 && tpr != 4 && tpr != 12 && tpr != 14) return kErrBadArgument;
     if (grid <= 0) {
         const int at_a_time = tpr > 10 ? tpr - 10 : tpr;
         grid = (tiles + at_a_time - 1) / at_a_time;
-        if (grid > 512) grid = 512;                     // two workgroups per compute unit
+        if (grid > 2 * compute_units()) grid = 2 * compute_units();    // two workgroups per compute unit
     }
     const bf16* W = static_cast<const bf16*>(w);
     if (norm_dtype == kBF16) {
@@ -494,8 +494,8 @@ extern "C" int llme_gemv_norm_rope(const float* h, const void* norm_w, int norm_
     const int N = (n_q + 2 * n_kv) * hd;
     if (static_cast<double>(N) * K * 2 >= 4294967296.0) return kErrUnsupported;   // 32-bit offsets into w
     const int tiles = N / 16;
-    const int tpr = tiles <= 256 ? 1 : 2;              // as the plain form
-    if (grid <= 0) grid = (tiles + tpr - 1) / tpr > 512 ? 512 : (tiles + tpr - 1) / tpr;
+    const int tpr = tiles <= compute_units() ? 1 : 2;  // as the plain form
+    if (grid <= 0) grid = (tiles + tpr - 1) / tpr > 2 * compute_units() ? 2 * compute_units() : (tiles + tpr - 1) / tpr;
     const RopeTarget rope{positions, seq_idx, block_table, max_blocks, cos_t, sin_t, static_cast<bf16*>(q_out),
                           static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache), n_q, n_kv, hd, page};
     const bf16* W = static_cast<const bf16*>(w);

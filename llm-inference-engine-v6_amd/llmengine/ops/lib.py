@@ -41,6 +41,7 @@ _SIGNATURES = {
                                _f, _i, _vp],
     "llme_argmax": [_vp, _vp, _vp, _vp, _i, _i, _vp],
     "llme_argmax_parts": [_i],
+    "llme_compute_units": [],
     "llme_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
 }
 

@@ -108,17 +108,28 @@ def work_queue(device: torch.device) -> torch.Tensor:
 
 
 # Workgroups (of four wavefronts) the decode kernel should have at most when it cuts the keys: one
-# per compute unit. Measured at batch 8 and a context of 4,096: 0.948 ms a step with 256, 0.969
-# with 512, 0.998 with 1,024, 1.036 with 128; with 384 (one and a half per compute unit) 1.000.
-DECODE_BLOCKS_WANTED = 256
+# per compute unit (None: the device is asked for their number). Measured on the 256 compute units
+# of an MI355X at batch 8 and a context of 4,096: 0.948 ms a step with 256, 0.969 with 512, 0.998
+# with 1,024, 1.036 with 128; with 384 (one and a half per compute unit) 1.000.
+DECODE_BLOCKS_WANTED: int | None = None
+_compute_units = 0
+
+
+def compute_units() -> int:
+    """Compute units of the current device (asked once)."""
+    global _compute_units
+    if _compute_units <= 0:
+        _compute_units = max(1, int(entry("llme_compute_units")()))
+    return _compute_units
+
 MIN_SPLIT = 128                     # keys per split at least: one 32-key block per wavefront
 MAX_SPLITS = 64                     # the join kernel's limit
 # Portions of prompts: work items (a span of rows x a group of heads) the prefill kernel should
 # have at least; with PREFILL_CUT_ITEMS or fewer (half a workgroup per compute unit; measured: 256
 # items cut in two were 3 % slower than whole), the longest item's keys are cut into that many
 # runs of at least PREFILL_MIN_RUN keys, and the others' into runs of the same length.
-PREFILL_ITEMS_WANTED = 512
-PREFILL_CUT_ITEMS = 128
+PREFILL_ITEMS_WANTED: int | None = None        # None: two per compute unit
+PREFILL_CUT_ITEMS: int | None = None           # None: half a workgroup per compute unit
 PREFILL_MIN_RUN = 512
 PREFILL_MAX_SPLITS = 16
 # (A whole prompt of 2,048 tokens, whose last rows' items walk twice the average, was also tried with
@@ -150,8 +161,9 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
         items = groups * (n_q // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
         keys = max(c + n for n, c in zip(new_lens, ctx_lens) if n >= 2)
         splits = 1
-        if items <= PREFILL_CUT_ITEMS:
-            splits = max(1, min(PREFILL_ITEMS_WANTED // items, keys // PREFILL_MIN_RUN, PREFILL_MAX_SPLITS))
+        if items <= (PREFILL_CUT_ITEMS or compute_units() // 2):
+            splits = max(1, min((PREFILL_ITEMS_WANTED or 2 * compute_units()) // items, keys // PREFILL_MIN_RUN,
+                                PREFILL_MAX_SPLITS))
             stretches = (keys + 63) // 64
             run = (stretches + splits - 1) // splits       # stretches of 64 keys per run
         if splits > 1:
@@ -159,7 +171,7 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
     if decode:
         longest = max(decode) if plan_len is None else max(plan_len, max(decode))
         pairs = len(decode) * n_kv * ((n_q // n_kv + 15) // 16)
-        nsplit = max(1, min(DECODE_BLOCKS_WANTED // pairs, (longest + MIN_SPLIT - 1) // MIN_SPLIT, MAX_SPLITS))
+        nsplit = max(1, min((DECODE_BLOCKS_WANTED or compute_units()) // pairs, (longest + MIN_SPLIT - 1) // MIN_SPLIT, MAX_SPLITS))
         split_len = ((longest + nsplit - 1) // nsplit + 31) // 32 * 32
         plan["split_len"] = split_len
         plan["nsplit"] = (longest + split_len - 1) // split_len

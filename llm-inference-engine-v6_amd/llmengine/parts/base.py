@@ -80,8 +80,12 @@ Getter = Callable[[str], torch.Tensor]      # local tensor name -> CPU tensor as
 class Part:
     # True if forward() issues the same launches, with the same arguments, for every step of
     # the same shape, reading what changes (tokens, positions, tables, slots) from the step's
-    # device arrays only. Steps of such parts can be recorded once and replayed as a HIP graph;
-    # a part that looks at the step's host-side lists while it runs must leave this False.
+    # device arrays only, and if running a step twice on the same inputs leaves the same cache
+    # and state as running it once (a step that is recorded runs plainly first, to size the scratch
+    # buffers, and once more while it is recorded: attention rewrites the same keys at the same
+    # places, a part that adds into its state would count the token twice). Steps of such parts
+    # can be recorded once and replayed as a HIP graph; a part that looks at the step's host-side
+    # lists while it runs, or whose step is not repeatable, must leave this False.
     graph_safe = False
 
     def param_specs(self) -> dict[str, ParamSpec]:

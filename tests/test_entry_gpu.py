@@ -188,7 +188,16 @@ def test_scheduler_greedy_equals_generate(dir_a, dtype):
     if dtype == "fp32":
         assert [(r.token_ids, r.finish_reason) for r in sched.results] == alone
     else:
-        assert sum(r.token_ids == a[0] for r, a in zip(sched.results, alone)) >= len(prompts) - 1
+        # In bfloat16 a near-tie may fall the other way in a batch than alone (other kernels add in
+        # another order), after which the streams differ: every token of every stream must be a
+        # maximum of the plain logits of its own history, up to the bfloat16 tolerance.
+        cfg, w = load_plain_model(dir_a)
+        for r, p in zip(sched.results, prompts):
+            assert r.token_ids[:len(p)] == p and len(r.token_ids) == len(p) + 12 and r.finish_reason == "length"
+            ref = plain_forward(cfg, w, r.token_ids, rounder=bf16_round)
+            for i in range(len(p), len(r.token_ids)):
+                row = ref[i - 1]
+                assert row[r.token_ids[i]] >= row.max() - 2e-2 * row.abs().max(), (r.seq_id, i)
     assert blocks.free_blocks == 64 and [r.seq_id for r in sched.results] == list(range(len(prompts)))
 
 
