@@ -76,6 +76,126 @@ __device__ __forceinline__ void deal_between_products() {
     }
 }
 
+// The end of a tile kernel: the wavefronts' accumulators go to `out` in the kernel's mode. The
+// result tile (i, j) of a lane is column wn + 16 j + r, rows wm + 16 i + 4 q + e: written straight
+// from there, a store instruction touches 4 rows with 64 bytes each. Where the tile fits into the
+// LDS that the operand slabs no longer need (LDS_BYTES of it; the caller has passed a barrier), it
+// goes through LDS instead, so that every thread stores 16 contiguous bytes of a row.
+template <int WMT, int WNT, int MODE, int LDS_BYTES, int WR = 2, int WC = 2>
+__device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned char* lds_raw, void* __restrict__ out,
+                                              int M, int N, int m0, int n0, int wm, int wn, int tid, int r, int q) {
+    constexpr int BM = WR * 16 * WMT, BN = WC * 16 * WNT, NT = 64 * WR * WC;
+
+    constexpr int SS = BN + 4;                           // floats per staged row
+    // A tile that is larger than the LDS goes through it in 2 or 4 passes of whole wavefront rows.
+    constexpr int WAVE_ROWS = 16 * WMT;
+    constexpr auto fits = [](int passes) {
+        return (BM / passes) % WAVE_ROWS == 0 && static_cast<size_t>(BM / passes) * SS * 4 <= static_cast<size_t>(LDS_BYTES);
+    };
+    constexpr int PASSES = fits(1) ? 1 : (WR % 2 == 0 && fits(2)) ? 2 : (WR % 4 == 0 && fits(4)) ? 4 : 0;
+    // (Atomic adds are faster scattered than packed into the same cache lines: they stay direct.)
+    constexpr bool STAGED = MODE != kAtomicF32 && PASSES > 0;
+    if (STAGED && N % 8 == 0) {
+        constexpr int HB = PASSES > 0 ? BM / (PASSES > 0 ? PASSES : 1) : BM;     // rows of a pass
+        float* stage = reinterpret_cast<float*>(lds_raw);
+#pragma unroll
+        for (int pass = 0; pass < PASSES; ++pass) {
+        if (pass > 0) __syncthreads();                  // the pass before has been stored
+        if (wm / HB == pass) {
+#pragma unroll
+            for (int i = 0; i < WMT; ++i)
+#pragma unroll
+                for (int j = 0; j < WNT; ++j)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        stage[(wm - pass * HB + i * 16 + q * 4 + e) * SS + wn + j * 16 + r] = acc[i][j][e];
+        }
+        __syncthreads();
+        const int mp = m0 + pass * HB;                  // the pass's first row
+        if (MODE == kGatedBF16) {
+            // a thread makes 8 units: their gates and ups lie 16 columns apart in a group of 32
+            constexpr int PER_ROW = BN / 16;             // 8-unit pieces per row
+            for (int idx = tid; idx < HB * PER_ROW; idx += NT) {
+                const int row = idx / PER_ROW, piece = idx % PER_ROW;
+                const int col = (piece / 2) * 32 + (piece % 2) * 8;
+                const int m = mp + row, n = n0 + col;
+                if (m >= M || n >= N) continue;
+                const float* gp = stage + row * SS + col;
+                bf16x8 o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float gt = gp[e], up = gp[16 + e];
+                    o[e] = static_cast<__bf16>((gt / (1.0f + expf(-gt))) * up);
+                }
+                const int unit = (n0 + (piece / 2) * 32) / 2 + (piece % 2) * 8;
+                *reinterpret_cast<bf16x8*>(static_cast<bf16*>(out) + static_cast<size_t>(m) * (N / 2) + unit) = o;
+            }
+        } else if (MODE == kStoreBF16) {
+            constexpr int PER_ROW = BN / 8;
+            for (int idx = tid; idx < HB * PER_ROW; idx += NT) {
+                const int row = idx / PER_ROW, col = (idx % PER_ROW) * 8;
+                const int m = mp + row, n = n0 + col;
+                if (m >= M || n >= N) continue;
+                const float* sp = stage + row * SS + col;
+                bf16x8 o;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[e] = static_cast<__bf16>(sp[e]);
+                *reinterpret_cast<bf16x8*>(static_cast<bf16*>(out) + static_cast<size_t>(m) * N + n) = o;
+            }
+        } else {
+            constexpr int PER_ROW = BN / 4;
+            for (int idx = tid; idx < HB * PER_ROW; idx += NT) {
+                const int row = idx / PER_ROW, col = (idx % PER_ROW) * 4;
+                const int m = mp + row, n = n0 + col;
+                if (m >= M || n >= N) continue;
+                const float4 v = *reinterpret_cast<const float4*>(stage + row * SS + col);
+                float* op = static_cast<float*>(out) + static_cast<size_t>(m) * N + n;
+                if (MODE == kStoreF32) {
+                    *reinterpret_cast<float4*>(op) = v;
+                } else if (MODE == kAddF32) {
+                    float4 cur = *reinterpret_cast<const float4*>(op);
+                    cur.x += v.x; cur.y += v.y; cur.z += v.z; cur.w += v.w;
+                    *reinterpret_cast<float4*>(op) = cur;
+                } else {
+                    atomicAdd(op, v.x); atomicAdd(op + 1, v.y); atomicAdd(op + 2, v.z); atomicAdd(op + 3, v.w);
+                }
+            }
+        }
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < WMT; ++i) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int m = m0 + wm + i * 16 + q * 4 + e;
+            if (m >= M) continue;
+            if (MODE == kGatedBF16) {
+#pragma unroll
+                for (int j = 0; j + 1 < WNT; j += 2) {
+                    const int unit = (n0 + wn + j * 16) / 2 + r;        // tile column pair (gate, up)
+                    if (2 * unit >= N) continue;
+                    const float gt = acc[i][j][e], up = acc[i][j + 1][e];
+                    static_cast<bf16*>(out)[static_cast<size_t>(m) * (N / 2) + unit] =
+                        static_cast<bf16>((gt / (1.0f + expf(-gt))) * up);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < WNT; ++j) {
+                    const int n = n0 + wn + j * 16 + r;
+                    if (n >= N) continue;
+                    const size_t idx = static_cast<size_t>(m) * N + n;
+                    const float v = acc[i][j][e];
+                    if (MODE == kStoreF32) static_cast<float*>(out)[idx] = v;
+                    else if (MODE == kAddF32) static_cast<float*>(out)[idx] += v;
+                    else if (MODE == kAtomicF32) atomicAdd(static_cast<float*>(out) + idx, v);
+                    else static_cast<bf16*>(out)[idx] = static_cast<bf16>(v);
+                }
+            }
+        }
+    }
+}
+
 // kGatedBF16: w holds gate and up rows interleaved in groups of 16, so that even MFMA tile
 // columns are gates and odd ones the ups of the same 16 units; out [M, N / 2] bfloat16 gets
 // silu(gate) * up (src/engine.cpp:213-216).
@@ -260,109 +380,202 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
         if ((kt_end - kt_begin) & 1) turn(kt, 0, s1);
     }
     __syncthreads();                                  // the epilogue reuses the slabs' LDS
-
-    // Epilogue. The result tile (i, j) of a lane is column wn + 16 j + r, rows wm + 16 i + 4 q + e:
-    // written straight from there, a store instruction touches 4 rows with 64 bytes each. Where
-    // the tile fits into the LDS that the operand slabs no longer need, it goes through LDS
-    // instead, so that every thread stores 16 contiguous bytes of a row.
-    constexpr int SS = BN + 4;                           // floats per staged row
-    // (Atomic adds are faster scattered than packed into the same cache lines: they stay direct.)
-    constexpr bool STAGED = MODE != kAtomicF32 &&
-                            static_cast<size_t>(BM) * SS * 4 <= static_cast<size_t>(tile_lds_bytes<WMT, WNT>());
-    if (STAGED && N % 8 == 0) {
-        float* stage = reinterpret_cast<float*>(lds_raw);
-#pragma unroll
-        for (int i = 0; i < WMT; ++i)
-#pragma unroll
-            for (int j = 0; j < WNT; ++j)
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    stage[(wm + i * 16 + q * 4 + e) * SS + wn + j * 16 + r] = acc[i][j][e];
-        __syncthreads();
-        if (MODE == kGatedBF16) {
-            // a thread makes 8 units: their gates and ups lie 16 columns apart in a group of 32
-            constexpr int PER_ROW = BN / 16;             // 8-unit pieces per row
-            for (int idx = tid; idx < BM * PER_ROW; idx += 256) {
-                const int row = idx / PER_ROW, piece = idx % PER_ROW;
-                const int col = (piece / 2) * 32 + (piece % 2) * 8;
-                const int m = m0 + row, n = n0 + col;
-                if (m >= M || n >= N) continue;
-                const float* gp = stage + row * SS + col;
-                bf16x8 o;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float gt = gp[e], up = gp[16 + e];
-                    o[e] = static_cast<__bf16>((gt / (1.0f + expf(-gt))) * up);
-                }
-                const int unit = (n0 + (piece / 2) * 32) / 2 + (piece % 2) * 8;
-                *reinterpret_cast<bf16x8*>(static_cast<bf16*>(out) + static_cast<size_t>(m) * (N / 2) + unit) = o;
-            }
-        } else if (MODE == kStoreBF16) {
-            constexpr int PER_ROW = BN / 8;
-            for (int idx = tid; idx < BM * PER_ROW; idx += 256) {
-                const int row = idx / PER_ROW, col = (idx % PER_ROW) * 8;
-                const int m = m0 + row, n = n0 + col;
-                if (m >= M || n >= N) continue;
-                const float* sp = stage + row * SS + col;
-                bf16x8 o;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) o[e] = static_cast<__bf16>(sp[e]);
-                *reinterpret_cast<bf16x8*>(static_cast<bf16*>(out) + static_cast<size_t>(m) * N + n) = o;
-            }
-        } else {
-            constexpr int PER_ROW = BN / 4;
-            for (int idx = tid; idx < BM * PER_ROW; idx += 256) {
-                const int row = idx / PER_ROW, col = (idx % PER_ROW) * 4;
-                const int m = m0 + row, n = n0 + col;
-                if (m >= M || n >= N) continue;
-                const float4 v = *reinterpret_cast<const float4*>(stage + row * SS + col);
-                float* op = static_cast<float*>(out) + static_cast<size_t>(m) * N + n;
-                if (MODE == kStoreF32) {
-                    *reinterpret_cast<float4*>(op) = v;
-                } else if (MODE == kAddF32) {
-                    float4 cur = *reinterpret_cast<const float4*>(op);
-                    cur.x += v.x; cur.y += v.y; cur.z += v.z; cur.w += v.w;
-                    *reinterpret_cast<float4*>(op) = cur;
-                } else {
-                    atomicAdd(op, v.x); atomicAdd(op + 1, v.y); atomicAdd(op + 2, v.z); atomicAdd(op + 3, v.w);
-                }
-            }
-        }
-        return;
-    }
-#pragma unroll
-    for (int i = 0; i < WMT; ++i) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int m = m0 + wm + i * 16 + q * 4 + e;
-            if (m >= M) continue;
-            if (MODE == kGatedBF16) {
-#pragma unroll
-                for (int j = 0; j + 1 < WNT; j += 2) {
-                    const int unit = (n0 + wn + j * 16) / 2 + r;        // tile column pair (gate, up)
-                    if (2 * unit >= N) continue;
-                    const float gt = acc[i][j][e], up = acc[i][j + 1][e];
-                    static_cast<bf16*>(out)[static_cast<size_t>(m) * (N / 2) + unit] =
-                        static_cast<bf16>((gt / (1.0f + expf(-gt))) * up);
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < WNT; ++j) {
-                    const int n = n0 + wn + j * 16 + r;
-                    if (n >= N) continue;
-                    const size_t idx = static_cast<size_t>(m) * N + n;
-                    const float v = acc[i][j][e];
-                    if (MODE == kStoreF32) static_cast<float*>(out)[idx] = v;
-                    else if (MODE == kAddF32) static_cast<float*>(out)[idx] += v;
-                    else if (MODE == kAtomicF32) atomicAdd(static_cast<float*>(out) + idx, v);
-                    else static_cast<bf16*>(out)[idx] = static_cast<bf16>(v);
-                }
-            }
-        }
-    }
+    tile_epilogue<WMT, WNT, MODE, tile_lds_bytes<WMT, WNT>()>(acc, lds_raw, out, M, N, m0, n0, wm, wn, tid, r, q);
 }
 
-template <auto KERNEL>
+// ----------------------------------------------------------------------------------------
+// The tile kernel with slabs that go from memory straight into LDS: on this chip a buffer load
+// can name LDS as its destination, 16 bytes per lane, lane l's bytes landing at the wavefront's
+// LDS base + 16 l. A wavefront's load is thus 1 KB of consecutive LDS:
+//  * W in the blocked layout: one operand block of the matrix instruction ([4 q][16 r][8]: lane
+//    16 q + r holds row r, k = 8 q ..), lane l loading the block's bytes 16 l ..; a wavefront reads
+//    it back as an operand with 1 KB of consecutive addresses.
+//  * A is row-major: a load takes 8 rows x 64 k, whole 128-byte lines (16 rows x 32 k, a block's own
+//    shape, touches twice as many lines per load, and the loads' path is what such a kernel is
+//    short of: measured 856 against 963 TFLOP/s). Lane 32 kb + 8 q + r loads row r, k = 32 kb + 8 q ..,
+//    so that LDS holds the chunk as [2 kb][4 q][8 r][8]: the upper or lower half of two operand
+//    blocks. Chunks lie 1,152 bytes apart, so that the two halves of an operand (rows 0 .. 7 and
+//    8 .. 15 of a block, in neighbouring chunks) fall into different banks.
+// No padding inside what a load writes, no registers and no LDS-write instructions on the way.
+// k advances in slabs of 64 through NSTAGE LDS buffers, NSTAGE - 1 slabs in flight; a turn waits
+// for its slab (the loads are counted by hand: nothing else of a turn goes through the vector
+// memory path), meets the barrier, asks for the slab NSTAGE - 1 turns ahead into the buffer that
+// the turn before has read, and multiplies.
+// Needs: W blocked (N a multiple of 16, K of 32); K a multiple of 8 as everywhere (a slab that
+// hangs over the end of k reads zeros there: the descriptors end with the rows).
+constexpr int DK = 64;
+constexpr int A_CHUNK = 1024 + 128;                    // bytes from one 8-row chunk of A to the next
+
+template <int WR, int WC, int WMT, int WNT>
+constexpr int direct_stage_bytes() {
+    constexpr int chunks = WR * 2 * WMT, blocks = WC * 2 * WNT, waves = WR * WC;    // per slab: 8-row chunks of A, blocks of W
+    constexpr int padded = (chunks + blocks + waves - 1) / waves * waves;           // (a wavefront with one load too many writes zeros there)
+    return chunks * A_CHUNK + (padded - chunks) * 1024;
+}
+template <int WR, int WC, int WMT, int WNT, int NSTAGE>
+constexpr int direct_lds_bytes() {
+    constexpr int slabs = NSTAGE * direct_stage_bytes<WR, WC, WMT, WNT>();
+    constexpr int staged = WR * 16 * WMT * (WC * 16 * WNT + 4) * 4;                 // the epilogue's staged tile
+    return (staged <= 160 * 1024 && staged > slabs) ? staged : slabs;
+}
+
+// Waits until at most N of this wavefront's vector memory loads are still on their way.
+template <int N> __device__ __forceinline__ void wait_vm() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }
+
+// A buffer descriptor for raw data, as four words (what __builtin_amdgcn_make_buffer_rsrc makes).
+__device__ __forceinline__ u32x4 raw_descriptor(const void* base, unsigned bytes) {
+    const unsigned long long p = reinterpret_cast<unsigned long long>(base);
+    return u32x4{static_cast<unsigned>(p), static_cast<unsigned>(p >> 32) & 0xFFFFu, bytes, static_cast<unsigned>(kBufferFlags)};
+}
+// 16 bytes per lane from rsrc at voffset (per lane) + soffset (scalar), straight into LDS: lane l's
+// bytes land at lds_base + 16 l (lds_base: the same in every lane, a byte address within LDS).
+// Written as assembly because the compiler, which cannot tell which LDS reads such a load may
+// alias, would wait for every load in flight in front of every LDS read.
+__device__ __forceinline__ void load_b128_to_lds(u32x4 rsrc, unsigned lds_base, unsigned voffset, unsigned soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
+                 : "memory", "m0");
+}
+
+template <int WR, int WC, int WMT, int WNT, int MODE, int NSTAGE>
+__global__ __launch_bounds__(64 * WR * WC, (WR * WC <= 4 ? 2 : 1)) void gemm_tile_direct_kernel(
+    const bf16* __restrict__ a, const bf16* __restrict__ w, void* __restrict__ out, int M, int N, int K, int tiles_m,
+    int tiles_n, int ksplit) {
+    constexpr int BM = WR * 16 * WMT, BN = WC * 16 * WNT, NW = WR * WC;
+    constexpr int AC = BM / 8, WB = BN / 16 * 2, NL = AC + WB;  // loads of a slab: A chunks, then W blocks
+    constexpr int LPW = (NL + NW - 1) / NW;                     // loads per wavefront and slab
+    constexpr int STAGE = direct_stage_bytes<WR, WC, WMT, WNT>();
+    static_assert(LPW * (NSTAGE - 1) < 64, "the count of loads in flight has six bits");
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+
+    const int per_split = tiles_m * tiles_n;
+    int pid = blockIdx.x % per_split;
+    const int split = blockIdx.x / per_split;
+    if (per_split % 8 == 0) pid = (pid % 8) * (per_split / 8) + pid / 8;      // (a die gets consecutive tiles)
+    constexpr int GROUP = 8;
+    const int per_group = GROUP * tiles_n;
+    const int g = pid / per_group;
+    const int first_m = g * GROUP;
+    const int gsize = (tiles_m - first_m < GROUP) ? tiles_m - first_m : GROUP;
+    const int tm = first_m + (pid % per_group) % gsize;
+    const int tn = (pid % per_group) / gsize;
+    const int m0 = tm * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, q = lane >> 4;
+    const int wm = (wave / WC) * (16 * WMT), wn = (wave % WC) * (16 * WNT);
+
+    const int nk_all = (K + DK - 1) / DK;
+    const int nk_per = (nk_all + ksplit - 1) / ksplit;
+    const int kt_begin = split * nk_per;
+    const int kt_end = (kt_begin + nk_per < nk_all) ? kt_begin + nk_per : nk_all;
+
+    // Descriptors that begin at the tile's first row and end behind its last row that exists: what
+    // lies behind reads as zeros, without a check, and so does the load that a wavefront has one
+    // too many of (its offset is behind everything). The last slab may hang over the end of k by 32:
+    // in the blocked W that is the next row group's first block, which must not be read, so W's
+    // loads of the slab's second half get an offset behind everything there (k_tail).
+    const int a_rows = M - m0 < BM ? M - m0 : BM, w_rows = N - n0 < BN ? N - n0 : BN;
+    const u32x4 a_rsrc = raw_descriptor(a + static_cast<size_t>(m0) * K, static_cast<unsigned>(a_rows) * K * 2);
+    const u32x4 w_rsrc = raw_descriptor(w + static_cast<size_t>(n0) * K, static_cast<unsigned>(w_rows) * K * 2);
+    // (the slabs' LDS starts at the workgroup's LDS address 0: the kernel has no other LDS)
+    const unsigned lds_origin = static_cast<unsigned>(reinterpret_cast<size_t>(
+        (__attribute__((address_space(3))) unsigned char*)lds_raw));
+    constexpr unsigned kNowhere = 0xFFFFFF00u;
+    unsigned off[LPW], tail_off[LPW], step[LPW], dst[LPW];      // per load: lane offset, the same in the last slab,
+    u32x4 rs[LPW];                                              // bytes from slab to slab, place in the stage
+    const bool k_tail = K % DK != 0;                            // (K is a multiple of 32 here: half a slab is left)
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+        const int j = wave + NW * i;                    // (the same in every lane: the choices below are scalar)
+        rs[i] = j < AC ? a_rsrc : w_rsrc;
+        step[i] = j < AC ? DK * 2 : 2048;
+        if (j < AC) {
+            // chunk j: rows 8 j .. 8 j + 7; lane 32 kb + 8 q' + r' loads row r', k = 32 kb + 8 q'
+            const int kb = lane >> 5, q8 = (lane >> 3) & 3, r8 = lane & 7;
+            off[i] = (static_cast<unsigned>(j * 8 + r8) * K + kb * 32 + q8 * 8) * 2;
+            tail_off[i] = kb == 0 ? off[i] : kNowhere;  // (row-major A: k past the end is the next row's start)
+            dst[i] = j * A_CHUNK;
+        } else if (j < NL) {
+            const int blk = j - AC, grp = blk >> 1, kb = blk & 1;
+            off[i] = (static_cast<unsigned>(grp) * (K / 32) + kb) * 1024u + lane * 16u;
+            tail_off[i] = kb == 0 ? off[i] : kNowhere;
+            dst[i] = AC * A_CHUNK + blk * 1024;
+        } else {
+            off[i] = tail_off[i] = kNowhere;
+            dst[i] = AC * A_CHUNK + (j - AC) * 1024;
+        }
+    }
+    auto ask = [&](int kt, int stage) {
+        if (kt >= kt_end) kt = kt_end - 1;              // (past the end: the last slab again, nobody reads it)
+        const bool tail = k_tail && kt == nk_all - 1;
+        const unsigned base = lds_origin + stage * STAGE;
+#pragma unroll
+        for (int i = 0; i < LPW; ++i) load_b128_to_lds(rs[i], base + dst[i], tail ? tail_off[i] : off[i], kt * step[i]);
+    };
+
+    f32x4 acc[WMT][WNT];
+#pragma unroll
+    for (int i = 0; i < WMT; ++i)
+#pragma unroll
+        for (int j = 0; j < WNT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    if (kt_begin < kt_end) {
+        // this lane's place in an operand of A: chunk 2 g + r / 8, then [kb][q][r % 8]
+        const unsigned a_lane = (wm / 8 + (r >> 3)) * A_CHUNK + q * 128 + (r & 7) * 16;
+        const unsigned w_lane = AC * A_CHUNK + (wn / 16) * 2048 + lane * 16;
+        auto read_frags = [&](int stage, int kk, bf16x8 (&fa)[WMT], bf16x8 (&fw)[WNT]) {
+            const unsigned char* sA = lds_raw + stage * STAGE + a_lane + kk * 512;
+            const unsigned char* sW = lds_raw + stage * STAGE + w_lane + kk * 1024;
+#pragma unroll
+            for (int i = 0; i < WMT; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(sA + i * 2 * A_CHUNK);
+#pragma unroll
+            for (int j = 0; j < WNT; ++j) fw[j] = *reinterpret_cast<const bf16x8*>(sW + j * 2048);
+        };
+        auto multiply = [&](const bf16x8 (&fa)[WMT], const bf16x8 (&fw)[WNT]) {
+#pragma unroll
+            for (int i = 0; i < WMT; ++i)
+#pragma unroll
+                for (int j = 0; j < WNT; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
+        };
+        // Every buffer is asked for at the start. A turn multiplies the first half of its slab (whose
+        // operands the turn before has read) while it reads the second half's; then it waits for
+        // the next slab, meets the barrier (every wavefront now holds the whole slab in registers),
+        // asks for the slab NSTAGE turns ahead into the buffer of its own, and multiplies the
+        // second half while it reads the next slab's first operands.
+#pragma unroll
+        for (int s0 = 0; s0 < NSTAGE; ++s0) ask(kt_begin + s0, s0);
+        wait_vm<LPW * (NSTAGE - 1)>();
+        lds_barrier();
+        bf16x8 fa0[WMT], fw0[WNT];
+        read_frags(0, 0, fa0, fw0);
+        int stage = 0;
+        for (int kt = kt_begin; kt < kt_end; ++kt) {
+            bf16x8 fa1[WMT], fw1[WNT];
+            read_frags(stage, 1, fa1, fw1);
+            multiply(fa0, fw0);
+            deal_between_products<kDsRead, WMT + WNT>();
+            __builtin_amdgcn_sched_barrier(0);
+            wait_vm<LPW * (NSTAGE - 2)>();              // the next slab has landed (the later ones may be on their way)
+            lds_barrier();                              // .. everybody's share of it, and everybody has read this one
+            ask(kt + NSTAGE, stage);
+            stage = stage + 1 == NSTAGE ? 0 : stage + 1;
+            read_frags(stage, 0, fa0, fw0);
+            multiply(fa1, fw1);
+            deal_between_products<kDsRead, WMT + WNT>();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    wait_vm<0>();                                       // (loads past the end are still on their way into LDS)
+    __syncthreads();                                    // the epilogue reuses the slabs' LDS
+    tile_epilogue<WMT, WNT, MODE, direct_lds_bytes<WR, WC, WMT, WNT, NSTAGE>(), WR, WC>(acc, lds_raw, out, M, N, m0, n0,
+                                                                                         wm, wn, tid, r, q);
+}
+
+template <auto KERNEL, int THREADS = 256>
 static int launch_tile_kernel(int LDS, int BM, int BN, const bf16* A, const bf16* W, void* out, int M, int N, int K,
                               int ksplit, hipStream_t stream) {
     static bool attr_set = false;                      // per kernel
@@ -373,7 +586,7 @@ static int launch_tile_kernel(int LDS, int BM, int BN, const bf16* A, const bf16
         attr_set = true;
     }
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
-    hipLaunchKernelGGL(KERNEL, dim3(tiles_m * tiles_n * ksplit), dim3(256), LDS, stream, A, W, out, M, N, K, tiles_m,
+    hipLaunchKernelGGL(KERNEL, dim3(tiles_m * tiles_n * ksplit), dim3(THREADS), LDS, stream, A, W, out, M, N, K, tiles_m,
                        tiles_n, ksplit);
     return launch_status();
 }
@@ -406,6 +619,24 @@ static int launch_tile(const bf16* A, const bf16* W, void* out, int M, int N, in
         case kGatedBF16: return launch_tile_mode<WMT, WNT, kGatedBF16>(A, W, out, M, N, K, 1, blocked, stream);
         default: return launch_tile_mode<WMT, WNT, kStoreBF16>(A, W, out, M, N, K, 1, blocked, stream);
     }
+}
+
+template <int WR, int WC, int WMT, int WNT, int NSTAGE>
+static int launch_tile_direct(const bf16* A, const bf16* W, void* out, int M, int N, int K, int mode, int ksplit,
+                              hipStream_t stream) {
+    constexpr int LDS = direct_lds_bytes<WR, WC, WMT, WNT, NSTAGE>();
+    constexpr int BM = WR * 16 * WMT, BN = WC * 16 * WNT;
+#define LLME_DIRECT(MODE) \
+    launch_tile_kernel<gemm_tile_direct_kernel<WR, WC, WMT, WNT, MODE, NSTAGE>, 64 * WR * WC>( \
+        LDS, BM, BN, A, W, out, M, N, K, MODE == kAtomicF32 ? ksplit : 1, stream)
+    switch (mode) {
+        case kStoreF32: return LLME_DIRECT(kStoreF32);
+        case kAddF32: return LLME_DIRECT(kAddF32);
+        case kAtomicF32: return LLME_DIRECT(kAtomicF32);
+        case kGatedBF16: return LLME_DIRECT(kGatedBF16);
+        default: return LLME_DIRECT(kStoreBF16);
+    }
+#undef LLME_DIRECT
 }
 
 // ----------------------------------------------------------------------------------------
@@ -522,10 +753,13 @@ using namespace llme;
 // nw, ksplit: 0 lets the entry point choose the skinny kernel's wavefronts per workgroup and
 // the split over k; tile_shape: 0 chooses, 64 / 128 force the tile kernel with that tile
 // edge also for small M (for tests and measurements). blocked: w is stored in 1 KB blocks of
-// 16 rows x 32 k (see the head of this file; N a multiple of 16, K of 32).
+// 16 rows x 32 k (see the head of this file; N a multiple of 16, K of 32). direct: the tile kernel
+// whose slabs go from memory straight into LDS (needs blocked; tile_shape also 256256 and 256128 then):
+// -1 where the entry point finds it faster, 0 never, 1 it must.
 extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
-                              int accumulate, int gated, int nw, int ksplit, int tile_shape, int blocked,
+                              int accumulate, int gated, int nw, int ksplit, int tile_shape, int blocked, int direct,
                               hipStream_t stream) {
+    if (direct < -1 || direct > 1 || (direct == 1 && !blocked)) return kErrBadArgument;
     if (M <= 0 || N <= 0) return 0;
     if (blocked && (N % 16 != 0 || K % 32 != 0)) return kErrUnsupported;
     if (K <= 0 || K % 8 != 0 || K >= (1 << 23)) return kErrUnsupported;   // 256 rows of K must stay below 2^32 bytes
@@ -580,6 +814,7 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     // workgroup per compute unit; a small output with a long k is cut over k instead (the
     // parts are added with atomics, so this needs an accumulating float32 output).
     if (gated) mode = kGatedBF16;
+    const bool auto_shape = tile_shape <= 0;
     if (tile_shape <= 0) {
         const long wg128 = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
         tile_shape = (M > 64 && wg128 >= 64) ? 128 : 64;
@@ -625,6 +860,25 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
         if (mode != kAddF32) return kErrBadArgument;
         mode = kAtomicF32;
     }
+    if (auto_shape && blocked && direct != 0 && mode != kAddF32 && mode != kAtomicF32) {
+        // Wide outputs that are stored, not added (gate/up, q/k/v of long prompts): tiles of 256 x 256
+        // by eight wavefronts, their slabs straight into LDS, load half the bytes per product; one
+        // workgroup fills a compute unit, so they pay where whole rounds of them cover the output
+        // (measured, 256 compute units: 1.07 to 1.16 times the 128 x 128 tiles' speed at 256, 512,
+        // 1,024 and more tiles, 0.9 at 384).
+        const long rounds = (static_cast<long>((M + 255) / 256) * ((N + 255) / 256) + cus - 1) / cus;
+        const double covered = static_cast<double>(M) * N / (static_cast<double>(rounds) * cus * 65536.0);
+        if (covered >= 0.85) return launch_tile_direct<4, 2, 4, 8, 2>(A, W, out, M, N, K, mode, ksplit, stream);
+    }
+    if (blocked && direct == 1 && tile_shape != 64) {
+        if (tile_shape == 128096) return launch_tile_direct<2, 2, 4, 3, 2>(A, W, out, M, N, K, mode, ksplit, stream);
+        if (tile_shape == 128064) return launch_tile_direct<2, 2, 4, 2, 2>(A, W, out, M, N, K, mode, ksplit, stream);
+        if (tile_shape == 128) return launch_tile_direct<2, 2, 4, 4, 2>(A, W, out, M, N, K, mode, ksplit, stream);
+        if (tile_shape == 256256) return launch_tile_direct<4, 2, 4, 8, 2>(A, W, out, M, N, K, mode, ksplit, stream);
+        if (tile_shape == 256128) return launch_tile_direct<4, 2, 4, 4, 3>(A, W, out, M, N, K, mode, ksplit, stream);
+        return kErrBadArgument;
+    }
+    if (direct == 1) return kErrUnsupported;
     if (tile_shape == 128096) return launch_tile<4, 3>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
     if (tile_shape == 128064) return launch_tile<4, 2>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
     if (tile_shape == 128) return launch_tile<4, 4>(A, W, out, M, N, K, mode, ksplit, blocked, stream);

@@ -12,7 +12,7 @@ from .lib import check, declare, entry, ptr, require, stream
 
 _vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
 
-declare("llme_gemm_bf16", [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp])
+declare("llme_gemm_bf16", [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp])
 
 
 def gemm_bf16_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool) -> bool:
@@ -25,11 +25,12 @@ def gemm_bf16_supported(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, acc
 
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False, *,
               gated: bool = False, waves: int = 0, ksplit: int = 0, tile: int = 0, force_tile: bool = False,
-              _supported: bool = False) -> None:
+              direct: int = -1, _supported: bool = False) -> None:
     """bfloat16 a [M, K] and w [N, K] -> out [M, N] (float32 or bfloat16), 32-bit accumulation.
     K must be a multiple of 8. gated: w holds gate and up rows interleaved in groups of 16 and
     out is bfloat16 [M, N / 2] = silu(gate) * up. waves / ksplit / tile (64, 128, 128096, 128064) /
-    force_tile override the launch choices (tests and measurements)."""
+    force_tile override the launch choices (tests and measurements); direct: whether the tile kernel's
+    slabs go from memory straight into LDS, which needs a blocked w (-1: where it can, 0: never, 1: it must)."""
     require(a, "a", torch.bfloat16, (None, None))
     M, K = a.shape
     N, _ = kernels._require_weight(w, "w", torch.bfloat16, K)
@@ -46,7 +47,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
         tile = 128
     check(entry("llme_gemm_bf16")(ptr(a), ptr(w), ptr(out), 0 if out.dtype == torch.float32 else 1, M, N, K,
                                   1 if accumulate else 0, 1 if gated else 0, waves, ksplit, tile,
-                                  1 if kernels.is_blocked(w) else 0, stream()),
+                                  1 if kernels.is_blocked(w) else 0, int(direct), stream()),
           "gemm_bf16")
 
 

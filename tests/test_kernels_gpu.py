@@ -269,6 +269,45 @@ def test_gemm_tile(ops, M, N, K, tile):
     assert _rel(half.cpu().double(), ref) < 5e-3
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 128, 64), (128, 128, 128), (300, 400, 96), (129, 112, 160), (257, 512, 32),
+                                   (2048, 3072, 2048), (1000, 2048, 8192), (333, 208, 2080)])
+@pytest.mark.parametrize("tile", [128, 128096, 128064, 256256, 256128])
+def test_gemm_tile_with_slabs_straight_into_lds(ops, M, N, K, tile):
+    """The tile kernel whose slabs go from memory into LDS without passing through registers
+    (blocked weights): every epilogue, sums cut over k, tiles that hang over the matrix's edges,
+    k of one slab and of many; against the plain product, and bit for bit against the kernel that
+    stages its slabs through registers (both add the same products in the same order)."""
+    a, w, ref = _bf16_pair(M, N, K, 35)
+    ad, wb = a.to(DEV), ops.block_weight(w.to(DEV))
+    for dtype, tol in ((torch.float32, 2e-5), (torch.bfloat16, 5e-3)):
+        direct = torch.full((M, N), 3.0, dtype=dtype, device=DEV)
+        staged = torch.full((M, N), 5.0, dtype=dtype, device=DEV)
+        ops.gemm_bf16(ad, wb, direct, tile=tile, direct=1)
+        ops.gemm_bf16(ad, wb, staged, tile=min(tile, 128), direct=0)
+        assert _rel(direct.cpu().double(), ref) < tol
+        assert torch.equal(direct, staged)
+    base = torch.randn(M, N, generator=_gen(36))
+    acc, acc0 = base.clone().to(DEV), base.clone().to(DEV)
+    ops.gemm_bf16(ad, wb, acc, accumulate=True, tile=tile, direct=1)
+    ops.gemm_bf16(ad, wb, acc0, accumulate=True, tile=min(tile, 128), direct=0)
+    assert _rel(acc.cpu().double(), ref + base.double()) < 2e-5 and torch.equal(acc, acc0)
+    for ksplit in (2, 5):
+        acc = base.clone().to(DEV)
+        ops.gemm_bf16(ad, wb, acc, accumulate=True, tile=tile, ksplit=ksplit, direct=1)
+        assert _rel(acc.cpu().double(), ref + base.double()) < 2e-5, ksplit
+    if N % 32 == 0:                                   # gate and up rows interleaved in groups of 16
+        gated = torch.empty(M, N // 2, dtype=torch.bfloat16, device=DEV)
+        gated0 = torch.empty(M, N // 2, dtype=torch.bfloat16, device=DEV)
+        ops.gemm_bf16(ad, wb, gated, gated=True, tile=tile, direct=1)
+        ops.gemm_bf16(ad, wb, gated0, gated=True, tile=min(tile, 128), direct=0)
+        gu = ref.view(M, N // 32, 2, 16)
+        want = (plain_silu(gu[:, :, 0]) * gu[:, :, 1]).reshape(M, N // 2)
+        assert _rel(gated.cpu().double(), want) < 8e-3 and torch.equal(gated, gated0)
+    from llmengine.ops import KernelError
+    with pytest.raises(KernelError):
+        ops.gemm_bf16(ad, w.to(DEV), torch.empty(M, N, device=DEV), tile=tile, direct=1)     # row-major weights
+
+
 @pytest.mark.parametrize("T,FF,K,tile", [(5, 176, 64, 0), (130, 256, 96, 64), (300, 208, 144, 128), (2048, 8192, 2048, 0),
                                          (257, 320, 128, 128096), (190, 352, 72, 128064), (64, 8192, 2048, 0)])
 def test_gemm_gated(ops, T, FF, K, tile):
