@@ -14,7 +14,8 @@ run at the configured context length. One JSON line goes to stdout.
 `--shape 3b` and `--shape 8b` take the layer sizes of Llama 3.2 3B and Llama 3.1 8B instead (for
 measurements at further sizes and context lengths; the default run is the 1B shape).
 
-`--phase serve` is another workload (with `--shape 3b`: 32 requests with prompts of 64 to 3,072
+`--phase mixed` times one step of continuous batching (a prompt portion beside decoded tokens of
+other requests), `--phase portion` portions of one long prompt. `--phase serve` is another workload (with `--shape 3b`: 32 requests with prompts of 64 to 3,072
 tokens and 128 to 512 new tokens each, 2,048 prompt tokens a step at most) through the
 continuous-batching scheduler, prompt portions beside decoded tokens in every step.
 
@@ -164,6 +165,60 @@ def portion(args, engine, cfg: dict, gen, page: int) -> int:
     return 0
 
 
+def mixed(args, engine, cfg: dict, gen, page: int) -> int:
+    """The step that continuous batching runs most: a prompt portion of --portion tokens of one
+    request (behind --context cached tokens) beside one decoded token of --batch other requests
+    (700 to 1,500 tokens each). Timed as the engine launches it, and once more with the same
+    launches recorded as a HIP graph and replayed, which is the GPU's time alone."""
+    import torch
+    from llmengine import StepEntry
+    V, n, nd = cfg["vocab_size"], args.portion, args.batch
+    steps = max(4, min(args.steps, 32))
+    lens = [700 + (800 * i) // max(nd, 1) for i in range(nd)]
+    cache = engine.new_cache((args.context + n + sum(lens)) // page + nd + 4, page, nd + 1)
+    for i, ln in enumerate(lens):
+        cache.admit(i)
+        engine.step(cache, [StepEntry(i, torch.randint(0, V, (ln,), generator=gen).tolist(), [])])
+    cache.admit("p")
+    for at in range(0, args.context, 2048):
+        engine.step(cache, [StepEntry("p", torch.randint(0, V, (min(2048, args.context - at),), generator=gen).tolist(), [])])
+    entries = [StepEntry("p", torch.randint(0, V, (n,), generator=gen).tolist(), [n - 1])] + [
+        StepEntry(i, [7], [0]) for i in range(nd)]
+    runner, mgr = engine.runner, cache.manager
+    # the same tokens at the same places every time: pages are reserved once and never committed
+    assert mgr.reserve_batch([(e.request_id, len(e.tokens)) for e in entries])
+    ctx, rows = runner._build_context(cache, entries)
+
+    def forward():
+        return runner.model.forward(ctx, cache.storage.layers, rows)
+    for _ in range(3):
+        forward()
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    for _ in range(steps):
+        forward()
+    torch.cuda.synchronize()
+    launched = (time.perf_counter() - t) / steps * 1e3
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        forward()
+    graph.replay()
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    gpu = (time.perf_counter() - t) / steps * 1e3
+    log(f"mixed step, {n} prompt tokens behind {args.context} beside {nd} decoded tokens: {launched:.3f} ms launched "
+        f"by the engine, {gpu:.3f} ms as a recorded graph")
+    print(json.dumps({"metric": "mixed_step_tokens_per_second", "value": round((n + nd) / (launched / 1e3), 1),
+                      "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype, "ms_per_step": round(launched, 3),
+                      "ms_per_step_gpu_only": round(gpu, 3), "steps": steps,
+                      "config": {"model": args.shape, "layers": args.layers, "context": args.context, "portion": n,
+                                 "decode_requests": nd, "page_size": page}}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -177,10 +232,11 @@ def main() -> int:
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode", "serve", "portion"],
+    ap.add_argument("--phase", default="all", choices=["all", "prefill", "decode", "serve", "portion", "mixed"],
                     help="run only one part (for profiling); the JSON line then lacks the other. 'serve' is another "
                          "workload: requests of mixed lengths through the continuous-batching scheduler; 'portion': "
-                         "steps of --portion prompt tokens of one request behind --context tokens")
+                         "steps of --portion prompt tokens of one request behind --context tokens; 'mixed': such a "
+                         "portion beside one decoded token of --batch other requests")
     ap.add_argument("--portion", type=int, default=256, help="portion: prompt tokens a step")
     ap.add_argument("--requests", type=int, default=32, help="serve: number of requests")
     ap.add_argument("--prompt-range", default="64,3072", help="serve: prompt lengths, uniform in [a, b]")
@@ -215,6 +271,8 @@ def main() -> int:
         return serve(args, engine, cfg, gen, page)
     if args.phase == "portion":
         return portion(args, engine, cfg, gen, page)
+    if args.phase == "mixed":
+        return mixed(args, engine, cfg, gen, page)
 
     # ---- prefill: one prompt, logits at its last place ----
     T = args.prefill_tokens
