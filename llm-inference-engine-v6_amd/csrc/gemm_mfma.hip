@@ -51,7 +51,24 @@ typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
 // The fourth word of a buffer descriptor for raw 32-bit data on this chip.
 constexpr int kBufferFlags = 0x00020000;
 
-enum OutMode : int { kStoreF32 = 0, kAddF32 = 1, kStoreBF16 = 2, kAtomicF32 = 3, kGatedBF16 = 4 };
+enum OutMode : int { kStoreF32 = 0, kAddF32 = 1, kStoreBF16 = 2, kAtomicF32 = 3, kGatedBF16 = 4, kRopeCache = 5 };
+
+// Where the q/k/v projection's epilogue (kRopeCache) puts its result: the columns are the heads
+// of q, then k, then v (hd columns each); q and k heads are rotated at the rows' positions (pairs
+// (i, i + hd / 2), src/kernels.cpp:189-203), q goes to q_out [M, n_q hd], k and v into the rows'
+// cache pages (k_cache [pages, n_kv, page, hd], v_cache [pages, n_kv, hd, page]), all bfloat16.
+struct QkvTarget {
+    const float* cos_t;         // [max_pos, hd / 2]
+    const float* sin_t;
+    const int* positions;       // [M]
+    const int* seq_idx;         // [M] row of the block table
+    const int* block_table;     // [n_seq, max_blocks]
+    int max_blocks;
+    bf16* q_out;
+    bf16* k_cache;
+    bf16* v_cache;
+    int n_q, n_kv, hd, page;
+};
 
 // ----------------------------------------------------------------------------------------
 // tile kernel: a workgroup of 2 x 2 wavefronts makes a (32 WMT) x (32 WNT) tile of the output,
@@ -83,7 +100,8 @@ __device__ __forceinline__ void deal_between_products() {
 // goes through LDS instead, so that every thread stores 16 contiguous bytes of a row.
 template <int WMT, int WNT, int MODE, int LDS_BYTES, int WR = 2, int WC = 2>
 __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned char* lds_raw, void* __restrict__ out,
-                                              int M, int N, int m0, int n0, int wm, int wn, int tid, int r, int q) {
+                                              int M, int N, int m0, int n0, int wm, int wn, int tid, int r, int q,
+                                              const QkvTarget& qt = QkvTarget{}) {
     constexpr int BM = WR * 16 * WMT, BN = WC * 16 * WNT, NT = 64 * WR * WC;
 
     constexpr int SS = BN + 4;                           // floats per staged row
@@ -112,7 +130,72 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
         }
         __syncthreads();
         const int mp = m0 + pass * HB;                  // the pass's first row
-        if (MODE == kGatedBF16) {
+        if (MODE == kRopeCache) {
+            // The tile holds whole heads (the entry point chose it so). q and k heads: a thread takes 8
+            // dims of a head's first half and their partners in the second, of one row.
+            const int hd = qt.hd, half = hd / 2, hv = half / 8, rotated = qt.n_q + qt.n_kv;
+            const int per_row = (BN / hd) * hv;
+            for (int idx = tid; idx < HB * per_row; idx += NT) {
+                const int row = idx / per_row, e = idx % per_row;
+                const int hh = e / hv, i = (e % hv) * 8;
+                const int m = mp + row, head = n0 / hd + hh;
+                if (m >= M || head >= rotated) continue;
+                const float* sp = stage + row * SS + hh * hd + i;
+                const int pos = qt.positions[m];
+                const float* cs = qt.cos_t + static_cast<size_t>(pos) * half + i;
+                const float* sn = qt.sin_t + static_cast<size_t>(pos) * half + i;
+                bf16x8 lo, hi;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float a = sp[j], b = sp[half + j], c = cs[j], sv = sn[j];
+                    lo[j] = static_cast<__bf16>(a * c - b * sv);
+                    hi[j] = static_cast<__bf16>(b * c + a * sv);
+                }
+                bf16* dst;
+                if (head < qt.n_q) {
+                    dst = qt.q_out + (static_cast<size_t>(m) * qt.n_q + head) * hd + i;
+                } else {
+                    const int pg = qt.block_table[static_cast<size_t>(qt.seq_idx[m]) * qt.max_blocks + pos / qt.page];
+                    dst = qt.k_cache + ((static_cast<size_t>(pg) * qt.n_kv + (head - qt.n_q)) * qt.page + pos % qt.page) * hd + i;
+                }
+                *reinterpret_cast<bf16x8*>(dst) = lo;
+                *reinterpret_cast<bf16x8*>(dst + half) = hi;
+            }
+            // v heads: a thread takes one dim of 16 consecutive rows. Where these are 16 consecutive
+            // positions of one request that begin at a multiple of 16 (the usual case in a prompt) they
+            // lie together in the transposed page and go out as one piece; otherwise one by one.
+            for (int idx = tid; idx < (HB / 16) * BN; idx += NT) {
+                const int g16 = idx / BN, col = idx % BN;
+                const int n = n0 + col, head = n / hd;
+                const int mg = mp + g16 * 16;
+                if (head < rotated || n >= N || mg >= M) continue;
+                const int kvh = head - rotated, d = n % hd;
+                const int nt = M - mg < 16 ? M - mg : 16;
+                const float* sp = stage + (g16 * 16) * SS + col;
+                const int pos0 = qt.positions[mg];
+                const bool together = nt == 16 && qt.seq_idx[mg] == qt.seq_idx[mg + 15] && pos0 % 16 == 0 &&
+                                      qt.page % 16 == 0 && qt.positions[mg + 15] == pos0 + 15;
+                if (together) {
+                    const int pg = qt.block_table[static_cast<size_t>(qt.seq_idx[mg]) * qt.max_blocks + pos0 / qt.page];
+                    bf16* dst = qt.v_cache + ((static_cast<size_t>(pg) * qt.n_kv + kvh) * hd + d) * qt.page + pos0 % qt.page;
+                    bf16x8 lo, hi;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        lo[j] = static_cast<__bf16>(sp[j * SS]);
+                        hi[j] = static_cast<__bf16>(sp[(j + 8) * SS]);
+                    }
+                    *reinterpret_cast<bf16x8*>(dst) = lo;
+                    *reinterpret_cast<bf16x8*>(dst + 8) = hi;
+                } else {
+                    for (int j = 0; j < nt; ++j) {
+                        const int pos = qt.positions[mg + j];
+                        const int pg = qt.block_table[static_cast<size_t>(qt.seq_idx[mg + j]) * qt.max_blocks + pos / qt.page];
+                        qt.v_cache[((static_cast<size_t>(pg) * qt.n_kv + kvh) * hd + d) * qt.page + pos % qt.page] =
+                            static_cast<__bf16>(sp[j * SS]);
+                    }
+                }
+            }
+        } else if (MODE == kGatedBF16) {
             // a thread makes 8 units: their gates and ups lie 16 columns apart in a group of 32
             constexpr int PER_ROW = BN / 16;             // 8-unit pieces per row
             for (int idx = tid; idx < HB * PER_ROW; idx += NT) {
@@ -164,6 +247,7 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
         }
         return;
     }
+    if (MODE == kRopeCache) return;                     // (always staged: its columns are whole heads of 16 dims and more)
 #pragma unroll
     for (int i = 0; i < WMT; ++i) {
 #pragma unroll
@@ -202,7 +286,7 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
 template <int WMT, int WNT, int MODE, bool KFULL, bool BLOCKED>
 __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restrict__ a, const bf16* __restrict__ w,
                                                         void* __restrict__ out, int M, int N, int K,
-                                                        int tiles_m, int tiles_n, int ksplit) {
+                                                        int tiles_m, int tiles_n, int ksplit, QkvTarget qt) {
     constexpr int BM = 32 * WMT, BN = 32 * WNT;
     constexpr int A_ELEMS = BM * TSTRIDE, W_ELEMS = BN * TSTRIDE;
     constexpr int CA = BM / 32, CW = BN / 32;        // 16-byte chunks per thread and slab
@@ -380,7 +464,7 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
         if ((kt_end - kt_begin) & 1) turn(kt, 0, s1);
     }
     __syncthreads();                                  // the epilogue reuses the slabs' LDS
-    tile_epilogue<WMT, WNT, MODE, tile_lds_bytes<WMT, WNT>()>(acc, lds_raw, out, M, N, m0, n0, wm, wn, tid, r, q);
+    tile_epilogue<WMT, WNT, MODE, tile_lds_bytes<WMT, WNT>()>(acc, lds_raw, out, M, N, m0, n0, wm, wn, tid, r, q, qt);
 }
 
 // ----------------------------------------------------------------------------------------
@@ -441,7 +525,7 @@ __device__ __forceinline__ void load_b128_to_lds(u32x4 rsrc, unsigned lds_base, 
 template <int WR, int WC, int WMT, int WNT, int MODE, int NSTAGE>
 __global__ __launch_bounds__(64 * WR * WC, (WR * WC <= 4 ? 2 : 1)) void gemm_tile_direct_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w, void* __restrict__ out, int M, int N, int K, int tiles_m,
-    int tiles_n, int ksplit) {
+    int tiles_n, int ksplit, QkvTarget qt) {
     constexpr int BM = WR * 16 * WMT, BN = WC * 16 * WNT, NW = WR * WC;
     constexpr int AC = BM / 8, WB = BN / 16 * 2, NL = AC + WB;  // loads of a slab: A chunks, then W blocks
     constexpr int LPW = (NL + NW - 1) / NW;                     // loads per wavefront and slab
@@ -572,12 +656,12 @@ __global__ __launch_bounds__(64 * WR * WC, (WR * WC <= 4 ? 2 : 1)) void gemm_til
     wait_vm<0>();                                       // (loads past the end are still on their way into LDS)
     __syncthreads();                                    // the epilogue reuses the slabs' LDS
     tile_epilogue<WMT, WNT, MODE, direct_lds_bytes<WR, WC, WMT, WNT, NSTAGE>(), WR, WC>(acc, lds_raw, out, M, N, m0, n0,
-                                                                                         wm, wn, tid, r, q);
+                                                                                         wm, wn, tid, r, q, qt);
 }
 
 template <auto KERNEL, int THREADS = 256>
 static int launch_tile_kernel(int LDS, int BM, int BN, const bf16* A, const bf16* W, void* out, int M, int N, int K,
-                              int ksplit, hipStream_t stream) {
+                              int ksplit, hipStream_t stream, const QkvTarget& qt = QkvTarget{}) {
     static bool attr_set = false;                      // per kernel
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(KERNEL),
@@ -587,7 +671,7 @@ static int launch_tile_kernel(int LDS, int BM, int BN, const bf16* A, const bf16
     }
     const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
     hipLaunchKernelGGL(KERNEL, dim3(tiles_m * tiles_n * ksplit), dim3(THREADS), LDS, stream, A, W, out, M, N, K, tiles_m,
-                       tiles_n, ksplit);
+                       tiles_n, ksplit, qt);
     return launch_status();
 }
 
@@ -641,6 +725,18 @@ static int launch_tile_direct(const bf16* A, const bf16* W, void* out, int M, in
 
 // ----------------------------------------------------------------------------------------
 // skinny kernel: MT row tiles of 16 (M <= 16 MT), NW wavefronts per workgroup splitting k
+template <int WMT, int WNT>
+static int launch_tile_rope(const bf16* A, const bf16* W, int M, int N, int K, int blocked, const QkvTarget& qt,
+                            hipStream_t stream) {
+    constexpr int LDS = tile_lds_bytes<WMT, WNT>();
+#define LLME_ROPE_TILE(KFULL, BLOCKED) \
+    launch_tile_kernel<gemm_tile_kernel<WMT, WNT, kRopeCache, KFULL, BLOCKED>>(LDS, 32 * WMT, 32 * WNT, A, W, nullptr, M, N, \
+                                                                                K, 1, stream, qt)
+    if (K % TK != 0) return blocked ? LLME_ROPE_TILE(false, true) : LLME_ROPE_TILE(false, false);
+    return blocked ? LLME_ROPE_TILE(true, true) : LLME_ROPE_TILE(true, false);
+#undef LLME_ROPE_TILE
+}
+
 constexpr int SK_U = 4;                  // 32-element k steps per wavefront iteration
 constexpr int SK_CHUNK = 32 * SK_U;      // 128 elements
 
@@ -817,7 +913,10 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     const bool auto_shape = tile_shape <= 0;
     if (tile_shape <= 0) {
         const long wg128 = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
-        tile_shape = (M > 64 && wg128 >= 64) ? 128 : 64;
+        // (a stored output with fewer than 96 tiles of 128 x 128 fills the chip better in 64 x 64 tiles:
+        // q/k/v of the 1B sizes at 273 rows 12.6 against 16.0 us; sums that are cut over k keep the larger tiles)
+        const long enough = (mode == kStoreF32 || mode == kStoreBF16) ? 96 : 64;
+        tile_shape = (M > 64 && wg128 >= enough) ? 128 : 64;
         if (tile_shape == 128 && wg128 < 4 * cus && !(mode == kAddF32 && wg128 <= cus && K >= 4096)) {
             // Medium outputs: narrower tiles can fill the compute units (two workgroups
             // each) more evenly. Estimated time: rounds of one workgroup per compute unit x tile area / measured
@@ -883,5 +982,43 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     if (tile_shape == 128064) return launch_tile<4, 2>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
     if (tile_shape == 128) return launch_tile<4, 4>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
     if (tile_shape == 64) return launch_tile<2, 2>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
+    return kErrBadArgument;
+}
+
+// The q/k/v projection of many rows (prompts) with rotation and cache write in its epilogue:
+// a [M, K] (the normed activations), w [(n_q + 2 n_kv) hd, K] (q heads, k heads, v heads), both
+// bfloat16; writes q_out [M, n_q hd] (rotated) and the rows' k (rotated) and v into the pages that
+// block_table[seq_idx[m]] names for positions[m]; cos/sin [max_pos, hd / 2] float32. Full rotation
+// only; hd 16, 32, 64 or 128 (a tile of 128 or 64 columns must hold whole heads). What the separate
+// kernels would store in between, the 32-bit q/k/v rows, never exists. tile_shape 0, 64, 128 or 128064.
+extern "C" int llme_gemm_bf16_qkv_rope(const void* a, const void* w, int M, int K, int blocked, const float* cos_t,
+                                       const float* sin_t, const int* positions, const int* seq_idx,
+                                       const int* block_table, int max_blocks, void* q_out, void* k_cache,
+                                       void* v_cache, int n_q, int n_kv, int hd, int page, int tile_shape,
+                                       hipStream_t stream) {
+    if (M <= 0) return 0;
+    if (n_q <= 0 || n_kv <= 0 || page <= 0 || max_blocks <= 0) return kErrBadArgument;
+    if (hd != 16 && hd != 32 && hd != 64 && hd != 128) return kErrUnsupported;
+    if (K <= 0 || K % 8 != 0 || K >= (1 << 23)) return kErrUnsupported;
+    if (blocked && K % 32 != 0) return kErrUnsupported;
+    if (!cos_t || !sin_t || !positions || !seq_idx || !block_table || !q_out || !k_cache || !v_cache) return kErrBadArgument;
+    if (reinterpret_cast<uintptr_t>(q_out) % 16 != 0 || reinterpret_cast<uintptr_t>(k_cache) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(v_cache) % 16 != 0)
+        return kErrUnsupported;
+    const int N = (n_q + 2 * n_kv) * hd;
+    const QkvTarget qt{cos_t, sin_t, positions, seq_idx, block_table, max_blocks, static_cast<bf16*>(q_out),
+                       static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache), n_q, n_kv, hd, page};
+    const bf16* A = static_cast<const bf16*>(a);
+    const bf16* W = static_cast<const bf16*>(w);
+    if (tile_shape <= 0) {
+        // 128 x 128 tiles once they cover the chip, 128 x 64 from 96 of the large ones on, else 64 x 64
+        // (measured at the 1B sizes: 273 rows 12.2 / 15.9 / 22.9 us with 64 x 64 / 128 x 64 / 128 x 128,
+        // 512 rows 19.0 / 16.5 / 23.8, 2,048 rows 55.5 / 40.1 / 38.9); a head of 128 needs the full width
+        const long wg128 = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
+        tile_shape = (hd > 64 || wg128 >= compute_units()) ? 128 : (M > 64 && wg128 >= 96) ? 128064 : 64;
+    }
+    if (tile_shape == 128) return launch_tile_rope<4, 4>(A, W, M, N, K, blocked, qt, stream);
+    if (tile_shape == 64 && hd <= 64) return launch_tile_rope<2, 2>(A, W, M, N, K, blocked, qt, stream);
+    if (tile_shape == 128064 && hd <= 64) return launch_tile_rope<4, 2>(A, W, M, N, K, blocked, qt, stream);
     return kErrBadArgument;
 }

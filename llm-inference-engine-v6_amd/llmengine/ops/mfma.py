@@ -66,6 +66,47 @@ def gemm_gated(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, grou
     kernels.swiglu(gu, out, group)
 
 
+declare("llme_gemm_bf16_qkv_rope", [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp])
+
+
+def gemm_qkv_rope_supported(x: torch.Tensor, w_qkv: torch.Tensor, k_cache: torch.Tensor, head_dim: int,
+                            rotary_dim: int) -> bool:
+    return (kernels.policy.fast_gemm and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16
+            and k_cache.dtype == torch.bfloat16 and head_dim in (16, 32, 64, 128) and rotary_dim == head_dim
+            and w_qkv.dim() in (2, 5) and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0 and w_qkv.data_ptr() % 16 == 0)
+
+
+def gemm_qkv_rope(x: torch.Tensor, w_qkv: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor,
+                  seq_idx: torch.Tensor, block_table: torch.Tensor, q_out: torch.Tensor, k_cache: torch.Tensor,
+                  v_cache: torch.Tensor, n_q: int, n_kv: int, head_dim: int, tile: int = 0) -> None:
+    """The q/k/v projection of a step's rows with rotation and cache write in the product's epilogue:
+    x [T, K] bfloat16 (normed), w_qkv [(n_q + 2 n_kv) hd, K] bfloat16 (row-major or blocked); q heads
+    and k heads are rotated at the rows' positions, q goes to q_out [T, n_q hd], k and v into the
+    rows' pages. The 32-bit q/k/v rows that the separate kernels pass between them never exist.
+    Full rotation, head size 16, 32, 64 or 128. tile: 0 (chosen), 64 or 128."""
+    require(x, "x", torch.bfloat16, (None, None))
+    T, K = x.shape
+    n_rows, _ = kernels._require_weight(w_qkv, "w_qkv", torch.bfloat16, K)
+    if n_rows != (n_q + 2 * n_kv) * head_dim:
+        raise kernels.KernelError(f"gemm_qkv_rope: w_qkv has {n_rows} rows, the heads need {(n_q + 2 * n_kv) * head_dim}")
+    require(positions, "positions", torch.int32, (T,))
+    require(seq_idx, "seq_idx", torch.int32, (T,))
+    require(block_table, "block_table", torch.int32, (None, None))
+    require(cos, "cos", torch.float32, (None, head_dim // 2))
+    require(sin, "sin", torch.float32, tuple(cos.shape))
+    require(q_out, "q_out", torch.bfloat16, (T, n_q * head_dim))
+    require(k_cache, "k_cache", torch.bfloat16, (None, n_kv, None, head_dim))
+    page = k_cache.shape[2]
+    require(v_cache, "v_cache", torch.bfloat16, (k_cache.shape[0], n_kv, head_dim, page))
+    if not gemm_qkv_rope_supported(x, w_qkv, k_cache, head_dim, head_dim):
+        raise kernels.KernelError(f"gemm_qkv_rope: head size {head_dim} (16, 32, 64 or 128), K={K} (multiple of 8) or the "
+                                  "operand types are not supported")
+    check(entry("llme_gemm_bf16_qkv_rope")(
+        ptr(x), ptr(w_qkv), T, K, 1 if kernels.is_blocked(w_qkv) else 0, ptr(cos), ptr(sin), ptr(positions), ptr(seq_idx),
+        ptr(block_table), block_table.shape[1], ptr(q_out), ptr(k_cache), ptr(v_cache), n_q, n_kv, head_dim, page,
+        int(tile), stream()), "gemm_qkv_rope")
+
+
 def _fast_gemm(a, w, out, accumulate, fixed_order=False) -> bool:
     if a.dim() != 2 or w.dim() not in (2, 5) or not gemm_bf16_supported(a, w, out, accumulate):
         return False

@@ -110,6 +110,11 @@ class Attention(Mixer):
             # decoding: norm, projection, rotation and the cache write are one kernel
             ops.gemv_norm_rope(x, rms[0], rms[1], self.w_qkv_paired, step.positions, step.seq_idx,
                                block_table, cos, sin, q, k_cache, v_cache, n_q, n_kv, hd)
+        elif (write_cache and rms is None and T > 64 and cos is not None
+              and ops.gemm_qkv_rope_supported(x, self.w_qkv, k_cache, hd, rot)):
+            # many rows (prompts): rotation and the cache write are the projection's epilogue
+            ops.gemm_qkv_rope(x, self.w_qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
+                              n_q, n_kv, hd)
         elif write_cache:
             qkv = step.buffer("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
             if (rms is None and 16 < T <= 64 and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16

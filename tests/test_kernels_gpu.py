@@ -730,3 +730,56 @@ def test_rope_write_of_many_tokens(ops, n_q, n_kv, hd, page, dtype, new):
         v_ref[pg, :, :, off] = v[t]
     assert float((k_cache.cpu().double() - k_ref).abs().max()) < tol * 8
     assert float((v_cache.cpu().double() - v_ref).abs().max()) < tol * 8
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,K,page", [(4, 2, 64, 128, 16), (32, 8, 64, 2048, 16), (3, 1, 128, 96, 32), (5, 3, 32, 72, 16),
+                                                 (6, 2, 16, 64, 48), (24, 8, 128, 512, 16)])
+@pytest.mark.parametrize("new", [[70, 130, 3, 16, 33], [300], [1, 90, 17]])
+@pytest.mark.parametrize("tile", [0, 64, 128, 128064])
+def test_gemm_qkv_rope(ops, n_q, n_kv, hd, K, page, new, tile):
+    """The q/k/v projection with rotation and cache write in its epilogue against the three kernels
+    it replaces (product into 32-bit rows, rotation + cache write): portions that start anywhere in
+    their requests, groups of 16 rows that span two requests or two pages, tiles that hang over the
+    rows and over the heads, row-major and blocked weights."""
+    if tile in (64, 128064) and hd > 64:
+        pytest.skip("a 64-column tile does not hold a head of 128")
+    g = _gen(90)
+    T = sum(new)
+    N = (n_q + 2 * n_kv) * hd
+    x = torch.randn(T, K, generator=g).to(torch.bfloat16)
+    w = (0.05 * torch.randn(N, K, generator=g)).to(torch.bfloat16)
+    ctx = [int(c) for c in torch.randint(0, 3 * page, (len(new),), generator=g)]       # tokens cached before
+    ctx[0] = 16                                                                          # one portion starts at a multiple of 16
+    positions = torch.cat([torch.arange(c, c + n) for c, n in zip(ctx, new)]).to(torch.int32)
+    seq_idx = torch.cat([torch.full((n,), s) for s, n in enumerate(new)]).to(torch.int32)
+    blocks = [(c + n + page - 1) // page for c, n in zip(ctx, new)]
+    perm = torch.randperm(sum(blocks) + 2, generator=g).tolist()
+    table = torch.zeros(len(new), max(blocks), dtype=torch.int32)
+    p = 0
+    for s, nb in enumerate(blocks):
+        for b in range(nb):
+            table[s, b] = perm[p]
+            p += 1
+    max_pos = max(c + n for c, n in zip(ctx, new))
+    inv = 1.0 / (10000.0 ** (torch.arange(hd // 2, dtype=torch.float64) * 2 / hd))
+    ang = torch.arange(max_pos, dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    pages = sum(blocks) + 2
+
+    def fresh():
+        return (torch.zeros(T, n_q * hd, dtype=torch.bfloat16, device=DEV),
+                torch.zeros(pages, n_kv, page, hd, dtype=torch.bfloat16, device=DEV),
+                torch.zeros(pages, n_kv, hd, page, dtype=torch.bfloat16, device=DEV))
+    xd, pd, sd, td = x.to(DEV), positions.to(DEV), seq_idx.to(DEV), table.to(DEV)
+    q0, k0, v0 = fresh()
+    qkv = torch.empty(T, N, device=DEV)
+    ops.gemm(xd, w.to(DEV), qkv)
+    ops.rope_kv_write(qkv, cos, sin, pd, sd, td, q0, k0, v0, n_q, n_kv, hd, hd)
+    for wd in ([w.to(DEV)] + ([ops.block_weight(w.to(DEV))] if K % 32 == 0 else [])):
+        q1, k1, v1 = fresh()
+        ops.gemm_qkv_rope(xd, wd, cos, sin, pd, sd, td, q1, k1, v1, n_q, n_kv, hd, tile=tile)
+        for got, want in ((q1, q0), (k1, k0), (v1, v0)):
+            # (the same sums; the rotation may contract a product and a difference into one rounding)
+            assert (got.float() - want.float()).abs().max() <= 1.6e-2 * want.float().abs().max()
+            assert ((got != want).float().mean()) < 2e-3
+            assert torch.equal(got == 0, want == 0)            # nothing else was written
