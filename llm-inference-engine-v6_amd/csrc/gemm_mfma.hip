@@ -468,40 +468,37 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
 }
 
 // ----------------------------------------------------------------------------------------
-// The tile kernel with slabs that go from memory straight into LDS: on this chip a buffer load
-// can name LDS as its destination, 16 bytes per lane, lane l's bytes landing at the wavefront's
-// LDS base + 16 l. A wavefront's load is thus 1 KB of consecutive LDS:
+// The tile kernel for wide outputs: tiles of 256 x 256 by eight wavefronts (64 x 128 each), whose slabs go
+// from memory straight into LDS. On this chip a buffer load can name LDS as its destination, 16
+// bytes per lane, lane l's bytes landing at the wavefront's LDS base + 16 l. A wavefront's load is
+// thus 1 KB of consecutive LDS:
 //  * W in the blocked layout: one operand block of the matrix instruction ([4 q][16 r][8]: lane
 //    16 q + r holds row r, k = 8 q ..), lane l loading the block's bytes 16 l ..; a wavefront reads
 //    it back as an operand with 1 KB of consecutive addresses.
 //  * A is row-major: a load takes 8 rows x 64 k, whole 128-byte lines (16 rows x 32 k, a block's own
-//    shape, touches twice as many lines per load, and the loads' path is what such a kernel is
-//    short of: measured 856 against 963 TFLOP/s). Lane 32 kb + 8 q + r loads row r, k = 32 kb + 8 q ..,
-//    so that LDS holds the chunk as [2 kb][4 q][8 r][8]: the upper or lower half of two operand
-//    blocks. Chunks lie 1,152 bytes apart, so that the two halves of an operand (rows 0 .. 7 and
-//    8 .. 15 of a block, in neighbouring chunks) fall into different banks.
-// No padding inside what a load writes, no registers and no LDS-write instructions on the way.
-// k advances in slabs of 64 through NSTAGE LDS buffers, NSTAGE - 1 slabs in flight; a turn waits
-// for its slab (the loads are counted by hand: nothing else of a turn goes through the vector
-// memory path), meets the barrier, asks for the slab NSTAGE - 1 turns ahead into the buffer that
-// the turn before has read, and multiplies.
-// Needs: W blocked (N a multiple of 16, K of 32); K a multiple of 8 as everywhere (a slab that
-// hangs over the end of k reads zeros there: the descriptors end with the rows).
+//    shape, touches twice as many lines per load: measured 856 against 963 TFLOP/s). Lane
+//    32 kb + 8 q + r loads row r, k = 32 kb + 8 q .., so that LDS holds the chunk as [2 kb][4 q][8 r][8]:
+//    the upper or lower half of two operand blocks. An operand's two halves (rows 0 .. 7 and 8 .. 15
+//    of a block) lie in neighbouring chunks, 1 KB apart, in the same banks; so the odd chunks hold
+//    their k quarters in the order 1, 0, 3, 2 (a lane of an odd chunk loads the neighbouring
+//    quarter's k), and the two halves of a read fall into different banks without padding.
+// No staging registers, no LDS-write instructions, no padding: that is what lets 160 KB of LDS hold
+// a tile that loads half the bytes per product of a 128 x 128 one. (The same kernel at 128 x 128 and
+// 256 x 128 was slower than the kernel above, which has three slabs in flight in registers; measured
+// 822 and 812 against 954 TFLOP/s at 16,384 x 2,048.)
+// LDS is cut into three buffers for A's slabs (64 k each) and four for halves of W's slabs (32 k:
+// one block per 16 rows), so that A is asked for two slabs ahead and W three half slabs: with two
+// buffers of whole slabs the loads, asked for one slab ahead, arrived late (from asking for A's
+// 32 KB to having them takes 1.06 us, W's 1.4 us, a slab's products 1.1 us; 1,060 against 1,111
+// TFLOP/s). The price is a barrier per half slab, at which a half buffer of W changes hands. The
+// loads are counted by hand (nothing else of a turn goes through the vector memory path).
+// Half turn h (k = 32 h ..) has its operands in registers when it starts. It waits for half slab
+// h + 1, meets the barrier, asks for W's half slab h + 4 into the buffer of h, which everybody has
+// read, and, if h is odd, for A's slab (h - 1) / 2 + 3 into the buffer of the slab that ends here;
+// then it reads the operands of h + 1 while it multiplies.
+// Needs: W blocked (N a multiple of 16, K of 32). A slab that hangs over the end of k reads zeros
+// there (the loads of A's second half get an offset behind the descriptor's end).
 constexpr int DK = 64;
-constexpr int A_CHUNK = 1024 + 128;                    // bytes from one 8-row chunk of A to the next
-
-template <int WR, int WC, int WMT, int WNT>
-constexpr int direct_stage_bytes() {
-    constexpr int chunks = WR * 2 * WMT, blocks = WC * 2 * WNT, waves = WR * WC;    // per slab: 8-row chunks of A, blocks of W
-    constexpr int padded = (chunks + blocks + waves - 1) / waves * waves;           // (a wavefront with one load too many writes zeros there)
-    return chunks * A_CHUNK + (padded - chunks) * 1024;
-}
-template <int WR, int WC, int WMT, int WNT, int NSTAGE>
-constexpr int direct_lds_bytes() {
-    constexpr int slabs = NSTAGE * direct_stage_bytes<WR, WC, WMT, WNT>();
-    constexpr int staged = WR * 16 * WMT * (WC * 16 * WNT + 4) * 4;                 // the epilogue's staged tile
-    return (staged <= 160 * 1024 && staged > slabs) ? staged : slabs;
-}
 
 // Waits until at most N of this wavefront's vector memory loads are still on their way.
 template <int N> __device__ __forceinline__ void wait_vm() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }
@@ -521,16 +518,18 @@ __device__ __forceinline__ void load_b128_to_lds(u32x4 rsrc, unsigned lds_base, 
                  : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
                  : "memory", "m0");
 }
-
-template <int WR, int WC, int WMT, int WNT, int MODE, int NSTAGE>
-__global__ __launch_bounds__(64 * WR * WC, (WR * WC <= 4 ? 2 : 1)) void gemm_tile_direct_kernel(
+template <int WR, int WC, int WMT, int WNT, int MODE>
+__global__ __launch_bounds__(64 * WR * WC, 1) void gemm_tile_direct_kernel(
     const bf16* __restrict__ a, const bf16* __restrict__ w, void* __restrict__ out, int M, int N, int K, int tiles_m,
     int tiles_n, int ksplit, QkvTarget qt) {
     constexpr int BM = WR * 16 * WMT, BN = WC * 16 * WNT, NW = WR * WC;
-    constexpr int AC = BM / 8, WB = BN / 16 * 2, NL = AC + WB;  // loads of a slab: A chunks, then W blocks
-    constexpr int LPW = (NL + NW - 1) / NW;                     // loads per wavefront and slab
-    constexpr int STAGE = direct_stage_bytes<WR, WC, WMT, WNT>();
-    static_assert(LPW * (NSTAGE - 1) < 64, "the count of loads in flight has six bits");
+    constexpr int AC = BM / 8, WB = BN / 16;                    // loads: chunks of a slab of A, blocks of half a slab of W
+    static_assert(AC % NW == 0 && WB % NW == 0, "every wavefront has the same loads");
+    constexpr int LA = AC / NW, LW = WB / NW;
+    constexpr int NSA = 3, NHW = 4;
+    constexpr int A_STAGE = AC * 1024, W_STAGE = WB * 1024, W_BASE = NSA * A_STAGE;
+    static_assert(W_BASE + NHW * W_STAGE <= 160 * 1024, "LDS");
+    static_assert(3 * LW + 2 * LA < 64, "the count of loads in flight has six bits");
     extern __shared__ __align__(16) unsigned char lds_raw[];
 
     const int per_split = tiles_m * tiles_n;
@@ -551,53 +550,44 @@ __global__ __launch_bounds__(64 * WR * WC, (WR * WC <= 4 ? 2 : 1)) void gemm_til
     const int r = lane & 15, q = lane >> 4;
     const int wm = (wave / WC) * (16 * WMT), wn = (wave % WC) * (16 * WNT);
 
+    // this workgroup's share of k, in half slabs (the shares are whole slabs, the last may end in a half)
+    const int nh_all = K / 32;
     const int nk_all = (K + DK - 1) / DK;
     const int nk_per = (nk_all + ksplit - 1) / ksplit;
-    const int kt_begin = split * nk_per;
-    const int kt_end = (kt_begin + nk_per < nk_all) ? kt_begin + nk_per : nk_all;
+    const int h_begin = 2 * split * nk_per;
+    const int h_end = (h_begin + 2 * nk_per < nh_all) ? h_begin + 2 * nk_per : nh_all;
 
-    // Descriptors that begin at the tile's first row and end behind its last row that exists: what
-    // lies behind reads as zeros, without a check, and so does the load that a wavefront has one
-    // too many of (its offset is behind everything). The last slab may hang over the end of k by 32:
-    // in the blocked W that is the next row group's first block, which must not be read, so W's
-    // loads of the slab's second half get an offset behind everything there (k_tail).
     const int a_rows = M - m0 < BM ? M - m0 : BM, w_rows = N - n0 < BN ? N - n0 : BN;
     const u32x4 a_rsrc = raw_descriptor(a + static_cast<size_t>(m0) * K, static_cast<unsigned>(a_rows) * K * 2);
     const u32x4 w_rsrc = raw_descriptor(w + static_cast<size_t>(n0) * K, static_cast<unsigned>(w_rows) * K * 2);
-    // (the slabs' LDS starts at the workgroup's LDS address 0: the kernel has no other LDS)
     const unsigned lds_origin = static_cast<unsigned>(reinterpret_cast<size_t>(
         (__attribute__((address_space(3))) unsigned char*)lds_raw));
     constexpr unsigned kNowhere = 0xFFFFFF00u;
-    unsigned off[LPW], tail_off[LPW], step[LPW], dst[LPW];      // per load: lane offset, the same in the last slab,
-    u32x4 rs[LPW];                                              // bytes from slab to slab, place in the stage
-    const bool k_tail = K % DK != 0;                            // (K is a multiple of 32 here: half a slab is left)
+    unsigned a_off[LA], a_tail[LA], w_off[LW];
 #pragma unroll
-    for (int i = 0; i < LPW; ++i) {
-        const int j = wave + NW * i;                    // (the same in every lane: the choices below are scalar)
-        rs[i] = j < AC ? a_rsrc : w_rsrc;
-        step[i] = j < AC ? DK * 2 : 2048;
-        if (j < AC) {
-            // chunk j: rows 8 j .. 8 j + 7; lane 32 kb + 8 q' + r' loads row r', k = 32 kb + 8 q'
-            const int kb = lane >> 5, q8 = (lane >> 3) & 3, r8 = lane & 7;
-            off[i] = (static_cast<unsigned>(j * 8 + r8) * K + kb * 32 + q8 * 8) * 2;
-            tail_off[i] = kb == 0 ? off[i] : kNowhere;  // (row-major A: k past the end is the next row's start)
-            dst[i] = j * A_CHUNK;
-        } else if (j < NL) {
-            const int blk = j - AC, grp = blk >> 1, kb = blk & 1;
-            off[i] = (static_cast<unsigned>(grp) * (K / 32) + kb) * 1024u + lane * 16u;
-            tail_off[i] = kb == 0 ? off[i] : kNowhere;
-            dst[i] = AC * A_CHUNK + blk * 1024;
-        } else {
-            off[i] = tail_off[i] = kNowhere;
-            dst[i] = AC * A_CHUNK + (j - AC) * 1024;
-        }
+    for (int i = 0; i < LA; ++i) {
+        // chunk j: rows 8 j .. 8 j + 7; lane 32 kb + 8 q' + r' loads row r', k = 32 kb + 8 q' (odd chunks: 8 (q' ^ 1))
+        const int j = wave + NW * i;
+        const int kb = lane >> 5, q8 = ((lane >> 3) & 3) ^ (j & 1), r8 = lane & 7;
+        a_off[i] = (static_cast<unsigned>(j * 8 + r8) * K + kb * 32 + q8 * 8) * 2;
+        a_tail[i] = kb == 0 ? a_off[i] : kNowhere;              // (row-major A: k past the end is the next row's start)
     }
-    auto ask = [&](int kt, int stage) {
-        if (kt >= kt_end) kt = kt_end - 1;              // (past the end: the last slab again, nobody reads it)
-        const bool tail = k_tail && kt == nk_all - 1;
-        const unsigned base = lds_origin + stage * STAGE;
 #pragma unroll
-        for (int i = 0; i < LPW; ++i) load_b128_to_lds(rs[i], base + dst[i], tail ? tail_off[i] : off[i], kt * step[i]);
+    for (int i = 0; i < LW; ++i) w_off[i] = static_cast<unsigned>(wave + NW * i) * (K / 32) * 1024u + lane * 16u;
+    // (past the end of the share: the last one again, nobody reads it)
+    auto ask_a = [&](int kt, int stage) {
+        const int last = (h_end - 1) >> 1;
+        if (kt > last) kt = last;
+        const bool tail = 2 * kt + 1 >= nh_all;                 // the slab is half a slab: k ends in it
+        const unsigned base = lds_origin + stage * A_STAGE + wave * 1024;
+#pragma unroll
+        for (int i = 0; i < LA; ++i) load_b128_to_lds(a_rsrc, base + i * (NW * 1024), tail ? a_tail[i] : a_off[i], kt * (DK * 2));
+    };
+    auto ask_w = [&](int h, int stage) {
+        if (h >= h_end) h = h_end - 1;
+        const unsigned base = lds_origin + W_BASE + stage * W_STAGE + wave * 1024;
+#pragma unroll
+        for (int i = 0; i < LW; ++i) load_b128_to_lds(w_rsrc, base + i * (NW * 1024), w_off[i], h * 1024);
     };
 
     f32x4 acc[WMT][WNT];
@@ -606,17 +596,17 @@ __global__ __launch_bounds__(64 * WR * WC, (WR * WC <= 4 ? 2 : 1)) void gemm_til
 #pragma unroll
         for (int j = 0; j < WNT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    if (kt_begin < kt_end) {
-        // this lane's place in an operand of A: chunk 2 g + r / 8, then [kb][q][r % 8]
-        const unsigned a_lane = (wm / 8 + (r >> 3)) * A_CHUNK + q * 128 + (r & 7) * 16;
-        const unsigned w_lane = AC * A_CHUNK + (wn / 16) * 2048 + lane * 16;
-        auto read_frags = [&](int stage, int kk, bf16x8 (&fa)[WMT], bf16x8 (&fw)[WNT]) {
-            const unsigned char* sA = lds_raw + stage * STAGE + a_lane + kk * 512;
-            const unsigned char* sW = lds_raw + stage * STAGE + w_lane + kk * 1024;
+    if (h_begin < h_end) {
+        // this lane's place in an operand of A: chunk 2 g + r / 8, then [kb][q, or q ^ 1 in odd chunks][r % 8]
+        const unsigned a_lane = (wm / 8 + (r >> 3)) * 1024 + (q ^ (r >> 3)) * 128 + (r & 7) * 16;
+        const unsigned w_lane = W_BASE + (wn / 16) * 1024 + lane * 16;
+        auto read_frags = [&](int sa, int kk, int sw, bf16x8 (&fa)[WMT], bf16x8 (&fw)[WNT]) {
+            const unsigned char* sA = lds_raw + sa * A_STAGE + a_lane + kk * 512;
+            const unsigned char* sW = lds_raw + sw * W_STAGE + w_lane;
 #pragma unroll
-            for (int i = 0; i < WMT; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(sA + i * 2 * A_CHUNK);
+            for (int i = 0; i < WMT; ++i) fa[i] = *reinterpret_cast<const bf16x8*>(sA + i * 2048);
 #pragma unroll
-            for (int j = 0; j < WNT; ++j) fw[j] = *reinterpret_cast<const bf16x8*>(sW + j * 2048);
+            for (int j = 0; j < WNT; ++j) fw[j] = *reinterpret_cast<const bf16x8*>(sW + j * 1024);
         };
         auto multiply = [&](const bf16x8 (&fa)[WMT], const bf16x8 (&fw)[WNT]) {
 #pragma unroll
@@ -625,38 +615,47 @@ __global__ __launch_bounds__(64 * WR * WC, (WR * WC <= 4 ? 2 : 1)) void gemm_til
                 for (int j = 0; j < WNT; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[i], fw[j], acc[i][j], 0, 0, 0);
         };
-        // Every buffer is asked for at the start. A turn multiplies the first half of its slab (whose
-        // operands the turn before has read) while it reads the second half's; then it waits for
-        // the next slab, meets the barrier (every wavefront now holds the whole slab in registers),
-        // asks for the slab NSTAGE turns ahead into the buffer of its own, and multiplies the
-        // second half while it reads the next slab's first operands.
-#pragma unroll
-        for (int s0 = 0; s0 < NSTAGE; ++s0) ask(kt_begin + s0, s0);
-        wait_vm<LPW * (NSTAGE - 1)>();
+        // In front of the loop, what the half turns -5 .. -1 would have asked for, in their order
+        // (W, then A): A(0); W(0); W(1), A(1); W(2); W(3), A(2). The waits count on this order: at an
+        // even half turn h the loads behind W(h + 1) are A, W(h + 2), W(h + 3), A; at an odd one
+        // W(h + 2), A, W(h + 3), and A's slab (h + 1) / 2 is older than W(h + 1).
+        const int kt0 = h_begin >> 1;
+        ask_a(kt0, 0);
+        ask_w(h_begin, 0);
+        ask_w(h_begin + 1, 1);
+        ask_a(kt0 + 1, 1);
+        ask_w(h_begin + 2, 2);
+        ask_w(h_begin + 3, 3);
+        ask_a(kt0 + 2, 2);
+        wait_vm<3 * LW + 2 * LA>();
         lds_barrier();
         bf16x8 fa0[WMT], fw0[WNT];
-        read_frags(0, 0, fa0, fw0);
-        int stage = 0;
-        for (int kt = kt_begin; kt < kt_end; ++kt) {
+        read_frags(0, 0, 0, fa0, fw0);
+        int sa = 0, pair = 0;                           // A's buffer of this slab; W's buffers of it are 2 pair and 2 pair + 1
+        for (int h = h_begin; h < h_end; h += 2) {
             bf16x8 fa1[WMT], fw1[WNT];
-            read_frags(stage, 1, fa1, fw1);
+            wait_vm<2 * LW + 2 * LA>();                 // half slab h + 1 has landed (the later ones may be on their way)
+            lds_barrier();                              // .. everybody's share of it, and everybody has read half slab h
+            ask_w(h + 4, 2 * pair);
+            read_frags(sa, 1, 2 * pair + 1, fa1, fw1);
             multiply(fa0, fw0);
             deal_between_products<kDsRead, WMT + WNT>();
             __builtin_amdgcn_sched_barrier(0);
-            wait_vm<LPW * (NSTAGE - 2)>();              // the next slab has landed (the later ones may be on their way)
-            lds_barrier();                              // .. everybody's share of it, and everybody has read this one
-            ask(kt + NSTAGE, stage);
-            stage = stage + 1 == NSTAGE ? 0 : stage + 1;
-            read_frags(stage, 0, fa0, fw0);
-            multiply(fa1, fw1);
+            wait_vm<2 * LW + LA>();
+            lds_barrier();
+            ask_w(h + 5, 2 * pair + 1);
+            ask_a((h >> 1) + 3, sa);
+            sa = sa + 1 == NSA ? 0 : sa + 1;
+            pair ^= 1;
+            read_frags(sa, 0, 2 * pair, fa0, fw0);
+            if (h + 1 < h_end) multiply(fa1, fw1);      // (a share that ends in half a slab: k ends there)
             deal_between_products<kDsRead, WMT + WNT>();
             __builtin_amdgcn_sched_barrier(0);
         }
     }
     wait_vm<0>();                                       // (loads past the end are still on their way into LDS)
     __syncthreads();                                    // the epilogue reuses the slabs' LDS
-    tile_epilogue<WMT, WNT, MODE, direct_lds_bytes<WR, WC, WMT, WNT, NSTAGE>(), WR, WC>(acc, lds_raw, out, M, N, m0, n0,
-                                                                                         wm, wn, tid, r, q, qt);
+    tile_epilogue<WMT, WNT, MODE, 160 * 1024, WR, WC>(acc, lds_raw, out, M, N, m0, n0, wm, wn, tid, r, q, qt);
 }
 
 template <auto KERNEL, int THREADS = 256>
@@ -705,13 +704,13 @@ static int launch_tile(const bf16* A, const bf16* W, void* out, int M, int N, in
     }
 }
 
-template <int WR, int WC, int WMT, int WNT, int NSTAGE>
+template <int WR, int WC, int WMT, int WNT>
 static int launch_tile_direct(const bf16* A, const bf16* W, void* out, int M, int N, int K, int mode, int ksplit,
-                              hipStream_t stream) {
-    constexpr int LDS = direct_lds_bytes<WR, WC, WMT, WNT, NSTAGE>();
+                                    hipStream_t stream) {
+    constexpr int LDS = 160 * 1024;
     constexpr int BM = WR * 16 * WMT, BN = WC * 16 * WNT;
 #define LLME_DIRECT(MODE) \
-    launch_tile_kernel<gemm_tile_direct_kernel<WR, WC, WMT, WNT, MODE, NSTAGE>, 64 * WR * WC>( \
+    launch_tile_kernel<gemm_tile_direct_kernel<WR, WC, WMT, WNT, MODE>, 64 * WR * WC>( \
         LDS, BM, BN, A, W, out, M, N, K, MODE == kAtomicF32 ? ksplit : 1, stream)
     switch (mode) {
         case kStoreF32: return LLME_DIRECT(kStoreF32);
@@ -850,8 +849,8 @@ using namespace llme;
 // the split over k; tile_shape: 0 chooses, 64 / 128 force the tile kernel with that tile
 // edge also for small M (for tests and measurements). blocked: w is stored in 1 KB blocks of
 // 16 rows x 32 k (see the head of this file; N a multiple of 16, K of 32). direct: the tile kernel
-// whose slabs go from memory straight into LDS (needs blocked; tile_shape also 256256 and 256128 then):
-// -1 where the entry point finds it faster, 0 never, 1 it must.
+// of 256 x 256 whose slabs go from memory straight into LDS (needs blocked): -1 where the entry point
+// finds it faster, 0 never, 1 it must (with tile_shape 256256).
 extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_dtype, int M, int N, int K,
                               int accumulate, int gated, int nw, int ksplit, int tile_shape, int blocked, int direct,
                               hipStream_t stream) {
@@ -967,16 +966,10 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
         // 1,024 and more tiles, 0.9 at 384).
         const long rounds = (static_cast<long>((M + 255) / 256) * ((N + 255) / 256) + cus - 1) / cus;
         const double covered = static_cast<double>(M) * N / (static_cast<double>(rounds) * cus * 65536.0);
-        if (covered >= 0.85) return launch_tile_direct<4, 2, 4, 8, 2>(A, W, out, M, N, K, mode, ksplit, stream);
+        if (covered >= 0.85) return launch_tile_direct<4, 2, 4, 8>(A, W, out, M, N, K, mode, ksplit, stream);
     }
-    if (blocked && direct == 1 && tile_shape != 64) {
-        if (tile_shape == 128096) return launch_tile_direct<2, 2, 4, 3, 2>(A, W, out, M, N, K, mode, ksplit, stream);
-        if (tile_shape == 128064) return launch_tile_direct<2, 2, 4, 2, 2>(A, W, out, M, N, K, mode, ksplit, stream);
-        if (tile_shape == 128) return launch_tile_direct<2, 2, 4, 4, 2>(A, W, out, M, N, K, mode, ksplit, stream);
-        if (tile_shape == 256256) return launch_tile_direct<4, 2, 4, 8, 2>(A, W, out, M, N, K, mode, ksplit, stream);
-        if (tile_shape == 256128) return launch_tile_direct<4, 2, 4, 4, 3>(A, W, out, M, N, K, mode, ksplit, stream);
-        return kErrBadArgument;
-    }
+    if (blocked && direct == 1 && tile_shape == 256256)
+        return launch_tile_direct<4, 2, 4, 8>(A, W, out, M, N, K, mode, ksplit, stream);
     if (direct == 1) return kErrUnsupported;
     if (tile_shape == 128096) return launch_tile<4, 3>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
     if (tile_shape == 128064) return launch_tile<4, 2>(A, W, out, M, N, K, mode, ksplit, blocked, stream);

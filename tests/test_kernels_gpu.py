@@ -270,13 +270,14 @@ def test_gemm_tile(ops, M, N, K, tile):
 
 
 @pytest.mark.parametrize("M,N,K", [(65, 128, 64), (128, 128, 128), (300, 400, 96), (129, 112, 160), (257, 512, 32),
-                                   (2048, 3072, 2048), (1000, 2048, 8192), (333, 208, 2080)])
-@pytest.mark.parametrize("tile", [128, 128096, 128064, 256256, 256128])
-def test_gemm_tile_with_slabs_straight_into_lds(ops, M, N, K, tile):
-    """The tile kernel whose slabs go from memory into LDS without passing through registers
-    (blocked weights): every epilogue, sums cut over k, tiles that hang over the matrix's edges,
-    k of one slab and of many; against the plain product, and bit for bit against the kernel that
-    stages its slabs through registers (both add the same products in the same order)."""
+                                   (2048, 3072, 2048), (1000, 2048, 8192), (333, 208, 2080), (513, 528, 192),
+                                   (700, 1040, 224), (256, 256, 256), (511, 272, 320)])
+def test_gemm_tile_with_slabs_straight_into_lds(ops, M, N, K, tile=256256):
+    """The 256 x 256 tile kernel whose slabs go from memory into LDS without passing through
+    registers (blocked weights): every epilogue, sums cut over k, tiles that hang over the
+    matrix's edges, k of half a slab, of one and of many, ending in half a slab or a whole one;
+    against the plain product, and bit for bit against the kernel that stages its slabs through
+    registers (both add the same products in the same order)."""
     a, w, ref = _bf16_pair(M, N, K, 35)
     ad, wb = a.to(DEV), ops.block_weight(w.to(DEV))
     for dtype, tol in ((torch.float32, 2e-5), (torch.bfloat16, 5e-3)):
