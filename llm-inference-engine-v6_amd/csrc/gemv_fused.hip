@@ -418,6 +418,7 @@ static int launch_gemv_norm_shape(int tpr, const float* h, const int* rows, cons
                                   hipStream_t stream) {
     const RopeTarget none{};
     // tpr: tiles at a time; 12 and 14: 2 and 4 tiles with 16 wavefronts instead of 8
+    if (tpr == 11) return launch_gemv_norm<16, 1, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, blocked, none, stream);
     if (tpr == 12) return launch_gemv_norm<16, 2, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, blocked, none, stream);
     if (tpr == 14) return launch_gemv_norm<16, 4, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, blocked, none, stream);
     if (tpr >= 4) return launch_gemv_norm<8, 4, EPI, TNW>(h, rows, norm_w, eps, w, out, M, N, K, grid, blocked, none, stream);
@@ -432,7 +433,8 @@ using namespace llme;
 // h [*, K] float32; rows: M indices into h or null; norm_w [K] (norm_dtype 0 float32, 1 bfloat16);
 // w bfloat16: plain [N, K], gated [2 N, K] with gate and up rows interleaved in groups of 16;
 // out: plain float32 [M, N], gated bfloat16 [M, N]. tpr (tiles a workgroup of 8 wavefronts works
-// on at a time: 1, 2 or 4) and grid (workgroups): 0 lets the entry point choose. blocked: w is
+// on at a time: 1, 2 or 4; 11, 12, 14: 1, 2, 4 tiles with 16 wavefronts) and grid (workgroups): 0 lets the
+// entry point choose. blocked: w is
 // stored in 1 KB blocks of 16 rows x 32 k (see the head of this file).
 extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_w, int norm_dtype, float eps,
                               const void* w, void* out, int M, int N, int K, int gated, int tpr, int grid,
@@ -449,11 +451,13 @@ extern "C" int llme_gemv_norm(const float* h, const int* rows, const void* norm_
         // few tiles: all 8 wavefronts on one tile, so that every tile has a workgroup of its own;
         // more tiles than compute units: 2 tiles at a time, 4 wavefronts each with several chunks of k
         tpr = tiles <= compute_units() ? 1 : 2;
+        // (one tile per workgroup: 16 wavefronts on it where their sums fit into LDS, see the rotating form)
+        if (tpr == 1 && static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(16) * 2 * 64 * 16 + 64 <= 160 * 1024) tpr = 11;
         // (measured: 16 wavefronts on 2 tiles, 14.2 against 14.8 us at 512 tiles; they need more LDS for their sums)
         const size_t lds16 = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(16) * 2 * 64 * 16 + 64;
         if (gated && tiles > compute_units() && tiles <= 4 * compute_units() && lds16 <= 160 * 1024) tpr = 12;
     }
-    if (tpr != 1 && tpr != 2 && tpr != 4 && tpr != 12 && tpr != 14) return kErrBadArgument;
+    if (tpr != 1 && tpr != 2 && tpr != 4 && tpr != 11 && tpr != 12 && tpr != 14) return kErrBadArgument;
     if (grid <= 0) {
         const int at_a_time = tpr > 10 ? tpr - 10 : tpr;
         grid = (tiles + at_a_time - 1) / at_a_time;
@@ -500,10 +504,19 @@ extern "C" int llme_gemv_norm_rope(const float* h, const void* norm_w, int norm_
                           static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache), n_q, n_kv, hd, page};
     const bf16* W = static_cast<const bf16*>(w);
     if (norm_dtype != kBF16 && norm_dtype != kF32) return kErrBadArgument;
-    if (tpr == 1)
+    if (tpr == 1) {
+        // One tile per workgroup leaves a compute unit to one workgroup: 16 wavefronts then norm up to
+        // 16 rows in one go (a row each) and cut k finer (measured at 192 tiles of k = 2,048, plain
+        // epilogue: 4.39 against 4.61 us at 1 row, 5.75 against 5.95 at 8, 7.12 against 8.88 at 16).
+        const size_t lds16 = static_cast<size_t>(16) * (K + 8) * 2 + static_cast<size_t>(16) * 64 * 16 + 64;
+        if (lds16 <= 160 * 1024)
+            return norm_dtype == kBF16
+                ? launch_gemv_norm<16, 1, kRope, bf16>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream)
+                : launch_gemv_norm<16, 1, kRope, float>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream);
         return norm_dtype == kBF16
             ? launch_gemv_norm<8, 1, kRope, bf16>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream)
             : launch_gemv_norm<8, 1, kRope, float>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream);
+    }
     return norm_dtype == kBF16
         ? launch_gemv_norm<8, 2, kRope, bf16>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream)
         : launch_gemv_norm<8, 2, kRope, float>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream);
