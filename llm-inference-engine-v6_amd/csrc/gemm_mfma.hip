@@ -847,7 +847,7 @@ using namespace llme;
 // groups of 16 and out is bfloat16 [M, N / 2] = silu(gate) * up (tile kernel only).
 // nw, ksplit: 0 lets the entry point choose the skinny kernel's wavefronts per workgroup and
 // the split over k; tile_shape: 0 chooses, 64 / 128 force the tile kernel with that tile
-// edge also for small M (for tests and measurements). blocked: w is stored in 1 KB blocks of
+// edge also for small M (for tests and measurements), 128096, 128064, 96128, 96064 tiles of 128 x 96 and so on. blocked: w is stored in 1 KB blocks of
 // 16 rows x 32 k (see the head of this file; N a multiple of 16, K of 32). direct: the tile kernel
 // of 256 x 256 whose slabs go from memory straight into LDS (needs blocked): -1 where the entry point
 // finds it faster, 0 never, 1 it must (with tile_shape 256256).
@@ -920,15 +920,17 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
             // Medium outputs: narrower tiles can fill the compute units (two workgroups
             // each) more evenly. Estimated time: rounds of one workgroup per compute unit x tile area / measured
             // efficiency of the shape; a workgroup alone on its compute unit overlaps nothing.
-            const long tm = (M + 127) / 128;
-            const int shapes[3] = {128, 128096, 128064};
-            const int widths[3] = {128, 96, 64};
-            const float eff[3] = {1.0f, 0.9f, 0.85f};
+            // (tiles of 96 rows where they cover the rows with less to spare: 273 rows are three row
+            // tiles either way; measured at the 1B sizes, gate/up 39.5 -> 32.6 us at 273 rows, 24.5 -> 21.7 at 192)
+            const int shapes[5] = {128, 128096, 128064, 96128, 96064};
+            const int heights[5] = {128, 128, 128, 96, 96};
+            const int widths[5] = {128, 96, 64, 128, 64};
+            const float eff[5] = {1.0f, 0.9f, 0.85f, 0.84f, 0.78f};
             float best = 0.f;
-            for (int c = 0; c < 3; ++c) {
-                const long wgs = tm * ((N + widths[c] - 1) / widths[c]);
+            for (int c = 0; c < 5; ++c) {
+                const long wgs = static_cast<long>((M + heights[c] - 1) / heights[c]) * ((N + widths[c] - 1) / widths[c]);
                 const long rounds = (wgs + cus - 1) / cus;
-                float cost = static_cast<float>(rounds) * 128.f * widths[c] / eff[c];
+                float cost = static_cast<float>(rounds) * heights[c] * widths[c] / eff[c];
                 // (less so for the gated product, whose epilogue is long: measured at 129 to 256 rows,
                 // 128 x 128 tiles 26.5 against 31 us at the 1B sizes, 36.6 against 43.7 at the 3B sizes)
                 if (wgs <= cus) cost *= (mode == kGatedBF16 ? 1.1f : 1.25f);
@@ -938,15 +940,22 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
                 }
             }
         }
+        // A long sum into few 64 x 64 tiles (down-proj at 129 to 288 rows): tiles of 96 x 64 where they
+        // need no more rows than those of 64, cut over k in 2 or 4 (measured at the 1B sizes and 273
+        // rows: 23.7 against 29.3 us; 18.4 against 21.3 at 192).
+        const bool tall = mode == kAddF32 && ksplit <= 0 && tile_shape == 64 && M > 128 && K >= 4096 &&
+                          (M + 95) / 96 * 96 <= (M + 63) / 64 * 64;
+        if (tall) tile_shape = 96064;
         if (mode == kAddF32 && ksplit <= 0) {
             // A sum that is joined anyway (the residual stream) is cut over k until the tiles fill
             // the chip: 64 x 64 tiles to about two workgroups per compute unit, the larger ones to
             // about one. (Measured at 96 to 512 rows, where the output has few tiles: down-proj of
             // the 1B sizes 48 us uncut against 15 to 33 us, o-proj 13.5 against 7.5 to 14 us.)
-            const int bm = tile_shape == 64 ? 64 : 128;
-            const int bn = tile_shape == 64 ? 64 : tile_shape == 128 ? 128 : tile_shape == 128096 ? 96 : 64;
+            const int bm = tile_shape == 64 ? 64 : (tile_shape == 96064 || tile_shape == 96128) ? 96 : 128;
+            const int bn = (tile_shape == 128 || tile_shape == 96128) ? 128 : tile_shape == 128096 ? 96 : 64;
             const long wgs = static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
             long ks = (tile_shape == 64 ? 2 * cus : cus) / wgs;
+            if (tall) ks = 3 * cus / (2 * wgs) >= 4 ? 4 : 3 * cus / (2 * wgs) >= 2 ? 2 : 1;
             if (tile_shape == 128 && wg128 <= cus && K >= 4096 && ks < 2) ks = 2;
             if (ks > K / 512) ks = K / 512;
             if (ks > 8) ks = 8;
@@ -971,6 +980,8 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     if (blocked && direct == 1 && tile_shape == 256256)
         return launch_tile_direct<4, 2, 4, 8>(A, W, out, M, N, K, mode, ksplit, stream);
     if (direct == 1) return kErrUnsupported;
+    if (tile_shape == 96064) return launch_tile<3, 2>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
+    if (tile_shape == 96128) return launch_tile<3, 4>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
     if (tile_shape == 128096) return launch_tile<4, 3>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
     if (tile_shape == 128064) return launch_tile<4, 2>(A, W, out, M, N, K, mode, ksplit, blocked, stream);
     if (tile_shape == 128) return launch_tile<4, 4>(A, W, out, M, N, K, mode, ksplit, blocked, stream);

@@ -28,7 +28,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
               direct: int = -1, _supported: bool = False) -> None:
     """bfloat16 a [M, K] and w [N, K] -> out [M, N] (float32 or bfloat16), 32-bit accumulation.
     K must be a multiple of 8. gated: w holds gate and up rows interleaved in groups of 16 and
-    out is bfloat16 [M, N / 2] = silu(gate) * up. waves / ksplit / tile (64, 128, 128096, 128064) /
+    out is bfloat16 [M, N / 2] = silu(gate) * up. waves / ksplit / tile (64, 128, 128096, 128064, 96128, 96064) /
     force_tile override the launch choices (tests and measurements); direct: whether the product may
     use the 256 x 256 tile kernel whose slabs go from memory straight into LDS, which needs a blocked w
     (-1: where it pays, 0: never, 1: it must, with tile 256256)."""
