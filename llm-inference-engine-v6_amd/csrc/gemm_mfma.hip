@@ -940,10 +940,11 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
                 }
             }
         }
-        // A long sum into few 64 x 64 tiles (down-proj at 129 to 288 rows): tiles of 96 x 64 where they
-        // need no more rows than those of 64, cut over k in 2 or 4 (measured at the 1B sizes and 273
-        // rows: 23.7 against 29.3 us; 18.4 against 21.3 at 192).
-        const bool tall = mode == kAddF32 && ksplit <= 0 && tile_shape == 64 && M > 128 && K >= 4096 &&
+        // A long sum into an output of few tiles (down-proj at 129 to 288 rows): tiles of 96 x 64 where
+        // they need no more rows than those of 64, cut over k in 2 or 4 up to three workgroups per
+        // compute unit (measured at 273 rows, down-proj of the 1B sizes 23.7 against 29.3 us, of the 8B
+        // sizes 53 against 66; at 192 rows 18.4 against 21.3 and 40 against 43).
+        const bool tall = mode == kAddF32 && ksplit <= 0 && M > 128 && K >= 4096 && wg128 <= cus &&
                           (M + 95) / 96 * 96 <= (M + 63) / 64 * 64;
         if (tall) tile_shape = 96064;
         if (mode == kAddF32 && ksplit <= 0) {
@@ -955,7 +956,7 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
             const int bn = (tile_shape == 128 || tile_shape == 96128) ? 128 : tile_shape == 128096 ? 96 : 64;
             const long wgs = static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
             long ks = (tile_shape == 64 ? 2 * cus : cus) / wgs;
-            if (tall) ks = 3 * cus / (2 * wgs) >= 4 ? 4 : 3 * cus / (2 * wgs) >= 2 ? 2 : 1;
+            if (tall) ks = 3 * cus / wgs >= 4 ? 4 : 3 * cus / wgs >= 2 ? 2 : 1;
             if (tile_shape == 128 && wg128 <= cus && K >= 4096 && ks < 2) ks = 2;
             if (ks > K / 512) ks = K / 512;
             if (ks > 8) ks = 8;
