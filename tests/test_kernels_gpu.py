@@ -309,12 +309,12 @@ def test_gemm_tile_with_slabs_straight_into_lds(ops, M, N, K, tile=256256):
         ops.gemm_bf16(ad, w.to(DEV), torch.empty(M, N, device=DEV), tile=tile, direct=1)     # row-major weights
 
 
-@pytest.mark.parametrize("M", [130, 160, 192, 200, 273, 288, 300])
+@pytest.mark.parametrize("M", [17, 24, 32, 33, 50, 64, 130, 160, 192, 200, 273, 288, 300])
 @pytest.mark.parametrize("N,K", [(2048, 8192), (2048, 2048), (3072, 4096)])
-def test_gemm_sums_of_a_few_hundred_rows(ops, M, N, K):
-    """Sums into the residual stream at the row counts of a prompt portion beside decoded tokens,
-    whatever tile and cut over k the entry point chooses there (tiles of 96 x 64 cut in 2 or 4 for
-    long sums at 129 to 288 rows)."""
+def test_gemm_sums_of_a_few_dozen_to_a_few_hundred_rows(ops, M, N, K):
+    """Sums into the residual stream at the row counts of decoding at larger batches and of a
+    prompt portion beside decoded tokens, whatever tile and cut over k the entry point chooses
+    there (tiles of 96 x 64 cut in 2 or 4 for long sums at 129 to 288 rows)."""
     a, w, ref = _bf16_pair(M, N, K, 37)
     base = torch.randn(M, N, generator=_gen(38))
     for weight in (w.to(DEV), ops.block_weight(w.to(DEV))):
@@ -326,7 +326,7 @@ def test_gemm_sums_of_a_few_hundred_rows(ops, M, N, K):
 @pytest.mark.parametrize("T,FF,K,tile", [(5, 176, 64, 0), (130, 256, 96, 64), (300, 208, 144, 128), (2048, 8192, 2048, 0),
                                          (257, 320, 128, 128096), (190, 352, 72, 128064), (64, 8192, 2048, 0),
                                          (273, 8192, 2048, 0), (192, 8192, 2048, 0), (190, 352, 72, 96064),
-                                         (257, 320, 128, 96128)])
+                                         (257, 320, 128, 96128), (33, 8192, 2048, 0), (20, 352, 72, 0)])
 def test_gemm_gated(ops, T, FF, K, tile):
     x = torch.randn(T, K, generator=_gen(33)).to(torch.bfloat16)
     wg = (0.1 * torch.randn(FF, K, generator=_gen(34))).to(torch.bfloat16)
