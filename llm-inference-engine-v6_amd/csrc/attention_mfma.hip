@@ -39,100 +39,16 @@
 namespace llme {
 
 // ------------------------------------------------------------------------------------------
-// decode: one token per request. A workgroup of four wavefronts takes one split of the keys
-// of one (request, kv head, tile of 16 query heads); its wavefronts take every fourth
-// 32-key block and add up through LDS.
-constexpr int DEC_WAVES = 4;
-
+// decode: one token per request; the work of a workgroup is decode_item (attention_tiles.h).
 template <int HD, bool STREAM>
 __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     bf16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
     int max_blocks, int n_q, int n_kv, int page, float scale, int window, int split_len, int nsplit) {
-    constexpr int DC = (HD + 31) / 32, DT = HD / 16;
-    __shared__ float sh_o[DEC_WAVES][16][HD];
-    __shared__ float sh_m[DEC_WAVES][16], sh_l[DEC_WAVES][16];
-    const int s = blockIdx.x;
-    // What the walk over the keys needs first is asked for together, before anything depends on
-    // it: the request's rows, its length, and the line of its block table that this split's first
-    // page ids lie in (the walk's own lookups then find it in the cache). One after the other
-    // these were three trips to memory in front of the first key.
-    const int row0 = q_start[s], row1 = q_start[s + 1];
-    const int pos = ctx_len[s];                         // the token's position; it sees keys lo..pos
-    const long first_block = static_cast<long>(blockIdx.z) * split_len / page;
-    const int table_line = block_table[static_cast<size_t>(s) * max_blocks +
-                                       (first_block < max_blocks ? first_block : max_blocks - 1)];
-    if (row1 - row0 != 1) return;                       // not a decoding request (whole workgroup)
-    asm volatile("" ::"v"(table_line));                 // (the load is wanted for its effect on the cache)
-    const int G = n_q / n_kv;
-    const int gtiles = (G + 15) / 16;
-    const int kvh = blockIdx.y / gtiles, gt = blockIdx.y % gtiles;
-    const int split = blockIdx.z;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g4 = lane >> 4;
-
-    const int lo_all = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-    int k_begin = split * split_len, k_end = k_begin + split_len;
-    if (k_end > pos + 1) k_end = pos + 1;
-    if (k_begin < (lo_all & ~31)) k_begin = lo_all & ~31;
-
-    const int head = kvh * G + gt * 16 + r;             // this lane's row is a query head
-    const bool row_ok = (gt * 16 + r) < G;
-    bf16x8 qf[1][DC];
-    load_q<HD>(q + (static_cast<size_t>(row0) * n_q + (row_ok ? head : 0)) * HD, row_ok, qf[0]);
-    const int row_pos[1] = {row_ok ? pos : -1};
-    const int row_lo[1] = {lo_all};
-    const int tile_free[1] = {-1};                      // few blocks, heads may be missing: always checked
-    float m[1] = {kNoMax}, l[1] = {0.f};
-    f32x4 o[1][DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD,
-               page_magic_of(page), static_cast<unsigned>(n_kv) * page * HD, static_cast<unsigned>(kvh) * page * HD};
-    const int first = k_begin + __builtin_amdgcn_readfirstlane(wave) * 32;
-    attend_range<HD, 1, STREAM>(kv, first, DEC_WAVES * 32, lo_all, k_end, qf, row_pos, row_lo, tile_free,
-                              scale * kLog2e, m, l, o);
-
-    float lt = l[0];
-    lt += __shfl_xor(lt, 16, 64);
-    lt += __shfl_xor(lt, 32, 64);
-    if (g4 == 0) {
-        sh_m[wave][r] = m[0];
-        sh_l[wave][r] = lt;
-    }
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) sh_o[wave][g4 * 4 + e][dt * 16 + r] = o[0][dt][e];
-    __syncthreads();
-    // join the wavefronts: thread -> (row, dims)
-    for (int item = threadIdx.x; item < 16 * HD; item += DEC_WAVES * 64) {
-        const int row = item / HD, d = item % HD;
-        if (gt * 16 + row >= G) continue;
-        float mx = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < DEC_WAVES; ++w) mx = fmaxf(mx, sh_m[w][row]);
-        float acc = 0.f, lsum = 0.f;
-#pragma unroll
-        for (int w = 0; w < DEC_WAVES; ++w) {
-            const float mw = sh_m[w][row];
-            const float f = (mw <= kNoMax) ? 0.f : exp2f(mw - mx);
-            acc += f * sh_o[w][row][d];
-            lsum += f * sh_l[w][row];
-        }
-        const int h = kvh * G + gt * 16 + row;
-        if (nsplit == 1) {
-            out[(static_cast<size_t>(row0) * n_q + h) * HD + d] = static_cast<bf16>(acc / lsum);
-        } else {
-            const size_t pidx = (static_cast<size_t>(s) * n_q + h) * nsplit + split;
-            part_o[pidx * HD + d] = acc;
-            if (d == 0) {
-                part_ml[pidx * 2] = mx;
-                part_ml[pidx * 2 + 1] = lsum;
-            }
-        }
-    }
+    __shared__ float sh[decode_lds_floats(HD)];
+    decode_item<HD, STREAM>(q, k_cache, v_cache, out, part_o, part_ml, q_start, ctx_len, block_table, max_blocks, n_q,
+                            n_kv, page, scale, window, split_len, nsplit, blockIdx.x, blockIdx.y, blockIdx.z, sh);
 }
 
 // Joins the splits of one (row, head): one wavefront, lanes over the splits for the statistics,
@@ -333,9 +249,14 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
                            int nsplit, int prefill_groups, int qt, int shared_rows, int* queue, int n_rows,
                            int prefill_splits, int prefill_run, float* pre_part_o, float* pre_part_ml,
                            const Tuning& tuning, hipStream_t stream) {
-    if (n_decode > 0) {
-        const int G = n_q / n_kv;
-        const dim3 grid(n_seq, n_kv * ((G + 15) / 16), nsplit);
+    const int head_tiles = n_kv * ((n_q / n_kv + 15) / 16);
+    // A step with decoded tokens and prompt portions: where the prompt kernel that shares K and V
+    // through LDS runs, it takes the decode work items into its launch (the two kinds of work do
+    // not depend on each other; measured at the 1B sizes, a 256-token portion beside 17 decoded
+    // tokens, one after the other they took 17.8 + 21.4 us a layer).
+    const bool together = n_decode > 0 && prefill_groups > 0 && shared_rows > 0 && decode_reads_once(tuning);
+    if (n_decode > 0 && !together) {
+        const dim3 grid(n_seq, head_tiles, nsplit);
         if (decode_reads_once(tuning))
             hipLaunchKernelGGL((attention_decode_kernel<HD, true>), grid, dim3(DEC_WAVES * 64), 0, stream, q, kc, vc, out,
                                part_o, part_ml, q_start, ctx_len, table, max_blocks, n_q, n_kv, page, scale, window,
@@ -350,11 +271,24 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
     }
     if (prefill_groups > 0) {
         if (shared_rows > 0) {
+            DecodeBeside beside;
+            if (together) {
+                beside.part_o = part_o;
+                beside.part_ml = part_ml;
+                beside.head_tiles = head_tiles;
+                beside.split_len = split_len;
+                beside.nsplit = nsplit;
+                beside.blocks = n_seq * head_tiles * nsplit;
+            }
             const int status = launch_prefill_shared(q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q,
                                                      n_kv, HD, page, scale, window, prefill_groups, shared_rows, queue,
                                                      prefill_splits, prefill_run, pre_part_o, pre_part_ml,
-                                                     tuning.key_waves, stream);
-            if (status != 0 || prefill_splits <= 1) return status;
+                                                     tuning.key_waves, beside, stream);
+            if (status != 0) return status;
+            if (together && nsplit > 1)
+                hipLaunchKernelGGL(attention_join_kernel, dim3(n_seq, n_q), dim3(64), 0, stream, part_o, part_ml, out,
+                                   q_start, n_q, HD, nsplit);
+            if (prefill_splits <= 1) return launch_status();
             hipLaunchKernelGGL(attention_join_rows_kernel, dim3(n_rows, n_q), dim3(64), 0, stream, pre_part_o,
                                pre_part_ml, out, q_start, ctx_len, n_seq, n_q, HD, prefill_splits, prefill_run,
                                shared_rows, window);

@@ -375,10 +375,20 @@ __global__ __launch_bounds__(256 * KW) void attention_prefill_shared_kernel(
     bf16* __restrict__ out, const int* __restrict__ q_start, const int* __restrict__ ctx_len,
     const int* __restrict__ block_table, int max_blocks, int n_seq, int n_q, int n_kv, int page, float scale,
     int window, int spans, int* __restrict__ queue, int nsplit, int run, float* __restrict__ part_o,
-    float* __restrict__ part_ml) {
+    float* __restrict__ part_ml, DecodeBeside beside) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     __shared__ int next_item;
     bf16* lds = reinterpret_cast<bf16*>(lds_raw);
+    if (static_cast<int>(blockIdx.x) < beside.blocks) {
+        // one of the step's decode work items: the workgroup's first four wavefronts, the stages' LDS
+        static_assert(decode_lds_floats(HD) * 4 <= StageLayout<HD>::BYTES, "the decode item's sums must fit into the stages");
+        if (threadIdx.x >= DEC_WAVES * 64) return;
+        const int b = blockIdx.x, per_seq = beside.head_tiles * beside.nsplit;
+        decode_item<HD, true>(q, k_cache, v_cache, out, beside.part_o, beside.part_ml, q_start, ctx_len, block_table,
+                              max_blocks, n_q, n_kv, page, scale, window, beside.split_len, beside.nsplit, b / per_seq,
+                              (b % per_seq) / beside.nsplit, b % beside.nsplit, reinterpret_cast<float*>(lds_raw));
+        return;
+    }
     const int head_groups = n_q / HPW;
     const int n_items = spans * head_groups * (SPLIT ? nsplit : 1);
     for (;;) {
@@ -395,7 +405,7 @@ __global__ __launch_bounds__(256 * KW) void attention_prefill_shared_kernel(
     if (threadIdx.x == 0) {
         // whoever leaves last has seen every other workgroup take its final number: nobody touches
         // the counter any more
-        if (atomicAdd(queue + 1, 1) == static_cast<int>(gridDim.x) - 1) {
+        if (atomicAdd(queue + 1, 1) == static_cast<int>(gridDim.x) - beside.blocks - 1) {
             atomicExch(queue, 0);
             atomicExch(queue + 1, 0);
         }
@@ -420,7 +430,7 @@ template <int HD, int QT, int HPW, int KW, bool SPLIT>
 static int launch_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, const int* q_start,
                          const int* ctx_len, const int* table, int max_blocks, int n_seq, int n_q, int n_kv, int page,
                          float scale, int window, int items, int* queue, int nsplit, int run, float* part_o,
-                         float* part_ml, hipStream_t stream) {
+                         float* part_ml, const DecodeBeside& beside, hipStream_t stream) {
     constexpr int LDS = StageLayout<HD>::BYTES;
     auto kernel = attention_prefill_shared_kernel<HD, QT, HPW, KW, SPLIT>;
     static bool attr_set = false;                      // per instantiation
@@ -442,16 +452,17 @@ static int launch_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* ou
         resident = cus * (per_cu > 0 ? per_cu : 1);
     }
     const int n_items = items * (n_q / HPW) * (SPLIT ? nsplit : 1);
-    hipLaunchKernelGGL(kernel, dim3(n_items < resident ? n_items : resident), dim3(256 * KW), LDS, stream, q, kc, vc, out,
-                       q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, page, scale, window, items, queue, nsplit,
-                       run, part_o, part_ml);
+    hipLaunchKernelGGL(kernel, dim3(beside.blocks + (n_items < resident ? n_items : resident)), dim3(256 * KW), LDS, stream,
+                       q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, page, scale, window, items,
+                       queue, nsplit, run, part_o, part_ml, beside);
     return launch_status();
 }
 
 int launch_prefill_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* out, const int* q_start,
                           const int* ctx_len, const int* table, int max_blocks, int n_seq, int n_q, int n_kv, int hd,
                           int page, float scale, int window, int items, int rows_per_item, int* queue, int nsplit,
-                          int run, float* part_o, float* part_ml, int key_waves, hipStream_t stream) {
+                          int run, float* part_o, float* part_ml, int key_waves, const DecodeBeside& beside,
+                          hipStream_t stream) {
     if (queue == nullptr) return kErrBadArgument;
     if (nsplit < 1 || (nsplit > 1 && (run < 1 || part_o == nullptr || part_ml == nullptr))) return kErrBadArgument;
     const int hpw = heads_per_workgroup(n_q, n_kv);
@@ -461,7 +472,7 @@ int launch_prefill_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* o
     int kw = static_cast<long>(items) * (n_q / hpw) <= kSplitBelowItems ? 2 : 1;
     if (key_waves == 1 || key_waves == 2) kw = key_waves;  // (forced by the caller: tests, measurements)
 #define LLME_SHARED_ARGS q, kc, vc, out, q_start, ctx_len, table, max_blocks, n_seq, n_q, n_kv, page, scale, window, \
-                         items, queue, nsplit, run, part_o, part_ml, stream
+                         items, queue, nsplit, run, part_o, part_ml, beside, stream
 #define LLME_SHARED(HD, QT, HPW)                                                       \
     if (hd == HD && rows == 16 * QT && hpw == HPW) {                                   \
         if (nsplit > 1)                                                                \

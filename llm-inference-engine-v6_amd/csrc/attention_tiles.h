@@ -349,16 +349,127 @@ __device__ __forceinline__ void load_q(const bf16* qrow, bool ok, bf16x8 (&qf)[(
 }
 
 
+// ------------------------------------------------------------------------------------------
+// decode: one token per request. A workgroup's four wavefronts (the first DEC_WAVES of it) take
+// one split of the keys of one (request s, kv head and tile of 16 query heads `head_tile`, split);
+// they take every fourth 32-key block each and add up through LDS (sh: decode_lds_floats(HD)
+// floats). A device function so that two kernels can hold it: the decode kernel, and the kernel
+// that runs a step's prompt portions beside its decoded tokens in one launch.
+constexpr int DEC_WAVES = 4;
+__host__ __device__ constexpr int decode_lds_floats(int hd) { return DEC_WAVES * 16 * hd + 2 * DEC_WAVES * 16; }
+
+template <int HD, bool STREAM>
+__device__ __forceinline__ void decode_item(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    bf16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
+    const int* __restrict__ q_start, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
+    int max_blocks, int n_q, int n_kv, int page, float scale, int window, int split_len, int nsplit, int s,
+    int head_tile, int split, float* sh) {
+    constexpr int DC = (HD + 31) / 32, DT = HD / 16;
+    float (*sh_o)[16][HD] = reinterpret_cast<float (*)[16][HD]>(sh);
+    float (*sh_m)[16] = reinterpret_cast<float (*)[16]>(sh + DEC_WAVES * 16 * HD);
+    float (*sh_l)[16] = sh_m + DEC_WAVES;
+    // What the walk over the keys needs first is asked for together, before anything depends on
+    // it: the request's rows, its length, and the line of its block table that this split's first
+    // page ids lie in (the walk's own lookups then find it in the cache). One after the other
+    // these were three trips to memory in front of the first key.
+    const int row0 = q_start[s], row1 = q_start[s + 1];
+    const int pos = ctx_len[s];                         // the token's position; it sees keys lo..pos
+    const long first_block = static_cast<long>(split) * split_len / page;
+    const int table_line = block_table[static_cast<size_t>(s) * max_blocks +
+                                       (first_block < max_blocks ? first_block : max_blocks - 1)];
+    if (row1 - row0 != 1) return;                       // not a decoding request (whole workgroup)
+    asm volatile("" ::"v"(table_line));                 // (the load is wanted for its effect on the cache)
+    const int G = n_q / n_kv;
+    const int gtiles = (G + 15) / 16;
+    const int kvh = head_tile / gtiles, gt = head_tile % gtiles;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g4 = lane >> 4;
+
+    const int lo_all = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    int k_begin = split * split_len, k_end = k_begin + split_len;
+    if (k_end > pos + 1) k_end = pos + 1;
+    if (k_begin < (lo_all & ~31)) k_begin = lo_all & ~31;
+
+    const int head = kvh * G + gt * 16 + r;             // this lane's row is a query head
+    const bool row_ok = (gt * 16 + r) < G;
+    bf16x8 qf[1][DC];
+    load_q<HD>(q + (static_cast<size_t>(row0) * n_q + (row_ok ? head : 0)) * HD, row_ok, qf[0]);
+    const int row_pos[1] = {row_ok ? pos : -1};
+    const int row_lo[1] = {lo_all};
+    const int tile_free[1] = {-1};                      // few blocks, heads may be missing: always checked
+    float m[1] = {kNoMax}, l[1] = {0.f};
+    f32x4 o[1][DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD,
+               page_magic_of(page), static_cast<unsigned>(n_kv) * page * HD, static_cast<unsigned>(kvh) * page * HD};
+    const int first = k_begin + __builtin_amdgcn_readfirstlane(wave) * 32;
+    attend_range<HD, 1, STREAM>(kv, first, DEC_WAVES * 32, lo_all, k_end, qf, row_pos, row_lo, tile_free,
+                              scale * kLog2e, m, l, o);
+
+    float lt = l[0];
+    lt += __shfl_xor(lt, 16, 64);
+    lt += __shfl_xor(lt, 32, 64);
+    if (g4 == 0) {
+        sh_m[wave][r] = m[0];
+        sh_l[wave][r] = lt;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sh_o[wave][g4 * 4 + e][dt * 16 + r] = o[0][dt][e];
+    __syncthreads();
+    // join the wavefronts: thread -> (row, dims)
+    for (int item = threadIdx.x; item < 16 * HD; item += DEC_WAVES * 64) {
+        const int row = item / HD, d = item % HD;
+        if (gt * 16 + row >= G) continue;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; ++w) mx = fmaxf(mx, sh_m[w][row]);
+        float acc = 0.f, lsum = 0.f;
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; ++w) {
+            const float mw = sh_m[w][row];
+            const float f = (mw <= kNoMax) ? 0.f : exp2f(mw - mx);
+            acc += f * sh_o[w][row][d];
+            lsum += f * sh_l[w][row];
+        }
+        const int h = kvh * G + gt * 16 + row;
+        if (nsplit == 1) {
+            out[(static_cast<size_t>(row0) * n_q + h) * HD + d] = static_cast<bf16>(acc / lsum);
+        } else {
+            const size_t pidx = (static_cast<size_t>(s) * n_q + h) * nsplit + split;
+            part_o[pidx * HD + d] = acc;
+            if (d == 0) {
+                part_ml[pidx * 2] = mx;
+                part_ml[pidx * 2 + 1] = lsum;
+            }
+        }
+    }
+}
+
+
 // The prefill kernel that shares K and V blocks among a workgroup's wavefronts through LDS
 // (attention_prefill.hip). rows_per_item: rows of one work item, see prefill_shared_rows; queue:
 // two integers that are zero and that no other launch in flight uses. nsplit > 1: an item's keys
 // are cut into key_runs(...) runs of `run` stretches; items with one run write out, the runs of
 // the others go to part_o [rows, n_q, nsplit, hd] and part_ml [rows, n_q, nsplit, 2] (by batch
 // row) and the caller joins them.
+// beside: the same step's decoded tokens, for the launch to hold as well (blocks = 0: none): its
+// first `blocks` workgroups each take one decode_item (read-once loads) and leave; the two kinds
+// of work do not depend on each other, and each alone leaves most of the chip waiting for loads.
+struct DecodeBeside {
+    float* part_o = nullptr;
+    float* part_ml = nullptr;
+    int head_tiles = 0, split_len = 0, nsplit = 0;      // grid of the decode kernel: (n_seq, head_tiles, nsplit)
+    int blocks = 0;                                     // n_seq * head_tiles * nsplit
+};
 int launch_prefill_shared(const bf16* q, const bf16* k_cache, const bf16* v_cache, bf16* out, const int* q_start,
                           const int* ctx_len, const int* block_table, int max_blocks, int n_seq, int n_q, int n_kv,
                           int hd, int page, float scale, int window, int items, int rows_per_item, int* queue,
-                          int nsplit, int run, float* part_o, float* part_ml, int key_waves, hipStream_t stream);
+                          int nsplit, int run, float* part_o, float* part_ml, int key_waves, const DecodeBeside& beside,
+                          hipStream_t stream);
 
 // Runs that the keys [k_begin, key_end) of a prefill work item are cut into: `run` stretches of 64
 // keys each, at most max_runs (the last run then takes the rest).
