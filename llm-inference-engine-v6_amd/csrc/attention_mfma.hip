@@ -91,29 +91,25 @@ __device__ __forceinline__ void join_splits(const float* __restrict__ part_o, co
     }
 }
 
-// The decode kernel's splits: grid (request, head); parts indexed by request.
-__global__ __launch_bounds__(64) void attention_join_kernel(const float* __restrict__ part_o,
-                                                            const float* __restrict__ part_ml, bf16* __restrict__ out,
-                                                            const int* __restrict__ q_start, int n_q, int hd, int nsplit) {
-    __shared__ float weight[64];
-    const int s = blockIdx.x, h = blockIdx.y;
+// The decode kernel's splits of (request s, head h); parts indexed by request.
+__device__ __forceinline__ void join_decode_splits(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                   bf16* __restrict__ out, const int* __restrict__ q_start, int n_q,
+                                                   int hd, int nsplit, int s, int h, float* weight) {
     const int row0 = q_start[s];
     if (q_start[s + 1] - row0 != 1) return;
     join_splits(part_o, part_ml, out + (static_cast<size_t>(row0) * n_q + h) * hd,
                 (static_cast<size_t>(s) * n_q + h) * nsplit, hd, nsplit, weight);
 }
 
-// The prefill kernel's key runs: grid (batch row, head); parts indexed by batch row. Rows of
+// The prefill kernel's key runs of (batch row, head h); parts indexed by batch row. Rows of
 // requests that bring one token belong to the decode kernel and are left alone, and so are rows
 // of work items with a single run, which wrote their output themselves. span_rows: rows of one
 // work item; the row's item and its number of runs are found as the prefill kernel finds them.
-__global__ __launch_bounds__(64) void attention_join_rows_kernel(const float* __restrict__ part_o,
-                                                                 const float* __restrict__ part_ml,
-                                                                 bf16* __restrict__ out, const int* __restrict__ q_start,
-                                                                 const int* __restrict__ ctx_len, int n_seq, int n_q,
-                                                                 int hd, int nsplit, int run, int span_rows, int window) {
-    __shared__ float weight[64];
-    const int row = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+__device__ __forceinline__ void join_row_runs(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                              bf16* __restrict__ out, const int* __restrict__ q_start,
+                                              const int* __restrict__ ctx_len, int n_seq, int n_q, int hd, int nsplit,
+                                              int run, int span_rows, int window, int row, int h, float* weight) {
+    const int lane = threadIdx.x;
     int first_row = -1, n_new = 0, ctx = 0;             // the row's request (the same in every lane)
     for (int first = 0; first < n_seq; first += 64) {
         const int i = first + lane;
@@ -142,6 +138,39 @@ __global__ __launch_bounds__(64) void attention_join_rows_kernel(const float* __
     if (runs == 1) return;
     join_splits(part_o, part_ml, out + (static_cast<size_t>(row) * n_q + h) * hd,
                 (static_cast<size_t>(row) * n_q + h) * nsplit, hd, runs, weight);
+}
+
+// grid (request, head)
+__global__ __launch_bounds__(64) void attention_join_kernel(const float* __restrict__ part_o,
+                                                            const float* __restrict__ part_ml, bf16* __restrict__ out,
+                                                            const int* __restrict__ q_start, int n_q, int hd, int nsplit) {
+    __shared__ float weight[64];
+    join_decode_splits(part_o, part_ml, out, q_start, n_q, hd, nsplit, blockIdx.x, blockIdx.y, weight);
+}
+
+// grid (batch row, head)
+__global__ __launch_bounds__(64) void attention_join_rows_kernel(const float* __restrict__ part_o,
+                                                                 const float* __restrict__ part_ml,
+                                                                 bf16* __restrict__ out, const int* __restrict__ q_start,
+                                                                 const int* __restrict__ ctx_len, int n_seq, int n_q,
+                                                                 int hd, int nsplit, int run, int span_rows, int window) {
+    __shared__ float weight[64];
+    join_row_runs(part_o, part_ml, out, q_start, ctx_len, n_seq, n_q, hd, nsplit, run, span_rows, window, blockIdx.x,
+                  blockIdx.y, weight);
+}
+
+// Both joins of a step that holds decoded tokens and prompt portions, in one launch: grid
+// (requests + batch rows, head); the first n_seq workgroups of a head join the decode splits.
+__global__ __launch_bounds__(64) void attention_join_both_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, int nsplit,
+    const float* __restrict__ pre_part_o, const float* __restrict__ pre_part_ml, int pre_nsplit, int run, int span_rows,
+    bf16* __restrict__ out, const int* __restrict__ q_start, const int* __restrict__ ctx_len, int n_seq, int n_q, int hd,
+    int window) {
+    __shared__ float weight[64];
+    const int x = blockIdx.x;
+    if (x < n_seq) join_decode_splits(part_o, part_ml, out, q_start, n_q, hd, nsplit, x, blockIdx.y, weight);
+    else join_row_runs(pre_part_o, pre_part_ml, out, q_start, ctx_len, n_seq, n_q, hd, pre_nsplit, run, span_rows, window,
+                       x - n_seq, blockIdx.y, weight);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -285,6 +314,12 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
                                                      prefill_splits, prefill_run, pre_part_o, pre_part_ml,
                                                      tuning.key_waves, beside, stream);
             if (status != 0) return status;
+            if (together && nsplit > 1 && prefill_splits > 1) {
+                hipLaunchKernelGGL(attention_join_both_kernel, dim3(n_seq + n_rows, n_q), dim3(64), 0, stream, part_o,
+                                   part_ml, nsplit, pre_part_o, pre_part_ml, prefill_splits, prefill_run, shared_rows, out,
+                                   q_start, ctx_len, n_seq, n_q, HD, window);
+                return launch_status();
+            }
             if (together && nsplit > 1)
                 hipLaunchKernelGGL(attention_join_kernel, dim3(n_seq, n_q), dim3(64), 0, stream, part_o, part_ml, out,
                                    q_start, n_q, HD, nsplit);

@@ -466,6 +466,22 @@ def test_attention_prefill_cut_keys(ops, n_q, n_kv, hd, page, splits, key_waves,
     assert _rel(out, ref) < 8e-3
 
 
+@pytest.mark.parametrize("n_q,n_kv,hd,page", [(8, 2, 64, 16), (32, 8, 64, 16), (6, 2, 128, 32), (6, 2, 48, 16)])
+@pytest.mark.parametrize("splits,key_waves", [(1, -1), (3, -1), (4, 3), (2, 2)])
+def test_attention_decoded_tokens_beside_prompt_portions(ops, n_q, n_kv, hd, page, splits, key_waves):
+    """A step with decoded tokens far into their requests (their keys cut into several splits) and
+    prompt portions (their keys whole or cut into runs): where the prompt kernel shares K and V
+    through LDS, one launch holds both kinds of work and one launch both joins; head size 48 takes
+    the separate kernels."""
+    lens = [900, 700, 1300, 2, 640, 33, 257]
+    news = [1, 40, 1, 2, 1, 1, 130]
+    out, ref, plan = _attn_case(ops, lens, news, n_q, n_kv, hd, page, seed=66, prefill_splits=splits if hd != 48 else None,
+                                prefill_run=3, tuning=ops.mfma.attention_tuning(shared=key_waves))
+    assert plan["n_decode"] == 4 and plan["nsplit"] > 1
+    assert not out.isnan().any()
+    assert _rel(out, ref) < 8e-3
+
+
 @pytest.mark.parametrize("window", [1, 64, 65, 200])
 def test_attention_prefill_cut_keys_window(ops, window):
     out, ref, _ = _attn_case(ops, [600, 70, 190], [140, 70, 2], 8, 2, 64, 16, window=window, seed=64, prefill_splits=4,
