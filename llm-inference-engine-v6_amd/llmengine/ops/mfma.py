@@ -175,6 +175,10 @@ PREFILL_ITEMS_WANTED: int | None = None        # None: two per compute unit
 PREFILL_CUT_ITEMS: int | None = None           # None: half a workgroup per compute unit
 PREFILL_MIN_RUN = 512
 PREFILL_MAX_SPLITS = 16
+PREFILL_MIN_SPLITS = 3
+# Two runs are not worth their join: a 256-token portion beside 17 decoded tokens at the 1B sizes takes
+# 2.18 ms in two runs against 2.07 whole behind 1,024 tokens, 2.28 against 2.27 behind 2,048 (four
+# runs: 2.20), and behind 3,000 tokens 2.32 in three or six runs against 2.49 whole.
 # (A whole prompt of 2,048 tokens, whose last rows' items walk twice the average, was also tried with
 # the items behind 1,024 keys cut in two: 6.5 to 6.6 ms against 5.95 whole; the partial outputs and
 # the join cost more than the evener load wins.)
@@ -207,6 +211,8 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
         if items <= (PREFILL_CUT_ITEMS or compute_units() // 2):
             splits = max(1, min((PREFILL_ITEMS_WANTED or 2 * compute_units()) // items, keys // PREFILL_MIN_RUN,
                                 PREFILL_MAX_SPLITS))
+            if splits < PREFILL_MIN_SPLITS:
+                splits = 1                                 # (two runs win less than their join costs)
             stretches = (keys + 63) // 64
             run = (stretches + splits - 1) // splits       # stretches of 64 keys per run
         if splits > 1:

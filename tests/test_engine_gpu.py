@@ -105,6 +105,7 @@ def test_prompt_portions_with_cut_keys_match_plain(zoo, name, schedule, min_run,
     from llmengine.ops import mfma
     monkeypatch.setattr(mfma, "PREFILL_MIN_RUN", min_run)
     monkeypatch.setattr(mfma, "PREFILL_MAX_SPLITS", max_splits)
+    monkeypatch.setattr(mfma, "PREFILL_MIN_SPLITS", 2)
     cut = []
     plan_attention = mfma.plan_attention
 
