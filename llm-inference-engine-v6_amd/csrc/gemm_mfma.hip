@@ -944,7 +944,8 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
         // they need no more rows than those of 64, cut over k in 2 or 4 up to three workgroups per
         // compute unit (measured at 273 rows, down-proj of the 1B sizes 23.7 against 29.3 us, of the 8B
         // sizes 53 against 66; at 192 rows 18.4 against 21.3 and 40 against 43).
-        const bool tall = mode == kAddF32 && ksplit <= 0 && M > 128 && K >= 4096 && wg128 <= cus &&
+        // (and at 65 to 96 rows, one row tile: down-proj of the 1B sizes 13.5 against 14.7 us, of the 3B sizes 16.6 against 21.1)
+        const bool tall = mode == kAddF32 && ksplit <= 0 && M > 64 && K >= 4096 && wg128 <= cus &&
                           (M + 95) / 96 * 96 <= (M + 63) / 64 * 64;
         if (tall) tile_shape = 96064;
         if (mode == kAddF32 && ksplit <= 0) {
@@ -956,7 +957,7 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
             const int bn = (tile_shape == 128 || tile_shape == 96128) ? 128 : tile_shape == 128096 ? 96 : 64;
             const long wgs = static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
             long ks = (tile_shape == 64 ? 2 * cus : cus) / wgs;
-            if (tall) ks = 3 * cus / wgs >= 4 ? 4 : 3 * cus / wgs >= 2 ? 2 : 1;
+            if (tall) ks = (M <= 96 && K >= 8192 && 3 * cus / wgs >= 8) ? 8 : 3 * cus / wgs >= 4 ? 4 : 3 * cus / wgs >= 2 ? 2 : 1;
             if (tile_shape == 128 && wg128 <= cus && K >= 4096 && ks < 2) ks = 2;
             if (ks > K / 512) ks = K / 512;
             if (ks > 8) ks = 8;

@@ -309,7 +309,7 @@ def test_gemm_tile_with_slabs_straight_into_lds(ops, M, N, K, tile=256256):
         ops.gemm_bf16(ad, w.to(DEV), torch.empty(M, N, device=DEV), tile=tile, direct=1)     # row-major weights
 
 
-@pytest.mark.parametrize("M", [17, 24, 32, 33, 50, 64, 130, 160, 192, 200, 273, 288, 300])
+@pytest.mark.parametrize("M", [17, 24, 32, 33, 50, 64, 65, 81, 96, 97, 130, 160, 192, 200, 273, 288, 300])
 @pytest.mark.parametrize("N,K", [(2048, 8192), (2048, 2048), (3072, 4096)])
 def test_gemm_sums_of_a_few_dozen_to_a_few_hundred_rows(ops, M, N, K):
     """Sums into the residual stream at the row counts of decoding at larger batches and of a
