@@ -258,9 +258,12 @@ __device__ __forceinline__ void load8(const float* src, float (&v)[8]) {
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
 }
 
-template <typename TQ, typename TC>
+// ZERO: every value of qkv is set to zero once it has been read (each is read by one thread, once, when
+// the cache is written too): a buffer that a product cut over k adds its parts into is then ready
+// for the next layer's product without a kernel that clears it.
+template <typename TQ, typename TC, bool ZERO>
 __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
-    const float* __restrict__ qkv, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    float* qkv, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
     const int* __restrict__ positions, const int* __restrict__ seq_idx, const int* __restrict__ block_table,
     int max_blocks, TQ* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache, int n_q, int n_kv,
     int hd, int page, int write_cache) {
@@ -272,20 +275,27 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
         off = pos % page;
     }
     const int half = hd / 2, hv = half / 8, dv = hd / 8;
-    const float* row = qkv + static_cast<size_t>(t) * (n_q + 2 * n_kv) * hd;
+    float* row = qkv + static_cast<size_t>(t) * (n_q + 2 * n_kv) * hd;
     const float* cs = cos_t + static_cast<size_t>(pos) * half;
     const float* sn = sin_t + static_cast<size_t>(pos) * half;
     const int q_items = n_q * hv, k_items = n_kv * hv, v_items = n_kv * dv;
     const int items = q_items + (write_cache ? k_items + v_items : 0);
+    const float4 zero4{0.f, 0.f, 0.f, 0.f};
     for (int it = threadIdx.x; it < items; it += blockDim.x) {
         if (it < q_items + k_items) {
             const bool is_q = it < q_items;
             const int e = is_q ? it : it - q_items;
             const int h = e / hv, i = (e % hv) * 8;
-            const float* src = row + (is_q ? 0 : n_q * hd) + h * hd + i;
+            float* src = row + (is_q ? 0 : n_q * hd) + h * hd + i;
             float a[8], b[8], c[8], sv[8], lo[8], hi[8];
             load8(src, a);
             load8(src + half, b);
+            if (ZERO) {
+                reinterpret_cast<float4*>(src)[0] = zero4;
+                reinterpret_cast<float4*>(src)[1] = zero4;
+                reinterpret_cast<float4*>(src + half)[0] = zero4;
+                reinterpret_cast<float4*>(src + half)[1] = zero4;
+            }
             load8(cs + i, c);
             load8(sn + i, sv);
 #pragma unroll
@@ -306,7 +316,12 @@ __global__ __launch_bounds__(256) void rope_kv_write_vec_kernel(
             const int e = it - q_items - k_items;
             const int h = e / dv, d0 = (e % dv) * 8;
             float v[8];
-            load8(row + (n_q + n_kv) * hd + h * hd + d0, v);
+            float* src = row + (n_q + n_kv) * hd + h * hd + d0;
+            load8(src, v);
+            if (ZERO) {
+                reinterpret_cast<float4*>(src)[0] = zero4;
+                reinterpret_cast<float4*>(src)[1] = zero4;
+            }
             TC* dst = v_cache + ((static_cast<size_t>(pg) * n_kv + h) * hd + d0) * page + off;
 #pragma unroll
             for (int j = 0; j < 8; ++j) dst[static_cast<size_t>(j) * page] = from_float<TC>(v[j]);
@@ -479,12 +494,15 @@ extern "C" int llme_swiglu(const void* gu, int in_dtype, void* out, int out_dtyp
     return launch_status();
 }
 
-extern "C" int llme_rope_kv_write(const float* qkv, const float* cos_t, const float* sin_t,
+// zero_input (with write_cache): qkv is all zeros afterwards (by the kernel itself where one thread
+// reads each value once, else by the clearing kernel behind it).
+extern "C" int llme_rope_kv_write(float* qkv, const float* cos_t, const float* sin_t,
                                   const int* positions, const int* seq_idx, const int* block_table,
                                   int max_blocks, void* q_out, int q_dtype, void* k_cache, void* v_cache,
                                   int cache_dtype, int T, int n_q, int n_kv, int hd, int rot, int page,
-                                  int write_cache, hipStream_t stream) {
+                                  int write_cache, int zero_input, hipStream_t stream) {
     if (T <= 0) return 0;
+    if (zero_input && !write_cache) return kErrBadArgument;
     if (rot < 0 || rot > hd || rot % 2 != 0 || page <= 0) return kErrBadArgument;
     // all dims rotated and head sizes in steps of 16: the kernel that moves 8 dims per thread
     const bool vec = rot == hd && hd % 16 == 0 && cos_t != nullptr && sin_t != nullptr &&
@@ -503,11 +521,16 @@ extern "C" int llme_rope_kv_write(const float* qkv, const float* cos_t, const fl
                                dim3(256), 0, stream, qkv, cos_t, sin_t, positions, seq_idx, block_table,    \
                                max_blocks, static_cast<TQ*>(q_out), static_cast<TC*>(k_cache),              \
                                static_cast<TC*>(v_cache), n_q, n_kv, hd, page, write_cache, T);             \
+        else if (vec && zero_input)                                                                         \
+            hipLaunchKernelGGL((rope_kv_write_vec_kernel<TQ, TC, true>), dim3(T), dim3(256), 0, stream, qkv, \
+                               cos_t, sin_t, positions, seq_idx, block_table, max_blocks,                  \
+                               static_cast<TQ*>(q_out), static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), \
+                               n_q, n_kv, hd, page, write_cache);                                           \
         else if (vec)                                                                                       \
-            hipLaunchKernelGGL((rope_kv_write_vec_kernel<TQ, TC>), dim3(T), dim3(256), 0, stream, qkv, cos_t, \
-                               sin_t, positions, seq_idx, block_table, max_blocks, static_cast<TQ*>(q_out), \
-                               static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), n_q, n_kv, hd, page,   \
-                               write_cache);                                                                \
+            hipLaunchKernelGGL((rope_kv_write_vec_kernel<TQ, TC, false>), dim3(T), dim3(256), 0, stream, qkv, \
+                               cos_t, sin_t, positions, seq_idx, block_table, max_blocks,                  \
+                               static_cast<TQ*>(q_out), static_cast<TC*>(k_cache), static_cast<TC*>(v_cache), \
+                               n_q, n_kv, hd, page, write_cache);                                           \
         else                                                                                                \
             hipLaunchKernelGGL((rope_kv_write_kernel<TQ, TC>), dim3(T), dim3(256), 0, stream, qkv, cos_t,   \
                                sin_t, positions, seq_idx, block_table, max_blocks, static_cast<TQ*>(q_out), \
@@ -520,5 +543,14 @@ extern "C" int llme_rope_kv_write(const float* qkv, const float* cos_t, const fl
     else if (q_dtype == kBF16 && cache_dtype == kF32) LLME_ROPE(bf16, float);
     else return kErrBadArgument;
 #undef LLME_ROPE
+    if (zero_input && !(vec && !grouped)) {
+        const int status = launch_status();
+        if (status != 0) return status;
+        const size_t n = static_cast<size_t>(T) * (n_q + 2 * n_kv) * hd;
+        if (n % 4 != 0 || reinterpret_cast<uintptr_t>(qkv) % 16 != 0) return kErrUnsupported;
+        const size_t n4 = n / 4;
+        const unsigned grid = static_cast<unsigned>(n4 / 256 + 1 < 1024 ? n4 / 256 + 1 : 1024);
+        hipLaunchKernelGGL(clear_kernel, dim3(grid), dim3(256), 0, stream, reinterpret_cast<float4*>(qkv), n4);
+    }
     return launch_status();
 }

@@ -121,10 +121,11 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor
                   positions: torch.Tensor, seq_idx: torch.Tensor, block_table: torch.Tensor,
                   q_out: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                   n_q: int, n_kv: int, head_dim: int, rotary_dim: int, write_cache: bool = True,
-                  max_position: int | None = None) -> None:
+                  max_position: int | None = None, zero_input: bool = False) -> None:
     """Rotates q and k heads of qkv [T, (n_q + 2 n_kv) hd] (32-bit) by the tables' rows
     at `positions`, writes q to q_out and k, v into the pages named by the block table.
-    k_cache [pages, n_kv, page, hd]; v_cache [pages, n_kv, hd, page]."""
+    k_cache [pages, n_kv, page, hd]; v_cache [pages, n_kv, hd, page]. zero_input: qkv is all
+    zeros afterwards (for a product that adds its parts into it)."""
     T = qkv.shape[0]
     require(qkv, "qkv", torch.float32, (T, (n_q + 2 * n_kv) * head_dim))
     require(positions, "positions", torch.int32, (T,))
@@ -144,8 +145,11 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor
     check(entry("llme_rope_kv_write")(
         ptr(qkv), ptr(cos), ptr(sin), ptr(positions), ptr(seq_idx), ptr(block_table), block_table.shape[1],
         ptr(q_out), code(q_out.dtype), ptr(k_cache), ptr(v_cache), code(k_cache.dtype), T, n_q, n_kv,
-        head_dim, rotary_dim if cos is not None else 0, page, 1 if write_cache else 0, stream()),
+        head_dim, rotary_dim if cos is not None else 0, page, 1 if write_cache else 0,
+        1 if zero_input and write_cache else 0, stream()),
         "rope_kv_write")
+    if zero_input and not write_cache:
+        clear(qkv)
 
 
 def rope_q_only(q32: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor | None,
@@ -160,7 +164,7 @@ def rope_q_only(q32: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor |
         require(sin, "sin", torch.float32, tuple(cos.shape))
     check(entry("llme_rope_kv_write")(
         ptr(q32), ptr(cos), ptr(sin), ptr(positions), None, None, 0, ptr(q_out), code(q_out.dtype), None, None,
-        code(q_out.dtype), T, n_q, 0, head_dim, rotary_dim if cos is not None else 0, 1, 0, stream()),
+        code(q_out.dtype), T, n_q, 0, head_dim, rotary_dim if cos is not None else 0, 1, 0, 0, stream()),
         "rope_q_only")
 
 

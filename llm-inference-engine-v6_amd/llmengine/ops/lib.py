@@ -35,7 +35,7 @@ _SIGNATURES = {
     "llme_rmsnorm": [_vp, _vp, _i, _vp, _i, _vp, _i, _i, _f, _vp],
     "llme_swiglu": [_vp, _i, _vp, _i, _i, _i, _i, _vp],
     "llme_rope_kv_write": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _i,
-                           _i, _i, _i, _i, _i, _i, _i, _vp],
+                           _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     "llme_gemm_generic": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "llme_attention_generic": [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
                                _f, _i, _vp],

@@ -117,12 +117,17 @@ class Attention(Mixer):
                               n_q, n_kv, hd)
         elif write_cache:
             qkv = step.buffer("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
-            if (rms is None and 16 < T <= 64 and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16
-                    and qkv.numel() % 4 == 0):
+            adds = (rms is None and 16 < T <= 64 and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16
+                    and qkv.numel() % 4 == 0)
+            if adds:
                 # a few dozen rows (decoding at larger batches): q/k/v has too few output tiles for the
                 # chip, so the product is cut over k and adds its parts into a cleared buffer
-                # (measured at 32 rows of the 3B sizes: 10.7 + clearing against 19.5 us)
-                ops.clear(qkv)
+                # (measured at 32 rows of the 3B sizes: 10.7 + clearing against 19.5 us). The buffer
+                # is cleared for the step's first such layer; the rotation kernel leaves it zero for
+                # the next one (a clearing kernel per layer took 4.6 us).
+                if step.extra.get("attn.qkv zero", (0, 0)) != (qkv.data_ptr(), qkv.numel()):
+                    ops.clear(qkv)
+                step.extra.pop("attn.qkv zero", None)
                 ops.gemm(x, self.w_qkv, qkv, accumulate=True, fixed_order=step.fixed_order)
             else:
                 project(self.w_qkv, qkv)
@@ -130,7 +135,9 @@ class Attention(Mixer):
                 self.position.apply(qkv[:, :self.q_dim].view(T, n_q, hd),
                                     qkv[:, self.q_dim:self.q_dim + self.kv_dim].view(T, n_kv, hd), step.positions)
             ops.rope_kv_write(qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
-                              n_q, n_kv, hd, rot, write_cache=True)
+                              n_q, n_kv, hd, rot, write_cache=True, zero_input=adds)
+            if adds:
+                step.extra["attn.qkv zero"] = (qkv.data_ptr(), qkv.numel())
         else:
             # A layer that reads another layer's cache projects queries only.
             q32 = step.buffer("attn.q32", (T, self.q_dim), torch.float32)
