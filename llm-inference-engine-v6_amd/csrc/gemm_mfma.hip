@@ -996,7 +996,7 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
 // bfloat16; writes q_out [M, n_q hd] (rotated) and the rows' k (rotated) and v into the pages that
 // block_table[seq_idx[m]] names for positions[m]; cos/sin [max_pos, hd / 2] float32. Full rotation
 // only; hd 16, 32, 64 or 128 (a tile of 128 or 64 columns must hold whole heads). What the separate
-// kernels would store in between, the 32-bit q/k/v rows, never exists. tile_shape 0, 64, 128 or 128064.
+// kernels would store in between, the 32-bit q/k/v rows, never exists. tile_shape 0, 64, 96064, 128064, 96128 or 128.
 extern "C" int llme_gemm_bf16_qkv_rope(const void* a, const void* w, int M, int K, int blocked, const float* cos_t,
                                        const float* sin_t, const int* positions, const int* seq_idx,
                                        const int* block_table, int max_blocks, void* q_out, void* k_cache,
@@ -1017,14 +1017,32 @@ extern "C" int llme_gemm_bf16_qkv_rope(const void* a, const void* w, int M, int 
     const bf16* A = static_cast<const bf16*>(a);
     const bf16* W = static_cast<const bf16*>(w);
     if (tile_shape <= 0) {
-        // 128 x 128 tiles once they cover the chip, 128 x 64 from 96 of the large ones on, else 64 x 64
-        // (measured at the 1B sizes: 273 rows 12.2 / 15.9 / 22.9 us with 64 x 64 / 128 x 64 / 128 x 128,
-        // 512 rows 19.0 / 16.5 / 23.8, 2,048 rows 55.5 / 40.1 / 38.9); a head of 128 needs the full width
-        const long wg128 = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
-        tile_shape = (hd > 64 || wg128 >= compute_units()) ? 128 : (M > 64 && wg128 >= 96) ? 128064 : 64;
+        // The tile with the least rounds of workgroups over the compute units x (a round's fixed cost,
+        // which grows with k, + the tile's area): fitted to measurements at 80 to 1,024 rows. 1B sizes
+        // (us with 64 x 64 / 96 x 64 / 128 x 64 / 128 x 128 tiles): 273 rows 12.1 / 13.8 / 16.0 / 22.8,
+        // 384 rows 17.8 / 14.1 / 16.2 / 22.8, 512 rows 18.6 / 20.9 / 16.6 / 23.6, 1,024 rows 28.0 / 29.1 /
+        // 25.8 / 25.5. A head of 128 needs the full width: 96 x 128 / 128 x 128 at the 3B sizes 26.3 / 31.4
+        // at 256 rows, 44.3 / 49.2 at 1,024; at the 8B sizes 33.0 / 40.1 at 384 rows, 52.7 / 40.8 at 512.
+        const int shapes[5] = {64, 96064, 128064, 96128, 128};
+        const int heights[5] = {64, 96, 128, 96, 128};
+        const int widths[5] = {64, 64, 64, 128, 128};
+        const int cus = compute_units();
+        const double fixed = 4.3 * K;
+        double best = 0.0;
+        for (int c = 0; c < 5; ++c) {
+            if (hd > widths[c]) continue;
+            const long wgs = static_cast<long>((M + heights[c] - 1) / heights[c]) * ((N + widths[c] - 1) / widths[c]);
+            const double cost = static_cast<double>((wgs + cus - 1) / cus) * (fixed + heights[c] * widths[c]);
+            if (tile_shape <= 0 || cost < best) {
+                best = cost;
+                tile_shape = shapes[c];
+            }
+        }
     }
     if (tile_shape == 128) return launch_tile_rope<4, 4>(A, W, M, N, K, blocked, qt, stream);
     if (tile_shape == 64 && hd <= 64) return launch_tile_rope<2, 2>(A, W, M, N, K, blocked, qt, stream);
     if (tile_shape == 128064 && hd <= 64) return launch_tile_rope<4, 2>(A, W, M, N, K, blocked, qt, stream);
+    if (tile_shape == 96064 && hd <= 64) return launch_tile_rope<3, 2>(A, W, M, N, K, blocked, qt, stream);
+    if (tile_shape == 96128) return launch_tile_rope<3, 4>(A, W, M, N, K, blocked, qt, stream);
     return kErrBadArgument;
 }

@@ -84,7 +84,7 @@ def gemm_qkv_rope(x: torch.Tensor, w_qkv: torch.Tensor, cos: torch.Tensor, sin: 
     x [T, K] bfloat16 (normed), w_qkv [(n_q + 2 n_kv) hd, K] bfloat16 (row-major or blocked); q heads
     and k heads are rotated at the rows' positions, q goes to q_out [T, n_q hd], k and v into the
     rows' pages. The 32-bit q/k/v rows that the separate kernels pass between them never exist.
-    Full rotation, head size 16, 32, 64 or 128. tile: 0 (chosen), 64 or 128."""
+    Full rotation, head size 16, 32, 64 or 128. tile: 0 (chosen), 64, 96064, 128064, 96128 or 128."""
     require(x, "x", torch.bfloat16, (None, None))
     T, K = x.shape
     n_rows, _ = kernels._require_weight(w_qkv, "w_qkv", torch.bfloat16, K)

@@ -768,13 +768,13 @@ def test_rope_write_of_many_tokens(ops, n_q, n_kv, hd, page, dtype, new):
 @pytest.mark.parametrize("n_q,n_kv,hd,K,page", [(4, 2, 64, 128, 16), (32, 8, 64, 2048, 16), (3, 1, 128, 96, 32), (5, 3, 32, 72, 16),
                                                  (6, 2, 16, 64, 48), (24, 8, 128, 512, 16)])
 @pytest.mark.parametrize("new", [[70, 130, 3, 16, 33], [300], [1, 90, 17]])
-@pytest.mark.parametrize("tile", [0, 64, 128, 128064])
+@pytest.mark.parametrize("tile", [0, 64, 128, 128064, 96064, 96128])
 def test_gemm_qkv_rope(ops, n_q, n_kv, hd, K, page, new, tile):
     """The q/k/v projection with rotation and cache write in its epilogue against the three kernels
     it replaces (product into 32-bit rows, rotation + cache write): portions that start anywhere in
     their requests, groups of 16 rows that span two requests or two pages, tiles that hang over the
     rows and over the heads, row-major and blocked weights."""
-    if tile in (64, 128064) and hd > 64:
+    if tile in (64, 128064, 96064) and hd > 64:
         pytest.skip("a 64-column tile does not hold a head of 128")
     g = _gen(90)
     T = sum(new)
