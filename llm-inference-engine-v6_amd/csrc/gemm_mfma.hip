@@ -910,6 +910,7 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
     // parts are added with atomics, so this needs an accumulating float32 output).
     if (gated) mode = kGatedBF16;
     const bool auto_shape = tile_shape <= 0;
+    float tiles_cost = -1.f;                           // of the chosen tile, in the units of the estimate below
     if (tile_shape <= 0) {
         const long wg128 = static_cast<long>((M + 127) / 128) * ((N + 127) / 128);
         // (a stored output with fewer than 96 tiles of 128 x 128 fills the chip better in 64 x 64 tiles:
@@ -925,7 +926,12 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
             const int shapes[5] = {128, 128096, 128064, 96128, 96064};
             const int heights[5] = {128, 128, 128, 96, 96};
             const int widths[5] = {128, 96, 64, 128, 64};
-            const float eff[5] = {1.0f, 0.9f, 0.85f, 0.84f, 0.78f};
+            // (efficiencies: sums that are added, from sweeps at 96 to 512 rows; stored and gated outputs, from the
+            // gate/up shapes of the 1B, 3B and 8B sizes at 100 to 1,536 rows, e.g. at 320 rows of the 1B sizes
+            // 36 / 44 / 38 / 34 / 39 us in the order of the shapes)
+            const float eff_added[5] = {1.0f, 0.9f, 0.85f, 0.84f, 0.78f};
+            const float eff_stored[5] = {1.0f, 0.9f, 0.70f, 0.83f, 0.67f};
+            const float* eff = mode == kAddF32 ? eff_added : eff_stored;
             float best = 0.f;
             for (int c = 0; c < 5; ++c) {
                 const long wgs = static_cast<long>((M + heights[c] - 1) / heights[c]) * ((N + widths[c] - 1) / widths[c]);
@@ -939,6 +945,9 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
                     tile_shape = shapes[c];
                 }
             }
+            tiles_cost = best;
+        } else if (tile_shape == 128) {
+            tiles_cost = static_cast<float>((wg128 + cus - 1) / cus) * 16384.f;
         }
         // A long sum into an output of few tiles (down-proj at 129 to 288 rows): tiles of 96 x 64 where
         // they need no more rows than those of 64, cut over k in 2 or 4 up to three workgroups per
@@ -969,15 +978,15 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
         if (mode != kAddF32) return kErrBadArgument;
         mode = kAtomicF32;
     }
-    if (auto_shape && blocked && direct != 0 && mode != kAddF32 && mode != kAtomicF32) {
+    if (auto_shape && blocked && direct != 0 && mode != kAddF32 && mode != kAtomicF32 && tiles_cost > 0.f) {
         // Wide outputs that are stored, not added (gate/up, q/k/v of long prompts): tiles of 256 x 256
         // by eight wavefronts, their slabs straight into LDS, load half the bytes per product; one
-        // workgroup fills a compute unit, so they pay where whole rounds of them cover the output
-        // (measured, 256 compute units: 1.07 to 1.16 times the 128 x 128 tiles' speed at 256, 512,
-        // 1,024 and more tiles, 0.9 at 384).
+        // workgroup fills a compute unit. In the units of the estimate above a round of them costs
+        // 65,536 / 1.15 (measured: 1.07 to 1.16 times the 128 x 128 tiles' speed where whole rounds cover
+        // the output; 8B gate/up at 448 rows, one round against 3.5 of 128 x 128: 105 against 129 us).
         const long rounds = (static_cast<long>((M + 255) / 256) * ((N + 255) / 256) + cus - 1) / cus;
-        const double covered = static_cast<double>(M) * N / (static_cast<double>(rounds) * cus * 65536.0);
-        if (covered >= 0.85) return launch_tile_direct<4, 2, 4, 8>(A, W, out, M, N, K, mode, ksplit, stream);
+        if (static_cast<float>(rounds) * 65536.f / 1.15f < tiles_cost)
+            return launch_tile_direct<4, 2, 4, 8>(A, W, out, M, N, K, mode, ksplit, stream);
     }
     if (blocked && direct == 1 && tile_shape == 256256)
         return launch_tile_direct<4, 2, 4, 8>(A, W, out, M, N, K, mode, ksplit, stream);
