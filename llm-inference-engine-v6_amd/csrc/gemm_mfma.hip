@@ -949,14 +949,21 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
         } else if (tile_shape == 128) {
             tiles_cost = static_cast<float>((wg128 + cus - 1) / cus) * 16384.f;
         }
-        // A long sum into an output of few tiles (down-proj at 129 to 288 rows): tiles of 96 x 64 where
-        // they need no more rows than those of 64, cut over k in 2 or 4 up to three workgroups per
-        // compute unit (measured at 273 rows, down-proj of the 1B sizes 23.7 against 29.3 us, of the 8B
-        // sizes 53 against 66; at 192 rows 18.4 against 21.3 and 40 against 43).
-        // (and at 65 to 96 rows, one row tile: down-proj of the 1B sizes 13.5 against 14.7 us, of the 3B sizes 16.6 against 21.1)
-        const bool tall = mode == kAddF32 && ksplit <= 0 && M > 64 && K >= 4096 && wg128 <= cus &&
-                          (M + 95) / 96 * 96 <= (M + 63) / 64 * 64;
-        if (tall) tile_shape = 96064;
+        // A long sum into an output of few tiles (down-proj at 65 to 288 rows): tiles of 64 columns whose
+        // 64, 96 or 128 rows leave the fewest rows to spare (the taller on a tie), cut over k in 2, 4 or 8
+        // up to three workgroups per compute unit. Measured (us, against tiles of 64 x 64 or the estimate
+        // above): down-proj of the 1B sizes at 273 rows 23.7 against 29.3, at 192 rows 18.4 against 21.3, at
+        // 81 rows 13.5 against 14.7; of the 3B sizes at 200 and 256 rows 27.5 and 29.7 against 37.0 and 39.6, at 81
+        // rows 16.6 against 21.1; of the 8B sizes at 273 rows 53 against 66, at 100 and 128 rows 28.9 and 30.6
+        // against 40.9.
+        bool tall = false;
+        if (mode == kAddF32 && ksplit <= 0 && M > 64 && M <= 288 && K >= 4096 && wg128 <= cus) {
+            const int rows64 = (M + 63) / 64 * 64, rows96 = (M + 95) / 96 * 96, rows128 = (M + 127) / 128 * 128;
+            if (rows128 <= rows96 && rows128 <= rows64) tile_shape = 128064;
+            else if (rows96 <= rows64) tile_shape = 96064;
+            else tile_shape = 64;
+            tall = tile_shape != 64;
+        }
         if (mode == kAddF32 && ksplit <= 0) {
             // A sum that is joined anyway (the residual stream) is cut over k until the tiles fill
             // the chip: 64 x 64 tiles to about two workgroups per compute unit, the larger ones to
@@ -966,7 +973,7 @@ extern "C" int llme_gemm_bf16(const void* a, const void* w, void* out, int out_d
             const int bn = (tile_shape == 128 || tile_shape == 96128) ? 128 : tile_shape == 128096 ? 96 : 64;
             const long wgs = static_cast<long>((M + bm - 1) / bm) * ((N + bn - 1) / bn);
             long ks = (tile_shape == 64 ? 2 * cus : cus) / wgs;
-            if (tall) ks = (M <= 96 && K >= 8192 && 3 * cus / wgs >= 8) ? 8 : 3 * cus / wgs >= 4 ? 4 : 3 * cus / wgs >= 2 ? 2 : 1;
+            if (tall) ks = (K >= 8192 && (M <= 96 || 8 * wgs <= cus) && 3 * cus / wgs >= 8) ? 8 : 3 * cus / wgs >= 4 ? 4 : 3 * cus / wgs >= 2 ? 2 : 1;
             if (tile_shape == 128 && wg128 <= cus && K >= 4096 && ks < 2) ks = 2;
             if (ks > K / 512) ks = K / 512;
             if (ks > 8) ks = 8;
