@@ -259,14 +259,16 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 //              per tile whatever the number of work items
 //   bits 12-13 1 + read_once: whether the decode kernel loads keys and values with the read-once
 //              hint: -1 the entry point chooses, 0 never, 1 always
+//   bit 14     the decode kernel's splits are left unjoined in part_o / part_ml: the caller joins them
+//              (llme_attention_join_project); only for steps without prompt portions
 struct Tuning {
-    int rows, shared, key_waves, read_once;
+    int rows, shared, key_waves, read_once, no_join;
 };
 static bool parse_tuning(int packed, Tuning* t) {
-    if (packed < 0 || packed >= (1 << 14)) return false;
+    if (packed < 0 || packed >= (1 << 15)) return false;
     const int rows = packed & 0xFF, shared = ((packed >> 8) & 0xF) - 1, read_once = ((packed >> 12) & 0x3) - 1;
     if (rows % 16 != 0 || rows > 64 || shared > 3 || read_once > 1) return false;
-    *t = Tuning{rows, shared > 1 ? 1 : shared, shared > 1 ? shared - 1 : 0, read_once};
+    *t = Tuning{rows, shared > 1 ? 1 : shared, shared > 1 ? shared - 1 : 0, read_once, (packed >> 14) & 1};
     return true;
 }
 static bool decode_reads_once(const Tuning& t) { return t.read_once != 0; }
@@ -294,7 +296,7 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
             hipLaunchKernelGGL((attention_decode_kernel<HD, false>), grid, dim3(DEC_WAVES * 64), 0, stream, q, kc, vc, out,
                                part_o, part_ml, q_start, ctx_len, table, max_blocks, n_q, n_kv, page, scale, window,
                                split_len, nsplit);
-        if (nsplit > 1)
+        if (nsplit > 1 && !tuning.no_join)
             hipLaunchKernelGGL(attention_join_kernel, dim3(n_seq, n_q), dim3(64), 0, stream, part_o, part_ml, out,
                                q_start, n_q, HD, nsplit);
     }
@@ -401,6 +403,7 @@ extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const voi
     if (static_cast<double>(max_blocks) * (page / 16) * (page / 16) >= 4294967296.0) return kErrUnsupported;
     if (static_cast<double>(n_kv) * page * hd >= 4294967296.0) return kErrUnsupported;   // a page's elements: 32 bits
     if (n_decode > 0 && (split_len <= 0 || split_len % 32 != 0 || nsplit <= 0 || nsplit > 64)) return kErrBadArgument;
+    if (tune.no_join && prefill_groups > 0) return kErrBadArgument;
     const int qt = direct_rows(hd, tune) / 16;
     const int shared_rows = shared_rows_for(hd, n_q, n_kv, tune);
 #define LLME_HEAD(HD)                                                                                           \

@@ -224,7 +224,9 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         int(window), stream()), "attention_generic")
 
 
-_fast_attention = None  # set by ops/mfma.py when the MFMA kernels are present
+# set by ops/mfma.py when the MFMA kernels are present
+_fast_attention = None
+_fast_attention_project = None
 
 
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor, step,
@@ -237,6 +239,19 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out
         return
     attention_generic(q, k_cache, v_cache, out, step.positions, step.seq_idx, block_table, n_q, n_kv,
                       head_dim, scale, window)
+
+
+def attention_project(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, o: torch.Tensor, step,
+                      block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int, scale: float, window: int,
+                      w_o: torch.Tensor, out: torch.Tensor, accumulate: bool) -> None:
+    """attention (as above, into o) and the output projection behind it: out (+)= o w_o^T. Where a
+    step of a few decoded tokens cuts its keys into splits, the splits' join and the projection are
+    one kernel, and o is not written."""
+    if policy.fast_attention and policy.fast_gemm and _fast_attention_project is not None and _fast_attention_project(
+            q, k_cache, v_cache, o, step, block_table, n_q, n_kv, head_dim, scale, window, w_o, out, accumulate):
+        return
+    attention(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, head_dim, scale, window)
+    gemm(o, w_o, out, accumulate, fixed_order=step.fixed_order)
 
 
 # --- sampling ------------------------------------------------------------------------

@@ -293,6 +293,57 @@ def _fast_attention(q, k_cache, v_cache, out, step, block_table, n_q, n_kv, head
 
 kernels._fast_attention = _fast_attention
 
+declare("llme_attention_join_project_supported", [_i, _i, _i, _i, _i])
+declare("llme_attention_join_project_pays", [_i, _i, _i, _i, _i])
+declare("llme_attention_join_project", [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp])
+TUNING_NO_JOIN = 1 << 14            # the decode kernel leaves its splits unjoined (see attention_mfma.hip)
+JOIN_PROJECT = True                 # (tests and measurements switch the fused kernel off here)
+
+
+def attention_join_project(part_o, part_ml, w_o, out, n_rows: int, n_q: int, head_dim: int, nsplit: int) -> None:
+    """out [n_rows, N] float32 += join(part_o, part_ml) w_o^T: the join of the decode kernel's key splits
+    (part_o [n_rows, n_q, nsplit, head_dim], part_ml [.., 2], as llme_attention_bf16 leaves them with
+    TUNING_NO_JOIN for requests of one token each) and the output projection, w_o blocked bfloat16."""
+    require(part_o, "part_o", torch.float32)
+    require(part_ml, "part_ml", torch.float32)
+    N, _ = kernels._require_weight(w_o, "w_o", torch.bfloat16, n_q * head_dim)
+    require(out, "out", torch.float32, (n_rows, N))
+    if (not kernels.is_blocked(w_o) or part_o.numel() < n_rows * n_q * nsplit * head_dim
+            or part_ml.numel() < n_rows * n_q * nsplit * 2
+            or not entry("llme_attention_join_project_supported")(n_rows, n_q, head_dim, nsplit, N)):
+        raise kernels.KernelError(f"attention_join_project: {n_rows} rows (at most 16), {n_q} heads of {head_dim}, "
+                                  f"{nsplit} splits or the projection's layout are not supported")
+    check(entry("llme_attention_join_project")(ptr(part_o), ptr(part_ml), ptr(w_o), ptr(out), n_rows, n_q, head_dim,
+                                               nsplit, N, stream()), "attention_join_project")
+
+
+def _fast_attention_project(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, head_dim, scale, window, w_o, out,
+                            accumulate) -> bool:
+    """A step of up to 16 decoded tokens whose keys are cut into splits: the splits stay unjoined and
+    one kernel joins them and projects. Everything else: not taken (the caller runs the two apart)."""
+    T = q.shape[0]
+    if (not JOIN_PROJECT or not accumulate or step.fixed_order or T > 16 or T != step.num_seqs
+            or out.dtype != torch.float32 or w_o.dtype != torch.bfloat16 or not kernels.is_blocked(w_o)
+            or not attention_bf16_supported(q, k_cache, head_dim) or o.dtype != torch.bfloat16):
+        return False
+    key = ("attention_plan", n_q, n_kv, head_dim)
+    plan = step.extra.get(key)
+    if plan is None:
+        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len)
+    N, K = kernels.weight_shape(w_o)
+    if (plan["n_decode"] != T or plan["groups"] or plan["nsplit"] <= 1 or K != n_q * head_dim
+            or not entry("llme_attention_join_project_pays")(T, n_q, head_dim, plan["nsplit"], N)):
+        return False
+    part_o = step.buffer("attn.part_o", (T * n_q * plan["nsplit"] * head_dim,), torch.float32)
+    part_ml = step.buffer("attn.part_ml", (T * n_q * plan["nsplit"] * 2,), torch.float32)
+    attention_bf16(q, k_cache, v_cache, o, step.q_start, step.ctx_len, block_table, n_q, n_kv, head_dim, scale, window,
+                   dict(plan, tuning=int(plan.get("tuning", 0)) | TUNING_NO_JOIN), part_o, part_ml)
+    attention_join_project(part_o, part_ml, w_o, out, T, n_q, head_dim, plan["nsplit"])
+    return True
+
+
+kernels._fast_attention_project = _fast_attention_project
+
 
 # --- projections fused with the norm in front of them (decoding) ---------------------------
 declare("llme_gemv_norm", [_vp, _vp, _vp, _i, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp])

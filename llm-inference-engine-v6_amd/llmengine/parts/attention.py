@@ -146,8 +146,8 @@ class Attention(Mixer):
                 self.position.apply(q32.view(T, n_q, hd), None, step.positions)
             ops.rope_q_only(q32, cos, sin, step.positions, q, n_q, hd, rot)
         o = step.buffer("attn.o", (T, self.q_dim), act)
-        ops.attention(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, hd, self.scale, self.window)
-        ops.gemm(o, self.w_o, out, accumulate, fixed_order=step.fixed_order)
+        ops.attention_project(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, hd, self.scale, self.window,
+                              self.w_o, out, accumulate)
 
 
 register_part("mixer", "attention", Attention)

@@ -308,6 +308,47 @@ def test_short_portions_far_into_a_long_prompt(zoo, dtype, monkeypatch):
         assert err < TOL[dtype], (pos, err)
 
 
+@pytest.mark.parametrize("n_live", [1, 3])
+def test_decoded_tokens_join_their_splits_inside_the_output_projection(zoo, n_live, monkeypatch):
+    """Decoding behind a few hundred tokens cuts the keys into splits; for up to 16 decoded tokens the
+    splits' join and the output projection are one kernel. It must have run, match the plain
+    implementation, and give what the join kernel and the projection give apart."""
+    from llmengine.ops import mfma
+    calls = []
+    join_project = mfma.attention_join_project
+
+    def noting(*args, **kw):
+        calls.append(args[4])
+        return join_project(*args, **kw)
+    monkeypatch.setattr(mfma, "attention_join_project", noting)
+    model_dir, _, _, page = zoo["C"]
+    reqs = {f"s{i}": random_tokens(420 + 90 * i, TINY_C["vocab_size"], 90 + i) for i in range(n_live)}
+    pcfg, pw = load_plain_model(model_dir)
+    engine = engine_for(model_dir, "bf16")
+    # every request's prompt but its last 24 tokens in one step, then 24 steps of one token of each
+    steps = [{"step": 0, "entries": [{"id": rid, "tokens": ids[:-24], "want": []} for rid, ids in reqs.items()], "end": []}]
+    for t in range(24, 0, -1):
+        steps.append({"step": len(steps), "end": list(reqs) if t == 1 else [],
+                      "entries": [{"id": rid, "tokens": [ids[-t]], "want": [0]} for rid, ids in reqs.items()]})
+    pages = replay.trace_peak_tokens(steps, round_to=page) // page
+
+    def run():
+        cache = engine.new_cache(pages, page, max_requests=n_live)
+        return replay.run_trace(engine, cache, steps)
+    got = run()
+    assert calls and max(calls) == n_live, "no decode step joined its splits in the projection"
+    monkeypatch.setattr(mfma, "JOIN_PROJECT", False)
+    n_calls = len(calls)
+    apart = run()
+    assert len(calls) == n_calls
+    for rid, ids in reqs.items():
+        ref = plain_forward(pcfg, pw, ids, rounder=bf16_round).numpy()
+        for pos in range(len(ids) - 24, len(ids)):
+            top = np.abs(ref[pos]).max()
+            assert np.abs(got[rid][pos].astype(np.float64) - ref[pos]).max() / top < TOL["bf16"], (rid, pos)
+            assert np.abs(got[rid][pos].astype(np.float64) - apart[rid][pos]).max() / top < 2e-3, (rid, pos)
+
+
 # A layer or two with the sizes of Llama 3.2 1B, 3.2 3B and 3.1 8B: the kernels that serving picks at
 # real widths (tiled products over several row tiles, the prefill attention with many work items, the
 # fused decode kernels at widths 2048, 3072 and 4096, the output head over the whole vocabulary).

@@ -415,6 +415,80 @@ def test_attention_mfma_decode_splits(ops, monkeypatch):
     assert plan1["nsplit"] == 1 and _rel(out1, ref1) < 8e-3
 
 
+def _plain_attention_last_row(q, k, v):
+    """plain_attention's formula for the last position alone (which sees every key): [n_q, hd]."""
+    n_q, hd = q.shape[1], q.shape[2]
+    group = n_q // k.shape[1]
+    out = torch.zeros(n_q, hd, dtype=torch.float64)
+    for h in range(n_q):
+        scores = (k[:, h // group] * q[-1, h]).sum(dim=-1) / math.sqrt(float(hd))
+        e = torch.exp(scores - scores.max())
+        out[h] = ((e / e.sum())[:, None] * v[:, h // group]).sum(dim=0)
+    return out
+
+
+@pytest.mark.parametrize("lens,n_q,n_kv,hd,N", [
+    ([4000], 32, 8, 64, 2048),                          # one row, 32 splits dealt out over four threads each
+    ([1500, 40], 8, 2, 64, 96),                         # two rows, one of them with a single split's worth of keys
+    ([600, 650, 700, 512, 513, 1, 300, 640], 32, 8, 64, 2064),   # the columns end inside a block of tiles
+    ([150 + 40 * i for i in range(16)], 6, 2, 48, 160),  # 16 rows; the last stretch of k has fewer heads
+    ([900, 100, 1000], 8, 2, 128, 528),
+    ([700, 701], 4, 2, 80, 64),
+    ([520, 300, 900, 50], 34, 2, 16, 48),               # 16 heads of 16 to a stretch of k, the last stretch one block
+    ([2000, 1800, 1900, 100, 2100], 24, 8, 128, 3072),  # three tiles per wavefront
+    ([800, 900, 1000, 1100, 1200], 32, 8, 64, 6160)])   # four, and the last block of tiles not whole
+def test_attention_join_project(ops, lens, n_q, n_kv, hd, N):
+    """The join of the decode kernel's splits and the output projection as one kernel, against the
+    join kernel followed by a 32-bit product of the joined rows, and against plain attention."""
+    page, S, K = 16, len(lens), n_q * hd
+    s = _paged_setup(ops, lens, n_q, n_kv, hd, page, torch.bfloat16, seed=61)
+    last = torch.tensor([sum(lens[:i + 1]) - 1 for i in range(S)], device=DEV)
+    q = s["q"][last].contiguous()
+    i32 = dict(dtype=torch.int32, device=DEV)
+    q_start, ctx = torch.arange(S + 1, **i32), torch.tensor([n - 1 for n in lens], **i32)
+    plan = ops.mfma.plan_attention([1] * S, [n - 1 for n in lens], n_q, n_kv, hd)
+    assert plan["nsplit"] > 1
+    g = torch.Generator().manual_seed(62)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16()
+    base = torch.randn(S, N, generator=g)
+    wd = ops.block_weight(w.to(DEV))
+    scale = 1.0 / math.sqrt(hd)
+
+    def parts():
+        return (torch.full((S * n_q * plan["nsplit"] * hd,), float("nan"), device=DEV),
+                torch.full((S * n_q * plan["nsplit"] * 2,), float("nan"), device=DEV))
+    part_o, part_ml = parts()
+    o = torch.zeros_like(q)
+    ops.mfma.attention_bf16(q, s["k_cache"], s["v_cache"], o, q_start, ctx, s["table"], n_q, n_kv, hd, scale, 0, plan,
+                            part_o, part_ml)
+    apart = base.double() + o.cpu().double() @ w.double().T
+    part_o2, part_ml2 = parts()
+    o2 = torch.zeros_like(q)
+    ops.mfma.attention_bf16(q, s["k_cache"], s["v_cache"], o2, q_start, ctx, s["table"], n_q, n_kv, hd, scale, 0,
+                            dict(plan, tuning=ops.mfma.TUNING_NO_JOIN), part_o2, part_ml2)
+    assert not o2.any()                                  # left unjoined: nothing wrote the rows
+    out = base.to(DEV)
+    ops.mfma.attention_join_project(part_o2, part_ml2, wd, out, S, n_q, hd, plan["nsplit"])
+    assert _rel(out.cpu().double(), apart) < 1e-4
+    ref = torch.cat([_plain_attention_last_row(qq, kk, vv).reshape(1, K) for (qq, kk, vv) in s["plain"]])
+    assert _rel(out.cpu().double(), base.double() + ref @ w.double().T) < 8e-3
+
+
+def test_attention_join_project_refuses(ops):
+    from llmengine.ops import KernelError
+    w = ops.block_weight(torch.zeros(64, 128, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(KernelError):                     # 17 rows
+        ops.mfma.attention_join_project(torch.zeros(17 * 2 * 2 * 64, device=DEV), torch.zeros(17 * 2 * 2 * 2, device=DEV), w,
+                                        torch.zeros(17, 64, device=DEV), 17, 2, 64, 2)
+    with pytest.raises(KernelError):                     # scratch too small for the splits
+        ops.mfma.attention_join_project(torch.zeros(2 * 2 * 64, device=DEV), torch.zeros(2 * 2 * 2, device=DEV), w,
+                                        torch.zeros(1, 64, device=DEV), 1, 2, 64, 4)
+    with pytest.raises(KernelError):                     # a projection that is not blocked
+        ops.mfma.attention_join_project(torch.zeros(2 * 2 * 64, device=DEV), torch.zeros(2 * 2 * 2, device=DEV),
+                                        torch.zeros(64, 128, dtype=torch.bfloat16, device=DEV),
+                                        torch.zeros(1, 64, device=DEV), 1, 2, 64, 2)
+
+
 @pytest.mark.parametrize("n_q,n_kv,hd,page", [(4, 2, 16, 16), (3, 1, 32, 16), (6, 2, 48, 32), (32, 8, 64, 16),
                                               (5, 5, 80, 16), (8, 2, 128, 16)])
 def test_attention_mfma_prefill_and_mixed(ops, n_q, n_kv, hd, page):
