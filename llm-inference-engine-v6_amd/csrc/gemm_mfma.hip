@@ -118,11 +118,18 @@ struct AddendsAhead {
     }
 };
 
+// Where row m0 + tid of the tile goes (rotating epilogue): its position and the page that holds it,
+// looked up by thread tid while the products run (see the kernel).
+struct RowPlace {
+    int pos = 0, page = 0;
+};
+
 template <int WMT, int WNT, int MODE, int LDS_BYTES, int WR = 2, int WC = 2, bool AHEAD = false>
 __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned char* lds_raw, void* __restrict__ out,
                                               int M, int N, int m0, int n0, int wm, int wn, int tid, int r, int q,
                                               const QkvTarget& qt = QkvTarget{},
-                                              const AddendsAhead<WR * 16 * WMT, WC * 16 * WNT, 64 * WR * WC>& ahead = {}) {
+                                              const AddendsAhead<WR * 16 * WMT, WC * 16 * WNT, 64 * WR * WC>& ahead = {},
+                                              const RowPlace& place = RowPlace{}) {
     constexpr int BM = WR * 16 * WMT, BN = WC * 16 * WNT, NT = 64 * WR * WC;
 
     constexpr int SS = BN + 4;                           // floats per staged row
@@ -137,6 +144,17 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
     if (STAGED && N % 8 == 0) {
         constexpr int HB = PASSES > 0 ? BM / (PASSES > 0 ? PASSES : 1) : BM;     // rows of a pass
         float* stage = reinterpret_cast<float*>(lds_raw);
+        // the rows' positions and pages, behind the stage: [BM] each (the rotating epilogue has one pass)
+        int* row_pos = reinterpret_cast<int*>(lds_raw + static_cast<size_t>(HB) * SS * 4);
+        int* row_page = row_pos + BM;
+        if (MODE == kRopeCache) {
+            static_assert(MODE != kRopeCache || (PASSES == 1 && static_cast<size_t>(BM) * SS * 4 + BM * 8 <= static_cast<size_t>(LDS_BYTES)),
+                          "the rows' places fit behind the stage");
+            if (tid < BM) {
+                row_pos[tid] = place.pos;
+                row_page[tid] = place.page;
+            }
+        }
 #pragma unroll
         for (int pass = 0; pass < PASSES; ++pass) {
         if (pass > 0) __syncthreads();                  // the pass before has been stored
@@ -162,7 +180,7 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
                 const int m = mp + row, head = n0 / hd + hh;
                 if (m >= M || head >= rotated) continue;
                 const float* sp = stage + row * SS + hh * hd + i;
-                const int pos = qt.positions[m];
+                const int pos = row_pos[row];
                 const float* cs = qt.cos_t + static_cast<size_t>(pos) * half + i;
                 const float* sn = qt.sin_t + static_cast<size_t>(pos) * half + i;
                 bf16x8 lo, hi;
@@ -176,7 +194,7 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
                 if (head < qt.n_q) {
                     dst = qt.q_out + (static_cast<size_t>(m) * qt.n_q + head) * hd + i;
                 } else {
-                    const int pg = qt.block_table[static_cast<size_t>(qt.seq_idx[m]) * qt.max_blocks + pos / qt.page];
+                    const int pg = row_page[row];
                     dst = qt.k_cache + ((static_cast<size_t>(pg) * qt.n_kv + (head - qt.n_q)) * qt.page + pos % qt.page) * hd + i;
                 }
                 *reinterpret_cast<bf16x8*>(dst) = lo;
@@ -193,11 +211,12 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
                 const int kvh = head - rotated, d = n % hd;
                 const int nt = M - mg < 16 ? M - mg : 16;
                 const float* sp = stage + (g16 * 16) * SS + col;
-                const int pos0 = qt.positions[mg];
-                const bool together = nt == 16 && qt.seq_idx[mg] == qt.seq_idx[mg + 15] && pos0 % 16 == 0 &&
-                                      qt.page % 16 == 0 && qt.positions[mg + 15] == pos0 + 15;
+                // (a page belongs to one request: the same page and 15 positions further on is the same request)
+                const int pos0 = row_pos[g16 * 16];
+                const bool together = nt == 16 && row_page[g16 * 16] == row_page[g16 * 16 + 15] && pos0 % 16 == 0 &&
+                                      qt.page % 16 == 0 && row_pos[g16 * 16 + 15] == pos0 + 15;
                 if (together) {
-                    const int pg = qt.block_table[static_cast<size_t>(qt.seq_idx[mg]) * qt.max_blocks + pos0 / qt.page];
+                    const int pg = row_page[g16 * 16];
                     bf16* dst = qt.v_cache + ((static_cast<size_t>(pg) * qt.n_kv + kvh) * hd + d) * qt.page + pos0 % qt.page;
                     bf16x8 lo, hi;
 #pragma unroll
@@ -209,8 +228,8 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[WMT][WNT], unsigned c
                     *reinterpret_cast<bf16x8*>(dst + 8) = hi;
                 } else {
                     for (int j = 0; j < nt; ++j) {
-                        const int pos = qt.positions[mg + j];
-                        const int pg = qt.block_table[static_cast<size_t>(qt.seq_idx[mg + j]) * qt.max_blocks + pos / qt.page];
+                        const int pos = row_pos[g16 * 16 + j];
+                        const int pg = row_page[g16 * 16 + j];
                         qt.v_cache[((static_cast<size_t>(pg) * qt.n_kv + kvh) * hd + d) * qt.page + pos % qt.page] =
                             static_cast<__bf16>(sp[j * SS]);
                     }
@@ -475,6 +494,18 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
         deal_between_products<kVmemRead, (WMT * WNT) / 2>();
         __builtin_amdgcn_sched_barrier(0);
     };
+    // Rotating epilogue: where the tile's rows go is looked up while the slabs travel: thread t asks
+    // for row m0 + t's position and request in front of the first slab (they come from L2 and hold
+    // nothing up) and for its page behind the second; the epilogue finds them in LDS. Looked up in
+    // the epilogue, row by row, the two dependent trips were a fifth of the kernel at 273 rows.
+    RowPlace place;
+    int place_seq = 0;
+    if (MODE == kRopeCache) {
+        const int mrow = m0 + tid < M ? m0 + tid : M - 1;         // (every thread loads: no load under a condition)
+        place.pos = qt.positions[mrow];
+        place_seq = qt.seq_idx[mrow];
+        __builtin_amdgcn_sched_barrier(0);
+    }
     if (kt_begin < kt_end) {
         Slab s0, s1;
         // (the scheduling barriers keep the three slabs' loads in this order: the loop's waits
@@ -483,6 +514,10 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
         __builtin_amdgcn_sched_barrier(0);
         load_global(kt_begin + 1, s1);
         __builtin_amdgcn_sched_barrier(0);
+        if (MODE == kRopeCache) {
+            place.page = qt.block_table[static_cast<size_t>(place_seq) * qt.max_blocks + place.pos / qt.page];
+            __builtin_amdgcn_sched_barrier(0);
+        }
         store_lds(0, s0);
         load_global(kt_begin + 2, s0);
         __builtin_amdgcn_sched_barrier(0);
@@ -503,7 +538,7 @@ __global__ __launch_bounds__(256, 2) void gemm_tile_kernel(const bf16* __restric
     if (AHEAD && N % 8 == 0) addends.load(out, M, N, m0, n0, tid);
     __syncthreads();                                  // the epilogue reuses the slabs' LDS
     tile_epilogue<WMT, WNT, MODE, tile_lds_bytes<WMT, WNT>(), 2, 2, AHEAD>(acc, lds_raw, out, M, N, m0, n0, wm, wn, tid, r, q,
-                                                                           qt, addends);
+                                                                           qt, addends, place);
 }
 
 // ----------------------------------------------------------------------------------------
