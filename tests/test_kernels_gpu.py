@@ -434,6 +434,9 @@ def _plain_attention_last_row(q, k, v):
     ([150 + 40 * i for i in range(16)], 6, 2, 48, 160),  # 16 rows; the last stretch of k has fewer heads
     ([900, 100, 1000], 8, 2, 128, 528),
     ([700, 701], 4, 2, 80, 64),
+    ([300, 301, 302], 4, 2, 112, 96),
+    ([700], 3, 1, 32, 48),                              # one stretch of k with fewer heads than it could hold
+    ([260, 500], 8, 4, 96, 112),
     ([520, 300, 900, 50], 34, 2, 16, 48),               # 16 heads of 16 to a stretch of k, the last stretch one block
     ([2000, 1800, 1900, 100, 2100], 24, 8, 128, 3072),  # three tiles per wavefront
     ([800, 900, 1000, 1100, 1200], 32, 8, 64, 6160)])   # four, and the last block of tiles not whole
