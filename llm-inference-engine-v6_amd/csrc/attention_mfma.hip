@@ -51,6 +51,21 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
                             n_kv, page, scale, window, split_len, nsplit, blockIdx.x, blockIdx.y, blockIdx.z, sh);
 }
 
+// The same for a step whose q/k/v rows are still as the projection left them (RAW in attention_tiles.h):
+// grid (request, kv head); a single split, so the output rows are written at once.
+template <int HD>
+__global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_raw_kernel(
+    float* qkv, const float* __restrict__ cos_t, const float* __restrict__ sin_t, bf16* k_cache, bf16* v_cache,
+    bf16* __restrict__ out, const int* __restrict__ q_start, const int* __restrict__ ctx_len,
+    const int* __restrict__ block_table, int max_blocks, int n_q, int n_kv, int page, float scale, int window,
+    int split_len) {
+    __shared__ float sh[decode_lds_floats(HD)];
+    const RawQkv raw{qkv, cos_t, sin_t, k_cache, v_cache};
+    decode_item<HD, true, true>(nullptr, k_cache, v_cache, out, nullptr, nullptr, q_start, ctx_len, block_table,
+                                max_blocks, n_q, n_kv, page, scale, window, split_len, 1, blockIdx.x, blockIdx.y, 0, sh,
+                                raw);
+}
+
 // Joins the splits of one (row, head): one wavefront, lanes over the splits for the statistics,
 // then over the head's dimensions for the weighted sum. nsplit <= 64. `base` is the first of the
 // nsplit parts. The partial outputs are asked for 16 splits at a time, the first 16 together with
@@ -419,6 +434,39 @@ extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const voi
         default: return kErrUnsupported;
     }
 #undef LLME_HEAD
+}
+
+// Decode attention over a step of single tokens whose q/k/v rows are still 32-bit and unrotated (what a
+// projection cut over k has added up): rotation, cache write and the clearing of the rows happen inside
+// the attention kernel, one workgroup per (request, kv head) and a single split of the keys. qkv
+// [n_seq, (n_q + 2 n_kv) hd] float32 (row s is request s; left zero), cos/sin [max_pos, hd / 2]; the caches
+// as in llme_attention_bf16, written at each request's position ctx_len[s]; out [n_seq, n_q hd] bfloat16.
+// Head size 64 or 128, up to 16 query heads per kv head; split_len a multiple of 32 that covers the longest
+// request.
+extern "C" int llme_attention_decode_rope_bf16(float* qkv, const float* cos_t, const float* sin_t, void* k_cache,
+                                               void* v_cache, void* out, const int* q_start, const int* ctx_len,
+                                               const int* block_table, int max_blocks, int n_seq, int n_q, int n_kv,
+                                               int hd, int page, float scale, int window, int split_len,
+                                               hipStream_t stream) {
+    if (n_seq <= 0) return 0;
+    if (!qkv || !cos_t || !sin_t || !k_cache || !v_cache || !out || !q_start || !ctx_len || !block_table) return kErrBadArgument;
+    if ((hd != 64 && hd != 128) || page % 16 != 0 || n_kv <= 0 || n_q % n_kv != 0 || n_q / n_kv > 16) return kErrUnsupported;
+    if (!(scale > 0.f) || split_len <= 0 || split_len % 32 != 0) return kErrBadArgument;
+    if (static_cast<double>(max_blocks) * (page / 16) * (page / 16) >= 4294967296.0) return kErrUnsupported;
+    if (static_cast<double>(n_kv) * page * hd >= 4294967296.0) return kErrUnsupported;
+    if (reinterpret_cast<uintptr_t>(qkv) % 16 != 0 || reinterpret_cast<uintptr_t>(cos_t) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(sin_t) % 16 != 0 || reinterpret_cast<uintptr_t>(k_cache) % 16 != 0)
+        return kErrUnsupported;
+    const dim3 grid(n_seq, n_kv);
+    if (hd == 64)
+        hipLaunchKernelGGL(attention_decode_raw_kernel<64>, grid, dim3(DEC_WAVES * 64), 0, stream, qkv, cos_t, sin_t,
+                           static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache), static_cast<bf16*>(out), q_start,
+                           ctx_len, block_table, max_blocks, n_q, n_kv, page, scale, window, split_len);
+    else
+        hipLaunchKernelGGL(attention_decode_raw_kernel<128>, grid, dim3(DEC_WAVES * 64), 0, stream, qkv, cos_t, sin_t,
+                           static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache), static_cast<bf16*>(out), q_start,
+                           ctx_len, block_table, max_blocks, n_q, n_kv, page, scale, window, split_len);
+    return launch_status();
 }
 
 // ------------------------------------------------------------------------------------------

@@ -358,13 +358,28 @@ __device__ __forceinline__ void load_q(const bf16* qrow, bool ok, bf16x8 (&qf)[(
 constexpr int DEC_WAVES = 4;
 __host__ __device__ constexpr int decode_lds_floats(int hd) { return DEC_WAVES * 16 * hd + 2 * DEC_WAVES * 16; }
 
-template <int HD, bool STREAM>
+// RAW: the step's q/k/v rows come as the projection left them, 32-bit and unrotated ([rows, (n_q + 2 n_kv)
+// hd], full rotation, head size 64 or 128), and the workgroup does what the rotation kernel would have
+// done for its request and kv head: it rotates its query heads into operand registers, rotates the new key,
+// writes key and value into the request's page, and sets what it has read of the row to zero (the buffer
+// is one that a product cut over k adds into). Only with a single split: every value of the row is then
+// read by one workgroup. The cache is non-const here: the new key and value go into it.
+struct RawQkv {
+    float* qkv = nullptr;            // [rows, (n_q + 2 n_kv) hd]
+    const float* cos_t = nullptr;    // [max_pos, hd / 2]
+    const float* sin_t = nullptr;
+    bf16* k_cache = nullptr;
+    bf16* v_cache = nullptr;
+};
+
+// (k_cache and v_cache carry no promise that nothing else points at them: RAW writes into them)
+template <int HD, bool STREAM, bool RAW = false>
 __device__ __forceinline__ void decode_item(
-    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    const bf16* __restrict__ q, const bf16* k_cache, const bf16* v_cache,
     bf16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ q_start, const int* __restrict__ ctx_len, const int* __restrict__ block_table,
     int max_blocks, int n_q, int n_kv, int page, float scale, int window, int split_len, int nsplit, int s,
-    int head_tile, int split, float* sh) {
+    int head_tile, int split, float* sh, const RawQkv& raw = RawQkv{}) {
     constexpr int DC = (HD + 31) / 32, DT = HD / 16;
     float (*sh_o)[16][HD] = reinterpret_cast<float (*)[16][HD]>(sh);
     float (*sh_m)[16] = reinterpret_cast<float (*)[16]>(sh + DEC_WAVES * 16 * HD);
@@ -393,7 +408,81 @@ __device__ __forceinline__ void decode_item(
     const int head = kvh * G + gt * 16 + r;             // this lane's row is a query head
     const bool row_ok = (gt * 16 + r) < G;
     bf16x8 qf[1][DC];
-    load_q<HD>(q + (static_cast<size_t>(row0) * n_q + (row_ok ? head : 0)) * HD, row_ok, qf[0]);
+    PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD,
+               page_magic_of(page), static_cast<unsigned>(n_kv) * page * HD, static_cast<unsigned>(kvh) * page * HD};
+    if constexpr (RAW) {
+        static_assert(!RAW || HD == 64 || HD == 128, "a lane holds a dim and its rotation partner");
+        constexpr int HALF = HD / 2;
+        float* qkv_row = raw.qkv + static_cast<size_t>(row0) * (n_q + 2 * n_kv) * HD;
+        const float* cs = raw.cos_t + static_cast<size_t>(pos) * HALF;
+        const float* sn = raw.sin_t + static_cast<size_t>(pos) * HALF;
+        // a + b i -> (a c - b s) + (b c + a s) i, as the rotation kernel computes it, then rounded
+        auto rotate8 = [&](const float* src, int d, bf16x8& lo, bf16x8& hi) {
+            const float4 a0 = *reinterpret_cast<const float4*>(src + d), a1 = *reinterpret_cast<const float4*>(src + d + 4);
+            const float4 b0 = *reinterpret_cast<const float4*>(src + d + HALF), b1 = *reinterpret_cast<const float4*>(src + d + HALF + 4);
+            const float4 c0 = *reinterpret_cast<const float4*>(cs + d), c1 = *reinterpret_cast<const float4*>(cs + d + 4);
+            const float4 s0 = *reinterpret_cast<const float4*>(sn + d), s1 = *reinterpret_cast<const float4*>(sn + d + 4);
+            const float a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+            const float b[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+            const float c[8] = {c0.x, c0.y, c0.z, c0.w, c1.x, c1.y, c1.z, c1.w};
+            const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                lo[j] = static_cast<__bf16>(a[j] * c[j] - b[j] * sv[j]);
+                hi[j] = static_cast<__bf16>(b[j] * c[j] + a[j] * sv[j]);
+            }
+        };
+        auto zero8 = [&](float* dst) {
+            const float4 z{0.f, 0.f, 0.f, 0.f};
+            reinterpret_cast<float4*>(dst)[0] = z;
+            reinterpret_cast<float4*>(dst)[1] = z;
+        };
+        // the query heads: lane (r, g4) holds dims 32 c + 8 g4 .. of head r, c < DC / 2, and their partners
+        float* qhead = qkv_row + static_cast<size_t>(row_ok ? head : 0) * HD;
+#pragma unroll
+        for (int c = 0; c < DC / 2; ++c) {
+            bf16x8 lo, hi;
+            rotate8(qhead, c * 32 + g4 * 8, lo, hi);
+            qf[0][c] = row_ok ? lo : zero_frag();
+            qf[0][c + DC / 2] = row_ok ? hi : zero_frag();
+        }
+        // the new key and value of this kv head: the first wavefront's lanes take 8 dims each
+        const PagePlace at = page_of(kv, pos);
+        const int pg = __builtin_amdgcn_readfirstlane(kv.table[at.block]);
+        if (wave == 0) {
+            float* krow = qkv_row + static_cast<size_t>(n_q + kvh) * HD;
+            float* vrow = qkv_row + static_cast<size_t>(n_q + n_kv + kvh) * HD;
+            if (lane < HALF / 8) {
+                bf16x8 lo, hi;
+                rotate8(krow, lane * 8, lo, hi);
+                bf16* dst = raw.k_cache + static_cast<size_t>(pg) * kv.page_stride + kv.head_off +
+                            static_cast<size_t>(at.offset) * HD + lane * 8;
+                *reinterpret_cast<bf16x8*>(dst) = lo;
+                *reinterpret_cast<bf16x8*>(dst + HALF) = hi;
+                zero8(krow + lane * 8);
+                zero8(krow + lane * 8 + HALF);
+            } else if (lane >= 32 && lane < 32 + HD / 8) {
+                const int d0 = (lane - 32) * 8;
+                const float4 v0 = *reinterpret_cast<const float4*>(vrow + d0), v1 = *reinterpret_cast<const float4*>(vrow + d0 + 4);
+                const float v[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+                bf16* dst = raw.v_cache + static_cast<size_t>(pg) * kv.page_stride + kv.head_off +
+                            static_cast<size_t>(d0) * page + at.offset;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) dst[static_cast<size_t>(j) * page] = static_cast<__bf16>(v[j]);
+                zero8(vrow + d0);
+            }
+        }
+        __syncthreads();                                // the key and the value are in the page; every wavefront has read q
+        if (wave == 0 && row_ok) {
+#pragma unroll
+            for (int c = 0; c < DC / 2; ++c) {
+                zero8(qhead + c * 32 + g4 * 8);
+                zero8(qhead + c * 32 + g4 * 8 + HALF);
+            }
+        }
+    } else {
+        load_q<HD>(q + (static_cast<size_t>(row0) * n_q + (row_ok ? head : 0)) * HD, row_ok, qf[0]);
+    }
     const int row_pos[1] = {row_ok ? pos : -1};
     const int row_lo[1] = {lo_all};
     const int tile_free[1] = {-1};                      // few blocks, heads may be missing: always checked
@@ -402,8 +491,6 @@ __device__ __forceinline__ void decode_item(
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[0][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    PagedKV kv{k_cache, v_cache, block_table + static_cast<size_t>(s) * max_blocks, page, n_kv, kvh, HD,
-               page_magic_of(page), static_cast<unsigned>(n_kv) * page * HD, static_cast<unsigned>(kvh) * page * HD};
     const int first = k_begin + __builtin_amdgcn_readfirstlane(wave) * 32;
     attend_range<HD, 1, STREAM>(kv, first, DEC_WAVES * 32, lo_all, k_end, qf, row_pos, row_lo, tile_free,
                               scale * kLog2e, m, l, o);

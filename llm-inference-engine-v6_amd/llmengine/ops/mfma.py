@@ -344,6 +344,45 @@ def _fast_attention_project(q, k_cache, v_cache, o, step, block_table, n_q, n_kv
 
 kernels._fast_attention_project = _fast_attention_project
 
+declare("llme_attention_decode_rope_bf16", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i,
+                                            _i, _vp])
+DECODE_ROPE = True                  # (tests and measurements switch the fused kernel off here)
+
+
+def attention_decode_rope(qkv, cos, sin, k_cache, v_cache, out, step, block_table, n_q: int, n_kv: int, head_dim: int,
+                          scale: float, window: int) -> bool:
+    """A step of single decoded tokens whose q/k/v rows [S, (n_q + 2 n_kv) head_dim] are still 32-bit and
+    unrotated: rotation, the cache write at each request's position, attention over the pages into out
+    [S, n_q head_dim] and the clearing of qkv, in the attention kernel (one workgroup per request and kv
+    head, the keys in a single split). False, and nothing done, where the step or the sizes are not such."""
+    T = qkv.shape[0]
+    if (not DECODE_ROPE or not kernels.policy.fast_attention or T != step.num_seqs or head_dim not in (64, 128)
+            or cos is None or cos.shape[1] * 2 != head_dim or n_q % n_kv or n_q // n_kv > 16
+            or qkv.dtype != torch.float32 or out.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16
+            or k_cache.shape[2] % 16 or qkv.data_ptr() % 16 or cos.data_ptr() % 16 or sin.data_ptr() % 16
+            or k_cache.data_ptr() % 16):
+        return False
+    key = ("attention_plan", n_q, n_kv, head_dim)
+    plan = step.extra.get(key)
+    if plan is None:
+        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len)
+    if plan["n_decode"] != T or plan["groups"] or plan["nsplit"] != 1:
+        return False
+    S = T
+    require(qkv, "qkv", torch.float32, (S, (n_q + 2 * n_kv) * head_dim))
+    require(cos, "cos", torch.float32, (None, head_dim // 2))
+    require(sin, "sin", torch.float32, tuple(cos.shape))
+    require(out, "out", torch.bfloat16, (S, n_q * head_dim))
+    require(k_cache, "k_cache", torch.bfloat16, (None, n_kv, None, head_dim))
+    page = k_cache.shape[2]
+    require(v_cache, "v_cache", torch.bfloat16, (k_cache.shape[0], n_kv, head_dim, page))
+    require(block_table, "block_table", torch.int32, (S, None))
+    check(entry("llme_attention_decode_rope_bf16")(
+        ptr(qkv), ptr(cos), ptr(sin), ptr(k_cache), ptr(v_cache), ptr(out), ptr(step.q_start), ptr(step.ctx_len),
+        ptr(block_table), block_table.shape[1], S, n_q, n_kv, head_dim, page, float(scale), int(window),
+        plan["split_len"], stream()), "attention_decode_rope")
+    return True
+
 
 # --- projections fused with the norm in front of them (decoding) ---------------------------
 declare("llme_gemv_norm", [_vp, _vp, _vp, _i, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp])

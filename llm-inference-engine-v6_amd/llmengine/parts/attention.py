@@ -134,6 +134,14 @@ class Attention(Mixer):
             if applies:
                 self.position.apply(qkv[:, :self.q_dim].view(T, n_q, hd),
                                     qkv[:, self.q_dim:self.q_dim + self.kv_dim].view(T, n_kv, hd), step.positions)
+            if adds and not applies and rot == hd:
+                # decoded tokens only: the attention kernel rotates, writes the cache and clears the rows itself
+                o = step.buffer("attn.o", (T, self.q_dim), act)
+                if ops.mfma.attention_decode_rope(qkv, cos, sin, k_cache, v_cache, o, step, block_table, n_q, n_kv, hd,
+                                                  self.scale, self.window):
+                    step.extra["attn.qkv zero"] = (qkv.data_ptr(), qkv.numel())
+                    ops.gemm(o, self.w_o, out, accumulate, fixed_order=step.fixed_order)
+                    return
             ops.rope_kv_write(qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
                               n_q, n_kv, hd, rot, write_cache=True, zero_input=adds)
             if adds:

@@ -349,6 +349,51 @@ def test_decoded_tokens_join_their_splits_inside_the_output_projection(zoo, n_li
             assert np.abs(got[rid][pos].astype(np.float64) - apart[rid][pos]).max() / top < 2e-3, (rid, pos)
 
 
+@pytest.mark.parametrize("name", ["C", "F"])
+def test_twenty_decoded_tokens_are_rotated_inside_the_attention_kernel(zoo, name, monkeypatch):
+    """17 to 64 decoded tokens a step: q/k/v is a product cut over k into a cleared 32-bit buffer, and where
+    the keys are in one split the attention kernel itself rotates, writes the cache and clears the rows.
+    It must have run, match the plain implementation, and give exactly what the rotation kernel and the
+    decode kernel give apart (also on the steps after the first, which find the buffer cleared)."""
+    from llmengine.ops import mfma
+    from tiny_models import TINY_F
+    calls = []
+    inside = mfma.attention_decode_rope
+
+    def noting(*args, **kw):
+        done = inside(*args, **kw)
+        calls.append(done)
+        return done
+    monkeypatch.setattr(mfma, "attention_decode_rope", noting)
+    # (a recorded step plans its splits for the width of its block table, 1,024 tokens and more: with the
+    # few kv heads of these models it would cut the keys; models with 8 kv heads do not from 17 requests on)
+    monkeypatch.setattr(mfma, "DECODE_BLOCKS_WANTED", 1)
+    model_dir, _, _, page = zoo[name]
+    cfg = TINY_C if name == "C" else TINY_F
+    reqs = {f"s{i}": random_tokens(60 + 3 * i, cfg["vocab_size"], 190 + i) for i in range(20)}
+    pcfg, pw = load_plain_model(model_dir)
+    engine = engine_for(model_dir, "bf16")
+    steps = [{"step": 0, "entries": [{"id": rid, "tokens": ids[:-12], "want": []} for rid, ids in reqs.items()], "end": []}]
+    for t in range(12, 0, -1):
+        steps.append({"step": len(steps), "end": list(reqs) if t == 1 else [],
+                      "entries": [{"id": rid, "tokens": [ids[-t]], "want": [0]} for rid, ids in reqs.items()]})
+    pages = replay.trace_peak_tokens(steps, round_to=page) // page
+
+    def run():
+        cache = engine.new_cache(pages, page, max_requests=20)
+        return replay.run_trace(engine, cache, steps)
+    got = run()
+    assert calls and all(calls), "the decode steps did not rotate inside the attention kernel"
+    monkeypatch.setattr(mfma, "DECODE_ROPE", False)
+    apart = run()
+    for rid, ids in reqs.items():
+        ref = plain_forward(pcfg, pw, ids, rounder=bf16_round).numpy()
+        for pos in range(len(ids) - 12, len(ids)):
+            top = np.abs(ref[pos]).max()
+            assert np.abs(got[rid][pos].astype(np.float64) - ref[pos]).max() / top < TOL["bf16"], (rid, pos)
+            assert np.abs(got[rid][pos].astype(np.float64) - apart[rid][pos]).max() / top < 2e-3, (rid, pos)
+
+
 # A layer or two with the sizes of Llama 3.2 1B, 3.2 3B and 3.1 8B: the kernels that serving picks at
 # real widths (tiled products over several row tiles, the prefill attention with many work items, the
 # fused decode kernels at widths 2048, 3072 and 4096, the output head over the whole vocabulary).

@@ -477,6 +477,86 @@ def test_attention_join_project(ops, lens, n_q, n_kv, hd, N):
     assert _rel(out.cpu().double(), base.double() + ref @ w.double().T) < 8e-3
 
 
+@pytest.mark.parametrize("lens,n_q,n_kv,hd,page,window", [
+    ([1, 2, 17, 33, 64, 65, 300, 77, 129] * 2, 32, 8, 64, 16, 0),
+    ([40 + 7 * i for i in range(24)], 24, 8, 128, 16, 0),
+    ([5, 90, 200, 31, 32, 33] * 3, 8, 8, 64, 32, 0),          # one query head per kv head, pages of 32
+    ([20 + 5 * i for i in range(20)], 16, 1, 128, 64, 0),      # 16 query heads on one kv head
+    ([30, 100, 120, 61] * 5, 8, 2, 64, 16, 48)])               # a window
+def test_attention_decode_with_rotation_inside(ops, lens, n_q, n_kv, hd, page, window):
+    """Decoded tokens whose q/k/v rows are still 32-bit and unrotated: the attention kernel rotates, writes
+    key and value into the pages, attends and clears the rows. Against the rotation kernel followed by
+    the decode kernel (same pages afterwards, same output) and against plain attention."""
+    import types
+    S, T = len(lens), sum(lens)
+    g = _gen(71)
+    width = (n_q + 2 * n_kv) * hd
+    qkv = torch.randn(T, width, generator=g)
+    half = hd // 2
+    inv = 1.0 / (10000.0 ** (torch.arange(half, dtype=torch.float64) * 2 / hd))
+    ang = torch.arange(max(lens) + 3, dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = torch.cos(ang).float().to(DEV), torch.sin(ang).float().to(DEV)
+    nblk = [(n + page - 1) // page for n in lens]
+    total_pages = sum(nblk) + 2
+    perm = torch.randperm(total_pages, generator=g).tolist()
+    table = torch.zeros(S, max(nblk), dtype=torch.int32)
+    p = 0
+    for s_, nb in enumerate(nblk):
+        for b in range(nb):
+            table[s_, b] = perm[p]
+            p += 1
+    table = table.to(DEV)
+    positions = torch.cat([torch.arange(n) for n in lens]).to(torch.int32)
+    seq_idx = torch.cat([torch.full((n,), s_) for s_, n in enumerate(lens)]).to(torch.int32)
+    last = torch.tensor([sum(lens[:i + 1]) - 1 for i in range(S)])
+    is_last = torch.zeros(T, dtype=torch.bool)
+    is_last[last] = True
+
+    def caches():
+        return (torch.zeros(total_pages, n_kv, page, hd, dtype=torch.bfloat16, device=DEV),
+                torch.zeros(total_pages, n_kv, hd, page, dtype=torch.bfloat16, device=DEV))
+    i32 = dict(dtype=torch.int32, device=DEV)
+    q_start, ctx = torch.arange(S + 1, **i32), torch.tensor([n - 1 for n in lens], **i32)
+    scale = 1.0 / math.sqrt(hd)
+    # apart: every token through the rotation kernel, then the decode kernel over the last ones
+    k1, v1 = caches()
+    q_all = torch.empty(T, n_q * hd, dtype=torch.bfloat16, device=DEV)
+    ops.rope_kv_write(qkv.to(DEV), cos, sin, positions.to(DEV), seq_idx.to(DEV), table, q_all, k1, v1, n_q, n_kv, hd, hd)
+    plan = ops.mfma.plan_attention([1] * S, [n - 1 for n in lens], n_q, n_kv, hd)
+    assert plan["nsplit"] == 1
+    apart = torch.zeros(S, n_q * hd, dtype=torch.bfloat16, device=DEV)
+    ops.mfma.attention_bf16(q_all[last.to(DEV)].contiguous(), k1, v1, apart, q_start, ctx, table, n_q, n_kv, hd, scale,
+                            window, plan)
+    # together: the earlier tokens through the rotation kernel, the last ones raw
+    k2, v2 = caches()
+    before = ~is_last
+    if before.any():
+        ops.rope_kv_write(qkv[before].contiguous().to(DEV), cos, sin, positions[before].contiguous().to(DEV),
+                          seq_idx[before].contiguous().to(DEV), table, torch.empty(int(before.sum()), n_q * hd,
+                          dtype=torch.bfloat16, device=DEV), k2, v2, n_q, n_kv, hd, hd)
+    raw = qkv[last].contiguous().to(DEV)
+    step = types.SimpleNamespace(num_seqs=S, new_lens=[1] * S, ctx_lens=[n - 1 for n in lens], plan_len=None, extra={},
+                                 q_start=q_start, ctx_len=ctx)
+    out = torch.zeros(S, n_q * hd, dtype=torch.bfloat16, device=DEV)
+    assert ops.mfma.attention_decode_rope(raw, cos, sin, k2, v2, out, step, table, n_q, n_kv, hd, scale, window)
+    assert not raw.any(), "the rows are left zero"
+    assert torch.equal(k1, k2) and torch.equal(v1, v2), "the pages hold what the rotation kernel writes"
+    assert torch.equal(out, apart)
+    # plain attention of the last rows
+    rows = []
+    for s_, n in enumerate(lens):
+        blk = qkv[last[s_] - n + 1:last[s_] + 1].double()
+        q = blk[:, :n_q * hd].reshape(n, n_q, hd)
+        k = blk[:, n_q * hd:(n_q + n_kv) * hd].reshape(n, n_kv, hd)
+        v = blk[:, (n_q + n_kv) * hd:].reshape(n, n_kv, hd)
+        c = torch.cat([cos[:n].cpu(), cos[:n].cpu()], dim=1).double()
+        sn = torch.cat([sin[:n].cpu(), sin[:n].cpu()], dim=1).double()
+        q, k = plain_apply_rope(q, c, sn), plain_apply_rope(k, c, sn)
+        lo = max(0, n - window) if window > 0 else 0
+        rows.append(_plain_attention_last_row(q[lo:], k[lo:], v[lo:]).reshape(1, n_q * hd))
+    assert _rel(out.cpu().double(), torch.cat(rows)) < 8e-3
+
+
 def test_attention_join_project_refuses(ops):
     from llmengine.ops import KernelError
     w = ops.block_weight(torch.zeros(64, 128, dtype=torch.bfloat16, device=DEV))
