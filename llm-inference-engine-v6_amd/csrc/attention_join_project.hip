@@ -17,8 +17,6 @@
 
 namespace llme {
 
-typedef __attribute__((ext_vector_type(4))) unsigned jp_u32x4;
-
 constexpr int JP_WAVES = 4;
 constexpr int JP_MAX_KP = 256;                       // dims of a workgroup's heads at most
 constexpr int JP_KB = JP_MAX_KP / 32;                // 32-wide k blocks of a stretch at most
