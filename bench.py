@@ -323,16 +323,15 @@ def main() -> int:
             f"({batch * start_ctx / t_fill:.0f} tok/s, token generation on the host included)")
         last = torch.randint(0, V, (batch,), generator=gen).tolist()
 
-        def one_step(tokens):
-            return engine.run_step(cache, [StepEntry(rid, [t], [0]) for rid, t in zip(ids, tokens)], None)
-        for _ in range(warmup):
-            last = one_step(last)
+        # greedy decoding as `Engine.generate` runs it: every step's tokens feed the next on the device, and
+        # the host fetches a step's tokens while the next step runs
+        last = engine.greedy_chain(cache, ids, last, warmup)[-1] if warmup > 0 else last
         sync()
         t = time.perf_counter()
-        for _ in range(steps):
-            last = one_step(last)
+        chosen = engine.greedy_chain(cache, ids, last, steps)
         sync()
         dt = time.perf_counter() - t
+        assert len(chosen) == steps and all(len(c) == batch for c in chosen)
         for rid in ids:
             cache.release(rid)
         mean_ctx = start_ctx + warmup + (steps + 1) / 2.0

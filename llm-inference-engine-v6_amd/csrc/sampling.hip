@@ -68,9 +68,13 @@ __global__ __launch_bounds__(kSampleThreads) void argmax_part_kernel(const float
     }
 }
 
+// out[slot R + row] (slot: a number the device holds, 0 without one), and also[row] where that is given:
+// a recorded decode step leaves its choice for the host in one of two places in turn, and for its own
+// next replay among its integer arrays.
 __global__ __launch_bounds__(kWave) void argmax_join_kernel(const float* __restrict__ part_val,
                                                             const int* __restrict__ part_idx, int* __restrict__ out,
-                                                            int parts) {
+                                                            int parts, int* __restrict__ also = nullptr,
+                                                            const int* __restrict__ slot = nullptr) {
     float bv = -INFINITY;
     int bi = 0x7fffffff;
     for (int p = threadIdx.x; p < parts; p += kWave)
@@ -81,7 +85,11 @@ __global__ __launch_bounds__(kWave) void argmax_join_kernel(const float* __restr
         const int oi = __shfl_xor(bi, off, kWave);
         argmax_combine(bv, bi, ov, oi);
     }
-    if (threadIdx.x == 0) out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
+    if (threadIdx.x == 0) {
+        const int token = (bi == 0x7fffffff) ? 0 : bi;
+        out[(slot ? *slot * static_cast<int>(gridDim.x) : 0) + blockIdx.x] = token;
+        if (also) also[blockIdx.x] = token;
+    }
 }
 
 // Temperature sampling in three stages over the same parts as the greedy choice. The first is
@@ -212,7 +220,22 @@ extern "C" int llme_argmax(const float* logits, int* out, float* part_val, int* 
     const int chunk = (V + parts - 1) / parts;
     hipLaunchKernelGGL(argmax_part_kernel, dim3(R, parts), dim3(kSampleThreads), 0, stream, logits, part_val,
                        part_idx, V, chunk);
-    hipLaunchKernelGGL(argmax_join_kernel, dim3(R), dim3(kWave), 0, stream, part_val, part_idx, out, parts);
+    hipLaunchKernelGGL(argmax_join_kernel, dim3(R), dim3(kWave), 0, stream, part_val, part_idx, out, parts,
+                       static_cast<int*>(nullptr), static_cast<const int*>(nullptr));
+    return launch_status();
+}
+
+// The same with the choice left in two places: out[*slot * R + row] (slot: an int in device memory that is 0
+// or 1; out holds 2 R ints) and also[row]. For a recorded step whose next replay reads the tokens it chose.
+extern "C" int llme_argmax_to(const float* logits, int* out, int* also, const int* slot, float* part_val,
+                              int* part_idx, int R, int V, hipStream_t stream) {
+    if (R <= 0) return 0;
+    if (V <= 0 || !out) return kErrBadArgument;
+    const int parts = llme_argmax_parts(V);
+    const int chunk = (V + parts - 1) / parts;
+    hipLaunchKernelGGL(argmax_part_kernel, dim3(R, parts), dim3(kSampleThreads), 0, stream, logits, part_val,
+                       part_idx, V, chunk);
+    hipLaunchKernelGGL(argmax_join_kernel, dim3(R), dim3(kWave), 0, stream, part_val, part_idx, out, parts, also, slot);
     return launch_status();
 }
 

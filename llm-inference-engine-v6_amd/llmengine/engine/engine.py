@@ -218,6 +218,38 @@ class Engine:
                 sampler = self._samplers[(float(temperature), int(seed))] = Sampler(temperature, seed)
             return sampler.choose(logits, draws)
 
+    def greedy_chain(self, cache: CacheContext, request_ids: Sequence, tokens: Sequence[int], steps: int
+                     ) -> list[list[int]]:
+        """`steps` greedy decode steps of the live requests `request_ids`, the first on `tokens` (one per
+        request), every later one on the tokens the step before it chose. Those stay on the device: a
+        step is launched before the host has fetched the tokens of the one before, so the host's work
+        for a step runs beside the device's. Returns every step's tokens. (Stopping is the caller's
+        business: `generate` runs the same loop with its own check.)"""
+        ids = list(request_ids)
+        first = self._validate_ids(tokens, "greedy_chain")
+        if len(first) != len(ids):
+            raise ValueError("greedy_chain: one token per request")
+        out: list[list[int]] = []
+        if steps <= 0:
+            return out
+        with self._lock, torch.cuda.device(self.runner.device):
+            runner = self.runner
+            if not runner.use_graphs:
+                last = first
+                for _ in range(steps):
+                    last = self.run_step(cache, [StepEntry(r, [t], [0]) for r, t in zip(ids, last)], None)
+                    out.append(last)
+                return out
+            pending = runner.greedy_launch(cache, ids, first, self.max_pos)
+            for i in range(1, steps + 1):
+                ahead = runner.greedy_launch(cache, ids, None, self.max_pos) if i < steps else None
+                last = runner.greedy_result(pending)
+                out.append(last)
+                if i < steps and ahead is None:          # (the recording changed: the tokens go through the host once)
+                    ahead = runner.greedy_launch(cache, ids, last, self.max_pos)
+                pending = ahead
+        return out
+
     # ---- whole-sequence logits (src/engine.cpp:694-716) ----
     def _validate_ids(self, ids: Sequence[int], what: str) -> list[int]:
         ids = [int(t) for t in ids]
@@ -289,14 +321,35 @@ class Engine:
                     logits = self.step(cache, [StepEntry(rid, part, [len(part) - 1] if last else [])])
                 finish = "length"
                 generated = 0
+                runner = self.runner
+                greedy = self.sampler.temperature == 0.0 and runner.use_graphs
+                pending = None
                 while generated < max_new_tokens:
-                    nxt = self.sampler.choose(logits, [(0, generated)])[0]
+                    if pending is None:
+                        nxt = self.sampler.choose(logits, [(0, generated)])[0]
+                    else:
+                        # greedy: the step behind this one is launched on the token the device holds
+                        # before the host has fetched it (one step more than needed if this one stops)
+                        more = generated + 1 < max_new_tokens     # the token being fetched is not the last wanted
+                        with torch.cuda.device(runner.device):
+                            ahead = runner.greedy_launch(cache, [rid], None, self.max_pos) if more else None
+                            nxt = runner.greedy_result(pending)[0]
                     if nxt in eos:
                         finish = "stop"
+                        if pending is not None and ahead is not None:
+                            runner.greedy_result(ahead)
                         break
                     out.append(nxt)
                     generated += 1
-                    if generated < max_new_tokens:
+                    if generated >= max_new_tokens:
+                        break
+                    if greedy:
+                        with torch.cuda.device(runner.device):
+                            if pending is not None and ahead is not None:
+                                pending = ahead
+                            else:
+                                pending = runner.greedy_launch(cache, [rid], [nxt], self.max_pos)
+                    else:
                         logits = self.step(cache, [StepEntry(rid, [nxt], [0])])
                 return out, finish
             finally:

@@ -140,17 +140,21 @@ class CacheContext:
         self.page_size = page_size
         self.max_requests = max_requests
         self.graphs: dict = {}          # recorded decode steps over this pool's tensors, by shape
+        self.chain = None               # the last greedy launch: (recording, requests, its key), see greedy_launch
 
     def admit(self, request_id) -> int:
+        self.chain = None
         slot = self.manager.admit(request_id)
         self.storage.clear_slot(slot)
         return slot
 
     def slot_admitted(self, slot: int) -> None:
         """A request was admitted by the host runtime itself (the scheduler): its state starts empty."""
+        self.chain = None
         self.storage.clear_slot(slot)
 
     def release(self, request_id) -> None:
+        self.chain = None
         self.manager.release(request_id)
 
 
@@ -164,15 +168,21 @@ class _DecodeRecord:
     def __init__(self, graph, logits, meta: torch.Tensor, S: int, width: int, groups: list[str],
                  tok_host: torch.Tensor | None = None):
         self.graph, self.logits, self.meta = graph, logits, meta
-        self.tok_host = tok_host                # pinned: where a greedy recording leaves the chosen tokens
-        self.tok_event = torch.cuda.Event() if tok_host is not None else None
+        # pinned, 2 S: where a greedy recording leaves the chosen tokens, in its two halves in turn (the
+        # half is named by the integer behind the arrays), so that a step can be launched before the
+        # tokens of the one before it have been read; the same tokens also land in the token array
+        # itself, where the next replay finds them without the host
+        self.tok_host = tok_host
+        self.tok_events = [torch.cuda.Event(), torch.cuda.Event()] if tok_host is not None else None
+        self.slot = 1                           # the half the last launch used
+        self.launches = [0, 0]                  # launches into each half so far
         self.S, self.width, self.groups = S, width, groups
         sizes = [S, S, S, S + 1, S, S] + [S * width] * len(groups) + [S]
         self.offsets = [0]
         for n in sizes:
             self.offsets.append(self.offsets[-1] + n)
         self.total = self.offsets[-1]
-        self.host = torch.zeros(self.total, dtype=torch.int32, pin_memory=True)
+        self.host = torch.zeros(self.total + 1, dtype=torch.int32, pin_memory=True)   # (+ the half's number)
         self.np = h = self.host.numpy()
         o, G = self.offsets, len(groups)
         h[o[2]:o[3]] = range(S)                 # request index of each token
@@ -185,7 +195,9 @@ class _DecodeRecord:
         self.event: torch.cuda.Event | None = None
         self.scratch = None
 
-    def refresh(self, mgr: CacheManager, entries: Sequence[StepEntry], keys=None) -> None:
+    def refresh(self, mgr: CacheManager, entries: Sequence[StepEntry] | None, keys=None, slot: int = 0) -> None:
+        """entries None: the tokens are the ones the last replay chose and left in the device's array;
+        everything else is rewritten as always."""
         if self.event is not None:
             self.event.synchronize()            # the last copy has read the host mirror
         S, width, o, h = self.S, self.width, self.offsets, self.np
@@ -196,7 +208,9 @@ class _DecodeRecord:
             if keys != self.key_list:
                 self.key_list = keys
                 self.keys = (ctypes.c_int64 * S)(*keys)
-        h[o[0]:o[1]] = [e.tokens[0] for e in entries]
+        if entries is not None:
+            h[o[0]:o[1]] = [e.tokens[0] for e in entries]
+        h[self.total] = slot
         # lengths (tokens cached before this step), slots and the block-table entries that are new,
         # straight from the C++ manager into the pinned mirror
         base = h.ctypes.data
@@ -205,10 +219,18 @@ class _DecodeRecord:
         if rc != 0:
             raise RuntimeError(f"a request of the recorded step is not live (code {rc})")
         h[o[1]:o[2]] = h[o[4]:o[5]]             # the new token's position
-        self.meta[:self.total].copy_(self.host, non_blocking=True)
+        first = 0 if entries is not None else o[1]
+        self.meta[first:self.total + 1].copy_(self.host[first:], non_blocking=True)
         if self.event is None:
             self.event = torch.cuda.Event()
         self.event.record()
+
+
+class PendingTokens:
+    """A launched greedy step whose tokens have not been fetched yet."""
+
+    def __init__(self, rec: _DecodeRecord, slot: int, launch: int):
+        self.rec, self.slot, self.launch = rec, slot, launch
 
 
 class ModelRunner:
@@ -246,6 +268,7 @@ class ModelRunner:
         mgr = cache.manager
         if not entries:
             return None
+        cache.chain = None                      # (a later greedy launch takes its tokens from the host again)
         vocab = self.model.vocab_size
         seen = set()
         for e in entries:
@@ -293,27 +316,34 @@ class ModelRunner:
         self.graph_replays += 1
         return rec.logits
 
-    def _decode_record(self, cache: CacheContext, entries: Sequence[StepEntry], longest: int, greedy: bool):
+    def _decode_key(self, cache: CacheContext, S: int, longest: int, greedy: bool):
+        need = (longest + cache.page_size) // cache.page_size
+        bucket = self.GRAPH_BLOCK_BUCKET
+        return (S, (need + bucket - 1) // bucket * bucket, greedy)
+
+    def _decode_record(self, cache: CacheContext, entries: Sequence[StepEntry] | None, longest: int, greedy: bool,
+                       S: int | None = None):
         """The recording for this many requests and this width of block tables (and, greedy, with
         the argmax behind the model and its result written into pinned host memory); made at its
-        first use."""
+        first use (which needs the entries)."""
         page = cache.page_size
         mgr = cache.manager
-        S = len(entries)
-        need = (longest + page) // page
-        bucket = self.GRAPH_BLOCK_BUCKET
-        width = (need + bucket - 1) // bucket * bucket
-        key = (S, width, greedy)
+        S = len(entries) if S is None else S
+        key = self._decode_key(cache, S, longest, greedy)
+        width = key[1]
         rec = cache.graphs.pop(key, None)
         if rec is not None:
             cache.graphs[key] = rec                      # (most recently used last)
         if rec is None:
+            if entries is None:
+                raise RuntimeError("a step that takes its tokens from the step before has no recording to run in")
             while len(cache.graphs) >= self.GRAPH_LIMIT:
                 del cache.graphs[next(iter(cache.graphs))]
             # First time: run it plainly (this also sizes the scratch buffers), then record.
             # The recorded step reads its integer arrays from a buffer of its own.
             groups = len(mgr.groups)
-            meta = torch.empty(7 * S + 1 + groups * S * width + 64, dtype=torch.int32, device=self.device)
+            total = 7 * S + 1 + groups * S * width
+            meta = torch.zeros(total + 64, dtype=torch.int32, device=self.device)
             ctx, logit_rows = self._build_context(cache, entries, max_blocks=width, plan_len=width * page, dev=meta)
             logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
             tok_host = scratch = None
@@ -321,16 +351,18 @@ class ModelRunner:
                 # pinned host memory is mapped into the device's address space: the kernel writes
                 # the tokens where the host reads them, without a copy of its own; the argmax's
                 # scratch belongs to the recording (the one that plain calls share may be replaced)
-                tok_host = torch.zeros(S, dtype=torch.int32, pin_memory=True)
+                tok_host = torch.zeros(2 * S, dtype=torch.int32, pin_memory=True)
                 scratch = ops.sampling_scratch(self.device, S, self.model.vocab_size)
-                ops.argmax_into(logits, tok_host.data_ptr(), scratch)
+                ops.argmax_into(logits, tok_host.data_ptr(), scratch, also_ptr=meta.data_ptr(),
+                                slot_ptr=meta.data_ptr() + 4 * total)
             torch.cuda.synchronize(self.device)
             self.workspace.keep_replaced = True
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
                 if greedy:
-                    ops.argmax_into(logits, tok_host.data_ptr(), scratch)
+                    ops.argmax_into(logits, tok_host.data_ptr(), scratch, also_ptr=meta.data_ptr(),
+                                    slot_ptr=meta.data_ptr() + 4 * total)
             cache.graphs[key] = rec = _DecodeRecord(graph, logits, meta, S, width, list(mgr.groups), tok_host)
             rec.scratch = scratch                       # (kept alive: the graph holds its addresses)
         return rec
@@ -351,12 +383,34 @@ class ModelRunner:
             if not 0 <= int(e.tokens[0]) < vocab:
                 raise ValueError(f"token id {e.tokens[0]} out of range [0, {vocab})")
             ids.append(e.request_id)
+        pending = self.greedy_launch(cache, ids, [int(e.tokens[0]) for e in entries], max_position)
+        return self.greedy_result(pending)
+
+    def greedy_launch(self, cache: CacheContext, ids: Sequence, tokens: Sequence[int] | None,
+                      max_position: int | None = None) -> "PendingTokens | None":
+        """Launches a step of one token for each of the live requests `ids` whose greedy choices
+        `greedy_result` fetches later. tokens None: every request's token is the one that the launch
+        before this one chose for it, taken where that step's argmax left it on the device, so that
+        this step can be launched before the host has seen those tokens (the host's work for a step,
+        some 40 us, then runs beside the device's instead of in front of it). That needs the launch
+        before to have been of the same requests in the same recording; where it was not (the first
+        step, or the block tables have outgrown the recording), None is returned and nothing is
+        done: the caller fetches the tokens and passes them. At most one launch may be waiting for
+        its `greedy_result` when another is made."""
         S = len(ids)
         if len(set(ids)) != S:
             raise ValueError("a request appears twice in one step")
         mgr = cache.manager
         keys = (ctypes.c_int64 * S)(*[mgr.key_of(r) for r in ids])
         lengths = (ctypes.c_int * S)()
+        if tokens is None:
+            # (asked before anything changes: a chain that cannot go on leaves the manager as it was)
+            last = cache.chain
+            if last is None or last[1] != list(ids):
+                return None
+            longest = max(mgr.length(r) for r in ids)
+            if self._decode_key(cache, S, longest, greedy=True) != last[2] or cache.graphs.get(last[2]) is not last[0]:
+                return None
         # lengths, the position limit and the pages in one call; a call that fails has changed nothing
         rc = mgr._lib.llme_cm_decode_begin(mgr.handle, S, keys, lengths, int(max_position or 0))
         if rc < 0:
@@ -368,14 +422,28 @@ class ModelRunner:
             need = {g: sum(mgr.pages_needed(r, 1)[g] for r in ids) for g in mgr.groups}
             raise CapacityError(f"the step needs {need} more pages, free are "
                                 f"{({g: mgr.free_pages(g) for g in mgr.groups})}")
-        rec = self._decode_record(cache, entries, longest, greedy=True)
-        rec.refresh(mgr, entries, keys)
+        entries = None if tokens is None else [StepEntry(r, [t], [0]) for r, t in zip(ids, tokens)]
+        rec = self._decode_record(cache, entries, longest, greedy=True, S=S)
+        slot = 1 - rec.slot
+        rec.refresh(mgr, entries, keys, slot=slot)
         rec.graph.replay()
-        rec.tok_event.record()
+        rec.tok_events[slot].record()
+        rec.slot = slot
+        rec.launches[slot] += 1                 # (what an older launch left in this half is gone)
         self.graph_replays += 1
         mgr._lib.llme_cm_commit_batch(mgr.handle, S, keys, 1)
-        rec.tok_event.synchronize()
-        return rec.tok_host.tolist()
+        cache.chain = (rec, list(ids), self._decode_key(cache, S, longest, greedy=True))
+        return PendingTokens(rec, slot, rec.launches[slot])
+
+    def greedy_result(self, pending: "PendingTokens") -> list[int]:
+        """The tokens a launched step chose (waits for it). They can be fetched until the launch
+        after the next one, which uses the same half of the recording's token buffer."""
+        rec, slot = pending.rec, pending.slot
+        if rec.launches[slot] != pending.launch:
+            raise RuntimeError("the tokens of this launch have been overwritten: two later steps were launched "
+                               "before they were fetched")
+        rec.tok_events[slot].synchronize()
+        return rec.tok_host[slot * rec.S:(slot + 1) * rec.S].tolist()
 
     # ------------------------------------------------------------------------------
     def _build_context(self, cache: CacheContext, entries: Sequence[StepEntry], max_blocks: int | None = None,

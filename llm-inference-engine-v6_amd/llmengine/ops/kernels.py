@@ -296,13 +296,19 @@ def argmax(logits: torch.Tensor, out: torch.Tensor, scratch=None) -> None:
     argmax_into(logits, ptr(out), scratch)
 
 
-def argmax_into(logits: torch.Tensor, out_ptr: int, scratch=None) -> None:
+def argmax_into(logits: torch.Tensor, out_ptr: int, scratch=None, also_ptr: int = 0, slot_ptr: int = 0) -> None:
     """argmax with the result (one int32 per row) written to an address the device can reach:
-    device memory, or pinned host memory, which the device sees at the same address."""
+    device memory, or pinned host memory, which the device sees at the same address. also_ptr: a
+    second place for the same result. slot_ptr: an int32 in device memory, 0 or 1: the result goes to
+    out_ptr + 4 * slot * rows (out then holds two results in turn)."""
     require(logits, "logits", torch.float32, (None, None))
     R, V = logits.shape
     val, idx, _ = _scratch_for(logits, scratch)
-    check(entry("llme_argmax")(ptr(logits), out_ptr, ptr(val), ptr(idx), R, V, stream()), "argmax")
+    if also_ptr or slot_ptr:
+        check(entry("llme_argmax_to")(ptr(logits), out_ptr, also_ptr or None, slot_ptr or None, ptr(val), ptr(idx), R, V,
+                                      stream()), "argmax")
+    else:
+        check(entry("llme_argmax")(ptr(logits), out_ptr, ptr(val), ptr(idx), R, V, stream()), "argmax")
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor,

@@ -40,6 +40,7 @@ _SIGNATURES = {
     "llme_attention_generic": [_vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
                                _f, _i, _vp],
     "llme_argmax": [_vp, _vp, _vp, _vp, _i, _i, _vp],
+    "llme_argmax_to": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
     "llme_argmax_parts": [_i],
     "llme_compute_units": [],
     "llme_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],

@@ -394,6 +394,44 @@ def test_twenty_decoded_tokens_are_rotated_inside_the_attention_kernel(zoo, name
             assert np.abs(got[rid][pos].astype(np.float64) - apart[rid][pos]).max() / top < 2e-3, (rid, pos)
 
 
+@pytest.mark.parametrize("dtype,deterministic", [("fp32", False), ("bf16", True)])
+def test_greedy_chain_equals_steps_fetched_one_by_one(zoo, dtype, deterministic):
+    """Steps launched before the tokens of the step before them are fetched (the tokens stay on the
+    device) choose what steps do whose tokens go through the host one by one; over the place where the
+    block tables outgrow the recording (1,024 tokens), where the chain passes the tokens through the
+    host once, and for a second chain over the same recording."""
+    from llmengine import Engine, StepEntry
+    model_dir, _, _, page = zoo["C"]
+    engine = Engine(model_dir, dtype, deterministic=deterministic)
+    prompts = {"a": random_tokens(1000, TINY_C["vocab_size"], 301), "b": random_tokens(40, TINY_C["vocab_size"], 302),
+               "c": random_tokens(515, TINY_C["vocab_size"], 303)}
+    ids = list(prompts)
+
+    def start():
+        cache = engine.new_cache(sum((len(p) + 80 + page - 1) // page for p in prompts.values()), page, max_requests=3)
+        first = []
+        for rid, p in prompts.items():
+            cache.admit(rid)
+            logits = engine.step(cache, [StepEntry(rid, p, [len(p) - 1])])
+            first.append(int(logits[0].argmax()))
+        return cache, first
+    cache, first = start()
+    one_by_one, last = [], first
+    for _ in range(60):
+        last = engine.run_step(cache, [StepEntry(r, [t], [0]) for r, t in zip(ids, last)], None)
+        one_by_one.append(last)
+    cache, first2 = start()
+    assert first2 == first
+    replays = engine.runner.graph_replays
+    chained = engine.greedy_chain(cache, ids, first, 35)
+    chained += engine.greedy_chain(cache, ids, chained[-1], 25)
+    assert engine.runner.graph_replays == replays + 60
+    assert chained == one_by_one
+    assert [cache.manager.length(r) for r in ids] == [len(prompts[r]) + 60 for r in ids]
+    with pytest.raises(ValueError):
+        engine.greedy_chain(cache, ids, [0, 1], 3)
+
+
 # A layer or two with the sizes of Llama 3.2 1B, 3.2 3B and 3.1 8B: the kernels that serving picks at
 # real widths (tiled products over several row tiles, the prefill attention with many work items, the
 # fused decode kernels at widths 2048, 3072 and 4096, the output head over the whole vocabulary).

@@ -55,7 +55,8 @@ def test_prompts_longer_than_a_prefill_step(dir_a, chunk):
         prompt = random_tokens(n, 256, 60 + i)
         steps.clear()
         assert engine.generate(prompt, 6) == plain_generate(cfg, w, prompt, 6)
-        assert steps[:-5] == [[chunk]] * (n // chunk) + ([[n % chunk]] if n % chunk else [])
+        # (the five decode steps behind the prompt are launched by the runner itself, from recorded graphs)
+        assert steps == [[chunk]] * (n // chunk) + ([[n % chunk]] if n % chunk else [])
     ids = random_tokens(41, 256, 70)
     steps.clear()
     got = engine.forward_logits(ids)
