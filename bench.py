@@ -7,7 +7,9 @@ By default the model has the layer sizes of Llama 3.2 1B (16 layers, width 2048,
 heads of 64, feed-forward 8192, vocabulary 128256, llama3 rope scaling, tied head) with seeded
 random bfloat16 weights; token ids are seeded uniform random numbers. A "step" is one decode
 step of the whole batch: the model over one token per request from the paged cache, the choice
-of the next token (greedy) and its way back to the host. Every request holds `context - steps -
+of the next token (greedy) and its way back to the host; as in `Engine.generate`, a step is launched
+on the tokens the device holds while the host still fetches those of the step before
+(`Engine.greedy_chain`). Every request holds `context - steps -
 warmup` tokens when decoding starts, put there by real prefill steps, so that the timed steps
 run at the configured context length. One JSON line goes to stdout.
 
