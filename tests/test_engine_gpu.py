@@ -430,6 +430,28 @@ def test_greedy_chain_equals_steps_fetched_one_by_one(zoo, dtype, deterministic)
     assert [cache.manager.length(r) for r in ids] == [len(prompts[r]) + 60 for r in ids]
     with pytest.raises(ValueError):
         engine.greedy_chain(cache, ids, [0, 1], 3)
+    # a request that ends and another under its name: the chain's tokens on the device are nobody's any more
+    assert cache.chain is not None
+    cache.release("b")
+    assert cache.chain is None
+    cache.admit("b")
+    again = random_tokens(33, TINY_C["vocab_size"], 304)
+    logits = engine.step(cache, [StepEntry("b", again, [len(again) - 1])])
+    tokens = [chained[-1][0], int(logits[0].argmax()), chained[-1][2]]
+    got = engine.greedy_chain(cache, ids, tokens, 6)
+    # the same from a pool of its own, token by token through the host
+    other = engine.new_cache(sum((len(p) + 80 + page - 1) // page for p in prompts.values()), page, max_requests=3)
+    lengths = {r: cache.manager.length(r) - 6 for r in ids}
+    history = {"a": prompts["a"] + [first[0]] + [c[0] for c in chained], "b": again,
+               "c": prompts["c"] + [first[2]] + [c[2] for c in chained]}
+    for r in ids:
+        other.admit(r)
+        engine.step(other, [StepEntry(r, history[r][:lengths[r]], [])])
+    want, last = [], tokens
+    for _ in range(6):
+        last = engine.run_step(other, [StepEntry(r, [t], [0]) for r, t in zip(ids, last)], None)
+        want.append(last)
+    assert got == want
 
 
 # A layer or two with the sizes of Llama 3.2 1B, 3.2 3B and 3.1 8B: the kernels that serving picks at
