@@ -247,8 +247,10 @@ def attention_project(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     """attention (as above, into o) and the output projection behind it: out (+)= o w_o^T. Where a
     step of a few decoded tokens cuts its keys into splits, the splits' join and the projection are
     one kernel, and o is not written."""
-    if policy.fast_attention and policy.fast_gemm and _fast_attention_project is not None and _fast_attention_project(
-            q, k_cache, v_cache, o, step, block_table, n_q, n_kv, head_dim, scale, window, w_o, out, accumulate):
+    # (only a step of up to 16 decoded tokens is asked about: steps launched kernel by kernel count their calls)
+    if (q.shape[0] <= 16 and policy.fast_attention and policy.fast_gemm and _fast_attention_project is not None
+            and _fast_attention_project(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, head_dim, scale, window,
+                                        w_o, out, accumulate)):
         return
     attention(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, head_dim, scale, window)
     gemm(o, w_o, out, accumulate, fixed_order=step.fixed_order)

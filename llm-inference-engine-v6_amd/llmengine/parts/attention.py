@@ -134,7 +134,7 @@ class Attention(Mixer):
             if applies:
                 self.position.apply(qkv[:, :self.q_dim].view(T, n_q, hd),
                                     qkv[:, self.q_dim:self.q_dim + self.kv_dim].view(T, n_kv, hd), step.positions)
-            if adds and not applies and rot == hd:
+            if adds and not applies and rot == hd and T == step.num_seqs:
                 # decoded tokens only: the attention kernel rotates, writes the cache and clears the rows itself
                 o = step.buffer("attn.o", (T, self.q_dim), act)
                 if ops.mfma.attention_decode_rope(qkv, cos, sin, k_cache, v_cache, o, step, block_table, n_q, n_kv, hd,
