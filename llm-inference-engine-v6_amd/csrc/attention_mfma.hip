@@ -276,14 +276,17 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 //              hint: -1 the entry point chooses, 0 never, 1 always
 //   bit 14     the decode kernel's splits are left unjoined in part_o / part_ml: the caller joins them
 //              (llme_attention_join_project); only for steps without prompt portions
+//   bit 15     the prefill kernel that shares K and V through LDS takes work items of half the rows (16
+//              per row group instead of 32): for steps with few items (see attention_prefill.hip)
 struct Tuning {
-    int rows, shared, key_waves, read_once, no_join;
+    int rows, shared, key_waves, read_once, no_join, half_rows;
 };
 static bool parse_tuning(int packed, Tuning* t) {
-    if (packed < 0 || packed >= (1 << 15)) return false;
+    if (packed < 0 || packed >= (1 << 16)) return false;
     const int rows = packed & 0xFF, shared = ((packed >> 8) & 0xF) - 1, read_once = ((packed >> 12) & 0x3) - 1;
     if (rows % 16 != 0 || rows > 64 || shared > 3 || read_once > 1) return false;
-    *t = Tuning{rows, shared > 1 ? 1 : shared, shared > 1 ? shared - 1 : 0, read_once, (packed >> 14) & 1};
+    *t = Tuning{rows, shared > 1 ? 1 : shared, shared > 1 ? shared - 1 : 0, read_once, (packed >> 14) & 1,
+                (packed >> 15) & 1};
     return true;
 }
 static bool decode_reads_once(const Tuning& t) { return t.read_once != 0; }
@@ -373,7 +376,8 @@ static int direct_rows(int hd, const Tuning& t) {
     return rows;
 }
 static int shared_rows_for(int hd, int n_q, int n_kv, const Tuning& t) {
-    return t.shared == 0 ? 0 : prefill_shared_rows(hd, n_q, n_kv);
+    const int rows = t.shared == 0 ? 0 : prefill_shared_rows(hd, n_q, n_kv);
+    return t.half_rows ? rows / 2 : rows;
 }
 extern "C" int llme_attention_bf16_rows(int hd, int n_q, int n_kv, int tuning) {
     Tuning t;

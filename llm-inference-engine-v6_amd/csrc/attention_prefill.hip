@@ -438,7 +438,13 @@ static int heads_per_workgroup(int n_q, int n_kv) {
 }
 
 // Rows per work item: 32 per row group (measured: 64 are no faster at any length, and leave
-// fewer items to spread over the chip), times the row groups of a workgroup.
+// fewer items to spread over the chip), times the row groups of a workgroup. The caller may halve
+// them (16 per row group) where a step has few items: an item's time is set by its walk over the
+// keys, a stretch after the other, and a stretch of 16 rows is shorter than one of 32. Measured on
+// whole prompts (us, 32 / 16 rows; 32 query and 8 kv heads): heads of 64, 256 tokens 9.6 / 7.2, 1,024
+// 20.7 / 17.1, 2,048 40.0 / 39.1, 3,072 80.8 / 73.6, 4,096 96.8 / 121; heads of 128, 512 tokens 19.0 /
+// 15.4, 1,024 30.0 / 29.0, 2,048 57.8 / 71.7: half the rows win until the items of 32 rows number
+// one workgroup less per compute unit than LDS lets it hold (four with heads of 64, two with 128).
 int prefill_shared_rows(int hd, int n_q, int n_kv) {
     if ((hd != 64 && hd != 128) || n_kv <= 0 || n_q % n_kv != 0) return 0;
     return 32 * (4 / heads_per_workgroup(n_q, n_kv));
@@ -505,6 +511,8 @@ int launch_prefill_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* o
     }
     LLME_SHARED(64, 2, 4) LLME_SHARED(64, 2, 2) LLME_SHARED(64, 2, 1)
     LLME_SHARED(128, 2, 4) LLME_SHARED(128, 2, 2) LLME_SHARED(128, 2, 1)
+    LLME_SHARED(64, 1, 4) LLME_SHARED(64, 1, 2) LLME_SHARED(64, 1, 1)
+    LLME_SHARED(128, 1, 4) LLME_SHARED(128, 1, 2) LLME_SHARED(128, 1, 1)
 #undef LLME_SHARED
 #undef LLME_SHARED_ARGS
     return kErrUnsupported;

@@ -126,16 +126,22 @@ declare("llme_attention_bf16", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i,
                                 _i, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp, _i, _vp])
 
 
-def attention_tuning(rows: int = 0, shared: int = -1, read_once: int = -1) -> int:
+def attention_tuning(rows: int = 0, shared: int = -1, read_once: int = -1, half_rows: bool = False) -> int:
     """Overrides of the attention kernels' launch choices for one call (tests, measurements), as
     the entry points take them; 0 leaves every choice to the entry point. rows: rows per work item
     of the prefill kernel without LDS (16, 32, 64; 0: by head size). shared: the prefill kernel that
     shares K and V through LDS: -1 where it takes the sizes, 0 never, 1 wherever it can, 2 / 3 with
     one / two wavefronts per tile whatever the number of items. read_once: the decode kernel's
-    cache hint on keys and values: -1 the entry point chooses, 0 off, 1 on."""
+    cache hint on keys and values: -1 the entry point chooses, 0 off, 1 on. half_rows: work items of
+    half the rows in the kernel that shares K and V (plan_attention sets it by itself for steps with
+    few items; PREFILL_HALF_ROWS False keeps it from that)."""
     if rows not in (0, 16, 32, 64) or not -1 <= shared <= 3 or not -1 <= read_once <= 1:
         raise kernels.KernelError(f"attention_tuning: rows {rows}, shared {shared}, read_once {read_once}")
-    return rows | (shared + 1) << 8 | (read_once + 1) << 12
+    return rows | (shared + 1) << 8 | (read_once + 1) << 12 | (TUNING_HALF_ROWS if half_rows else 0)
+
+
+TUNING_HALF_ROWS = 1 << 15
+PREFILL_HALF_ROWS = True            # (tests and measurements switch the choice off here)
 
 _work_queues: dict = {}
 
@@ -203,9 +209,9 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
     plan = {"n_decode": len(decode), "groups": groups, "split_len": 32, "nsplit": 1, "prefill_splits": 1,
             "prefill_run": 1, "tuning": tuning}
     if groups and entry("llme_attention_bf16_splits_prefill")(head_dim, n_q, n_kv, tuning):
-        # few rows over long contexts: too few work items for the chip, each with many keys
         group = n_q // n_kv
         items = groups * (n_q // (4 if group % 4 == 0 else 2 if group % 2 == 0 else 1))
+        # few rows over long contexts: too few work items for the chip, each with many keys
         keys = max(c + n for n, c in zip(new_lens, ctx_lens) if n >= 2)
         splits = 1
         if items <= (PREFILL_CUT_ITEMS or compute_units() // 2):
@@ -217,6 +223,17 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
             run = (stretches + splits - 1) // splits       # stretches of 64 keys per run
         if splits > 1:
             plan["prefill_splits"], plan["prefill_run"] = splits, run
+        elif (PREFILL_HALF_ROWS and not tuning & TUNING_HALF_ROWS
+              and items <= (3 if head_dim == 64 else 1) * compute_units()):
+            # few items whose keys are not cut (short prompts, portions early in a prompt): work items of
+            # half the rows, until the items of whole rows number one workgroup less per compute unit than
+            # LDS lets it hold (measurements in attention_prefill.hip). Where the keys are cut the items are
+            # many already, and half rows were no faster (256 tokens behind 16,128: 2.75 against 2.66 ms a step).
+            tuning |= TUNING_HALF_ROWS
+        if tuning & TUNING_HALF_ROWS:
+            rows = entry("llme_attention_bf16_rows")(head_dim, n_q, n_kv, tuning)
+            plan["groups"] = sum((n + rows - 1) // rows for n in new_lens if n >= 2)
+            plan["tuning"] = tuning
     if decode:
         longest = max(decode) if plan_len is None else max(plan_len, max(decode))
         pairs = len(decode) * n_kv * ((n_q // n_kv + 15) // 16)
