@@ -375,13 +375,10 @@ class ModelRunner:
         and a sampler do it)."""
         if not self.use_graphs or not entries:
             return None
-        vocab = self.model.vocab_size
         ids = []
         for e in entries:
             if len(e.tokens) != 1 or len(e.want) != 1 or e.want[0] != 0:
                 return None
-            if not 0 <= int(e.tokens[0]) < vocab:
-                raise ValueError(f"token id {e.tokens[0]} out of range [0, {vocab})")
             ids.append(e.request_id)
         pending = self.greedy_launch(cache, ids, [int(e.tokens[0]) for e in entries], max_position)
         return self.greedy_result(pending)
@@ -400,6 +397,13 @@ class ModelRunner:
         S = len(ids)
         if len(set(ids)) != S:
             raise ValueError("a request appears twice in one step")
+        if tokens is not None:
+            vocab = self.model.vocab_size
+            if len(tokens) != S:
+                raise ValueError(f"{len(tokens)} tokens for {S} requests")
+            for t in tokens:
+                if not 0 <= int(t) < vocab:
+                    raise ValueError(f"token id {t} out of range [0, {vocab})")
         mgr = cache.manager
         keys = (ctypes.c_int64 * S)(*[mgr.key_of(r) for r in ids])
         lengths = (ctypes.c_int * S)()
