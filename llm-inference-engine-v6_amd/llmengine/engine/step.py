@@ -195,9 +195,10 @@ class _DecodeRecord:
         self.event: torch.cuda.Event | None = None
         self.scratch = None
 
-    def refresh(self, mgr: CacheManager, entries: Sequence[StepEntry] | None, keys=None, slot: int = 0) -> None:
-        """entries None: the tokens are the ones the last replay chose and left in the device's array;
-        everything else is rewritten as always."""
+    def refresh(self, mgr: CacheManager, entries: Sequence[StepEntry] | None, keys=None, slot: int = 0,
+                tokens: Sequence[int] | None = None) -> None:
+        """The step's tokens come in `entries` or in `tokens`; with neither they are the ones the last
+        replay chose and left in the device's array. Everything else is rewritten as always."""
         if self.event is not None:
             self.event.synchronize()            # the last copy has read the host mirror
         S, width, o, h = self.S, self.width, self.offsets, self.np
@@ -209,7 +210,9 @@ class _DecodeRecord:
                 self.key_list = keys
                 self.keys = (ctypes.c_int64 * S)(*keys)
         if entries is not None:
-            h[o[0]:o[1]] = [e.tokens[0] for e in entries]
+            tokens = [e.tokens[0] for e in entries]
+        if tokens is not None:
+            h[o[0]:o[1]] = tokens
         h[self.total] = slot
         # lengths (tokens cached before this step), slots and the block-table entries that are new,
         # straight from the C++ manager into the pinned mirror
@@ -219,7 +222,7 @@ class _DecodeRecord:
         if rc != 0:
             raise RuntimeError(f"a request of the recorded step is not live (code {rc})")
         h[o[1]:o[2]] = h[o[4]:o[5]]             # the new token's position
-        first = 0 if entries is not None else o[1]
+        first = 0 if tokens is not None else o[1]
         self.meta[first:self.total + 1].copy_(self.host[first:], non_blocking=True)
         if self.event is None:
             self.event = torch.cuda.Event()
@@ -426,17 +429,21 @@ class ModelRunner:
             need = {g: sum(mgr.pages_needed(r, 1)[g] for r in ids) for g in mgr.groups}
             raise CapacityError(f"the step needs {need} more pages, free are "
                                 f"{({g: mgr.free_pages(g) for g in mgr.groups})}")
-        entries = None if tokens is None else [StepEntry(r, [t], [0]) for r, t in zip(ids, tokens)]
-        rec = self._decode_record(cache, entries, longest, greedy=True, S=S)
+        key = self._decode_key(cache, S, longest, greedy=True)
+        if key in cache.graphs or tokens is None:
+            rec = self._decode_record(cache, None, longest, greedy=True, S=S)
+        else:                                   # (a new recording runs the step once from entries)
+            rec = self._decode_record(cache, [StepEntry(r, [t], [0]) for r, t in zip(ids, tokens)], longest,
+                                      greedy=True)
         slot = 1 - rec.slot
-        rec.refresh(mgr, entries, keys, slot=slot)
+        rec.refresh(mgr, None, keys, slot=slot, tokens=tokens)
         rec.graph.replay()
         rec.tok_events[slot].record()
         rec.slot = slot
         rec.launches[slot] += 1                 # (what an older launch left in this half is gone)
         self.graph_replays += 1
         mgr._lib.llme_cm_commit_batch(mgr.handle, S, keys, 1)
-        cache.chain = (rec, list(ids), self._decode_key(cache, S, longest, greedy=True))
+        cache.chain = (rec, list(ids), key)
         return PendingTokens(rec, slot, rec.launches[slot])
 
     def greedy_result(self, pending: "PendingTokens") -> list[int]:
