@@ -147,3 +147,5 @@ extern "C" int llme_attention_generic(const void* q, int q_dtype, const void* k_
 #undef LLME_ATTN
     return launch_status();
 }
+
+LLME_LOAD_ENTRY(attention_generic)

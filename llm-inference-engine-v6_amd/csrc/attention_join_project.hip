@@ -364,3 +364,5 @@ extern "C" int llme_attention_join_project(const float* part_o, const float* par
 #undef LLME_JOIN_PROJECT
     return launch_status();
 }
+
+LLME_LOAD_ENTRY(attention_join_project)

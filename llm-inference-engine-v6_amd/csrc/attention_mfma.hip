@@ -542,3 +542,5 @@ extern "C" int llme_attention_decode_noalloc(const void* q, const void* k_cache,
                                /*prefill_groups=*/0, /*queue=*/nullptr, /*n_rows=*/n_seq, /*prefill_splits=*/1,
                                /*prefill_run=*/1, nullptr, nullptr, /*tuning=*/0, stream);
 }
+
+LLME_LOAD_ENTRY(attention_mfma)

@@ -519,3 +519,5 @@ int launch_prefill_shared(const bf16* q, const bf16* kc, const bf16* vc, bf16* o
 }
 
 }  // namespace llme
+
+LLME_LOAD_ENTRY(attention_prefill)

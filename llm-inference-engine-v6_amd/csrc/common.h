@@ -81,3 +81,13 @@ constexpr int kErrBadArgument = 10001;
 constexpr int kErrUnsupported = 10002;
 
 }  // namespace llme
+
+// The runtime loads a source file's device code when one of its kernels is first launched (or asked
+// about). LLME_LOAD_ENTRY(name) gives the file an entry point llme_load_<name> that makes this happen,
+// so that a caller can have every file's code on the device before it records launches into a graph.
+#define LLME_LOAD_ENTRY(name)                                                                        \
+    namespace { __global__ void load_probe_##name() {} }                                            \
+    extern "C" int llme_load_##name(void) {                                                          \
+        hipFuncAttributes attr;                                                                      \
+        return static_cast<int>(hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(&load_probe_##name))); \
+    }

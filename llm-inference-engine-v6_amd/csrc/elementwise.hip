@@ -554,3 +554,5 @@ extern "C" int llme_rope_kv_write(float* qkv, const float* cos_t, const float* s
     }
     return launch_status();
 }
+
+LLME_LOAD_ENTRY(elementwise)

@@ -207,3 +207,5 @@ extern "C" int llme_gemm_generic(const void* a, int a_dtype, const void* w, int 
         default: return kErrBadArgument;
     }
 }
+
+LLME_LOAD_ENTRY(gemm_generic)

@@ -1139,3 +1139,5 @@ extern "C" int llme_gemm_bf16_qkv_rope(const void* a, const void* w, int M, int 
     if (tile_shape == 96128) return launch_tile_rope<3, 4>(A, W, M, N, K, blocked, qt, stream);
     return kErrBadArgument;
 }
+
+LLME_LOAD_ENTRY(gemm_mfma)

@@ -521,3 +521,5 @@ extern "C" int llme_gemv_norm_rope(const float* h, const void* norm_w, int norm_
         ? launch_gemv_norm<8, 2, kRope, bf16>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream)
         : launch_gemv_norm<8, 2, kRope, float>(h, nullptr, norm_w, eps, W, nullptr, M, N, K, grid, blocked, rope, stream);
 }
+
+LLME_LOAD_ENTRY(gemv_fused)

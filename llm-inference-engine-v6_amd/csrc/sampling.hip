@@ -254,3 +254,5 @@ extern "C" int llme_sample(const float* logits, const float* temperature, const 
                        part_val, part_idx, part_sum, out, V, chunk, parts);
     return launch_status();
 }
+
+LLME_LOAD_ENTRY(sampling)

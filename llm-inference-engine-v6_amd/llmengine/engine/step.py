@@ -43,6 +43,9 @@ class Workspace:
         self._buffers: dict[tuple[str, torch.dtype], torch.Tensor] = {}
         self.keep_replaced = False      # set once a recorded graph holds addresses of these buffers
         self._replaced: list[torch.Tensor] = []
+        # buffers that were first asked for (or outgrown) while a graph was being recorded: their memory then
+        # belongs to that recording's own pool (see `made_while_recording`)
+        self._recorded: dict[tuple[str, torch.dtype], int] = {}
         # the shaped views handed out, by (name, dtype, shape): a step asks for the same ones layer after layer
         self._views: dict[tuple, torch.Tensor] = {}
 
@@ -59,6 +62,8 @@ class Workspace:
         if buf is None or buf.numel() < n:
             if buf is not None and self.keep_replaced:
                 self._replaced.append(buf)          # a recorded graph may still read and write it
+            if torch.cuda.is_current_stream_capturing():
+                self._recorded[key] = max(n, 1)
             buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._buffers[key] = buf
             self._views = {k: v for k, v in self._views.items() if k[:2] != key}
@@ -66,6 +71,18 @@ class Workspace:
             self._views.clear()
         view = self._views[(name, dtype, shape)] = buf[:n].view(shape)
         return view
+
+    def made_while_recording(self) -> bool:
+        """Call outside any recording. True if the last recording made buffers: they are replaced by
+        buffers of the same sizes made in the ordinary way, and the recording, which holds the old
+        addresses, must be thrown away and made again."""
+        if not self._recorded:
+            return False
+        for key, n in self._recorded.items():
+            self._buffers[key] = torch.empty(n, dtype=key[1], device=self.device)
+        self._views = {k: v for k, v in self._views.items() if k[:2] not in self._recorded}
+        self._recorded = {}
+        return True
 
 
 @dataclass
@@ -342,13 +359,14 @@ class ModelRunner:
                 raise RuntimeError("a step that takes its tokens from the step before has no recording to run in")
             while len(cache.graphs) >= self.GRAPH_LIMIT:
                 del cache.graphs[next(iter(cache.graphs))]
-            # First time: run it plainly (this also sizes the scratch buffers), then record.
+            # The step is recorded without having run: a part's step need not be repeatable (a mixer that
+            # advances a state would count the token twice), and the first replay is its first run.
             # The recorded step reads its integer arrays from a buffer of its own.
+            ops.load_kernels()                          # (no code object is loaded inside a recording)
             groups = len(mgr.groups)
             total = 7 * S + 1 + groups * S * width
             meta = torch.zeros(total + 64, dtype=torch.int32, device=self.device)
             ctx, logit_rows = self._build_context(cache, entries, max_blocks=width, plan_len=width * page, dev=meta)
-            logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
             tok_host = scratch = None
             if greedy:
                 # pinned host memory is mapped into the device's address space: the kernel writes
@@ -356,16 +374,24 @@ class ModelRunner:
                 # scratch belongs to the recording (the one that plain calls share may be replaced)
                 tok_host = torch.zeros(2 * S, dtype=torch.int32, pin_memory=True)
                 scratch = ops.sampling_scratch(self.device, S, self.model.vocab_size)
-                ops.argmax_into(logits, tok_host.data_ptr(), scratch, also_ptr=meta.data_ptr(),
-                                slot_ptr=meta.data_ptr() + 4 * total)
             torch.cuda.synchronize(self.device)
             self.workspace.keep_replaced = True
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
-                if greedy:
-                    ops.argmax_into(logits, tok_host.data_ptr(), scratch, also_ptr=meta.data_ptr(),
-                                    slot_ptr=meta.data_ptr() + 4 * total)
+            # Scratch buffers that the step is the first to ask for are made while it is recorded and
+            # belong to the recording's own memory pool, which later steps of other kinds must not be
+            # handed: they are made again outside, and the step is recorded once more with those.
+            for attempt in range(3):
+                ctx.extra.clear()                       # (notes of the pass before: launch plans, what was left cleared)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
+                    if greedy:
+                        ops.argmax_into(logits, tok_host.data_ptr(), scratch, also_ptr=meta.data_ptr(),
+                                        slot_ptr=meta.data_ptr() + 4 * total)
+                if not self.workspace.made_while_recording():
+                    break
+                del graph, logits
+            else:
+                raise RuntimeError("a decode step asks for new scratch buffers every time it is recorded")
             cache.graphs[key] = rec = _DecodeRecord(graph, logits, meta, S, width, list(mgr.groups), tok_host)
             rec.scratch = scratch                       # (kept alive: the graph holds its addresses)
         return rec

@@ -89,6 +89,25 @@ def entry(name: str):
         raise KernelLibraryError(f"the kernel library has no entry point {name}") from None
 
 
+_loaded_on: set = set()
+
+
+def load_kernels() -> None:
+    """Has the device code of every kernel file loaded onto the current device (the runtime would
+    load a file's code at the first launch of one of its kernels, which must not happen while
+    launches are being recorded into a graph). Cheap after the first call on a device."""
+    device = torch.cuda.current_device()
+    if device in _loaded_on:
+        return
+    import os
+    for src in _build.sources():
+        name = "llme_load_" + os.path.basename(src)[:-4]
+        fn = entry(name)
+        fn.argtypes, fn.restype = [], ctypes.c_int
+        check(fn(), name)
+    _loaded_on.add(device)
+
+
 def code(dtype: torch.dtype) -> int:
     try:
         return _CODES[dtype]

@@ -410,6 +410,10 @@ def attention_decode_rope(qkv, cos, sin, k_cache, v_cache, out, step, block_tabl
 declare("llme_gemv_norm", [_vp, _vp, _vp, _i, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp])
 
 GEMV_NORM_MAX_ROWS = 16
+# Steps of more rows than that and of at most this many cut their q/k/v product over k and add the parts
+# into a cleared 32-bit buffer (too few output tiles for the chip otherwise); steps of more rows rotate
+# and write the cache in the product's epilogue.
+QKV_SUM_MAX_ROWS = 64
 
 
 def gemv_norm_supported(h: torch.Tensor, norm_weight: torch.Tensor, w: torch.Tensor, rows_out: int,

@@ -110,24 +110,27 @@ class Attention(Mixer):
             # decoding: norm, projection, rotation and the cache write are one kernel
             ops.gemv_norm_rope(x, rms[0], rms[1], self.w_qkv_paired, step.positions, step.seq_idx,
                                block_table, cos, sin, q, k_cache, v_cache, n_q, n_kv, hd)
-        elif (write_cache and rms is None and T > 64 and cos is not None
+        elif (write_cache and rms is None and T > ops.mfma.QKV_SUM_MAX_ROWS and cos is not None
               and ops.gemm_qkv_rope_supported(x, self.w_qkv, k_cache, hd, rot)):
             # many rows (prompts): rotation and the cache write are the projection's epilogue
             ops.gemm_qkv_rope(x, self.w_qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
                               n_q, n_kv, hd)
         elif write_cache:
-            qkv = step.buffer("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
-            adds = (rms is None and 16 < T <= 64 and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16
-                    and qkv.numel() % 4 == 0)
+            adds = (rms is None and ops.mfma.GEMV_NORM_MAX_ROWS < T <= ops.mfma.QKV_SUM_MAX_ROWS
+                    and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16
+                    and (T * (self.q_dim + 2 * self.kv_dim)) % 4 == 0)
+            # (the product that adds has a buffer that nothing else writes: what it is left holding is known)
+            qkv = step.buffer("attn.qkv_sum" if adds else "attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
             if adds:
                 # a few dozen rows (decoding at larger batches): q/k/v has too few output tiles for the
                 # chip, so the product is cut over k and adds its parts into a cleared buffer
                 # (measured at 32 rows of the 3B sizes: 10.7 + clearing against 19.5 us). The buffer
                 # is cleared for the step's first such layer; the rotation kernel leaves it zero for
-                # the next one (a clearing kernel per layer took 4.6 us).
-                if step.extra.get("attn.qkv zero", (0, 0)) != (qkv.data_ptr(), qkv.numel()):
+                # the next one (a clearing kernel per layer took 4.6 us). The note of that is the
+                # step's: every step, and every recording of one, clears for itself.
+                if step.extra.get("attn.qkv_sum zero", (0, 0)) != (qkv.data_ptr(), qkv.numel()):
                     ops.clear(qkv)
-                step.extra.pop("attn.qkv zero", None)
+                step.extra.pop("attn.qkv_sum zero", None)
                 ops.gemm(x, self.w_qkv, qkv, accumulate=True, fixed_order=step.fixed_order)
             else:
                 project(self.w_qkv, qkv)
@@ -139,13 +142,13 @@ class Attention(Mixer):
                 o = step.buffer("attn.o", (T, self.q_dim), act)
                 if ops.mfma.attention_decode_rope(qkv, cos, sin, k_cache, v_cache, o, step, block_table, n_q, n_kv, hd,
                                                   self.scale, self.window):
-                    step.extra["attn.qkv zero"] = (qkv.data_ptr(), qkv.numel())
+                    step.extra["attn.qkv_sum zero"] = (qkv.data_ptr(), qkv.numel())
                     ops.gemm(o, self.w_o, out, accumulate, fixed_order=step.fixed_order)
                     return
             ops.rope_kv_write(qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
                               n_q, n_kv, hd, rot, write_cache=True, zero_input=adds)
             if adds:
-                step.extra["attn.qkv zero"] = (qkv.data_ptr(), qkv.numel())
+                step.extra["attn.qkv_sum zero"] = (qkv.data_ptr(), qkv.numel())
         else:
             # A layer that reads another layer's cache projects queries only.
             q32 = step.buffer("attn.q32", (T, self.q_dim), torch.float32)

@@ -78,14 +78,13 @@ Getter = Callable[[str], torch.Tensor]      # local tensor name -> CPU tensor as
 
 
 class Part:
-    # True if forward() issues the same launches, with the same arguments, for every step of
-    # the same shape, reading what changes (tokens, positions, tables, slots) from the step's
-    # device arrays only, and if running a step twice on the same inputs leaves the same cache
-    # and state as running it once (a step that is recorded runs plainly first, to size the scratch
-    # buffers, and once more while it is recorded: attention rewrites the same keys at the same
-    # places, a part that adds into its state would count the token twice). Steps of such parts
-    # can be recorded once and replayed as a HIP graph; a part that looks at the step's host-side
-    # lists while it runs, or whose step is not repeatable, must leave this False.
+    # True if, for a step of one token of each request that wants its logits, forward() issues the
+    # same launches with the same arguments whatever the requests are, reading what changes (tokens,
+    # positions, tables, slots) from the step's device arrays only and never from its host-side
+    # lists. Such steps are recorded once as a HIP graph and replayed. The step is recorded without
+    # being run (the first replay is its first run), so it may advance state of its own. Tensors
+    # that forward() makes while it is recorded belong to the recording; scratch memory from
+    # `step.buffer` is the runner's.
     graph_safe = False
 
     def param_specs(self) -> dict[str, ParamSpec]:

@@ -221,3 +221,95 @@ def test_fp32_logits_do_not_depend_on_pages(zoo, name):
         results.append(_flat(replay.run_trace(engine, cache, steps)))
     for other in results[1:]:
         assert np.array_equal(results[0], other)
+
+
+# --- recorded decode steps between steps of other kinds ---------------------------------------
+# A recorded decode step of 17 to 64 requests cuts its q/k/v product over k and adds the parts into a
+# 32-bit buffer. Other kinds of step use the same scratch memory and leave values behind: a prompt
+# portion of more than 64 rows where the projection cannot rotate in its epilogue (head sizes that are
+# no power of two), a step of up to 16 rows where the fused decode kernel is refused (a width beyond
+# what its LDS holds). The replay behind such a step must give what the plain implementation gives.
+HEAD_96 = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": 192,
+           "intermediate_size": 320, "num_hidden_layers": 2, "num_attention_heads": 4,
+           "num_key_value_heads": 2, "head_dim": 96, "vocab_size": 300, "max_position_embeddings": 512,
+           "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "tie_word_embeddings": True}
+WIDTH_5120 = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": 5120,
+              "intermediate_size": 1024, "num_hidden_layers": 1, "num_attention_heads": 40,
+              "num_key_value_heads": 8, "head_dim": 128, "vocab_size": 300, "max_position_embeddings": 512,
+              "rms_norm_eps": 1e-5, "rope_theta": 500000.0, "tie_word_embeddings": False}
+HEAD_48 = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": 144,
+           "intermediate_size": 208, "num_hidden_layers": 2, "num_attention_heads": 6,
+           "num_key_value_heads": 2, "head_dim": 48, "vocab_size": 331, "max_position_embeddings": 512,
+           "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "tie_word_embeddings": False}
+DISTURBED = {"head96": (HEAD_96, dict(seed=21, std=0.05, norm_mean=1.0, norm_std=0.1)),
+             "width5120": (WIDTH_5120, dict(seed=22, std=0.01, norm_mean=1.0, norm_std=0.05)),
+             "head48": (HEAD_48, dict(seed=23, std=0.05, norm_mean=1.0, norm_std=0.1))}
+
+
+def disturbed_schedule(ids: dict, live: int, late: int, prompt: int = 8, portion: int = 70, dip: int = 10,
+                       run: int = 3) -> tuple[list[dict], dict]:
+    """`live` requests: their prompts in one step, then `run` decode steps of all of them (the first
+    is recorded). Then `late` times: a new request's prompt portion of `portion` tokens beside the
+    decoded tokens of all live ones (one of which ends there, so that the number stays), `run`
+    decode steps, a decode step of only `dip` of the requests, `run` decode steps. Returns the
+    steps and every request cut to the tokens that were fed."""
+    names = list(ids)
+    main, waiting = names[:live], names[live:live + late]
+    pos = {rid: 0 for rid in names}
+    steps: list[dict] = []
+
+    def entry(rid, n):
+        e = {"id": rid, "tokens": ids[rid][pos[rid]:pos[rid] + n], "want": list(range(n))}
+        assert len(e["tokens"]) == n, f"{rid} is too short"
+        pos[rid] += n
+        return e
+
+    def add(entries, end=()):
+        steps.append({"step": len(steps), "entries": entries, "end": list(end)})
+
+    add([entry(r, prompt) for r in main])
+    for _ in range(run):
+        add([entry(r, 1) for r in main])
+    for new in waiting:
+        victim = main.pop(0)
+        add([entry(r, 1) for r in [victim] + main] + [entry(new, portion)], end=[victim])
+        main.append(new)
+        for _ in range(run):
+            add([entry(r, 1) for r in main])
+        add([entry(r, 1) for r in main[:dip]])
+        for _ in range(run):
+            add([entry(r, 1) for r in main])
+    steps[-1]["end"] = list(main)
+    return steps, {rid: ids[rid][:pos[rid]] for rid in names if pos[rid]}
+
+
+@pytest.mark.parametrize("graphs", [True, False], ids=["recorded", "plain"])
+@pytest.mark.parametrize("name", list(DISTURBED))
+def test_recorded_decode_steps_between_other_steps(name, graphs):
+    from llmengine import Engine
+    from llmengine.weights import random_state
+    cfg, init = DISTURBED[name]
+    tensors = dict(random_state(cfg, init["seed"], torch.bfloat16, init["std"], init["norm_mean"], init["norm_std"]))
+    live, late = 24, 3
+    ids = {f"r{i}": random_tokens(120, cfg["vocab_size"], 900 + i) for i in range(live + late)}
+    steps, reqs = disturbed_schedule(ids, live, late)
+    sizes = [(len(st["entries"]), sum(len(e["tokens"]) for e in st["entries"])) for st in steps]
+    assert sizes[0][1] > max(t for _, t in sizes[1:]) > 64          # the first step sizes the scratch memory
+    assert sum(1 for s, t in sizes if s == t == live) >= 6 * late + 3 and any(s == t <= 16 for s, t in sizes)
+    rows = {rid: list(range(len(t))) for rid, t in reqs.items()}
+    plain = plain_rows(name, cfg, tensors, reqs, rows, "bf16")
+    engine = Engine(None, "bf16", _config=cfg, _tensors=dict(tensors), block_size=16, use_graphs=graphs)
+    cache = engine.new_cache(replay.trace_peak_tokens(steps, round_to=16) // 16, 16, max_requests=live + 1)
+    got = replay.run_trace(engine, cache, steps)
+    if graphs:
+        assert engine.runner.graph_replays >= 6 * late + 3
+    worst = (0.0, None)
+    for rid, t in reqs.items():
+        for pos in range(len(t)):
+            ref = plain[rid][pos]
+            err = np.abs(got[rid][pos].astype(np.float64) - ref).max() / np.abs(ref).max()
+            worst = max(worst, (err, (rid, pos)))
+    assert worst[0] < TOL["bf16"], f"request and position {worst[1]}: relative error {worst[0]:.3e}"
+    assert all(cache.manager.free_pages(g) == cache.manager.num_pages(g) for g in cache.manager.groups)
+    del engine
+    torch.cuda.empty_cache()

@@ -237,10 +237,14 @@ def test_windowed_attention_gives_pages_back():
 
 
 # --- a toy mixer with state of its own ---------------------------------------------------
-def test_a_toy_mixer_with_state_registers_builds_and_steps():
+@pytest.mark.parametrize("recordable", [False, True], ids=["launched", "recorded"])
+def test_a_toy_mixer_with_state_registers_builds_and_steps(recordable):
     """A mixer that keeps no pages but a running sum and a count per request:
     y_t = W mean(x_0..x_t). Layer 0 uses it, layer 1 is ordinary attention: different mixers in
-    different layers of one model. Defined here, registered through the public registries."""
+    different layers of one model. Defined here, registered through the public registries.
+    recorded: the mixer says that its steps of single tokens can be recorded as a graph (it then
+    reads the slots from the step's device array). Its step advances the state, so it must run
+    exactly once for a token: a recording that ran the step to try it would count tokens twice."""
     from llmengine import Engine
     from llmengine.config import register_architecture
     from llmengine.models.model import DecoderModel
@@ -249,6 +253,8 @@ def test_a_toy_mixer_with_state_registers_builds_and_steps():
     from llmengine.weights import random_state
 
     class RunningMean(Mixer):
+        graph_safe = recordable
+
         def __init__(self, hidden_size):
             self.hidden_size = hidden_size
             self.w = None
@@ -263,6 +269,17 @@ def test_a_toy_mixer_with_state_registers_builds_and_steps():
             return CacheSpec(state={"sum": ((self.hidden_size,), torch.float32), "count": ((1,), torch.float32)})
 
         def forward(self, x, step, cache, out, accumulate, write_cache=True):
+            if recordable and step.num_tokens == step.num_seqs:
+                # one token of every request: the same launches whatever the requests, nothing from host lists
+                slots = step.slots.long()
+                cache.state["sum"].index_add_(0, slots, x.float())
+                cache.state["count"].index_add_(0, slots, torch.ones_like(x[:, :1], dtype=torch.float32))
+                y = (cache.state["sum"][slots] / cache.state["count"][slots]) @ self.w.T
+                if accumulate:
+                    out.add_(y)
+                else:
+                    out.copy_(y)
+                return
             row = 0
             for n, slot in zip(step.new_lens, step.slot_list):        # tokens of a request in order
                 xs = x[row:row + n].float()
@@ -307,6 +324,7 @@ def test_a_toy_mixer_with_state_registers_builds_and_steps():
     engine = Engine(None, "fp32", _config=cfg, _tensors=dict(tensors), block_size=8)
     specs = engine.model.cache_specs()
     assert specs[0].state and not specs[0].paged and specs[1].paged
+    assert engine.runner.use_graphs == recordable
 
     def plain_toy(ids):
         w = {k: v.double() for k, v in tensors.items()}
@@ -338,6 +356,7 @@ def test_a_toy_mixer_with_state_registers_builds_and_steps():
         for rid, ids in reqs.items():
             for pos in range(len(ids)):
                 assert _rel(got[rid][pos], plain[rid][pos]) < 1e-5, (rid, pos)
+    assert (engine.runner.graph_replays > 40) == recordable
     out, finish = engine.generate(reqs["t1"], 5)
     assert finish == "length" and len(out) == 13
 
