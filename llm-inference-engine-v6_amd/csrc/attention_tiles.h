@@ -245,9 +245,9 @@ __device__ __forceinline__ void block_weights(f32x4 (&s)[QT][2], int t0, const i
         for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const float p = fast_exp2(fmaf(s[qt][hf][e], c, neg_m));
-                psum += p;
-                pf[qt][hf * 4 + e] = static_cast<__bf16>(p);
+                const __bf16 p = static_cast<__bf16>(fast_exp2(fmaf(s[qt][hf][e], c, neg_m)));
+                psum += static_cast<float>(p);          // (the sum of the weights as the product sees them)
+                pf[qt][hf * 4 + e] = p;
             }
         l[qt] += psum;
     }

@@ -22,8 +22,12 @@
 // prompts move on by the portions that ran, sequences move on or finish, pages go back). If the
 // model run fails, the caller calls abort() instead of complete(): the planned portions have not
 // run, the prompts stay where they were, and the next plan() offers them again. (What plan()
-// decided apart from the batch stands: admissions, and requests ended for want of pages.) The cache manager is the one the step function
-// reserves and commits in; sequence ids are its request keys.
+// decided apart from the batch stands: admissions, and requests ended for want of pages.) If the
+// batch ran, so that the cache holds its tokens, and only what came after failed (the choice of the
+// next tokens, the copy to the host), the caller calls fail(): no sequence of the batch can go on
+// from a token that is not known, so each of them ends with "error" and keeps what it had.
+// The cache manager is the one the step function reserves and commits in; sequence ids are its
+// request keys.
 #include "host_api.h"
 
 #include <algorithm>
@@ -44,7 +48,7 @@ int llme_cm_release(void* h, int64_t key);
 namespace llme_host {
 
 enum State : int { kWaiting = 0, kPrefilling = 1, kRunning = 2, kFinished = 3 };
-enum Reason : int { kNone = 0, kStop = 1, kLength = 2, kCapacity = 3 };
+enum Reason : int { kNone = 0, kStop = 1, kLength = 2, kCapacity = 3, kError = 4 };
 
 struct Seq {
     int64_t id = 0;
@@ -90,6 +94,7 @@ public:
         owners_.clear();
         prompt_ends_.clear();
         portions_.clear();
+        batch_.clear();
         *n_admitted = 0;
         // admission: no page check, as in the reference
         while (!waiting_.empty() && static_cast<int>(prefilling_.size() + running_.size()) < max_concurrent_) {
@@ -120,6 +125,7 @@ public:
             std::copy(s.tokens.begin() + first, s.tokens.begin() + first + n, tokens + used);
             used += n;
             ++E;
+            batch_.push_back(&s);
             if (want) owners_.push_back(&s);
             return true;
         };
@@ -183,6 +189,47 @@ public:
             running_.push_back(std::move(*it));
             prefilling_.erase(it);
         }
+        owners_.clear();
+        prompt_ends_.clear();
+        batch_.clear();
+        return retire();
+    }
+
+    // The planned step ran, but its tokens never arrived: every sequence of the batch ends with
+    // "error", with the tokens it had, and its pages go back. Returns how many ended.
+    int fail() {
+        if (!planned_) return LLME_HOST_BAD_ARGUMENT;
+        planned_ = false;
+        for (Seq* s : batch_) finish(*s, kError);
+        owners_.clear();
+        prompt_ends_.clear();
+        portions_.clear();
+        batch_.clear();
+        return retire();
+    }
+
+    // The planned step did not run: forget the batch, keep every prompt where it was.
+    void abort() {
+        planned_ = false;
+        owners_.clear();
+        prompt_ends_.clear();
+        portions_.clear();
+        batch_.clear();
+    }
+
+    int num_results() const { return static_cast<int>(results_.size()); }
+    const Seq* result(int i) const {
+        return i >= 0 && i < num_results() ? results_[static_cast<size_t>(i)].get() : nullptr;
+    }
+    void clear_results() { results_.clear(); }
+
+private:
+    static void finish(Seq& s, Reason r) {
+        s.state = kFinished;
+        s.reason = r;
+    }
+    // Finished sequences leave the lists, give their pages back and become results (in enqueue order).
+    int retire() {
         int finished = 0;
         for (auto* list : {&prefilling_, &running_}) {
             std::vector<std::unique_ptr<Seq>> keep;
@@ -200,29 +247,7 @@ public:
         if (finished)
             std::sort(results_.begin(), results_.end(),
                       [](const std::unique_ptr<Seq>& a, const std::unique_ptr<Seq>& b) { return a->id < b->id; });
-        owners_.clear();
-        prompt_ends_.clear();
         return finished;
-    }
-
-    // The planned step did not run: forget the batch, keep every prompt where it was.
-    void abort() {
-        planned_ = false;
-        owners_.clear();
-        prompt_ends_.clear();
-        portions_.clear();
-    }
-
-    int num_results() const { return static_cast<int>(results_.size()); }
-    const Seq* result(int i) const {
-        return i >= 0 && i < num_results() ? results_[static_cast<size_t>(i)].get() : nullptr;
-    }
-    void clear_results() { results_.clear(); }
-
-private:
-    static void finish(Seq& s, Reason r) {
-        s.state = kFinished;
-        s.reason = r;
     }
     void* cm_;
     int max_concurrent_;
@@ -231,7 +256,7 @@ private:
     bool planned_ = false;
     std::deque<std::unique_ptr<Seq>> waiting_;
     std::vector<std::unique_ptr<Seq>> prefilling_, running_, results_;
-    std::vector<Seq*> owners_, prompt_ends_;       // between plan() and complete()
+    std::vector<Seq*> owners_, prompt_ends_, batch_;   // between plan() and complete(): who gets a token, whose prompt ends, who takes part
     std::vector<std::pair<Seq*, long>> portions_;  // prompt tokens that the planned step carries
 };
 
@@ -266,8 +291,9 @@ int llme_sched_complete(void* h, const int* sampled, int n, const int* eos, int 
     return static_cast<Scheduler*>(h)->complete(sampled, n, eos, n_eos);
 }
 void llme_sched_abort(void* h) { static_cast<Scheduler*>(h)->abort(); }
+int llme_sched_fail(void* h) { return static_cast<Scheduler*>(h)->fail(); }
 int llme_sched_num_results(void* h) { return static_cast<Scheduler*>(h)->num_results(); }
-// reason: 1 "stop", 2 "length", 3 "capacity"
+// reason: 1 "stop", 2 "length", 3 "capacity", 4 "error"
 int llme_sched_result_info(void* h, int i, int64_t* seq_id, long* prompt_len, long* n_tokens, int* reason) {
     const auto* s = static_cast<Scheduler*>(h)->result(i);
     if (!s) return LLME_HOST_BAD_ARGUMENT;

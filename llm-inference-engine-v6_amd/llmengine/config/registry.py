@@ -17,7 +17,7 @@ from .base import ConfigError, read_model_json
 class Architecture:
     name: str
     parse_config: Callable[..., Any]     # (config dict, generation dict | None, architecture=name) -> config
-    build_model: Callable[..., Any]      # (config, dtype, device) -> DecoderModel
+    build_model: Callable[..., Any]      # (config) -> DecoderModel, its tensors not yet loaded
 
 
 _ARCHITECTURES: dict[str, Architecture] = {}

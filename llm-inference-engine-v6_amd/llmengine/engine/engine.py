@@ -23,7 +23,7 @@ from ..config.registry import architecture_name, parse_config, resolve
 from ..parts.base import Placement
 from ..sampling import Sampler
 from ..weights import TensorIndex, load_model_weights, load_state_dict, random_state
-from .step import CacheContext, CapacityError, ModelRunner, StepEntry
+from .step import CacheContext, CapacityError, ModelRunner, StepCommittedError, StepEntry
 
 _DTYPES = {"fp32": torch.float32, "float32": torch.float32, "bf16": torch.bfloat16,
            "bfloat16": torch.bfloat16}
@@ -75,7 +75,7 @@ class Engine:
     def __init__(self, model_dir: str | None, dtype: str = "fp32", *, device: str = "cuda:0",
                  max_prefill_tokens_per_step: int = 8192, temperature: float = 0.0, sampler_seed: int = 0,
                  block_size: int = 16, use_graphs: bool = True, max_context: int | None = None,
-                 deterministic: bool = False, _config: dict | None = None, _tensors=None):
+                 deterministic: bool = False, kernel_choices=None, _config: dict | None = None, _tensors=None):
         self._dtype_name = {"float32": "fp32", "bfloat16": "bf16"}.get(dtype, dtype)
         self._torch_dtype = parse_dtype(dtype)
         if _config is None:
@@ -113,6 +113,9 @@ class Engine:
         # every run (bfloat16 products into the residual stream are otherwise cut over k and joined
         # with atomics in the order the workgroups happen to finish).
         self.deterministic = bool(deterministic)
+        # which kernels the operations may choose and where launch plans change shape (ops.KernelChoices;
+        # None: the defaults): for tests and measurements
+        self.kernel_choices = kernel_choices
 
     # ---- construction from random weights ----
     @classmethod
@@ -164,6 +167,9 @@ class Engine:
                 from ..ops import library
                 library()                               # fails loudly if the kernels are missing
                 model = self._arch.build_model(self.cfg)
+                refused = model.tree_refusals()
+                if refused:
+                    raise ValueError("this engine's kernels do not take this model: " + "; ".join(refused))
                 placement = Placement(device, self._torch_dtype)
                 with torch.cuda.device(device):
                     if self._tensors is not None:
@@ -172,7 +178,7 @@ class Engine:
                     else:
                         load_model_weights(model, self.model_dir, placement)
                 self._runner = ModelRunner(model, self._torch_dtype, device, use_graphs=self.use_graphs,
-                                           deterministic=self.deterministic)
+                                           deterministic=self.deterministic, choices=self.kernel_choices)
             return self._runner
 
     @property
@@ -202,7 +208,9 @@ class Engine:
             return self.runner.step(cache, entries, max_position=self.max_pos)
 
     def run_step(self, cache: CacheContext, entries, draws, temperature: float = 0.0, seed: int = 0) -> list[int]:
-        """A step plus the choice of a token for every wanted row (the scheduler's call)."""
+        """A step plus the choice of a token for every wanted row (the scheduler's call). A failure
+        before the step is committed to the cache raises what it is and has changed nothing; one
+        behind that raises StepCommittedError."""
         with self._lock, torch.cuda.device(self.runner.device):
             if temperature == 0.0:
                 tokens = self.runner.step_greedy(cache, entries, max_position=self.max_pos)
@@ -211,12 +219,15 @@ class Engine:
             logits = self.runner.step(cache, entries, max_position=self.max_pos)
             if logits is None:
                 return []
-            sampler = self._samplers.get((float(temperature), int(seed)))
-            if sampler is None:
-                if len(self._samplers) >= 64:
-                    self._samplers = {(self.sampler.temperature, self.sampler.seed): self.sampler}
-                sampler = self._samplers[(float(temperature), int(seed))] = Sampler(temperature, seed)
-            return sampler.choose(logits, draws)
+            try:
+                sampler = self._samplers.get((float(temperature), int(seed)))
+                if sampler is None:
+                    if len(self._samplers) >= 64:
+                        self._samplers = {(self.sampler.temperature, self.sampler.seed): self.sampler}
+                    sampler = self._samplers[(float(temperature), int(seed))] = Sampler(temperature, seed)
+                return sampler.choose(logits, draws)
+            except BaseException as e:                  # (the cache has moved on: the caller must not run the step again)
+                raise StepCommittedError(f"the step ran, but no tokens were chosen: {e}") from e
 
     def greedy_chain(self, cache: CacheContext, request_ids: Sequence, tokens: Sequence[int], steps: int
                      ) -> list[list[int]]:

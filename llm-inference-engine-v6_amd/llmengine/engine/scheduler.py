@@ -8,6 +8,8 @@ then decode one token per step; a sequence ends with "stop" (an EOS id was
 sampled; it is not appended), "length" (`max_new_tokens` reached, or 0 asked) or
 "capacity" (the page pool cannot hold its next tokens; what it generated so far is
 kept; nothing is preempted or recomputed). Results come back in enqueue order.
+One more reason, "error", has no counterpart there: a step ran, but the choice of
+its next tokens failed afterwards; its sequences cannot go on and keep what they had.
 
 What differs from the reference: a step is ONE mixed batch. Prompt portions and
 the single tokens of decoding requests go through the model together, and because
@@ -26,9 +28,9 @@ from dataclasses import dataclass
 from typing import Protocol, Sequence
 
 from ..runtime import native
-from .step import StepEntry
+from .step import StepCommittedError, StepEntry
 
-_REASONS = {1: "stop", 2: "length", 3: "capacity"}
+_REASONS = {1: "stop", 2: "length", 3: "capacity", 4: "error"}
 
 
 @dataclass
@@ -191,10 +193,16 @@ class ContinuousBatchScheduler:
             try:
                 sampled = self.engine.run_step(self._cache, entries, draws, self.temperature, self.seed)
                 if len(sampled) != len(draws):
-                    raise RuntimeError(f"the step returned {len(sampled)} tokens for {len(draws)} wanted rows")
+                    raise StepCommittedError(f"the step returned {len(sampled)} tokens for {len(draws)} wanted rows")
+            except StepCommittedError:
+                # the batch ran and the cache holds its tokens, but the next tokens never arrived: no
+                # sequence of the batch can go on, each ends with "error" and keeps what it had
+                self._lib.llme_sched_fail(self._h)
+                raise
             except BaseException:
                 # the batch did not run: the prompts stay where they were and the next step offers
-                # the same portions again (the step function changes nothing when it fails)
+                # the same portions again (the step function changes nothing when it fails before
+                # it commits)
                 self._lib.llme_sched_abort(self._h)
                 raise
             self.steps += 1

@@ -27,6 +27,11 @@ class CapacityError(RuntimeError):
     """The page pool cannot hold the tokens of a step."""
 
 
+class StepCommittedError(RuntimeError):
+    """A step ran and the cache holds its tokens, but what came after it failed (the choice of the
+    next tokens, their copy to the host): running the same step again would cache its tokens twice."""
+
+
 @dataclass
 class StepEntry:
     request_id: object
@@ -113,6 +118,7 @@ class StepContext:
     # sum has one fixed order, and a step gives the same bits every time it runs.
     fixed_order: bool = False
     extra: dict = field(default_factory=dict)          # per-step notes of kernels (launch plans)
+    choices: "ops.KernelChoices | None" = None          # which kernels the operations may choose (the runner's)
 
     def buffer(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         return self.workspace.get(name, shape, dtype)
@@ -260,8 +266,10 @@ class ModelRunner:
     GRAPH_LIMIT = 192               # recorded steps kept per page pool; the least recently used one goes first
 
     def __init__(self, model: DecoderModel, dtype: torch.dtype, device: torch.device, use_graphs: bool = True,
-                 deterministic: bool = False):
+                 deterministic: bool = False, choices: "ops.KernelChoices | None" = None):
         self.model = model
+        # what the operations may choose for this runner's steps (a copy of its own: see ops/choices.py)
+        self.choices = choices if choices is not None else ops.KernelChoices()
         self.deterministic = bool(deterministic)
         self.dtype = dtype
         self.device = device
@@ -339,7 +347,8 @@ class ModelRunner:
     def _decode_key(self, cache: CacheContext, S: int, longest: int, greedy: bool):
         need = (longest + cache.page_size) // cache.page_size
         bucket = self.GRAPH_BLOCK_BUCKET
-        return (S, (need + bucket - 1) // bucket * bucket, greedy)
+        # (a recording holds the launches that the choices of its time led to)
+        return (S, (need + bucket - 1) // bucket * bucket, greedy, self.choices.key())
 
     def _decode_record(self, cache: CacheContext, entries: Sequence[StepEntry] | None, longest: int, greedy: bool,
                        S: int | None = None):
@@ -410,7 +419,10 @@ class ModelRunner:
                 return None
             ids.append(e.request_id)
         pending = self.greedy_launch(cache, ids, [int(e.tokens[0]) for e in entries], max_position)
-        return self.greedy_result(pending)
+        try:
+            return self.greedy_result(pending)
+        except BaseException as e:
+            raise StepCommittedError(f"the step ran, but its tokens could not be fetched: {e}") from e
 
     def greedy_launch(self, cache: CacheContext, ids: Sequence, tokens: Sequence[int] | None,
                       max_position: int | None = None) -> "PendingTokens | None":
@@ -555,6 +567,6 @@ class ModelRunner:
             block_tables={g: view(6 + gi, (S, max_blocks)) for gi, g in enumerate(groups)},
             act_dtype=self.dtype, workspace=self.workspace, new_lens=new_lens, ctx_lens=ctx_lens,
             slot_list=slot_list, max_position=max(c + n for c, n in zip(ctx_lens, new_lens)) - 1,
-            plan_len=plan_len, fixed_order=self.deterministic)
+            plan_len=plan_len, fixed_order=self.deterministic, choices=self.choices)
         logit_rows = view(len(sizes) - 1) if R else None
         return ctx, logit_rows

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 from ..config.llama import LlamaConfig
 from ..config.registry import register_architecture
-from ..parts import (Embedding, LayerSpec, OutputHead, PartChoice, RMSNorm, build_layer)
+from ..parts import LayerSpec, PartChoice, build_layer, make_part
 from .model import DecoderModel
 
 
@@ -36,9 +36,11 @@ def llama_layer_specs(cfg: LlamaConfig) -> list[LayerSpec]:
 def build_llama(cfg: LlamaConfig) -> DecoderModel:
     shared: dict = {}
     layers = [build_layer(spec, shared) for spec in llama_layer_specs(cfg)]
-    embedding = Embedding(cfg.vocab_size, cfg.hidden_size)
-    head = OutputHead(cfg.vocab_size, cfg.hidden_size, tied_to=embedding if cfg.tie_word_embeddings else None)
-    return DecoderModel(cfg, embedding, layers, RMSNorm(cfg.hidden_size, cfg.rms_norm_eps), head)
+    embedding = make_part("embedding", "table", vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size)
+    head = make_part("head", "linear", vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size,
+                     tied_to=embedding if cfg.tie_word_embeddings else None)
+    final_norm = make_part("norm", "rmsnorm", size=cfg.hidden_size, eps=cfg.rms_norm_eps)
+    return DecoderModel(cfg, embedding, layers, final_norm, head)
 
 
 register_architecture("LlamaForCausalLM", LlamaConfig.from_dict, build_llama)

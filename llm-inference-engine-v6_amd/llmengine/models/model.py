@@ -13,8 +13,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ..parts.base import Block, CacheSpec, Norm, Part
-from ..parts.embedding import Embedding, OutputHead
+from ..parts.base import Block, CacheSpec, Head, Norm, Part, TokenEmbedding
 
 
 @dataclass(frozen=True)
@@ -31,8 +30,8 @@ class LayerCall:
 class DecoderModel(Part):
     graph_safe = True
 
-    def __init__(self, config, embedding: Embedding, layers: list[Block], final_norm: Norm,
-                 head: OutputHead, schedule: list[LayerCall] | None = None, names: dict | None = None):
+    def __init__(self, config, embedding: TokenEmbedding, layers: list[Block], final_norm: Norm,
+                 head: Head, schedule: list[LayerCall] | None = None, names: dict | None = None):
         self.config = config
         self.embedding, self.layers, self.final_norm, self.head = embedding, list(layers), final_norm, head
         self.schedule = list(schedule) if schedule is not None else [LayerCall(i) for i in range(len(layers))]
@@ -57,7 +56,7 @@ class DecoderModel(Part):
     def aliases(self):
         # A tied head is the embedding table under a second name (src/weights.cpp:244-267): a
         # checkpoint may store it under both, and then both must agree in shape and type.
-        if self.head.tied_to is self.embedding:
+        if getattr(self.head, "tied_to", None) is self.embedding:
             return {f"{self.names['head']}.weight": f"{self.names['embedding']}.weight"}
         return {}
 
@@ -87,17 +86,17 @@ class DecoderModel(Part):
         [len(logit_rows), vocab] for the wanted rows (None if none is wanted)."""
         T = step.num_tokens
         h = step.buffer("model.hidden", (T, self.hidden_size), torch.float32)
-        self.embedding.forward(step.tokens, h)
+        self.embedding.forward(step.tokens, h, step)
         for call in self.schedule:
             self.layers[call.layer].forward(h, step, caches[call.cache_id], call.write_cache)
         if logit_rows is None or logit_rows.shape[0] == 0:
             return None
         R = logit_rows.shape[0]
         logits = step.buffer("model.logits", (R, self.vocab_size), torch.float32)
-        if self.head.fuses_norm(h, self.final_norm, R, step.act_dtype):
-            self.head.forward_normed_rows(h, logit_rows, self.final_norm, logits)
+        if self.head.fuses_norm(h, self.final_norm, R, step):
+            self.head.forward_normed_rows(h, logit_rows, self.final_norm, logits, step)
         else:
             x = step.buffer("model.head_in", (R, self.hidden_size), step.act_dtype)
             self.final_norm.forward(h, x, rows=logit_rows)
-            self.head.forward(x, logits)
+            self.head.forward(x, logits, step)
         return logits

@@ -1,0 +1,56 @@
+"""What the dispatching operations may choose, and the sizes at which launch plans change their
+shape: one object per model runner, handed to the operations through the step.
+
+Nothing here changes what is computed, only which kernel computes it and how its work is cut.
+Tests and measurements make an object with other values for an engine of their own; two engines in
+one process do not share it, and a recorded decode step is kept under the values it was recorded
+with."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+
+@dataclass
+class KernelChoices:
+    # the matrix-instruction kernels where operand types and sizes fit them; off: every product /
+    # every attention goes through the plain-precision kernels (the 32-bit model's always do)
+    fast_gemm: bool = True
+    fast_attention: bool = True
+    # decoding, up to 16 tokens whose keys are cut into splits: the splits' join inside the output projection
+    join_project: bool = True
+    # decoding, 17 to 64 tokens with the keys in one split: rotation and cache write inside the attention kernel
+    decode_rope: bool = True
+    # prompt attention: work items of half the rows where a step has few items
+    prefill_half_rows: bool = True
+    # Workgroups (of four wavefronts) the decode kernel should have at most when it cuts the keys: one
+    # per compute unit (None: the device is asked for their number). Measured on the 256 compute units
+    # of an MI355X at batch 8 and a context of 4,096: 0.948 ms a step with 256, 0.969 with 512, 0.998
+    # with 1,024, 1.036 with 128; with 384 (one and a half per compute unit) 1.000.
+    decode_blocks_wanted: int | None = None
+    # Portions of prompts: work items (a span of rows x a group of heads) the prefill kernel should
+    # have at least (None: two per compute unit); with prefill_cut_items or fewer (None: half a
+    # workgroup per compute unit; measured: 256 items cut in two were 3 % slower than whole), the longest
+    # item's keys are cut into that many runs of at least prefill_min_run keys, and the others' into
+    # runs of the same length.
+    prefill_items_wanted: int | None = None
+    prefill_cut_items: int | None = None
+    prefill_min_run: int = 512
+    prefill_max_splits: int = 16
+    # Two runs are not worth their join: a 256-token portion beside 17 decoded tokens at the 1B sizes takes
+    # 2.18 ms in two runs against 2.07 whole behind 1,024 tokens, 2.28 against 2.27 behind 2,048 (four
+    # runs: 2.20), and behind 3,000 tokens 2.32 in three or six runs against 2.49 whole.
+    # (A whole prompt of 2,048 tokens, whose last rows' items walk twice the average, was also tried with
+    # the items behind 1,024 keys cut in two: 6.5 to 6.6 ms against 5.95 whole; the partial outputs and
+    # the join cost more than the evener load wins.)
+    prefill_min_splits: int = 3
+
+    def key(self) -> tuple:
+        return tuple(self.__dict__.values())
+
+
+# What an operation uses when it is called without a step (a kernel on its own).
+DEFAULT = KernelChoices()
+
+
+def choices_of(step) -> KernelChoices:
+    return getattr(step, "choices", None) or DEFAULT

@@ -12,18 +12,10 @@ from .lib import BF16, F32, KernelError, check, code, entry, ptr, require, strea
 _FLOATS = (torch.float32, torch.bfloat16)
 
 
-class Policy:
-    """Which kernel family the dispatching operations may choose.
+from .choices import DEFAULT, KernelChoices, choices_of  # noqa: E402,F401
 
-    `fast_gemm` / `fast_attention`: allow the MFMA kernels where operand types and
-    sizes fit them; off, every product and every attention goes through the
-    plain-precision kernels (the 32-bit model always does)."""
-
-    fast_gemm = True
-    fast_attention = True
-
-
-policy = Policy()
+# The choices of operations that are called without a step (kernels on their own).
+policy = DEFAULT
 
 
 # --- weight layouts ------------------------------------------------------------------
@@ -191,17 +183,20 @@ _fast_gemm = None       # set by ops/mfma.py when the MFMA kernels are present
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
-         fixed_order: bool = False) -> None:
+         fixed_order: bool = False, choices: KernelChoices | None = None) -> None:
     """out[m, n] (+)= sum_k a[m, k] w[n, k]; 32-bit accumulation whatever the types. A sum that
     adds into `out` may be cut over k into parts that several workgroups add with atomics, in
     whatever order they finish: the result then differs from run to run in its last bits.
     fixed_order forbids that cut (every output element is summed by one workgroup in one order)."""
-    if policy.fast_gemm and _fast_gemm is not None and _fast_gemm(a, w, out, accumulate, fixed_order):
+    if (choices or DEFAULT).fast_gemm and _fast_gemm is not None and _fast_gemm(a, w, out, accumulate, fixed_order):
         return
     gemm_generic(a, w, out, accumulate)
 
 
 # --- attention -----------------------------------------------------------------------
+ATTENTION_MAX_HEAD_DIM = 256        # (a lane of attention_generic holds head_dim / 64 values of a row)
+
+
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                       positions: torch.Tensor, seq_idx: torch.Tensor, block_table: torch.Tensor,
                       n_q: int, n_kv: int, head_dim: int, scale: float, window: int = 0) -> None:
@@ -214,8 +209,8 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     require(positions, "positions", torch.int32, (T,))
     require(seq_idx, "seq_idx", torch.int32, (T,))
     require(block_table, "block_table", torch.int32, (None, None))
-    if head_dim > 256:
-        raise KernelError(f"attention: head_dim {head_dim} is beyond the kernel's limit of 256")
+    if head_dim > ATTENTION_MAX_HEAD_DIM:
+        raise KernelError(f"attention: head_dim {head_dim} is beyond the kernel's limit of {ATTENTION_MAX_HEAD_DIM}")
     if n_q % n_kv:
         raise KernelError(f"attention: {n_q} query heads do not divide into {n_kv} key/value heads")
     check(entry("llme_attention_generic")(
@@ -234,7 +229,7 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out
               window: int = 0) -> None:
     """Attention of every token of the step over its request's pages. `step` carries
     positions, request index per token and, on the host, how the batch is cut."""
-    if policy.fast_attention and _fast_attention is not None and _fast_attention(
+    if choices_of(step).fast_attention and _fast_attention is not None and _fast_attention(
             q, k_cache, v_cache, out, step, block_table, n_q, n_kv, head_dim, scale, window):
         return
     attention_generic(q, k_cache, v_cache, out, step.positions, step.seq_idx, block_table, n_q, n_kv,
@@ -248,12 +243,13 @@ def attention_project(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     step of a few decoded tokens cuts its keys into splits, the splits' join and the projection are
     one kernel, and o is not written."""
     # (only a step of up to 16 decoded tokens is asked about: steps launched kernel by kernel count their calls)
-    if (q.shape[0] <= 16 and policy.fast_attention and policy.fast_gemm and _fast_attention_project is not None
+    choices = choices_of(step)
+    if (q.shape[0] <= 16 and choices.fast_attention and choices.fast_gemm and _fast_attention_project is not None
             and _fast_attention_project(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, head_dim, scale, window,
                                         w_o, out, accumulate)):
         return
     attention(q, k_cache, v_cache, o, step, block_table, n_q, n_kv, head_dim, scale, window)
-    gemm(o, w_o, out, accumulate, fixed_order=step.fixed_order)
+    gemm(o, w_o, out, accumulate, fixed_order=step.fixed_order, choices=choices)
 
 
 # --- sampling ------------------------------------------------------------------------

@@ -8,6 +8,7 @@ import ctypes
 import torch
 
 from . import kernels
+from .choices import DEFAULT, KernelChoices, choices_of
 from .lib import check, declare, entry, ptr, require, stream
 
 _vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
@@ -52,18 +53,19 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
           "gemm_bf16")
 
 
-def gemm_gated(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, group: int, scratch) -> None:
+def gemm_gated(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor, group: int, scratch,
+               choices: KernelChoices | None = None) -> None:
     """out [T, FF] = silu(x Wg^T) * (x Wu^T), the gate and up rows interleaved in groups of `group`
     rows of w_gate_up [2 FF, K]. One MFMA kernel where the types and sizes fit it; otherwise the
     product into a 32-bit scratch [T, 2 FF] (scratch(shape, dtype) provides it) and the
     activation kernel."""
     T, FF = out.shape
-    if (kernels.policy.fast_gemm and group == 16 and out.dtype == torch.bfloat16 and (2 * FF) % 32 == 0
+    if ((choices or DEFAULT).fast_gemm and group == 16 and out.dtype == torch.bfloat16 and (2 * FF) % 32 == 0
             and x.dtype == torch.bfloat16 and gemm_bf16_supported(x, w_gate_up, out, False)):
         gemm_bf16(x, w_gate_up, out, gated=True, _supported=True)
         return
     gu = scratch((T, 2 * FF), torch.float32)
-    kernels.gemm(x, w_gate_up, gu)
+    kernels.gemm(x, w_gate_up, gu, choices=choices)
     kernels.swiglu(gu, out, group)
 
 
@@ -71,8 +73,13 @@ declare("llme_gemm_bf16_qkv_rope", [_vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _v
 
 
 def gemm_qkv_rope_supported(x: torch.Tensor, w_qkv: torch.Tensor, k_cache: torch.Tensor, head_dim: int,
-                            rotary_dim: int) -> bool:
-    return (kernels.policy.fast_gemm and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16
+                            rotary_dim: int, choices: KernelChoices | None = None) -> bool:
+    """Whether a step may take gemm_qkv_rope: the kernel takes the operands, and the choices allow it."""
+    return (choices or DEFAULT).fast_gemm and _gemm_qkv_rope_fits(x, w_qkv, k_cache, head_dim, rotary_dim)
+
+
+def _gemm_qkv_rope_fits(x, w_qkv, k_cache, head_dim: int, rotary_dim: int) -> bool:
+    return (x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16
             and k_cache.dtype == torch.bfloat16 and head_dim in (16, 32, 64, 128) and rotary_dim == head_dim
             and w_qkv.dim() in (2, 5) and x.shape[1] % 8 == 0 and x.data_ptr() % 16 == 0 and w_qkv.data_ptr() % 16 == 0)
 
@@ -99,7 +106,7 @@ def gemm_qkv_rope(x: torch.Tensor, w_qkv: torch.Tensor, cos: torch.Tensor, sin: 
     require(k_cache, "k_cache", torch.bfloat16, (None, n_kv, None, head_dim))
     page = k_cache.shape[2]
     require(v_cache, "v_cache", torch.bfloat16, (k_cache.shape[0], n_kv, head_dim, page))
-    if not gemm_qkv_rope_supported(x, w_qkv, k_cache, head_dim, head_dim):
+    if not _gemm_qkv_rope_fits(x, w_qkv, k_cache, head_dim, head_dim):
         raise kernels.KernelError(f"gemm_qkv_rope: head size {head_dim} (16, 32, 64 or 128), K={K} (multiple of 8) or the "
                                   "operand types are not supported")
     check(entry("llme_gemm_bf16_qkv_rope")(
@@ -134,14 +141,13 @@ def attention_tuning(rows: int = 0, shared: int = -1, read_once: int = -1, half_
     one / two wavefronts per tile whatever the number of items. read_once: the decode kernel's
     cache hint on keys and values: -1 the entry point chooses, 0 off, 1 on. half_rows: work items of
     half the rows in the kernel that shares K and V (plan_attention sets it by itself for steps with
-    few items; PREFILL_HALF_ROWS False keeps it from that)."""
+    few items; the choice prefill_half_rows False keeps it from that)."""
     if rows not in (0, 16, 32, 64) or not -1 <= shared <= 3 or not -1 <= read_once <= 1:
         raise kernels.KernelError(f"attention_tuning: rows {rows}, shared {shared}, read_once {read_once}")
     return rows | (shared + 1) << 8 | (read_once + 1) << 12 | (TUNING_HALF_ROWS if half_rows else 0)
 
 
 TUNING_HALF_ROWS = 1 << 15
-PREFILL_HALF_ROWS = True            # (tests and measurements switch the choice off here)
 
 _work_queues: dict = {}
 
@@ -156,11 +162,6 @@ def work_queue(device: torch.device) -> torch.Tensor:
     return q
 
 
-# Workgroups (of four wavefronts) the decode kernel should have at most when it cuts the keys: one
-# per compute unit (None: the device is asked for their number). Measured on the 256 compute units
-# of an MI355X at batch 8 and a context of 4,096: 0.948 ms a step with 256, 0.969 with 512, 0.998
-# with 1,024, 1.036 with 128; with 384 (one and a half per compute unit) 1.000.
-DECODE_BLOCKS_WANTED: int | None = None
 _compute_units = 0
 
 
@@ -173,21 +174,6 @@ def compute_units() -> int:
 
 MIN_SPLIT = 128                     # keys per split at least: one 32-key block per wavefront
 MAX_SPLITS = 64                     # the join kernel's limit
-# Portions of prompts: work items (a span of rows x a group of heads) the prefill kernel should
-# have at least; with PREFILL_CUT_ITEMS or fewer (half a workgroup per compute unit; measured: 256
-# items cut in two were 3 % slower than whole), the longest item's keys are cut into that many
-# runs of at least PREFILL_MIN_RUN keys, and the others' into runs of the same length.
-PREFILL_ITEMS_WANTED: int | None = None        # None: two per compute unit
-PREFILL_CUT_ITEMS: int | None = None           # None: half a workgroup per compute unit
-PREFILL_MIN_RUN = 512
-PREFILL_MAX_SPLITS = 16
-PREFILL_MIN_SPLITS = 3
-# Two runs are not worth their join: a 256-token portion beside 17 decoded tokens at the 1B sizes takes
-# 2.18 ms in two runs against 2.07 whole behind 1,024 tokens, 2.28 against 2.27 behind 2,048 (four
-# runs: 2.20), and behind 3,000 tokens 2.32 in three or six runs against 2.49 whole.
-# (A whole prompt of 2,048 tokens, whose last rows' items walk twice the average, was also tried with
-# the items behind 1,024 keys cut in two: 6.5 to 6.6 ms against 5.95 whole; the partial outputs and
-# the join cost more than the evener load wins.)
 
 
 def attention_bf16_supported(q, k_cache, head_dim: int) -> bool:
@@ -197,10 +183,12 @@ def attention_bf16_supported(q, k_cache, head_dim: int) -> bool:
 
 
 def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_len: int | None = None,
-                   tuning: int = 0) -> dict:
+                   tuning: int = 0, choices: KernelChoices | None = None) -> dict:
     """Launch sizes for a step, from how its batch is cut (host-side numbers only). plan_len:
     plan the decode splits for requests of up to this many tokens, whatever their length now
-    (a recorded step is replayed while the requests grow). tuning: see attention_tuning."""
+    (a recorded step is replayed while the requests grow). tuning: see attention_tuning. choices:
+    the sizes at which the plan changes its shape."""
+    ch = choices or DEFAULT
     rows = entry("llme_attention_bf16_rows")(head_dim, n_q, n_kv, tuning)
     if rows <= 0:
         raise kernels.KernelError(f"plan_attention: tuning {tuning} is not one that attention_tuning makes")
@@ -214,16 +202,16 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
         # few rows over long contexts: too few work items for the chip, each with many keys
         keys = max(c + n for n, c in zip(new_lens, ctx_lens) if n >= 2)
         splits = 1
-        if items <= (PREFILL_CUT_ITEMS or compute_units() // 2):
-            splits = max(1, min((PREFILL_ITEMS_WANTED or 2 * compute_units()) // items, keys // PREFILL_MIN_RUN,
-                                PREFILL_MAX_SPLITS))
-            if splits < PREFILL_MIN_SPLITS:
+        if items <= (ch.prefill_cut_items or compute_units() // 2):
+            splits = max(1, min((ch.prefill_items_wanted or 2 * compute_units()) // items, keys // ch.prefill_min_run,
+                                ch.prefill_max_splits))
+            if splits < ch.prefill_min_splits:
                 splits = 1                                 # (two runs win less than their join costs)
             stretches = (keys + 63) // 64
             run = (stretches + splits - 1) // splits       # stretches of 64 keys per run
         if splits > 1:
             plan["prefill_splits"], plan["prefill_run"] = splits, run
-        elif (PREFILL_HALF_ROWS and not tuning & TUNING_HALF_ROWS
+        elif (ch.prefill_half_rows and not tuning & TUNING_HALF_ROWS
               and items <= (3 if head_dim == 64 else 1) * compute_units()):
             # few items whose keys are not cut (short prompts, portions early in a prompt): work items of
             # half the rows, until the items of whole rows number one workgroup less per compute unit than
@@ -237,7 +225,7 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
     if decode:
         longest = max(decode) if plan_len is None else max(plan_len, max(decode))
         pairs = len(decode) * n_kv * ((n_q // n_kv + 15) // 16)
-        nsplit = max(1, min((DECODE_BLOCKS_WANTED or compute_units()) // pairs, (longest + MIN_SPLIT - 1) // MIN_SPLIT, MAX_SPLITS))
+        nsplit = max(1, min((ch.decode_blocks_wanted or compute_units()) // pairs, (longest + MIN_SPLIT - 1) // MIN_SPLIT, MAX_SPLITS))
         split_len = ((longest + nsplit - 1) // nsplit + 31) // 32 * 32
         plan["split_len"] = split_len
         plan["nsplit"] = (longest + split_len - 1) // split_len
@@ -292,7 +280,8 @@ def _fast_attention(q, k_cache, v_cache, out, step, block_table, n_q, n_kv, head
     key = ("attention_plan", n_q, n_kv, head_dim)
     plan = step.extra.get(key)
     if plan is None:
-        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len)
+        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len,
+                                                      choices=choices_of(step))
     part_o = part_ml = None
     if plan["n_decode"] and plan["nsplit"] > 1:
         S = step.num_seqs
@@ -314,7 +303,6 @@ declare("llme_attention_join_project_supported", [_i, _i, _i, _i, _i])
 declare("llme_attention_join_project_pays", [_i, _i, _i, _i, _i])
 declare("llme_attention_join_project", [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp])
 TUNING_NO_JOIN = 1 << 14            # the decode kernel leaves its splits unjoined (see attention_mfma.hip)
-JOIN_PROJECT = True                 # (tests and measurements switch the fused kernel off here)
 
 
 def attention_join_project(part_o, part_ml, w_o, out, n_rows: int, n_q: int, head_dim: int, nsplit: int) -> None:
@@ -339,14 +327,15 @@ def _fast_attention_project(q, k_cache, v_cache, o, step, block_table, n_q, n_kv
     """A step of up to 16 decoded tokens whose keys are cut into splits: the splits stay unjoined and
     one kernel joins them and projects. Everything else: not taken (the caller runs the two apart)."""
     T = q.shape[0]
-    if (not JOIN_PROJECT or not accumulate or step.fixed_order or T > 16 or T != step.num_seqs
+    if (not choices_of(step).join_project or not accumulate or step.fixed_order or T > 16 or T != step.num_seqs
             or out.dtype != torch.float32 or w_o.dtype != torch.bfloat16 or not kernels.is_blocked(w_o)
             or not attention_bf16_supported(q, k_cache, head_dim) or o.dtype != torch.bfloat16):
         return False
     key = ("attention_plan", n_q, n_kv, head_dim)
     plan = step.extra.get(key)
     if plan is None:
-        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len)
+        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len,
+                                                      choices=choices_of(step))
     N, K = kernels.weight_shape(w_o)
     if (plan["n_decode"] != T or plan["groups"] or plan["nsplit"] <= 1 or K != n_q * head_dim
             or not entry("llme_attention_join_project_pays")(T, n_q, head_dim, plan["nsplit"], N)):
@@ -363,7 +352,6 @@ kernels._fast_attention_project = _fast_attention_project
 
 declare("llme_attention_decode_rope_bf16", [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i,
                                             _i, _vp])
-DECODE_ROPE = True                  # (tests and measurements switch the fused kernel off here)
 
 
 def attention_decode_rope(qkv, cos, sin, k_cache, v_cache, out, step, block_table, n_q: int, n_kv: int, head_dim: int,
@@ -373,7 +361,8 @@ def attention_decode_rope(qkv, cos, sin, k_cache, v_cache, out, step, block_tabl
     [S, n_q head_dim] and the clearing of qkv, in the attention kernel (one workgroup per request and kv
     head, the keys in a single split). False, and nothing done, where the step or the sizes are not such."""
     T = qkv.shape[0]
-    if (not DECODE_ROPE or not kernels.policy.fast_attention or T != step.num_seqs or head_dim not in (64, 128)
+    ch = choices_of(step)
+    if (not ch.decode_rope or not ch.fast_attention or T != step.num_seqs or head_dim not in (64, 128)
             or cos is None or cos.shape[1] * 2 != head_dim or n_q % n_kv or n_q // n_kv > 16
             or qkv.dtype != torch.float32 or out.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16
             or k_cache.shape[2] % 16 or qkv.data_ptr() % 16 or cos.data_ptr() % 16 or sin.data_ptr() % 16
@@ -382,7 +371,8 @@ def attention_decode_rope(qkv, cos, sin, k_cache, v_cache, out, step, block_tabl
     key = ("attention_plan", n_q, n_kv, head_dim)
     plan = step.extra.get(key)
     if plan is None:
-        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len)
+        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len,
+                                                      choices=choices_of(step))
     if plan["n_decode"] != T or plan["groups"] or plan["nsplit"] != 1:
         return False
     # (measured, ms a decode step at a context of 2,048, apart / inside: 1B sizes 1.238 / 1.203 at 17 requests,
@@ -417,13 +407,18 @@ QKV_SUM_MAX_ROWS = 64
 
 
 def gemv_norm_supported(h: torch.Tensor, norm_weight: torch.Tensor, w: torch.Tensor, rows_out: int,
-                        gated: bool) -> bool:
+                        gated: bool, choices: KernelChoices | None = None) -> bool:
+    """Whether a step may take gemv_norm: the kernel takes the operands, and the choices allow it."""
+    return (choices or DEFAULT).fast_gemm and _gemv_norm_fits(h, norm_weight, w, rows_out, gated)
+
+
+def _gemv_norm_fits(h, norm_weight, w, rows_out: int, gated: bool) -> bool:
     K = h.shape[1]
     if w.dim() not in (2, 5):
         return False
     n_rows, k_w = kernels.weight_shape(w)
     n_out = n_rows // 2 if gated else n_rows
-    return (kernels.policy.fast_gemm and h.dtype == torch.float32 and w.dtype == torch.bfloat16
+    return (h.dtype == torch.float32 and w.dtype == torch.bfloat16
             and norm_weight.dtype in (torch.float32, torch.bfloat16) and 0 < rows_out <= GEMV_NORM_MAX_ROWS
             and K % 8 == 0 and 16 * (K + 8) * 2 <= 132 * 1024 and k_w == K
             and (not gated or n_out % 16 == 0) and w.data_ptr() % 16 == 0 and h.data_ptr() % 16 == 0
@@ -444,7 +439,7 @@ def gemv_norm(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.T
     n_rows, _ = kernels._require_weight(w, "w", torch.bfloat16, K)
     N = n_rows // 2 if gated else n_rows
     require(out, "out", torch.bfloat16 if gated else torch.float32, (M, N))
-    if not gemv_norm_supported(h, norm_weight, w, M, gated):
+    if not _gemv_norm_fits(h, norm_weight, w, M, gated):
         raise kernels.KernelError(f"gemv_norm: {M} rows (at most 16), K={K} (multiple of 8, 16 rows must fit "
                                   "into LDS) or the operand types are not supported")
     check(entry("llme_gemv_norm")(ptr(h), ptr(rows), ptr(norm_weight), 0 if norm_weight.dtype == torch.float32 else 1,
@@ -457,8 +452,9 @@ declare("llme_gemv_norm_rope", [_vp, _vp, _i, _f, _vp, _vp, _vp, _vp, _i, _vp, _
                                 _i, _i, _i, _i, _i, _i, _i, _i, _vp])
 
 
-def gemv_norm_rope_supported(h, norm_weight, w_qkv, k_cache, n_tokens: int, head_dim: int, rotary_dim: int) -> bool:
-    return (gemv_norm_supported(h, norm_weight, w_qkv, n_tokens, gated=False) and rotary_dim == head_dim
+def gemv_norm_rope_supported(h, norm_weight, w_qkv, k_cache, n_tokens: int, head_dim: int, rotary_dim: int,
+                             choices: KernelChoices | None = None) -> bool:
+    return (gemv_norm_supported(h, norm_weight, w_qkv, n_tokens, gated=False, choices=choices) and rotary_dim == head_dim
             and head_dim % 16 == 0 and k_cache.dtype == torch.bfloat16)
 
 
@@ -502,7 +498,7 @@ def gemv_norm_rope(h: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv
     require(k_cache, "k_cache", torch.bfloat16, (None, n_kv, None, head_dim))
     page = k_cache.shape[2]
     require(v_cache, "v_cache", torch.bfloat16, (k_cache.shape[0], n_kv, head_dim, page))
-    if not gemv_norm_rope_supported(h, norm_weight, w_qkv, k_cache, M, head_dim, head_dim):
+    if not (_gemv_norm_fits(h, norm_weight, w_qkv, M, False) and head_dim % 16 == 0 and k_cache.dtype == torch.bfloat16):
         raise kernels.KernelError(f"gemv_norm_rope: {M} rows (at most 16), head size {head_dim} (multiple of 16) or "
                                   "the operand types are not supported")
     check(entry("llme_gemv_norm_rope")(

@@ -1,5 +1,5 @@
-from .base import (PAGE, Block, CacheSpec, FeedForward, LayerCache, Mixer, Norm, ParamSpec, Part, Placement,
-                   PositionEncoding)
+from .base import (PAGE, Block, CacheSpec, FeedForward, Head, LayerCache, Mixer, Norm, ParamSpec, Part, Placement,
+                   PositionEncoding, TokenEmbedding)
 from .registry import LayerSpec, PartChoice, build_layer, make_part, register_part, registered
 from .norm import RMSNorm
 from .rope import RotaryEmbedding, inverse_frequencies
@@ -9,6 +9,6 @@ from .attention import Attention
 from .block import PreNormBlock
 
 __all__ = ["PAGE", "Block", "CacheSpec", "FeedForward", "LayerCache", "Mixer", "Norm", "ParamSpec", "Part",
-           "Placement", "PositionEncoding", "LayerSpec", "PartChoice", "build_layer", "make_part",
+           "Placement", "PositionEncoding", "TokenEmbedding", "Head", "LayerSpec", "PartChoice", "build_layer", "make_part",
            "register_part", "registered", "RMSNorm", "RotaryEmbedding", "inverse_frequencies", "Embedding",
            "OutputHead", "GatedMLP", "Attention", "PreNormBlock"]

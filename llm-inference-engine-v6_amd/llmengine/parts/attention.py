@@ -68,6 +68,11 @@ class Attention(Mixer):
                 ops.pair_rows_for_rotation(fused, self.num_heads + self.num_kv_heads, self.head_dim))
         self.w_o = placement.place_matrix(get("o_proj.weight"))
 
+    def refusals(self):
+        if self.head_dim > ops.ATTENTION_MAX_HEAD_DIM:
+            return [f"head_dim={self.head_dim}: the attention kernels take head sizes up to {ops.ATTENTION_MAX_HEAD_DIM}"]
+        return []
+
     def tree_graph_safe(self) -> bool:
         # (the position encoding is no child with tensors of its own, but it runs inside forward)
         return super().tree_graph_safe() and (self.position is None or self.position.tree_graph_safe())
@@ -81,7 +86,7 @@ class Attention(Mixer):
         # A few rows (decoding): the q/k/v projection applies the norm itself.
         rms = norm.fused_rms()
         return (rms is not None and step.act_dtype == torch.bfloat16
-                and ops.gemv_norm_supported(h, rms[0], self.w_qkv, h.shape[0], gated=False))
+                and ops.gemv_norm_supported(h, rms[0], self.w_qkv, h.shape[0], gated=False, choices=step.choices))
 
     def forward(self, x, step, cache, out, accumulate, write_cache=True, pre_norm=None):
         """pre_norm: the norm in front of this mixer when `fuses_norm` said yes; x is then the
@@ -104,14 +109,14 @@ class Attention(Mixer):
             if rms is not None:
                 ops.gemv_norm(x, rms[0], rms[1], weight, dst)
             else:
-                ops.gemm(x, weight, dst)
+                ops.gemm(x, weight, dst, choices=step.choices)
         if (write_cache and rms is not None and cos is not None and self.w_qkv_paired is not None
-                and ops.gemv_norm_rope_supported(x, rms[0], self.w_qkv_paired, k_cache, T, hd, rot)):
+                and ops.gemv_norm_rope_supported(x, rms[0], self.w_qkv_paired, k_cache, T, hd, rot, step.choices)):
             # decoding: norm, projection, rotation and the cache write are one kernel
             ops.gemv_norm_rope(x, rms[0], rms[1], self.w_qkv_paired, step.positions, step.seq_idx,
                                block_table, cos, sin, q, k_cache, v_cache, n_q, n_kv, hd)
         elif (write_cache and rms is None and T > ops.mfma.QKV_SUM_MAX_ROWS and cos is not None
-              and ops.gemm_qkv_rope_supported(x, self.w_qkv, k_cache, hd, rot)):
+              and ops.gemm_qkv_rope_supported(x, self.w_qkv, k_cache, hd, rot, step.choices)):
             # many rows (prompts): rotation and the cache write are the projection's epilogue
             ops.gemm_qkv_rope(x, self.w_qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
                               n_q, n_kv, hd)
@@ -131,7 +136,7 @@ class Attention(Mixer):
                 if step.extra.get("attn.qkv_sum zero", (0, 0)) != (qkv.data_ptr(), qkv.numel()):
                     ops.clear(qkv)
                 step.extra.pop("attn.qkv_sum zero", None)
-                ops.gemm(x, self.w_qkv, qkv, accumulate=True, fixed_order=step.fixed_order)
+                ops.gemm(x, self.w_qkv, qkv, accumulate=True, fixed_order=step.fixed_order, choices=step.choices)
             else:
                 project(self.w_qkv, qkv)
             if applies:
@@ -143,7 +148,7 @@ class Attention(Mixer):
                 if ops.mfma.attention_decode_rope(qkv, cos, sin, k_cache, v_cache, o, step, block_table, n_q, n_kv, hd,
                                                   self.scale, self.window):
                     step.extra["attn.qkv_sum zero"] = (qkv.data_ptr(), qkv.numel())
-                    ops.gemm(o, self.w_o, out, accumulate, fixed_order=step.fixed_order)
+                    ops.gemm(o, self.w_o, out, accumulate, fixed_order=step.fixed_order, choices=step.choices)
                     return
             ops.rope_kv_write(qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
                               n_q, n_kv, hd, rot, write_cache=True, zero_input=adds)

@@ -16,6 +16,9 @@ Kinds of parts and what each must provide:
 * `FeedForward`: forward(x [T, H], step, out32 [T, H], accumulate)
 * `Block`:     the arrangement of the four above around the 32-bit residual stream:
                forward(h32 [T, H], step, cache, write_cache)
+* `TokenEmbedding`: forward(tokens [T] int32, out32 [T, H], step): the stream's first value
+* `Head`:      forward(x [R, H], out32 [R, V], step) on normed rows; optionally
+               fuses_norm(h32, norm, n_rows, step) / forward_normed_rows(h32, rows, norm, out32, step)
 
 `step` is the engine's `StepContext` (tokens, positions, request index per token,
 block tables, slots, scratch buffers); `cache` is the `LayerCache` that the cache
@@ -106,6 +109,18 @@ class Part:
 
     def load_params(self, get: Getter, placement: Placement) -> None:
         """Reads the part's own tensors (children are loaded by the walker)."""
+
+    def refusals(self) -> list[str]:
+        """Sizes of this part that no kernel takes, each as a sentence that names the argument; asked
+        when a runner is made, before any tensor is read, so that such a model is refused with the
+        name of the size and not at its first step."""
+        return []
+
+    def tree_refusals(self, prefix: str = "") -> list[str]:
+        out = [f"{prefix.rstrip('.') or 'model'}: {r}" for r in self.refusals()]
+        for name, child in self.children().items():
+            out += child.tree_refusals(f"{prefix}{name}.")
+        return out
 
     # ---- walking a tree of parts ----
     def named_specs(self, prefix: str = "") -> dict[str, ParamSpec]:
@@ -245,4 +260,39 @@ class Block(Part):
     mixer: Mixer
 
     def forward(self, h: torch.Tensor, step, cache: LayerCache | None, write_cache: bool = True) -> None:
+        raise NotImplementedError
+
+
+class TokenEmbedding(Part):
+    """Token ids to the first value of the 32-bit residual stream. `vocab_size` and `hidden_size`
+    are attributes. An embedding whose table an output head may share (tied weights) keeps it as
+    `weight`, a matrix [vocab, hidden] in a layout that `ops.gemm` reads."""
+    vocab_size: int
+    hidden_size: int
+    weight: torch.Tensor | None = None
+
+    def forward(self, tokens: torch.Tensor, out: torch.Tensor, step=None) -> None:
+        """out [T, H] (32-bit) = the rows of tokens [T] (int32, on the device), with whatever
+        multiplier the architecture has."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    """The normed last rows of the stream to 32-bit logits. `vocab_size` is an attribute."""
+    vocab_size: int
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor, step=None) -> None:
+        """out [R, V] (32-bit) from x [R, H], rows that the final norm has been applied to."""
+        raise NotImplementedError
+
+    def fuses_norm(self, h: torch.Tensor, norm: "Norm", n_rows: int, step) -> bool:
+        """True if, for `n_rows` wanted rows of this step, the head wants the un-normed 32-bit stream
+        h [T, H] and applies `norm` itself in `forward_normed_rows` (a kernel of its own does both).
+        The default never does: the model then norms the wanted rows and calls `forward`."""
+        return False
+
+    def forward_normed_rows(self, h: torch.Tensor, rows: torch.Tensor, norm: "Norm", out: torch.Tensor,
+                            step=None) -> None:
+        """out [R, V] = head(norm(h[rows])), rows [R] int32 on the device. Only called after
+        `fuses_norm` said yes for the same step."""
         raise NotImplementedError

@@ -9,10 +9,11 @@ from __future__ import annotations
 import torch
 
 from .. import ops
-from .base import Getter, ParamSpec, Part, Placement
+from .base import Getter, Head, ParamSpec, Placement, TokenEmbedding
+from .registry import register_part
 
 
-class Embedding(Part):
+class Embedding(TokenEmbedding):
     graph_safe = True
 
     def __init__(self, vocab_size: int, hidden_size: int):
@@ -26,14 +27,14 @@ class Embedding(Part):
         # (a tied head reads the table as a weight matrix: the gather takes either layout)
         self.weight = placement.place_matrix(get("weight"))
 
-    def forward(self, tokens: torch.Tensor, out: torch.Tensor) -> None:
+    def forward(self, tokens: torch.Tensor, out: torch.Tensor, step=None) -> None:
         ops.embed_gather(self.weight, tokens, out)
 
 
-class OutputHead(Part):
+class OutputHead(Head):
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied_to: Embedding | None = None):
+    def __init__(self, vocab_size: int, hidden_size: int, tied_to: TokenEmbedding | None = None):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.tied_to = tied_to
         self._weight: torch.Tensor | None = None
@@ -51,15 +52,19 @@ class OutputHead(Part):
     def weight(self) -> torch.Tensor:
         return self.tied_to.weight if self.tied_to is not None else self._weight
 
-    def fuses_norm(self, h: torch.Tensor, norm, n_rows: int, act_dtype) -> bool:
+    def fuses_norm(self, h: torch.Tensor, norm, n_rows: int, step) -> bool:
         rms = norm.fused_rms()
-        return (rms is not None and act_dtype == torch.bfloat16
-                and ops.gemv_norm_supported(h, rms[0], self.weight, n_rows, gated=False))
+        return (rms is not None and step.act_dtype == torch.bfloat16
+                and ops.gemv_norm_supported(h, rms[0], self.weight, n_rows, gated=False, choices=step.choices))
 
-    def forward(self, x: torch.Tensor, out: torch.Tensor) -> None:
-        ops.gemm(x, self.weight, out)
+    def forward(self, x: torch.Tensor, out: torch.Tensor, step=None) -> None:
+        ops.gemm(x, self.weight, out, choices=getattr(step, "choices", None))
 
-    def forward_normed_rows(self, h: torch.Tensor, rows: torch.Tensor, norm, out: torch.Tensor) -> None:
+    def forward_normed_rows(self, h: torch.Tensor, rows: torch.Tensor, norm, out: torch.Tensor, step=None) -> None:
         """Logits of the chosen rows of the 32-bit stream, the final norm applied inside the product."""
         weight, eps = norm.fused_rms()
         ops.gemv_norm(h, weight, eps, self.weight, out, rows=rows)
+
+
+register_part("embedding", "table", Embedding)
+register_part("head", "linear", OutputHead)

@@ -43,7 +43,7 @@ class GatedMLP(FeedForward):
         # A few rows (decoding): one kernel applies the norm, both projections and the activation.
         rms = norm.fused_rms()
         return (rms is not None and self.group == 16 and step.act_dtype == torch.bfloat16
-                and ops.gemv_norm_supported(h, rms[0], self.w_gate_up, h.shape[0], gated=True))
+                and ops.gemv_norm_supported(h, rms[0], self.w_gate_up, h.shape[0], gated=True, choices=step.choices))
 
     def forward(self, x, step, out, accumulate, pre_norm=None):
         T = x.shape[0]
@@ -55,8 +55,8 @@ class GatedMLP(FeedForward):
         else:
             act = step.buffer("mlp.act", (T, FF), x.dtype)
             ops.gemm_gated(x, self.w_gate_up, act, self.group,
-                           lambda shape, dtype: step.buffer("mlp.gate_up", shape, dtype))
-        ops.gemm(act, self.w_down, out, accumulate, fixed_order=step.fixed_order)
+                           lambda shape, dtype: step.buffer("mlp.gate_up", shape, dtype), choices=step.choices)
+        ops.gemm(act, self.w_down, out, accumulate, fixed_order=step.fixed_order, choices=step.choices)
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

@@ -30,7 +30,15 @@ WIDE_1B = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden
                             "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}}
 WIDE_INIT = dict(seed=11, std=0.02, norm_mean=1.0, norm_std=0.05)
 
-MODELS = {"A": (TINY_A, A_INIT, 16), "B": (TINY_B, B_INIT, 16), "1b": (WIDE_1B, WIDE_INIT, 16)}
+# one layer of the 3B and of the 8B sizes: products over k of 3,072 / 8,192 and 4,096 / 14,336 at 17 to 64
+# and more rows, heads of 128 with three and four query heads to a key/value head
+WIDE_3B = dict(WIDE_1B, hidden_size=3072, intermediate_size=8192, num_attention_heads=24, head_dim=128)
+WIDE_8B = dict(WIDE_1B, hidden_size=4096, intermediate_size=14336, num_attention_heads=32, head_dim=128,
+               tie_word_embeddings=False,
+               rope_scaling=dict(WIDE_1B["rope_scaling"], factor=8.0))
+
+MODELS = {"A": (TINY_A, A_INIT, 16), "B": (TINY_B, B_INIT, 16), "1b": (WIDE_1B, WIDE_INIT, 16),
+          "3b": (WIDE_3B, dict(WIDE_INIT, seed=12), 16), "8b": (WIDE_8B, dict(WIDE_INIT, seed=13), 16)}
 
 
 def batch_schedule(requests: dict, max_live: int, portion: int = 24, seed: int = 0) -> list[dict]:
@@ -77,9 +85,11 @@ _PLAIN: dict = {}
 def plain_rows(name, cfg, tensors, reqs, rows, dtype):
     key = (name, dtype, tuple(sorted((rid, len(ids)) for rid, ids in reqs.items())))
     if key not in _PLAIN:
-        wide = {k: v.double() for k, v in tensors.items()}
+        # (against bfloat16 the plain sums need no 64 bits: half the time at the real widths)
+        arith = torch.float32 if dtype == "bf16" and cfg["hidden_size"] >= 2048 else torch.float64
+        wide = {k: v.to(arith) for k, v in tensors.items()}
         rounder = bf16_round if dtype == "bf16" else None
-        _PLAIN[key] = {rid: plain_forward(cfg, wide, ids, rounder=rounder, rows=rows[rid]).numpy()
+        _PLAIN[key] = {rid: plain_forward(cfg, wide, ids, dtype=arith, rounder=rounder, rows=rows[rid]).double().numpy()
                        for rid, ids in reqs.items()}
     return _PLAIN[key]
 
@@ -105,14 +115,20 @@ def _count_product_rows(monkeypatch):
 @pytest.mark.parametrize("graphs", [True, False], ids=["recorded", "plain"])
 @pytest.mark.parametrize("dtype", ["fp32", "bf16"])
 @pytest.mark.parametrize("name,max_live,count", [("A", 24, 40), ("B", 24, 40), ("A", 70, 100), ("B", 70, 100),
-                                                 ("1b", 24, 36), ("1b", 70, 90)])
+                                                 ("1b", 24, 36), ("1b", 70, 90), ("3b", 24, 30), ("3b", 70, 80),
+                                                 ("8b", 24, 30), ("8b", 70, 80)])
 def test_many_live_requests_match_plain(zoo, name, max_live, count, dtype, graphs, monkeypatch):
     from llmengine import Engine
+    if name in ("3b", "8b") and not graphs:
+        pytest.skip("the larger widths run with recorded decode steps only (the plain implementation's time)")
     cfg, tensors, page = zoo[name]
-    reqs = _requests(cfg, count, 62, 100, seed=max_live)            # 40 and more decoded tokens each
+    if name in ("3b", "8b"):                                        # (the same requests under both numbers of live ones)
+        reqs = dict(list(_requests(cfg, 80, 62, 76, seed=5).items())[:count])
+    else:
+        reqs = _requests(cfg, count, 62, 100, seed=max_live)        # 40 and more decoded tokens each
     steps = batch_schedule(reqs, max_live, seed=max_live)
-    # all rows of the tiny models; of the wide one the first two, the prompt's last and every decoded one
-    if name == "1b":
+    # all rows of the tiny models; of the wide ones the first two, the prompt's last and every decoded one
+    if cfg["hidden_size"] >= 2048:
         rows = {rid: sorted({0, 1} | set(range(max(2, len(ids) // 3) - 1, len(ids)))) for rid, ids in reqs.items()}
         steps = replay.want_only(steps, rows)
     else:
@@ -125,7 +141,7 @@ def test_many_live_requests_match_plain(zoo, name, max_live, count, dtype, graph
     got = replay.run_trace(engine, cache, steps)
     sizes = [sum(len(e["tokens"]) for e in st["entries"]) for st in steps]
     decode_steps = [len(st["entries"]) for st in steps if all(len(e["tokens"]) == 1 for e in st["entries"])]
-    assert max(decode_steps) == max_live and len([s for s in decode_steps if s > 16]) >= 40
+    assert max(decode_steps) == max_live and len([s for s in decode_steps if s > 16]) >= 38
     # a portion beside more than 16 decoded tokens
     assert any(sum(len(e["tokens"]) == 1 for e in st["entries"]) > 16 and any(len(e["tokens"]) > 1 for e in st["entries"])
                for st in steps)
@@ -312,4 +328,33 @@ def test_recorded_decode_steps_between_other_steps(name, graphs):
     assert worst[0] < TOL["bf16"], f"request and position {worst[1]}: relative error {worst[0]:.3e}"
     assert all(cache.manager.free_pages(g) == cache.manager.num_pages(g) for g in cache.manager.groups)
     del engine
+    torch.cuda.empty_cache()
+
+
+# --- random configurations with many live requests ---------------------------------------------
+@pytest.mark.parametrize("case", list(range(14)) + [90])
+def test_random_configurations_with_many_live_requests(case):
+    """The random configurations of test_engine_gpu (head sizes from 16 to 256, odd numbers of heads
+    and groups, widths in and out of the blocked layout, any page size) with 24 live requests and
+    recorded decode steps: every route that a step of 17 to 64 rows, or a portion beside two dozen
+    decoded tokens, can take at sizes that are not Llama's."""
+    from llmengine import Engine
+    from llmengine.weights import random_state
+    from test_engine_gpu import _random_configuration
+    cfg, page, _ = _random_configuration(case)
+    tensors = dict(random_state(cfg, case, torch.bfloat16, 0.08, 1.0, 0.1))
+    wide = {k: v.double() for k, v in tensors.items()}
+    reqs = _requests(cfg, 34, 30, 64, seed=case)
+    steps = batch_schedule(reqs, 24, portion=80, seed=case)
+    for dtype, rounder in (("fp32", None), ("bf16", bf16_round)):
+        plain = {rid: plain_forward(cfg, wide, ids, rounder=rounder).numpy() for rid, ids in reqs.items()}
+        engine = Engine(None, dtype, _config=cfg, _tensors=dict(tensors), block_size=page)
+        cache = engine.new_cache(replay.trace_peak_tokens(steps, round_to=page) // page, page, max_requests=24)
+        got = replay.run_trace(engine, cache, steps)
+        assert engine.runner.graph_replays > 10
+        worst = max((np.abs(got[rid][pos].astype(np.float64) - plain[rid][pos]).max() / np.abs(plain[rid][pos]).max(),
+                     rid, pos) for rid, ids in reqs.items() for pos in range(len(ids)))
+        assert worst[0] < TOL[dtype], f"{cfg} page {page} {dtype}: request {worst[1]} position {worst[2]}: {worst[0]:.3e}"
+        assert all(cache.manager.free_pages(g) == cache.manager.num_pages(g) for g in cache.manager.groups)
+        del engine
     torch.cuda.empty_cache()

@@ -292,6 +292,54 @@ def test_threads_get_the_serial_answers(dir_a):
     assert got == serial
 
 
+def test_schedulers_beside_generate_on_one_engine(dir_b):
+    """Two schedulers (each with a block manager of its own) step while two other threads call
+    generate on the same engine, as in the reference's tests/test_engine_thread_safety.py:65-125:
+    the runner's scratch memory, its recorded decode steps and the stream are shared, and every
+    stream of tokens must be the serial one (32-bit: no near ties between the batched and the
+    single steps)."""
+    from llmengine import BlockManager, ContinuousBatchScheduler, Engine
+    engine = Engine(dir_b, "fp32", block_size=8)
+    assert engine.runner.use_graphs
+    prompts = [random_tokens(5 + 4 * i, 384, 950 + i) for i in range(4)]
+    serial = [engine.generate(p, 9) for p in prompts]
+    errors, from_sched, from_gen = [], [None, None], [None, None]
+
+    def run_sched(k):
+        try:
+            sched = ContinuousBatchScheduler(engine, BlockManager(24, 8), max_concurrent=3, max_prefill_tokens_per_step=6)
+            for p in prompts:
+                sched.enqueue(p, 9)
+            sched.run_until_idle()
+            from_sched[k] = [(r.token_ids, r.finish_reason) for r in sched.results]
+        except Exception as e:          # noqa: BLE001
+            errors.append(e)
+
+    def run_gen(k):
+        try:
+            from_gen[k] = [engine.generate(p, 9) for _ in range(2) for p in prompts]
+        except Exception as e:          # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=run_sched, args=(k,)) for k in range(2)]
+    threads += [threading.Thread(target=run_gen, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert from_sched[0] == serial and from_sched[1] == serial
+    assert from_gen[0] == serial + serial and from_gen[1] == serial + serial
+
+
+def test_a_head_size_beyond_the_kernels_is_refused_when_the_model_is_built():
+    from llmengine import Engine
+    cfg = dict(TINY_A, head_dim=512, hidden_size=64)
+    engine = Engine(None, "fp32", _config=cfg, _tensors={})
+    with pytest.raises(ValueError, match=r"self_attn: head_dim=512.*up to 256"):
+        engine.runner
+
+
 def test_command_line(dir_a, tmp_path):
     from llmengine import Engine
     prompt = [5, 17, 3, 99]

@@ -410,7 +410,7 @@ def test_attention_mfma_decode_splits(ops, monkeypatch):
     out, ref, plan = _attn_case(ops, [1500, 40], [1, 1], 8, 2, 64, 16)
     assert plan["nsplit"] > 4
     assert _rel(out, ref) < 8e-3
-    monkeypatch.setattr(ops.mfma, "DECODE_BLOCKS_WANTED", 1)
+    monkeypatch.setattr(ops.policy, "decode_blocks_wanted", 1)     # (the choices of calls without a step)
     out1, ref1, plan1 = _attn_case(ops, [1500, 40], [1, 1], 8, 2, 64, 16)
     assert plan1["nsplit"] == 1 and _rel(out1, ref1) < 8e-3
 

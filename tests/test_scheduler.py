@@ -234,3 +234,48 @@ def test_one_scheduler_per_block_manager():
     second.enqueue([4, 5], 3)
     second.run_until_idle()
     assert second.results[0].token_ids[:2] == [4, 5]
+
+
+def test_a_step_that_fails_after_it_ran_ends_its_sequences():
+    """The batch runs and the cache holds its tokens, but the choice of the next tokens fails: the
+    sequences of that batch cannot go on (offering the same tokens again would cache them twice).
+    Each ends with "error" and the tokens it had, its pages go back, and requests that were not in
+    the batch are served as if nothing had happened."""
+    from llmengine import StepCommittedError
+    prompts = [[1, 2, 3], list(range(20, 50)), list(range(5, 25)), [9], [4, 4, 4, 4]]
+
+    class FailsBehind(FakeEngine):
+        def __init__(self, fail_at):
+            super().__init__()
+            self.fail_at, self.calls, self.lost = fail_at, 0, []
+
+        def run_step(self, cache, entries, draws, temperature, seed):
+            out = super().run_step(cache, entries, draws, temperature, seed)
+            self.calls += 1
+            if self.calls == self.fail_at:
+                self.lost = [e.request_id for e in entries]
+                raise StepCommittedError("the tokens were not chosen")
+            return out
+
+    for fail_at in (1, 2, 4, 6):
+        eng, bm = FailsBehind(fail_at), FakeBlocks(64, 4)
+        s = ContinuousBatchScheduler(eng, bm, max_concurrent=3, max_prefill_tokens_per_step=8)
+        for p in prompts:
+            s.enqueue(p, 7)
+        failures = 0
+        while True:
+            try:
+                if not s.step():
+                    break
+            except StepCommittedError:
+                failures += 1
+        assert failures == 1 and eng.lost
+        for r, p in zip(s.results, prompts):
+            whole = single_generate(p, 7)
+            if r.seq_id in eng.lost:
+                assert r.finish_reason == "error"
+                assert r.token_ids == whole[0][:len(r.token_ids)] and len(r.token_ids) >= len(p)
+            else:
+                assert (r.token_ids, r.finish_reason) == whole, (fail_at, r.seq_id)
+        assert bm.free_blocks == bm.num_blocks and s.idle
+        bm.cache.manager.check()
