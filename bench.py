@@ -202,8 +202,13 @@ def mixed(args, engine, cfg: dict, gen, page: int) -> int:
     torch.cuda.synchronize()
     launched = (time.perf_counter() - t) / steps * 1e3
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
-        forward()
+    import gc
+    gc.disable()                            # (a collection must not free device memory while launches are recorded)
+    try:
+        with torch.cuda.graph(graph):
+            forward()
+    finally:
+        gc.enable()
     graph.replay()
     torch.cuda.synchronize()
     t = time.perf_counter()

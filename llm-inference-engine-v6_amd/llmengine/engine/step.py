@@ -11,6 +11,7 @@ the request's pages, and returns 32-bit logits at the wanted places.
 from __future__ import annotations
 
 import ctypes
+import gc
 
 from dataclasses import dataclass, field
 from typing import Sequence
@@ -388,19 +389,28 @@ class ModelRunner:
             # Scratch buffers that the step is the first to ask for are made while it is recorded and
             # belong to the recording's own memory pool, which later steps of other kinds must not be
             # handed: they are made again outside, and the step is recorded once more with those.
-            for attempt in range(3):
-                ctx.extra.clear()                       # (notes of the pass before: launch plans, what was left cleared)
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph):
-                    logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
-                    if greedy:
-                        ops.argmax_into(logits, tok_host.data_ptr(), scratch, also_ptr=meta.data_ptr(),
-                                        slot_ptr=meta.data_ptr() + 4 * total)
-                if not self.workspace.made_while_recording():
-                    break
-                del graph, logits
-            else:
-                raise RuntimeError("a decode step asks for new scratch buffers every time it is recorded")
+            # No garbage collection while launches are recorded: a collection that finds an engine nobody
+            # holds any more destroys its recordings and frees their memory, which the runtime refuses
+            # while a stream is being recorded (the process then ends in the destructor's error).
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                for attempt in range(3):
+                    ctx.extra.clear()                   # (notes of the pass before: launch plans, what was left cleared)
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
+                        if greedy:
+                            ops.argmax_into(logits, tok_host.data_ptr(), scratch, also_ptr=meta.data_ptr(),
+                                            slot_ptr=meta.data_ptr() + 4 * total)
+                    if not self.workspace.made_while_recording():
+                        break
+                    del graph, logits
+                else:
+                    raise RuntimeError("a decode step asks for new scratch buffers every time it is recorded")
+            finally:
+                if collecting:
+                    gc.enable()
             cache.graphs[key] = rec = _DecodeRecord(graph, logits, meta, S, width, list(mgr.groups), tok_host)
             rec.scratch = scratch                       # (kept alive: the graph holds its addresses)
         return rec
