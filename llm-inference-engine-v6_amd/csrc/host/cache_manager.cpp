@@ -405,4 +405,54 @@ int llme_cm_fill_decode(void* h, int S, const int64_t* keys, int width, int* len
     return 0;
 }
 
+// Tokens cached for each of S live requests. Returns 0 or an error code.
+int llme_cm_lengths(void* h, int S, const int64_t* keys, long* out) {
+    auto* m = static_cast<CacheManager*>(h);
+    for (int i = 0; i < S; ++i) {
+        auto* r = m->find(keys[i]);
+        if (!r) return LLME_HOST_NOT_LIVE;
+        out[i] = r->length;
+    }
+    return 0;
+}
+
+// The integer arrays of a step of any kind, for S requests that bring new_lens[i] tokens each: the
+// tokens' positions and request indices (T = sum of new_lens values each), the first row of every
+// request (S + 1), the tokens cached before the step (S), the slots (S), and for every group the rows
+// of the block table, `width` entries each (entries behind a request's last page are 0; pages of a
+// window group that were given back stay -1: no token of the step reads them). The arrays are
+// written in the caller's one buffer at the given places. Returns the highest position of the
+// step, or an error code (negative).
+long llme_cm_fill_step(void* h, int S, const int64_t* keys, const int* new_lens, int width, int* positions,
+                       int* seq_idx, int* q_start, int* ctx_len, int* slots, int* tables) {
+    auto* m = static_cast<CacheManager*>(h);
+    const int G = m->num_groups();
+    long row = 0, top = -1;
+    for (int i = 0; i < S; ++i) {
+        auto* r = m->find(keys[i]);
+        if (!r) return LLME_HOST_NOT_LIVE;
+        const int n = new_lens[i];
+        if (n <= 0) return LLME_HOST_BAD_ARGUMENT;
+        const long c = r->length;
+        q_start[i] = static_cast<int>(row);
+        ctx_len[i] = static_cast<int>(c);
+        slots[i] = r->slot;
+        for (int t = 0; t < n; ++t) {
+            positions[row + t] = static_cast<int>(c + t);
+            seq_idx[row + t] = i;
+        }
+        row += n;
+        top = std::max(top, c + n - 1);
+        for (int g = 0; g < G; ++g) {
+            const std::vector<int>& t = r->tables[static_cast<size_t>(g)];
+            const int nb = static_cast<int>(std::min<size_t>(t.size(), static_cast<size_t>(width)));
+            int* out = tables + (static_cast<size_t>(g) * S + i) * width;
+            for (int b = 0; b < nb; ++b) out[b] = t[static_cast<size_t>(b)];
+            for (int b = nb; b < width; ++b) out[b] = 0;
+        }
+    }
+    q_start[S] = static_cast<int>(row);
+    return top;
+}
+
 }  // extern "C"

@@ -40,6 +40,60 @@ class StepEntry:
     want: Sequence[int] = ()        # places among `tokens` whose logits are wanted
 
 
+def step_layout(mgr: CacheManager, entries: Sequence[StepEntry], page: int, max_blocks: int | None = None):
+    """Where a step's integer arrays lie in its one buffer: tokens, positions, request index per
+    token, first row of every request (S + 1), tokens cached before the step, slots, one block
+    table per group (rows of max_blocks entries; by default as many as the longest request needs),
+    the wanted rows. Returns (new_lens, ctx_lens, max_blocks, offsets, sizes, total, T, R, keys,
+    wanted)."""
+    S = len(entries)
+    new_lens = [len(e.tokens) for e in entries]
+    keys = (ctypes.c_int64 * S)(*[mgr.key_of(e.request_id) for e in entries])
+    lengths = (ctypes.c_long * S)()
+    if mgr._lib.llme_cm_lengths(mgr.handle, S, keys, lengths) != 0:
+        raise RuntimeError("a request of the step is not live")
+    ctx_lens = list(lengths)
+    T = sum(new_lens)
+    if max_blocks is None:
+        max_blocks = max(1, max((c + n + page - 1) // page for c, n in zip(ctx_lens, new_lens)))
+    wanted: list[int] = []
+    row = 0
+    for e, n in zip(entries, new_lens):
+        if e.want:
+            wanted += [row + int(w) for w in e.want]
+        row += n
+    R = len(wanted)
+    sizes = [T, T, T, S + 1, S, S] + [S * max_blocks] * len(mgr.groups) + [R]
+    offsets = [0]
+    for s in sizes:
+        offsets.append(offsets[-1] + s)
+    return new_lens, ctx_lens, max_blocks, offsets, sizes, offsets[-1], T, R, keys, wanted
+
+
+def fill_step_arrays(mgr: CacheManager, entries: Sequence[StepEntry], layout, h) -> tuple[list[int], int]:
+    """Writes the arrays of `step_layout` into the int32 numpy buffer h: the tokens and the wanted
+    rows here, everything that the cache manager knows (positions, request indices, first rows,
+    lengths, slots and the block tables' rows) by the manager in one call. Returns the requests'
+    slots and the step's highest position."""
+    new_lens, _, max_blocks, offsets, _, total, _, R, keys, wanted = layout
+    if h.shape[0] < total:
+        raise RuntimeError("the buffer for the step's integer arrays is too small")
+    S = len(entries)
+    pos = offsets[0]
+    for e, n in zip(entries, new_lens):
+        h[pos:pos + n] = e.tokens
+        pos += n
+    base = h.ctypes.data
+    top = mgr._lib.llme_cm_fill_step(mgr.handle, S, keys, (ctypes.c_int * S)(*new_lens), max_blocks,
+                                     base + 4 * offsets[1], base + 4 * offsets[2], base + 4 * offsets[3],
+                                     base + 4 * offsets[4], base + 4 * offsets[5], base + 4 * offsets[6])
+    if top < 0:
+        raise RuntimeError(f"the cache manager could not describe the step (code {top})")
+    if R:
+        h[offsets[-2]:offsets[-1]] = wanted
+    return h[offsets[5]:offsets[6]].tolist(), int(top)
+
+
 class Workspace:
     """Scratch buffers by name, grown on demand and kept, so that steps of the same
     size reuse the same device addresses."""
@@ -306,9 +360,9 @@ class ModelRunner:
             if e.request_id in seen:
                 raise ValueError(f"request {e.request_id!r} appears twice in one step")
             seen.add(e.request_id)
-            for t in e.tokens:
-                if not 0 <= int(t) < vocab:
-                    raise ValueError(f"token id {t} out of range [0, {vocab})")
+            if min(e.tokens) < 0 or max(e.tokens) >= vocab:         # (the passing case without a loop in Python)
+                bad = next(t for t in e.tokens if not 0 <= int(t) < vocab)
+                raise ValueError(f"token id {bad} out of range [0, {vocab})")
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):
                     raise ValueError(f"request {e.request_id!r}: wanted place {w} is not among "
@@ -508,55 +562,12 @@ class ModelRunner:
     def _build_context(self, cache: CacheContext, entries: Sequence[StepEntry], max_blocks: int | None = None,
                        plan_len: int | None = None, dev: torch.Tensor | None = None):
         mgr = cache.manager
-        page = cache.page_size
         S = len(entries)
-        new_lens = [len(e.tokens) for e in entries]
-        ctx_lens = [mgr.length(e.request_id) for e in entries]
-        T = sum(new_lens)
         groups = list(mgr.groups)
-        if max_blocks is None:
-            max_blocks = max(1, max((c + n + page - 1) // page for c, n in zip(ctx_lens, new_lens)))
-        wanted: list[int] = []
-        row = 0
-        for e, n in zip(entries, new_lens):
-            wanted += [row + int(w) for w in e.want]
-            row += n
-        R = len(wanted)
-
-        # layout of the one integer buffer: tokens, positions, seq_idx, q_start, ctx_len, slots,
-        # one block table per group, logit rows
-        sizes = [T, T, T, S + 1, S, S] + [S * max_blocks] * len(groups) + [R]
-        offsets = [0]
-        for s in sizes:
-            offsets.append(offsets[-1] + s)
-        total = offsets[-1]
+        layout = step_layout(mgr, entries, cache.page_size, max_blocks)
+        new_lens, ctx_lens, max_blocks, offsets, sizes, total, T, R = layout[:8]
         host, idx = self._staging.take(total)
-        h = host.numpy()
-        pos = 0
-        tok_o, pos_o, seq_o, qs_o, ctx_o, slot_o = offsets[:6]
-        slot_list = []
-        for i, (e, n, c) in enumerate(zip(entries, new_lens, ctx_lens)):
-            h[tok_o + pos:tok_o + pos + n] = e.tokens
-            h[pos_o + pos:pos_o + pos + n] = range(c, c + n)
-            h[seq_o + pos:seq_o + pos + n] = i
-            h[qs_o + i] = pos
-            h[ctx_o + i] = c
-            slot = mgr.slot(e.request_id)
-            h[slot_o + i] = slot
-            slot_list.append(slot)
-            pos += n
-        h[qs_o + S] = T
-        for gi, g in enumerate(groups):
-            base = offsets[6 + gi]
-            for i, e in enumerate(entries):
-                table = mgr.block_table(e.request_id, g)
-                row_base = base + i * max_blocks
-                nb = min(len(table), max_blocks)
-                # pages given back (-1) are never read: every key a token may see has a page
-                h[row_base:row_base + nb] = table[:nb]
-                h[row_base + nb:row_base + max_blocks] = 0
-        if R:
-            h[offsets[-2]:offsets[-1]] = wanted
+        slot_list, top = fill_step_arrays(mgr, entries, layout, host.numpy())
 
         if dev is None:
             if self._meta_dev is None or self._meta_dev.numel() < total:
@@ -576,7 +587,7 @@ class ModelRunner:
             ctx_len=view(4), slots=view(5),
             block_tables={g: view(6 + gi, (S, max_blocks)) for gi, g in enumerate(groups)},
             act_dtype=self.dtype, workspace=self.workspace, new_lens=new_lens, ctx_lens=ctx_lens,
-            slot_list=slot_list, max_position=max(c + n for c, n in zip(ctx_lens, new_lens)) - 1,
+            slot_list=slot_list, max_position=top,
             plan_len=plan_len, fixed_order=self.deterministic, choices=self.choices)
         logit_rows = view(len(sizes) - 1) if R else None
         return ctx, logit_rows

@@ -130,6 +130,8 @@ _SIGNATURES = {
     "llme_cm_free_pages": (_i, [_vp, _i]), "llme_cm_num_pages": (_i, [_vp, _i]), "llme_cm_check": (_i, [_vp]),
     "llme_cm_decode_begin": (_i, [_vp, _i, _pi64, _pi, _l]), "llme_cm_commit_batch": (_i, [_vp, _i, _pi64, _l]),
     "llme_cm_fill_decode": (_i, [_vp, _i, _pi64, _i, _vp, _vp, _vp, _pi, _pi64]),
+    "llme_cm_lengths": (_i, [_vp, _i, _pi64, _pl]),
+    "llme_cm_fill_step": (_l, [_vp, _i, _pi64, _pi, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "llme_sched_create": (_vp, [_vp, _i, _l]), "llme_sched_destroy": (None, [_vp]),
     "llme_sched_set_budget": (_i, [_vp, _l]), "llme_sched_enqueue": (_l, [_vp, _pi, _l, _l]),
     "llme_sched_idle": (_i, [_vp]), "llme_sched_counts": (None, [_vp, _pi]),

@@ -240,3 +240,65 @@ def test_decode_begin_checks_the_position_limit_before_it_reserves():
     assert m._lib.llme_cm_commit_batch(m.handle, 3, keys, 1) == 0
     m.check()
     assert m._lib.llme_cm_decode_begin(m.handle, 3, keys, lengths, 0) == 1       # 0: no limit
+
+
+def test_a_steps_integer_arrays_are_what_the_manager_knows():
+    """The arrays a step hands to the kernels (positions, request index per token, first rows,
+    lengths, slots, block tables by group, wanted rows) as the C++ manager writes them in one call,
+    against the same arrays put together here from the manager's single answers, for random
+    batches over a full and a window group, with pages given back and used again."""
+    import random
+    import numpy as np
+    from llmengine.engine.step import StepEntry, fill_step_arrays, step_layout
+    rng = random.Random(5)
+    page = 4
+    mgr = CacheManager([GroupSpec("full", "full", 0, 1200), GroupSpec("window8", "window", 8, 200)], page, 12)
+    live = {}
+    for step_no in range(200):
+        for rid in [r for r, n in live.items() if n > 250 or rng.random() < 0.05]:
+            mgr.release(rid)
+            del live[rid]
+        while len(live) < 2 or (len(live) < 12 and rng.random() < 0.3):
+            rid = rng.choice([f"r{step_no}_{len(live)}", 1000 * step_no + len(live)])      # text and integer ids
+            mgr.admit(rid)
+            live[rid] = 0
+        chosen = rng.sample(sorted(live, key=str), rng.randint(1, len(live)))
+        entries = []
+        for rid in chosen:
+            n = rng.choice([1, 1, 1, 2, 5, 9, 23])
+            toks = [rng.randrange(50) for _ in range(n)]
+            entries.append(StepEntry(rid, toks, sorted(rng.sample(range(n), rng.randint(0, min(n, 3))))))
+        assert mgr.reserve_batch([(e.request_id, len(e.tokens)) for e in entries])
+        for width in (None, 40):
+            layout = step_layout(mgr, entries, page, width)
+            new_lens, ctx_lens, max_blocks, offsets, sizes, total, T, R = layout[:8]
+            h = np.full(total + 5, -9, dtype=np.int32)
+            slots, top = fill_step_arrays(mgr, entries, layout, h)
+            assert (h[total:] == -9).all()
+            # the same from single answers
+            want = np.zeros(total, dtype=np.int32)
+            pos, r0 = 0, 0
+            for i, e in enumerate(entries):
+                n, c = len(e.tokens), mgr.length(e.request_id)
+                want[offsets[0] + pos:offsets[0] + pos + n] = e.tokens
+                want[offsets[1] + pos:offsets[1] + pos + n] = range(c, c + n)
+                want[offsets[2] + pos:offsets[2] + pos + n] = i
+                want[offsets[3] + i] = pos
+                want[offsets[4] + i] = c
+                want[offsets[5] + i] = mgr.slot(e.request_id)
+                for gi, g in enumerate(mgr.groups):
+                    table = mgr.block_table(e.request_id, g)[:max_blocks]
+                    at = offsets[6 + gi] + i * max_blocks
+                    want[at:at + len(table)] = table
+                want[offsets[-2] + r0:offsets[-2] + r0 + len(e.want)] = [pos + w for w in e.want]
+                r0 += len(e.want)
+                pos += n
+            want[offsets[3] + len(entries)] = pos
+            assert np.array_equal(h[:total], want), (step_no, width)
+            assert ctx_lens == [mgr.length(e.request_id) for e in entries]
+            assert slots == [mgr.slot(e.request_id) for e in entries]
+            assert top == max(c + n for c, n in zip(ctx_lens, new_lens)) - 1 and T == pos and R == r0
+        for e in entries:
+            mgr.commit(e.request_id, len(e.tokens))
+            live[e.request_id] += len(e.tokens)
+        mgr.check()
