@@ -110,7 +110,8 @@ def serve(args, engine, cfg: dict, gen, page: int) -> int:
     manager = BlockManager(pages, page)                        # one pool for both runs: the second finds the decode
     for rep in range(2):                                       # steps' HIP graphs that the first recorded over it
         sched = ContinuousBatchScheduler(engine, manager, max_concurrent=args.max_concurrent,
-                                         max_prefill_tokens_per_step=args.prefill_budget)
+                                         max_prefill_tokens_per_step=args.prefill_budget,
+                                         temperature=args.temperature, seed=args.seed)
         for p, n in zip(prompts, news):
             sched.enqueue(p, n)
         torch.cuda.synchronize()
@@ -135,7 +136,7 @@ def serve(args, engine, cfg: dict, gen, page: int) -> int:
         "config": {"model": args.shape, "layers": cfg["num_hidden_layers"], "requests": args.requests,
                    "prompt_range": args.prompt_range, "new_range": args.new_range, "prompt_tokens": prompt_tokens,
                    "generated_tokens": generated, "prefill_budget": args.prefill_budget,
-                   "max_concurrent": args.max_concurrent, "page_size": page},
+                   "max_concurrent": args.max_concurrent, "page_size": page, "temperature": args.temperature},
     }), flush=True)
     return 0
 
@@ -250,6 +251,7 @@ def main() -> int:
     ap.add_argument("--new-range", default="128,512", help="serve: new tokens per request, uniform in [a, b]")
     ap.add_argument("--prefill-budget", type=int, default=2048, help="serve: max_prefill_tokens_per_step")
     ap.add_argument("--max-concurrent", type=int, default=32, help="serve: live requests at a time")
+    ap.add_argument("--temperature", type=float, default=0.0, help="serve: sampling temperature (0 is greedy)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")

@@ -141,17 +141,22 @@ __global__ __launch_bounds__(kSampleThreads) void sample_pick_kernel(const float
                                                                      const int* __restrict__ part_idx,
                                                                      const float* __restrict__ part_sum,
                                                                      int* __restrict__ out, int V, int chunk,
-                                                                     int parts) {
+                                                                     int parts, int* __restrict__ also = nullptr,
+                                                                     const int* __restrict__ slot = nullptr) {
     __shared__ float wave_total[kSampleThreads / kWave];
     __shared__ int pick;
     const int r = blockIdx.x;
     const float temp = temperature[r];
+    // (the choice goes to out[slot R + row] and, where given, to also[row], as in argmax_join_kernel)
+    const int out_at = (slot ? *slot * static_cast<int>(gridDim.x) : 0) + r;
     if (!(temp > 0.f)) {
         if (threadIdx.x == 0) {
             float bv = -INFINITY;
             int bi = 0x7fffffff;
             for (int p = 0; p < parts; ++p) argmax_combine(bv, bi, part_val[r * parts + p], part_idx[r * parts + p]);
-            out[r] = (bi == 0x7fffffff) ? 0 : bi;
+            const int token = (bi == 0x7fffffff) ? 0 : bi;
+            out[out_at] = token;
+            if (also) also[r] = token;
         }
         return;
     }
@@ -198,7 +203,11 @@ __global__ __launch_bounds__(kSampleThreads) void sample_pick_kernel(const float
     }
     __syncthreads();
     // Rounding left the target beyond the last cumulative sum: the last id of the part.
-    if (threadIdx.x == 0) out[r] = (pick == 0x7fffffff) ? end - 1 : pick;
+    if (threadIdx.x == 0) {
+        const int token = (pick == 0x7fffffff) ? end - 1 : pick;
+        out[out_at] = token;
+        if (also) also[r] = token;
+    }
 }
 
 }  // namespace llme
@@ -251,7 +260,26 @@ extern "C" int llme_sample(const float* logits, const float* temperature, const 
     hipLaunchKernelGGL(sample_sum_kernel, dim3(R, parts), dim3(kSampleThreads), 0, stream, logits, temperature,
                        part_val, part_sum, V, chunk);
     hipLaunchKernelGGL(sample_pick_kernel, dim3(R), dim3(kSampleThreads), 0, stream, logits, temperature, uniform,
-                       part_val, part_idx, part_sum, out, V, chunk, parts);
+                       part_val, part_idx, part_sum, out, V, chunk, parts, static_cast<int*>(nullptr),
+                       static_cast<const int*>(nullptr));
+    return launch_status();
+}
+
+// The same with the choice left in two places, as llme_argmax_to leaves it: out[*slot * R + row] (out holds
+// 2 R ints; slot may be null: then out[row]) and also[row] (may be null).
+extern "C" int llme_sample_to(const float* logits, const float* temperature, const float* uniform, int* out,
+                              int* also, const int* slot, float* part_val, int* part_idx, float* part_sum, int R,
+                              int V, hipStream_t stream) {
+    if (R <= 0) return 0;
+    if (V <= 0 || !out || !temperature || !uniform) return kErrBadArgument;
+    const int parts = llme_argmax_parts(V);
+    const int chunk = (V + parts - 1) / parts;
+    hipLaunchKernelGGL(argmax_part_kernel, dim3(R, parts), dim3(kSampleThreads), 0, stream, logits, part_val,
+                       part_idx, V, chunk);
+    hipLaunchKernelGGL(sample_sum_kernel, dim3(R, parts), dim3(kSampleThreads), 0, stream, logits, temperature,
+                       part_val, part_sum, V, chunk);
+    hipLaunchKernelGGL(sample_pick_kernel, dim3(R), dim3(kSampleThreads), 0, stream, logits, temperature, uniform,
+                       part_val, part_idx, part_sum, out, V, chunk, parts, also, slot);
     return launch_status();
 }
 

@@ -21,7 +21,7 @@ import torch
 from ..config.base import read_model_json
 from ..config.registry import architecture_name, parse_config, resolve
 from ..parts.base import Placement
-from ..sampling import Sampler
+from ..sampling import Sampler, uniform_draw
 from ..weights import TensorIndex, load_model_weights, load_state_dict, random_state
 from .step import CacheContext, CapacityError, ModelRunner, StepCommittedError, StepEntry
 
@@ -212,10 +212,14 @@ class Engine:
         before the step is committed to the cache raises what it is and has changed nothing; one
         behind that raises StepCommittedError."""
         with self._lock, torch.cuda.device(self.runner.device):
-            if temperature == 0.0:
-                tokens = self.runner.step_greedy(cache, entries, max_position=self.max_pos)
-                if tokens is not None:
-                    return tokens
+            # a step of single decoded tokens is one recorded launch that ends in the choice of the tokens
+            uniforms = None
+            if temperature > 0.0 and self.runner.use_graphs and len(draws) == len(entries):
+                uniforms = [uniform_draw(seed, r, i) for r, i in draws]
+            tokens = self.runner.step_greedy(cache, entries, max_position=self.max_pos, temperature=temperature,
+                                             uniforms=uniforms)
+            if tokens is not None:
+                return tokens
             logits = self.runner.step(cache, entries, max_position=self.max_pos)
             if logits is None:
                 return []
@@ -333,17 +337,22 @@ class Engine:
                 finish = "length"
                 generated = 0
                 runner = self.runner
-                greedy = self.sampler.temperature == 0.0 and runner.use_graphs
+                recorded = runner.use_graphs      # decode steps are recorded launches that end in the choice
+                temperature, seed = self.sampler.temperature, self.sampler.seed
+
+                def draw(index: int):
+                    return [uniform_draw(seed, 0, index)] if temperature > 0.0 else None
                 pending = None
                 while generated < max_new_tokens:
                     if pending is None:
                         nxt = self.sampler.choose(logits, [(0, generated)])[0]
                     else:
-                        # greedy: the step behind this one is launched on the token the device holds
-                        # before the host has fetched it (one step more than needed if this one stops)
+                        # the step behind this one is launched on the token the device holds before the
+                        # host has fetched it (one step more than needed if this one stops)
                         more = generated + 1 < max_new_tokens     # the token being fetched is not the last wanted
                         with torch.cuda.device(runner.device):
-                            ahead = runner.greedy_launch(cache, [rid], None, self.max_pos) if more else None
+                            ahead = runner.greedy_launch(cache, [rid], None, self.max_pos, temperature,
+                                                         draw(generated + 1)) if more else None
                             nxt = runner.greedy_result(pending)[0]
                     if nxt in eos:
                         finish = "stop"
@@ -354,12 +363,13 @@ class Engine:
                     generated += 1
                     if generated >= max_new_tokens:
                         break
-                    if greedy:
+                    if recorded:
                         with torch.cuda.device(runner.device):
                             if pending is not None and ahead is not None:
                                 pending = ahead
                             else:
-                                pending = runner.greedy_launch(cache, [rid], [nxt], self.max_pos)
+                                pending = runner.greedy_launch(cache, [rid], [nxt], self.max_pos, temperature,
+                                                               draw(generated))
                     else:
                         logits = self.step(cache, [StepEntry(rid, [nxt], [0])])
                 return out, finish

@@ -244,8 +244,11 @@ class _DecodeRecord:
     everything when other requests take part."""
 
     def __init__(self, graph, logits, meta: torch.Tensor, S: int, width: int, groups: list[str],
-                 tok_host: torch.Tensor | None = None):
+                 tok_host: torch.Tensor | None = None, draws: bool = False):
         self.graph, self.logits, self.meta = graph, logits, meta
+        # a recording that samples reads a temperature and a uniform draw per request from behind the
+        # integer arrays (2 S floats that the host sends up with them)
+        self.draws = 2 * S if draws else 0
         # pinned, 2 S: where a greedy recording leaves the chosen tokens, in its two halves in turn (the
         # half is named by the integer behind the arrays), so that a step can be launched before the
         # tokens of the one before it have been read; the same tokens also land in the token array
@@ -260,8 +263,9 @@ class _DecodeRecord:
         for n in sizes:
             self.offsets.append(self.offsets[-1] + n)
         self.total = self.offsets[-1]
-        self.host = torch.zeros(self.total + 1, dtype=torch.int32, pin_memory=True)   # (+ the half's number)
+        self.host = torch.zeros(self.total + 1 + self.draws, dtype=torch.int32, pin_memory=True)   # (+ the half's number, the draws)
         self.np = h = self.host.numpy()
+        self.np_draws = self.host.view(torch.float32).numpy()[self.total + 1:]
         o, G = self.offsets, len(groups)
         h[o[2]:o[3]] = range(S)                 # request index of each token
         h[o[3]:o[4]] = range(S + 1)             # first row of each request
@@ -274,9 +278,11 @@ class _DecodeRecord:
         self.scratch = None
 
     def refresh(self, mgr: CacheManager, entries: Sequence[StepEntry] | None, keys=None, slot: int = 0,
-                tokens: Sequence[int] | None = None) -> None:
+                tokens: Sequence[int] | None = None, temperature: float = 0.0,
+                uniforms: Sequence[float] | None = None) -> None:
         """The step's tokens come in `entries` or in `tokens`; with neither they are the ones the last
-        replay chose and left in the device's array. Everything else is rewritten as always."""
+        replay chose and left in the device's array. Everything else is rewritten as always.
+        temperature, uniforms: for a recording that samples, the step's temperature and draws."""
         if self.event is not None:
             self.event.synchronize()            # the last copy has read the host mirror
         S, width, o, h = self.S, self.width, self.offsets, self.np
@@ -292,6 +298,11 @@ class _DecodeRecord:
         if tokens is not None:
             h[o[0]:o[1]] = tokens
         h[self.total] = slot
+        if self.draws:
+            if uniforms is None or len(uniforms) != S:
+                raise ValueError("a recording that samples needs a draw per request")
+            self.np_draws[:S] = temperature
+            self.np_draws[S:] = uniforms
         # lengths (tokens cached before this step), slots and the block-table entries that are new,
         # straight from the C++ manager into the pinned mirror
         base = h.ctypes.data
@@ -301,7 +312,7 @@ class _DecodeRecord:
             raise RuntimeError(f"a request of the recorded step is not live (code {rc})")
         h[o[1]:o[2]] = h[o[4]:o[5]]             # the new token's position
         first = 0 if tokens is not None else o[1]
-        self.meta[first:self.total + 1].copy_(self.host[first:], non_blocking=True)
+        self.meta[first:self.total + 1 + self.draws].copy_(self.host[first:], non_blocking=True)
         if self.event is None:
             self.event = torch.cuda.Event()
         self.event.record()
@@ -393,27 +404,29 @@ class ModelRunner:
         recorded once as a HIP graph and replayed; only the integer arrays change."""
         mgr = cache.manager
         lengths = [mgr.length(e.request_id) for e in entries]
-        rec = self._decode_record(cache, entries, max(lengths), greedy=False)
+        rec = self._decode_record(cache, entries, max(lengths), choose=None)
         rec.refresh(mgr, entries)
         rec.graph.replay()
         self.graph_replays += 1
         return rec.logits
 
-    def _decode_key(self, cache: CacheContext, S: int, longest: int, greedy: bool):
+    def _decode_key(self, cache: CacheContext, S: int, longest: int, choose: str | None):
         need = (longest + cache.page_size) // cache.page_size
         bucket = self.GRAPH_BLOCK_BUCKET
         # (a recording holds the launches that the choices of its time led to)
-        return (S, (need + bucket - 1) // bucket * bucket, greedy, self.choices.key())
+        return (S, (need + bucket - 1) // bucket * bucket, choose, self.choices.key())
 
-    def _decode_record(self, cache: CacheContext, entries: Sequence[StepEntry] | None, longest: int, greedy: bool,
-                       S: int | None = None):
-        """The recording for this many requests and this width of block tables (and, greedy, with
-        the argmax behind the model and its result written into pinned host memory); made at its
-        first use (which needs the entries)."""
+    def _decode_record(self, cache: CacheContext, entries: Sequence[StepEntry] | None, longest: int,
+                       choose: str | None, S: int | None = None):
+        """The recording for this many requests and this width of block tables. choose None: it ends
+        at the logits. "greedy": the argmax is behind the model, its result written into pinned host
+        memory. "sampled": the sampling kernels instead, with a temperature and a uniform draw per
+        request that the host sends up with the integer arrays. Made at its first use (which needs
+        the entries)."""
         page = cache.page_size
         mgr = cache.manager
         S = len(entries) if S is None else S
-        key = self._decode_key(cache, S, longest, greedy)
+        key = self._decode_key(cache, S, longest, choose)
         width = key[1]
         rec = cache.graphs.pop(key, None)
         if rec is not None:
@@ -429,10 +442,13 @@ class ModelRunner:
             ops.load_kernels()                          # (no code object is loaded inside a recording)
             groups = len(mgr.groups)
             total = 7 * S + 1 + groups * S * width
-            meta = torch.zeros(total + 64, dtype=torch.int32, device=self.device)
+            meta = torch.zeros(total + 1 + 2 * S + 64, dtype=torch.int32, device=self.device)
             ctx, logit_rows = self._build_context(cache, entries, max_blocks=width, plan_len=width * page, dev=meta)
-            tok_host = scratch = None
-            if greedy:
+            tok_host = scratch = temp_dev = uni_dev = None
+            if choose == "sampled":
+                temp_dev = meta[total + 1:total + 1 + S].view(torch.float32)
+                uni_dev = meta[total + 1 + S:total + 1 + 2 * S].view(torch.float32)
+            if choose:
                 # pinned host memory is mapped into the device's address space: the kernel writes
                 # the tokens where the host reads them, without a copy of its own; the argmax's
                 # scratch belongs to the recording (the one that plain calls share may be replaced)
@@ -454,7 +470,10 @@ class ModelRunner:
                     graph = torch.cuda.CUDAGraph()
                     with torch.cuda.graph(graph):
                         logits = self.model.forward(ctx, cache.storage.layers, logit_rows)
-                        if greedy:
+                        if choose == "sampled":
+                            ops.sample_into(logits, temp_dev, uni_dev, tok_host.data_ptr(), scratch,
+                                            also_ptr=meta.data_ptr(), slot_ptr=meta.data_ptr() + 4 * total)
+                        elif choose:
                             ops.argmax_into(logits, tok_host.data_ptr(), scratch, also_ptr=meta.data_ptr(),
                                             slot_ptr=meta.data_ptr() + 4 * total)
                     if not self.workspace.made_while_recording():
@@ -465,33 +484,37 @@ class ModelRunner:
             finally:
                 if collecting:
                     gc.enable()
-            cache.graphs[key] = rec = _DecodeRecord(graph, logits, meta, S, width, list(mgr.groups), tok_host)
+            cache.graphs[key] = rec = _DecodeRecord(graph, logits, meta, S, width, list(mgr.groups), tok_host,
+                                                    draws=choose == "sampled")
             rec.scratch = scratch                       # (kept alive: the graph holds its addresses)
         return rec
 
-    def step_greedy(self, cache: CacheContext, entries: Sequence[StepEntry], max_position: int | None = None
-                    ) -> list[int] | None:
-        """The greedy next token of every entry, for a step of single decoded tokens that all want
-        one: bookkeeping in two calls into the host runtime, the argmax inside the recorded graph,
-        its result read from pinned memory. None if the step is not of that kind (then `step`
-        and a sampler do it)."""
-        if not self.use_graphs or not entries:
+    def step_greedy(self, cache: CacheContext, entries: Sequence[StepEntry], max_position: int | None = None,
+                    temperature: float = 0.0, uniforms: Sequence[float] | None = None) -> list[int] | None:
+        """The next token of every entry, greedy or (temperature > 0, a uniform draw per entry in
+        `uniforms`) sampled, for a step of single decoded tokens that all want one: bookkeeping in two
+        calls into the host runtime, the choice inside the recorded graph, its result read from pinned
+        memory. None if the step is not of that kind (then `step` and a sampler do it)."""
+        if not self.use_graphs or not entries or (temperature > 0 and uniforms is None):
             return None
         ids = []
         for e in entries:
             if len(e.tokens) != 1 or len(e.want) != 1 or e.want[0] != 0:
                 return None
             ids.append(e.request_id)
-        pending = self.greedy_launch(cache, ids, [int(e.tokens[0]) for e in entries], max_position)
+        pending = self.greedy_launch(cache, ids, [int(e.tokens[0]) for e in entries], max_position,
+                                     temperature=temperature, uniforms=uniforms)
         try:
             return self.greedy_result(pending)
         except BaseException as e:
             raise StepCommittedError(f"the step ran, but its tokens could not be fetched: {e}") from e
 
     def greedy_launch(self, cache: CacheContext, ids: Sequence, tokens: Sequence[int] | None,
-                      max_position: int | None = None) -> "PendingTokens | None":
-        """Launches a step of one token for each of the live requests `ids` whose greedy choices
-        `greedy_result` fetches later. tokens None: every request's token is the one that the launch
+                      max_position: int | None = None, temperature: float = 0.0,
+                      uniforms: Sequence[float] | None = None) -> "PendingTokens | None":
+        """Launches a step of one token for each of the live requests `ids` whose choices (greedy, or
+        sampled at `temperature` with the draws `uniforms`, one per request) `greedy_result` fetches
+        later. tokens None: every request's token is the one that the launch
         before this one chose for it, taken where that step's argmax left it on the device, so that
         this step can be launched before the host has seen those tokens (the host's work for a step,
         some 40 us, then runs beside the device's instead of in front of it). That needs the launch
@@ -502,6 +525,9 @@ class ModelRunner:
         S = len(ids)
         if len(set(ids)) != S:
             raise ValueError("a request appears twice in one step")
+        choose = "sampled" if temperature and temperature > 0 else "greedy"
+        if choose == "sampled" and (uniforms is None or len(uniforms) != S):
+            raise ValueError("sampling needs a uniform draw per request")
         if tokens is not None:
             vocab = self.model.vocab_size
             if len(tokens) != S:
@@ -518,7 +544,7 @@ class ModelRunner:
             if last is None or last[1] != list(ids):
                 return None
             longest = max(mgr.length(r) for r in ids)
-            if self._decode_key(cache, S, longest, greedy=True) != last[2] or cache.graphs.get(last[2]) is not last[0]:
+            if self._decode_key(cache, S, longest, choose) != last[2] or cache.graphs.get(last[2]) is not last[0]:
                 return None
         # lengths, the position limit and the pages in one call; a call that fails has changed nothing
         rc = mgr._lib.llme_cm_decode_begin(mgr.handle, S, keys, lengths, int(max_position or 0))
@@ -531,14 +557,13 @@ class ModelRunner:
             need = {g: sum(mgr.pages_needed(r, 1)[g] for r in ids) for g in mgr.groups}
             raise CapacityError(f"the step needs {need} more pages, free are "
                                 f"{({g: mgr.free_pages(g) for g in mgr.groups})}")
-        key = self._decode_key(cache, S, longest, greedy=True)
+        key = self._decode_key(cache, S, longest, choose)
         if key in cache.graphs or tokens is None:
-            rec = self._decode_record(cache, None, longest, greedy=True, S=S)
-        else:                                   # (a new recording runs the step once from entries)
-            rec = self._decode_record(cache, [StepEntry(r, [t], [0]) for r, t in zip(ids, tokens)], longest,
-                                      greedy=True)
+            rec = self._decode_record(cache, None, longest, choose, S=S)
+        else:                                   # (a new recording is made from entries)
+            rec = self._decode_record(cache, [StepEntry(r, [t], [0]) for r, t in zip(ids, tokens)], longest, choose)
         slot = 1 - rec.slot
-        rec.refresh(mgr, None, keys, slot=slot, tokens=tokens)
+        rec.refresh(mgr, None, keys, slot=slot, tokens=tokens, temperature=float(temperature or 0.0), uniforms=uniforms)
         rec.graph.replay()
         rec.tok_events[slot].record()
         rec.slot = slot

@@ -309,6 +309,19 @@ def argmax_into(logits: torch.Tensor, out_ptr: int, scratch=None, also_ptr: int 
         check(entry("llme_argmax")(ptr(logits), out_ptr, ptr(val), ptr(idx), R, V, stream()), "argmax")
 
 
+def sample_into(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor, out_ptr: int, scratch=None,
+                also_ptr: int = 0, slot_ptr: int = 0) -> None:
+    """sample with the result written as argmax_into writes it: to out_ptr + 4 * slot * rows (device
+    memory, or pinned host memory), and to also_ptr where given."""
+    require(logits, "logits", torch.float32, (None, None))
+    R, V = logits.shape
+    require(temperature, "temperature", torch.float32, (R,))
+    require(uniform, "uniform", torch.float32, (R,))
+    val, idx, sums = _scratch_for(logits, scratch)
+    check(entry("llme_sample_to")(ptr(logits), ptr(temperature), ptr(uniform), out_ptr, also_ptr or None, slot_ptr or None,
+                                  ptr(val), ptr(idx), ptr(sums), R, V, stream()), "sample")
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, uniform: torch.Tensor, out: torch.Tensor,
            scratch=None) -> None:
     require(logits, "logits", torch.float32, (None, None))

@@ -44,6 +44,7 @@ _SIGNATURES = {
     "llme_argmax_parts": [_i],
     "llme_compute_units": [],
     "llme_sample": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
+    "llme_sample_to": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
 }
 
 

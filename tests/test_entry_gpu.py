@@ -202,6 +202,60 @@ def test_scheduler_greedy_equals_generate(dir_a, dtype):
     assert blocks.free_blocks == 64 and [r.seq_id for r in sched.results] == list(range(len(prompts)))
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_sampled_step_with_the_choice_in_the_recording(dir_b, dtype):
+    """run_step at a temperature takes decode steps through a recording that ends in the sampling
+    kernels, the temperature and the draws sent up with the step's integer arrays: the same tokens
+    as the sampler chooses from the logits of an engine without recordings, with requests that come
+    and go, two temperatures in turn through the same recording, and a greedy step between."""
+    from llmengine import Engine, StepEntry
+    from llmengine.sampling import Sampler
+    engine, plain = Engine(dir_b, dtype), Engine(dir_b, dtype, use_graphs=False)
+    prompts = {"x": random_tokens(19, 384, 1), "y": random_tokens(8, 384, 2), 7: random_tokens(33, 384, 3)}
+    caches = [e.new_cache(12, 8, 3) for e in (engine, plain)]
+    last = {}
+    for rid, p in prompts.items():
+        for c, e in zip(caches, (engine, plain)):
+            c.admit(rid)
+            lg = e.step(c, [StepEntry(rid, p, [len(p) - 1])])
+        last[rid] = int(lg.argmax())
+    number = {"x": 0, "y": 1, 7: 2}
+    recordings = set()
+    for turn in range(14):
+        ids = list(last) if turn % 4 else list(last)[::-1]
+        entries = [StepEntry(r, [last[r]], [0]) for r in ids]
+        temperature = (0.7, 1.6, 0.0)[turn % 3]
+        draws = [(number[r], turn) for r in ids]
+        got = engine.run_step(caches[0], entries, draws, temperature, seed=11)
+        want = Sampler(temperature, 11).choose(plain.step(caches[1], entries), draws)
+        assert got == want, (turn, temperature)
+        last = dict(zip(ids, got))
+        recordings |= {k[:3] for k in caches[0].graphs}
+        if turn == 6:
+            for c in caches:
+                c.release("y")
+            del last["y"]
+    assert engine.runner.graph_replays >= 14 and plain.runner.graph_replays == 0
+    # one recording for each number of requests and kind of choice, whatever the temperature
+    assert sorted(k[2] for k in recordings) == ["greedy", "greedy", "sampled", "sampled"]
+
+
+def test_generate_at_a_temperature_is_the_same_with_and_without_recordings(dir_a, dir_b):
+    """generate() launches each sampled step before it has fetched the token of the step before;
+    the stream is the one an engine without recordings samples, and the one the plain logits allow."""
+    from types import SimpleNamespace
+    from llmengine import Engine
+    for folder, vocab in ((dir_a, 256), (dir_b, 384)):
+        cfg, w = load_plain_model(folder)
+        for seed in (3, 4):
+            kw = dict(temperature=0.9, sampler_seed=seed)
+            prompt = random_tokens(11 + seed, vocab, seed)
+            with_rec, finish = Engine(folder, "fp32", **kw).generate(prompt, 20)
+            without, _ = Engine(folder, "fp32", use_graphs=False, **kw).generate(prompt, 20)
+            assert with_rec == without and len(with_rec) > len(prompt)
+            _check_sampled(cfg, w, SimpleNamespace(token_ids=with_rec, prompt_len=len(prompt), seq_id=0), 0.9, seed, 1e-4)
+
+
 def test_greedy_step_with_the_argmax_in_the_recording(dir_b):
     """run_step at temperature 0 takes decode steps through a recording that ends in the argmax:
     same tokens as the logits' own argmax, a clear error when the pages run out, and requests
