@@ -739,11 +739,13 @@ def test_attention_mfma_finds_one_far_key(ops):
 
 # --- projections fused with the norm in front of them -----------------------------------
 @pytest.mark.parametrize("M,N,K", [(1, 48, 64), (8, 3072, 2048), (16, 100, 96), (5, 331, 144), (3, 128256, 2048),
-                                   (7, 64, 4096)])
+                                   (7, 64, 4096), (8, 5120, 3072), (9, 5120, 3072), (6, 6144, 4096)])
 @pytest.mark.parametrize("wdtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("tpr,grid", [(0, 0), (1, 0), (2, 3), (4, 0), (4, 5)])
 def test_gemv_norm(ops, M, N, K, wdtype, tpr, grid):
     if N > 10000 and (tpr, grid) not in ((0, 0), (4, 0)):
+        pytest.skip("large case twice")
+    if N > 4000 and K > 2048 and (tpr, grid) not in ((0, 0), (2, 3)):
         pytest.skip("large case twice")
     h = 2 * torch.randn(M + 3, K, generator=_gen(60))
     nw = (1 + 0.1 * torch.randn(K, generator=_gen(61))).to(wdtype)
@@ -829,7 +831,9 @@ def test_gemv_norm_refusals(ops):
 
 @pytest.mark.parametrize("M,n_q,n_kv,hd,K,page", [(1, 4, 2, 32, 64, 16), (8, 32, 8, 64, 2048, 16), (16, 3, 1, 96, 96, 32),
                                                   (5, 6, 2, 128, 144, 16), (3, 40, 8, 64, 256, 64), (4, 5, 1, 48, 72, 16),
-                                                  (2, 2, 2, 16, 40, 16), (7, 24, 8, 128, 512, 16)])
+                                                  (2, 2, 2, 16, 40, 16), (7, 24, 8, 128, 512, 16),
+                                                  (8, 24, 8, 128, 3072, 16), (11, 24, 8, 128, 3072, 16),
+                                                  (5, 32, 8, 128, 4096, 16)])
 @pytest.mark.parametrize("grid", [0, 3])
 def test_gemv_norm_rope(ops, M, n_q, n_kv, hd, K, page, grid):
     """The fused kernel against its parts: norm, projection, rotation, cache write."""
