@@ -150,6 +150,8 @@ _SIGNATURES = {
     "llme_plain_attention": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "llme_plain_argmax": (_i, [_vp, _i]),
     "llme_plain_sample": (_i, [_vp, _i, _f, _f]),
+    # the whole model out of them (csrc/host/plain_model.cpp)
+    "llme_plain_llama_forward": (_i, [_vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp]),
 }
 
 # codes of csrc/host/host_api.h

@@ -111,3 +111,36 @@ def argmax(row: torch.Tensor) -> int:
 def sample(row: torch.Tensor, temperature: float, u: float) -> int:
     row = _f32(row)
     return _check(native.library().llme_plain_sample(row.data_ptr(), row.numel(), float(temperature), float(u)), "sample")
+
+
+def llama_forward(cfg, weights: dict, tokens, positions=None, window: int = 0) -> torch.Tensor:
+    """Logits [T, V] of one whole sequence through the plain C++ backend of the Llama decoder
+    (csrc/host/plain_model.cpp): every tensor in 32-bit, serial loops, no cache. cfg: the typed
+    configuration (config.llama.LlamaConfig); weights: checkpoint names -> tensors."""
+    import ctypes
+    tokens = _i32(tokens)
+    T = tokens.numel()
+    positions = _i32(range(T) if positions is None else positions)
+    if positions.numel() != T:
+        raise ValueError("llama_forward: one position per token")
+    w = {k: _f32(v) for k, v in weights.items()}
+    per_layer = ("input_layernorm.weight", "self_attn.q_proj.weight", "self_attn.k_proj.weight",
+                 "self_attn.v_proj.weight", "self_attn.o_proj.weight", "post_attention_layernorm.weight",
+                 "mlp.gate_proj.weight", "mlp.up_proj.weight", "mlp.down_proj.weight")
+    L = cfg.num_hidden_layers
+    pointers = (ctypes.c_void_p * (9 * L))(*[w[f"model.layers.{l}.{n}"].data_ptr() for l in range(L) for n in per_layer])
+    sizes = _i32([L, cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads, cfg.num_key_value_heads,
+                  cfg.head_dim, cfg.vocab_size, int(window)])
+    sc = cfg.rope_scaling
+    rope = torch.tensor([cfg.rope_theta, 0.0 if sc is None else 1.0] +
+                        ([1.0, 1.0, 1.0, 0.0] if sc is None else
+                         [sc.factor, sc.low_freq_factor, sc.high_freq_factor, float(sc.original_max_position_embeddings)]),
+                        dtype=torch.float64)
+    embed = w["model.embed_tokens.weight"]
+    head = embed if cfg.tie_word_embeddings else w["lm_head.weight"]
+    logits = torch.empty(T, cfg.vocab_size, dtype=torch.float32)
+    _check(native.library().llme_plain_llama_forward(sizes.data_ptr(), rope.data_ptr(), float(cfg.rms_norm_eps),
+                                                     embed.data_ptr(), w["model.norm.weight"].data_ptr(), head.data_ptr(),
+                                                     pointers, tokens.data_ptr(), positions.data_ptr(), T,
+                                                     logits.data_ptr()), "llama_forward")
+    return logits

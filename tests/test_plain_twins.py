@@ -1,7 +1,8 @@
 """The plain C++ twins of the device kernels (csrc/host/plain_kernels.cpp) against the plain
 Python implementation of this folder: two independent readings of the reference's formulas,
 one serial 32-bit C++ loop nest and one 64-bit tensor expression per operation, have to agree
-to 32-bit rounding. Sizes are the reference's own test sizes and some that are no power of
+to 32-bit rounding; so have the whole model put together from each (csrc/host/plain_model.cpp, the
+plain backend, against plain_forward). Sizes are the reference's own test sizes and some that are no power of
 two. The GPU half holds device kernels against the twins."""
 import math
 
@@ -154,6 +155,73 @@ def test_device_argmax_and_sample_against_twins(ops):
         # the device sums in 32-bit: its token is the twin's for a draw within rounding of u
         near = {twin.sample(logits[r], 0.7, min(max(u[r].item() + d, 0.0), 0.9999999)) for d in (-2e-5, 0.0, 2e-5)}
         assert out[r].item() in near or min(near) <= out[r].item() <= max(near)
+
+
+def _tiny(name):
+    import tiny_models
+    from llmengine.config.registry import parse_config
+    from llmengine.weights import random_state
+    cfg, init = getattr(tiny_models, f"TINY_{name}"), getattr(tiny_models, f"{name}_INIT")
+    tensors = dict(random_state(cfg, init["seed"], torch.float32, init["std"], init["norm_mean"], init["norm_std"]))
+    return cfg, parse_config(cfg), tensors
+
+
+@pytest.mark.parametrize("name,T", [("A", 40), ("B", 70), ("D", 33), ("E", 25), ("F", 30)])
+def test_whole_model_backend_against_plain_forward(name, T):
+    """The plain C++ backend (all layers, whole sequence, 32-bit) and the plain Python forward in
+    64-bit agree to 32-bit rounding at every position; a shift of all positions moves both alike
+    (B and F blend rope bands, so a shift is no identity there)."""
+    from plain_llama import plain_forward
+    from tiny_models import random_tokens
+    cfg, typed, tensors = _tiny(name)
+    tokens = random_tokens(T, cfg["vocab_size"], 77)
+    got = twin.llama_forward(typed, tensors, tokens)
+    ref = plain_forward(cfg, tensors, tokens)
+    rows = (got.double() - ref).abs().amax(dim=1) / ref.abs().amax(dim=1)
+    assert float(rows.max()) < 5e-6, (name, float(rows.max()))
+    shifted = list(range(9, 9 + T))
+    got_s = twin.llama_forward(typed, tensors, tokens, positions=shifted)
+    ref_s = plain_forward(cfg, tensors, tokens, positions=shifted)
+    assert float(((got_s.double() - ref_s).abs().amax(dim=1) / ref_s.abs().amax(dim=1)).max()) < 5e-6
+
+
+def test_whole_model_backend_window_and_refusals():
+    from plain_llama import plain_forward
+    from tiny_models import random_tokens
+    cfg, typed, tensors = _tiny("A")
+    tokens = random_tokens(30, 256, 5)
+    got = twin.llama_forward(typed, tensors, tokens, window=7)
+    ref = plain_forward(cfg, tensors, tokens, window=7)
+    assert float(((got.double() - ref).abs().amax(dim=1) / ref.abs().amax(dim=1)).max()) < 5e-6
+    assert float((got.double() - plain_forward(cfg, tensors, tokens)).abs().max()) > 1e-4       # the window matters
+    with pytest.raises(ValueError):
+        twin.llama_forward(typed, tensors, tokens + [256])                                       # an id out of range
+    with pytest.raises(ValueError):
+        twin.llama_forward(typed, tensors, tokens, positions=[0, 1])
+    with pytest.raises(KeyError):
+        twin.llama_forward(typed, {k: v for k, v in tensors.items() if "layers.1.mlp.up_proj" not in k}, tokens)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["A", "B", "F"])
+def test_device_32_bit_path_against_the_whole_model_backend(name):
+    """The engine's 32-bit path (pages, steps of changing size, its own kernels) against the plain
+    C++ backend's whole sequences: 1e-5 of a row's largest logit, the same greedy tokens."""
+    import replay
+    from llmengine import Engine
+    from tiny_models import random_tokens
+    cfg, typed, tensors = _tiny(name)
+    reqs = {f"r{i}": random_tokens(n, cfg["vocab_size"], 40 + i) for i, n in enumerate((45, 70, 9))}
+    ref = {rid: twin.llama_forward(typed, tensors, ids) for rid, ids in reqs.items()}
+    engine = Engine(None, "fp32", _config=cfg, _tensors=dict(tensors), block_size=16)
+    for steps in (replay.whole(reqs), replay.portions(reqs), replay.mixed(reqs, max_live=2, seed=4)):
+        cache = engine.new_cache(replay.trace_peak_tokens(steps, round_to=16) // 16, 16, max_requests=3)
+        got = replay.run_trace(engine, cache, steps)
+        for rid, ids in reqs.items():
+            for p in range(len(ids)):
+                row, want = torch.as_tensor(got[rid][p]).double(), ref[rid][p].double()
+                assert float((row - want).abs().max() / want.abs().max()) < 1e-5, (name, rid, p)
+                assert int(row.argmax()) == int(want.argmax()) or float(want.max() - want[int(row.argmax())]) < 1e-5 * float(want.abs().max())
 
 
 @pytest.mark.gpu
