@@ -643,3 +643,97 @@ def test_toy_interleaved_encoding_shifted_norm_and_wide_pages(dtype):
         for rid, ids in reqs.items():
             for pos in range(len(ids)):
                 assert _rel(got[rid][pos], plain[rid][pos]) < tol, (rid, pos)
+
+
+# --- an embedding with a multiplier and a head with a cap, through the registries' own kinds ---
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_toy_scaled_embedding_and_capped_head(dtype):
+    """The two ends of a model are parts like the others: an embedding that multiplies its rows by
+    sqrt(hidden) and a head that caps its logits (cap tanh(z / cap)), defined here against the base
+    classes `TokenEmbedding` and `Head`, registered under the kinds "embedding" and "head", built
+    into an architecture of their own beside ordinary Llama layers, and stepped under all schedules,
+    decode steps recorded. The plain forward gets the multiplier in its table and the cap behind."""
+    from llmengine import Engine
+    from llmengine.config import register_architecture
+    from llmengine.config.llama import LlamaConfig
+    from llmengine.models.llama import llama_layer_specs
+    from llmengine.models.model import DecoderModel
+    from llmengine.parts import ParamSpec, build_layer, make_part, register_part
+    from llmengine.parts.base import Head, TokenEmbedding
+    from llmengine.weights import random_state
+    from plain_llama import bf16_round
+
+    CAP = 3.0
+
+    class ScaledEmbedding(TokenEmbedding):
+        graph_safe = True                                   # reads the step's device arrays only
+
+        def __init__(self, vocab_size, hidden_size, multiplier):
+            self.vocab_size, self.hidden_size, self.multiplier = vocab_size, hidden_size, multiplier
+            self.weight = None
+
+        def param_specs(self):
+            return {"weight": ParamSpec((self.vocab_size, self.hidden_size), "linear")}
+
+        def load_params(self, get, placement):
+            self.weight = placement.place(get("weight"))
+
+        def forward(self, tokens, out, step=None):
+            out.copy_(self.weight[tokens.long()].float() * self.multiplier)
+
+    class CappedHead(Head):
+        graph_safe = True
+
+        def __init__(self, vocab_size, hidden_size, cap):
+            self.vocab_size, self.hidden_size, self.cap = vocab_size, hidden_size, cap
+            self.w = None
+
+        def param_specs(self):
+            return {"weight": ParamSpec((self.vocab_size, self.hidden_size), "linear")}
+
+        def load_params(self, get, placement):
+            self.w = placement.place(get("weight"), torch.float32)
+
+        def forward(self, x, out, step=None):
+            out.copy_(self.cap * torch.tanh((x.float() @ self.w.T) / self.cap))
+
+    register_part("embedding", "toy_scaled", ScaledEmbedding, replace=True)
+    register_part("head", "toy_capped", CappedHead, replace=True)
+
+    def build(c):
+        shared = {}
+        layers = [build_layer(spec, shared) for spec in llama_layer_specs(c)]
+        emb = make_part("embedding", "toy_scaled", vocab_size=c.vocab_size, hidden_size=c.hidden_size,
+                        multiplier=math.sqrt(c.hidden_size))
+        head = make_part("head", "toy_capped", vocab_size=c.vocab_size, hidden_size=c.hidden_size, cap=CAP)
+        return DecoderModel(c, emb, layers, make_part("norm", "rmsnorm", size=c.hidden_size, eps=c.rms_norm_eps), head)
+
+    register_architecture("ToyCappedForCausalLM", LlamaConfig.from_dict, build, replace=True)
+    cfg = dict(TINY_B, architectures=["ToyCappedForCausalLM"])
+    store = torch.float32 if dtype == "fp32" else torch.bfloat16
+    tensors = dict(random_state(cfg, 41, store, 0.05, 1.0, 0.1))
+    assert "lm_head.weight" in tensors and "model.embed_tokens.weight" in tensors
+    engine = Engine(None, dtype, _config=cfg, _tensors=dict(tensors), block_size=8)
+    assert engine.runner.use_graphs and not engine.model.head.fuses_norm(None, None, 1, None)
+
+    as_llama = {k: v.double() for k, v in tensors.items()}
+    as_llama["model.embed_tokens.weight"] = as_llama["model.embed_tokens.weight"] * math.sqrt(cfg["hidden_size"])
+    reqs = {f"c{i}": random_tokens(n, cfg["vocab_size"], 200 + i) for i, n in enumerate((40, 7, 66, 21))}
+    plain = {}
+    for rid, ids in reqs.items():
+        z = plain_forward(TINY_B, as_llama, ids, rounder=bf16_round if dtype == "bf16" else None)
+        plain[rid] = (CAP * torch.tanh(z / CAP)).numpy()
+    assert max(float(np.abs(v).max()) for v in plain.values()) > 0.5 * CAP          # the cap bends something
+    tol = 1e-5 if dtype == "fp32" else 2e-2
+    for steps in (replay.whole(reqs), replay.tail_one_by_one(reqs, 32), replay.portions(reqs),
+                  replay.mixed(reqs, max_live=3, seed=6)):
+        cache = engine.new_cache(replay.trace_peak_tokens(steps, 8) // 8, 8, 3)
+        got = replay.run_trace(engine, cache, steps)
+        for rid, ids in reqs.items():
+            for pos in range(len(ids)):
+                assert _rel(got[rid][pos], plain[rid][pos]) < tol, (rid, pos)
+    assert engine.runner.graph_replays > 0
+    # greedy generation through the entry point takes the recorded steps that end in the argmax
+    ids, finish = engine.generate(reqs["c1"], 6)
+    z = plain_forward(TINY_B, as_llama, ids[:-1], rounder=bf16_round if dtype == "bf16" else None)[-1]
+    assert finish == "length" and z[ids[-1]] >= z.max() - (1e-5 if dtype == "fp32" else 2e-2) * z.abs().max()
