@@ -216,7 +216,7 @@ class Engine:
             uniforms = None
             if temperature > 0.0 and self.runner.use_graphs and len(draws) == len(entries):
                 uniforms = [uniform_draw(seed, r, i) for r, i in draws]
-            tokens = self.runner.step_greedy(cache, entries, max_position=self.max_pos, temperature=temperature,
+            tokens = self.runner.step_choosing(cache, entries, max_position=self.max_pos, temperature=temperature,
                                              uniforms=uniforms)
             if tokens is not None:
                 return tokens
@@ -255,13 +255,13 @@ class Engine:
                     last = self.run_step(cache, [StepEntry(r, [t], [0]) for r, t in zip(ids, last)], None)
                     out.append(last)
                 return out
-            pending = runner.greedy_launch(cache, ids, first, self.max_pos)
+            pending = runner.launch_choosing(cache, ids, first, self.max_pos)
             for i in range(1, steps + 1):
-                ahead = runner.greedy_launch(cache, ids, None, self.max_pos) if i < steps else None
-                last = runner.greedy_result(pending)
+                ahead = runner.launch_choosing(cache, ids, None, self.max_pos) if i < steps else None
+                last = runner.chosen_tokens(pending)
                 out.append(last)
                 if i < steps and ahead is None:          # (the recording changed: the tokens go through the host once)
-                    ahead = runner.greedy_launch(cache, ids, last, self.max_pos)
+                    ahead = runner.launch_choosing(cache, ids, last, self.max_pos)
                 pending = ahead
         return out
 
@@ -351,13 +351,13 @@ class Engine:
                         # host has fetched it (one step more than needed if this one stops)
                         more = generated + 1 < max_new_tokens     # the token being fetched is not the last wanted
                         with torch.cuda.device(runner.device):
-                            ahead = runner.greedy_launch(cache, [rid], None, self.max_pos, temperature,
+                            ahead = runner.launch_choosing(cache, [rid], None, self.max_pos, temperature,
                                                          draw(generated + 1)) if more else None
-                            nxt = runner.greedy_result(pending)[0]
+                            nxt = runner.chosen_tokens(pending)[0]
                     if nxt in eos:
                         finish = "stop"
                         if pending is not None and ahead is not None:
-                            runner.greedy_result(ahead)
+                            runner.chosen_tokens(ahead)
                         break
                     out.append(nxt)
                     generated += 1
@@ -368,7 +368,7 @@ class Engine:
                             if pending is not None and ahead is not None:
                                 pending = ahead
                             else:
-                                pending = runner.greedy_launch(cache, [rid], [nxt], self.max_pos, temperature,
+                                pending = runner.launch_choosing(cache, [rid], [nxt], self.max_pos, temperature,
                                                                draw(generated))
                     else:
                         logits = self.step(cache, [StepEntry(rid, [nxt], [0])])

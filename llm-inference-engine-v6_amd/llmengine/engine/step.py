@@ -218,7 +218,7 @@ class CacheContext:
         self.page_size = page_size
         self.max_requests = max_requests
         self.graphs: dict = {}          # recorded decode steps over this pool's tensors, by shape
-        self.chain = None               # the last greedy launch: (recording, requests, its key), see greedy_launch
+        self.chain = None               # the last launch that chose its tokens: (recording, requests, its key), see launch_choosing
 
     def admit(self, request_id) -> int:
         self.chain = None
@@ -249,7 +249,7 @@ class _DecodeRecord:
         # a recording that samples reads a temperature and a uniform draw per request from behind the
         # integer arrays (2 S floats that the host sends up with them)
         self.draws = 2 * S if draws else 0
-        # pinned, 2 S: where a greedy recording leaves the chosen tokens, in its two halves in turn (the
+        # pinned, 2 S: where a recording that chooses leaves the chosen tokens, in its two halves in turn (the
         # half is named by the integer behind the arrays), so that a step can be launched before the
         # tokens of the one before it have been read; the same tokens also land in the token array
         # itself, where the next replay finds them without the host
@@ -319,7 +319,7 @@ class _DecodeRecord:
 
 
 class PendingTokens:
-    """A launched greedy step whose tokens have not been fetched yet."""
+    """A launched step that chooses its tokens itself, which have not been fetched yet."""
 
     def __init__(self, rec: _DecodeRecord, slot: int, launch: int):
         self.rec, self.slot, self.launch = rec, slot, launch
@@ -362,7 +362,7 @@ class ModelRunner:
         mgr = cache.manager
         if not entries:
             return None
-        cache.chain = None                      # (a later greedy launch takes its tokens from the host again)
+        cache.chain = None                      # (a later launch that chooses takes its tokens from the host again)
         vocab = self.model.vocab_size
         seen = set()
         for e in entries:
@@ -489,7 +489,7 @@ class ModelRunner:
             rec.scratch = scratch                       # (kept alive: the graph holds its addresses)
         return rec
 
-    def step_greedy(self, cache: CacheContext, entries: Sequence[StepEntry], max_position: int | None = None,
+    def step_choosing(self, cache: CacheContext, entries: Sequence[StepEntry], max_position: int | None = None,
                     temperature: float = 0.0, uniforms: Sequence[float] | None = None) -> list[int] | None:
         """The next token of every entry, greedy or (temperature > 0, a uniform draw per entry in
         `uniforms`) sampled, for a step of single decoded tokens that all want one: bookkeeping in two
@@ -502,18 +502,18 @@ class ModelRunner:
             if len(e.tokens) != 1 or len(e.want) != 1 or e.want[0] != 0:
                 return None
             ids.append(e.request_id)
-        pending = self.greedy_launch(cache, ids, [int(e.tokens[0]) for e in entries], max_position,
+        pending = self.launch_choosing(cache, ids, [int(e.tokens[0]) for e in entries], max_position,
                                      temperature=temperature, uniforms=uniforms)
         try:
-            return self.greedy_result(pending)
+            return self.chosen_tokens(pending)
         except BaseException as e:
             raise StepCommittedError(f"the step ran, but its tokens could not be fetched: {e}") from e
 
-    def greedy_launch(self, cache: CacheContext, ids: Sequence, tokens: Sequence[int] | None,
+    def launch_choosing(self, cache: CacheContext, ids: Sequence, tokens: Sequence[int] | None,
                       max_position: int | None = None, temperature: float = 0.0,
                       uniforms: Sequence[float] | None = None) -> "PendingTokens | None":
         """Launches a step of one token for each of the live requests `ids` whose choices (greedy, or
-        sampled at `temperature` with the draws `uniforms`, one per request) `greedy_result` fetches
+        sampled at `temperature` with the draws `uniforms`, one per request) `chosen_tokens` fetches
         later. tokens None: every request's token is the one that the launch
         before this one chose for it, taken where that step's argmax left it on the device, so that
         this step can be launched before the host has seen those tokens (the host's work for a step,
@@ -521,7 +521,7 @@ class ModelRunner:
         before to have been of the same requests in the same recording; where it was not (the first
         step, or the block tables have outgrown the recording), None is returned and nothing is
         done: the caller fetches the tokens and passes them. At most one launch may be waiting for
-        its `greedy_result` when another is made."""
+        its `chosen_tokens` when another is made."""
         S = len(ids)
         if len(set(ids)) != S:
             raise ValueError("a request appears twice in one step")
@@ -573,7 +573,7 @@ class ModelRunner:
         cache.chain = (rec, list(ids), key)
         return PendingTokens(rec, slot, rec.launches[slot])
 
-    def greedy_result(self, pending: "PendingTokens") -> list[int]:
+    def chosen_tokens(self, pending: "PendingTokens") -> list[int]:
         """The tokens a launched step chose (waits for it). They can be fetched until the launch
         after the next one, which uses the same half of the recording's token buffer."""
         rec, slot = pending.rec, pending.slot
