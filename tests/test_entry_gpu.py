@@ -240,6 +240,35 @@ def test_sampled_step_with_the_choice_in_the_recording(dir_b, dtype):
     assert sorted(k[2] for k in recordings) == ["greedy", "greedy", "sampled", "sampled"]
 
 
+def test_scheduler_at_a_temperature_with_many_live_requests(dir_a):
+    """28 requests, up to 24 live, at temperature 1.1: the decode steps' recordings (of every number of
+    live requests that occurs, each ending in the sampling kernels) choose the tokens that an engine
+    without recordings samples from its logits, request by request, and every token lies in its
+    draw's interval under the plain logits."""
+    from llmengine import BlockManager, ContinuousBatchScheduler, Engine
+    cfg, w = load_plain_model(dir_a)
+    prompts = [random_tokens(3 + (7 * i) % 40, 256, 500 + i) for i in range(28)]
+    news = [6 + (5 * i) % 17 for i in range(28)]
+    streams = []
+    for graphs in (True, False):
+        engine = Engine(dir_a, "fp32", use_graphs=graphs)
+        blocks = BlockManager(400, 8, 2, 2, 16)
+        sched = ContinuousBatchScheduler(engine, blocks, max_concurrent=24, max_prefill_tokens_per_step=48,
+                                         temperature=1.1, seed=13)
+        for p, n in zip(prompts, news):
+            sched.enqueue(p, n)
+        sched.run_until_idle()
+        assert blocks.free_blocks == 400
+        streams.append([(r.seq_id, r.token_ids, r.finish_reason) for r in sched.results])
+        if graphs:
+            kinds = {k[2] for k in sched._cache.graphs}
+            sizes = {k[0] for k in sched._cache.graphs}
+            assert kinds == {"sampled"} and max(sizes) > 16 and len(sizes) > 3
+            for r in sched.results:
+                _check_sampled(cfg, w, r, 1.1, 13, 1e-4)
+    assert streams[0] == streams[1]
+
+
 def test_generate_at_a_temperature_is_the_same_with_and_without_recordings(dir_a, dir_b):
     """generate() launches each sampled step before it has fetched the token of the step before;
     the stream is the one an engine without recordings samples, and the one the plain logits allow."""
