@@ -556,6 +556,30 @@ def test_random_configurations(case):
         del engine
 
 
+@pytest.mark.parametrize("hd,n_q,n_kv,hidden,ff,vocab", [(6, 3, 1, 48, 72, 101), (24, 4, 2, 96, 100, 130),
+                                                         (100, 2, 1, 104, 120, 99), (250, 1, 1, 64, 80, 70)])
+def test_head_sizes_that_are_no_multiple_of_16(hd, n_q, n_kv, hidden, ff, vocab):
+    """The configuration allows every even head size (rotary pairs); the kernels with matrix instructions
+    take multiples of 16, the others go through the plain-precision kernels, in bfloat16 too: the same
+    bounds, under every schedule."""
+    from llmengine import Engine
+    from llmengine.weights import random_state
+    cfg = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "head_dim": hd, "hidden_size": hidden,
+           "intermediate_size": ff, "num_hidden_layers": 2, "num_attention_heads": n_q, "num_key_value_heads": n_kv,
+           "vocab_size": vocab, "max_position_embeddings": 256, "rms_norm_eps": 1e-5, "rope_theta": 10000.0,
+           "tie_word_embeddings": True}
+    tensors = dict(random_state(cfg, hd, torch.bfloat16, 0.08, 1.0, 0.1))
+    wide = {k: v.double() for k, v in tensors.items()}
+    reqs = {f"r{i}": random_tokens(n, vocab, 100 + i) for i, n in enumerate((50, 9, 77))}
+    plain = {"fp32": {rid: plain_forward(cfg, wide, ids).numpy() for rid, ids in reqs.items()},
+             "bf16": {rid: plain_forward(cfg, wide, ids, rounder=bf16_round).numpy() for rid, ids in reqs.items()}}
+    for dtype in ("fp32", "bf16"):
+        engine = Engine(None, dtype, _config=cfg, _tensors=dict(tensors), block_size=16)
+        for steps in (replay.whole(reqs), replay.tail_one_by_one(reqs, 20), replay.mixed(reqs, max_live=3, seed=hd)):
+            cache = engine.new_cache(replay.trace_peak_tokens(steps, round_to=16) // 16, 16, max_requests=3)
+            check_against_plain(replay.run_trace(engine, cache, steps), plain[dtype], reqs, dtype)
+
+
 def test_two_heads_of_128_in_a_narrow_model():
     """Case 90 of the random configurations (heads of 128 in a width of 288, two of them, three
     layers): where bfloat16 shows most. The matrix-instruction attention rounds its softmax weights
