@@ -43,6 +43,14 @@ class KernelChoices:
     # the items behind 1,024 keys cut in two: 6.5 to 6.6 ms against 5.95 whole; the partial outputs and
     # the join cost more than the evener load wins.)
     prefill_min_splits: int = 3
+    # More than a quarter of a workgroup per compute unit (65 to 128 items on 256 units: portions of 257
+    # to 512 tokens of 32 heads): the keys are cut only where an item has at least this many keys for
+    # every item of the step, since whole keys in items of half the rows are faster until then and the
+    # join costs 13 us a layer whatever the length. Measured at the 1B sizes beside 17 decoded tokens (ms a
+    # step, cut / whole): 320 tokens behind 2,048: 2.55 / 2.32, behind 4,096: 2.61 / 2.63, behind 8,192:
+    # 2.91 / 3.29; 512 tokens behind 1,024: 2.83 / 2.49, behind 4,096: 3.10 / 2.95, behind 8,192: 3.55 / 3.62,
+    # behind 16,384: 4.44 / 4.97. (Up to 64 items the cut never lost: 256 tokens behind 8,192: 2.53 / 3.09.)
+    prefill_cut_keys_per_item: int = 64
 
     def key(self) -> tuple:
         return tuple(self.__dict__.values())
