@@ -28,10 +28,11 @@ class KernelChoices:
     # with 1,024, 1.036 with 128; with 384 (one and a half per compute unit) 1.000.
     decode_blocks_wanted: int | None = None
     # Portions of prompts: work items (a span of rows x a group of heads) the prefill kernel should
-    # have at least (None: two per compute unit); with prefill_cut_items or fewer (None: half a
-    # workgroup per compute unit; measured: 256 items cut in two were 3 % slower than whole), the longest
-    # item's keys are cut into that many runs of at least prefill_min_run keys, and the others' into
-    # runs of the same length.
+    # have at least (None: two per compute unit, three where the step has more than half a compute unit's
+    # number already); with prefill_cut_items or fewer (None: three quarters of the compute units' number;
+    # measured: 256 items cut in two were 3 % slower than whole, and 224 to 256 items cut in three or four
+    # no faster even behind 32,768 tokens), the longest item's keys are cut into that many runs of at least
+    # prefill_min_run keys, and the others' into runs of the same length.
     prefill_items_wanted: int | None = None
     prefill_cut_items: int | None = None
     prefill_min_run: int = 512
@@ -49,7 +50,9 @@ class KernelChoices:
     # join costs 13 us a layer whatever the length. Measured at the 1B sizes beside 17 decoded tokens (ms a
     # step, cut / whole): 320 tokens behind 2,048: 2.55 / 2.32, behind 4,096: 2.61 / 2.63, behind 8,192:
     # 2.91 / 3.29; 512 tokens behind 1,024: 2.83 / 2.49, behind 4,096: 3.10 / 2.95, behind 8,192: 3.55 / 3.62,
-    # behind 16,384: 4.44 / 4.97. (Up to 64 items the cut never lost: 256 tokens behind 8,192: 2.53 / 3.09.)
+    # behind 16,384: 4.44 / 4.97; 768 tokens (192 items, cut in four) behind 8,192: 4.85 / 4.85, behind 16,384:
+    # 6.31 / 6.85, behind 32,768: 9.12 / 10.91. (Up to 64 items the cut never lost: 256 tokens behind 8,192:
+    # 2.53 / 3.09.)
     prefill_cut_keys_per_item: int = 64
 
     def key(self) -> tuple:

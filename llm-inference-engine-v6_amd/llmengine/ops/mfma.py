@@ -202,9 +202,11 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
         # few rows over long contexts: too few work items for the chip, each with many keys
         keys = max(c + n for n, c in zip(new_lens, ctx_lens) if n >= 2)
         splits = 1
-        if items <= (ch.prefill_cut_items or compute_units() // 2):
-            splits = max(1, min((ch.prefill_items_wanted or 2 * compute_units()) // items, keys // ch.prefill_min_run,
-                                ch.prefill_max_splits))
+        if items <= (ch.prefill_cut_items or 3 * compute_units() // 4):
+            # (items wanted: two per compute unit; three where the step has more than half a compute unit's number
+            # already, which two would cut in two or not at all)
+            wanted = ch.prefill_items_wanted or (2 if 2 * items <= compute_units() else 3) * compute_units()
+            splits = max(1, min(wanted // items, keys // ch.prefill_min_run, ch.prefill_max_splits))
             if splits < ch.prefill_min_splits:
                 splits = 1                                 # (two runs win less than their join costs)
             if items * 4 > compute_units() and keys < ch.prefill_cut_keys_per_item * items:

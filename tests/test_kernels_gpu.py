@@ -668,7 +668,8 @@ def test_attention_plan_cuts_only_few_rows_over_many_keys(ops):
     assert ops.mfma.plan_attention([1, 1], [5000, 9000], 32, 8, 64)["prefill_splits"] == 1
     # more than a quarter of an item per compute unit: whole keys (in items of half the rows) until the keys are long
     for rows, behind, cut in ((512, 1024, False), (512, 4096, False), (512, 8192, True), (320, 2048, False),
-                              (320, 8192, True), (256, 4096, True), (256, 8192, True)):
+                              (320, 8192, True), (256, 4096, True), (256, 8192, True), (768, 8192, False),
+                              (768, 16384, True), (896, 32768, False)):
         plan = ops.mfma.plan_attention([rows, 1, 1], [behind, 700, 900], 32, 8, 64)
         assert (plan["prefill_splits"] > 1) == cut, (rows, behind, plan)
         assert cut or plan["tuning"] & ops.mfma.TUNING_HALF_ROWS
