@@ -53,6 +53,9 @@ class KernelChoices:
     # behind 16,384: 4.44 / 4.97; 768 tokens (192 items, cut in four) behind 8,192: 4.85 / 4.85, behind 16,384:
     # 6.31 / 6.85, behind 32,768: 9.12 / 10.91. (Up to 64 items the cut never lost: 256 tokens behind 8,192:
     # 2.53 / 3.09.)
+    # For heads of 64; a key of a head of 128 is twice the work, and half as many keys are long: at the 8B
+    # sizes (8 layers) 768 tokens behind 8,192: 5.46 / 6.32, at the 3B sizes 3.53 / 4.68, behind 1,024 whole
+    # keys win at both (4.33 / 4.42 and 2.64 / 2.73 whole / cut).
     prefill_cut_keys_per_item: int = 64
 
     def key(self) -> tuple:

@@ -209,7 +209,7 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
             splits = max(1, min(wanted // items, keys // ch.prefill_min_run, ch.prefill_max_splits))
             if splits < ch.prefill_min_splits:
                 splits = 1                                 # (two runs win less than their join costs)
-            if items * 4 > compute_units() and keys < ch.prefill_cut_keys_per_item * items:
+            if items * 4 > compute_units() and keys * head_dim < ch.prefill_cut_keys_per_item * 64 * items:
                 splits = 1                                 # (many items with keys that are not long: whole keys, half rows)
             stretches = (keys + 63) // 64
             run = (stretches + splits - 1) // splits       # stretches of 64 keys per run
