@@ -16,6 +16,10 @@ class KernelChoices:
     # every attention goes through the plain-precision kernels (the 32-bit model's always do)
     fast_gemm: bool = True
     fast_attention: bool = True
+    # products of a few rows more than a multiple of 1,024 (at most tail_rows_most): those rows in a launch of
+    # their own (ops.mfma.tail_rows)
+    tail_rows_apart: bool = True
+    tail_rows_most: int = 64
     # decoding, up to 16 tokens whose keys are cut into splits: the splits' join inside the output projection
     join_project: bool = True
     # decoding, 17 to 64 tokens with the keys in one split: rotation and cache write inside the attention kernel

@@ -188,7 +188,8 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
     adds into `out` may be cut over k into parts that several workgroups add with atomics, in
     whatever order they finish: the result then differs from run to run in its last bits.
     fixed_order forbids that cut (every output element is summed by one workgroup in one order)."""
-    if (choices or DEFAULT).fast_gemm and _fast_gemm is not None and _fast_gemm(a, w, out, accumulate, fixed_order):
+    if ((choices or DEFAULT).fast_gemm and _fast_gemm is not None
+            and _fast_gemm(a, w, out, accumulate, fixed_order, choices)):
         return
     gemm_generic(a, w, out, accumulate)
 

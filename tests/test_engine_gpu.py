@@ -580,6 +580,44 @@ def test_head_sizes_that_are_no_multiple_of_16(hd, n_q, n_kv, hidden, ff, vocab)
             check_against_plain(replay.run_trace(engine, cache, steps), plain[dtype], reqs, dtype)
 
 
+def test_a_few_rows_more_than_1024_take_the_products_apart():
+    """A step of 1,024 prompt tokens beside three decoded tokens, and whole prompts of 1,030 and 1,060 tokens:
+    the products run the rows behind the multiple of 1,024 in a launch of their own. Every wanted row
+    against the plain implementation, and against the same engine with one launch."""
+    from llmengine import Engine
+    from llmengine.ops import KernelChoices, mfma
+    from llmengine.weights import random_state
+    assert [mfma.tail_rows(m) for m in (1024, 1025, 1088, 1089, 1160, 2048, 2060, 700)] == [0, 1, 64, 0, 0, 0, 12, 0]
+    cfg = TINY_C
+    tensors = dict(random_state(cfg, C_INIT["seed"], torch.bfloat16, C_INIT["std"], C_INIT["norm_mean"], C_INIT["norm_std"]))
+    wide = {k: v.double() for k, v in tensors.items()}
+    V = cfg["vocab_size"]
+    reqs = {"a": random_tokens(31, V, 1), "b": random_tokens(41, V, 2), "c": random_tokens(12, V, 3),
+            "long": random_tokens(1500, V, 4), "p30": random_tokens(1030, V, 5), "p60": random_tokens(1060, V, 6)}
+    steps = [{"entries": [{"id": r, "tokens": reqs[r][:-1], "want": []} for r in ("a", "b", "c")], "end": []},
+             {"entries": [{"id": "long", "tokens": reqs["long"][:1024], "want": [1023]}] +
+                         [{"id": r, "tokens": reqs[r][-1:], "want": [0]} for r in ("a", "b", "c")], "end": ["a", "b", "c"]},
+             {"entries": [{"id": "long", "tokens": reqs["long"][1024:], "want": [475]}], "end": ["long"]},
+             {"entries": [{"id": "p30", "tokens": reqs["p30"], "want": [0, 1023, 1024, 1029]}], "end": ["p30"]},
+             {"entries": [{"id": "p60", "tokens": reqs["p60"], "want": [1059]}], "end": ["p60"]}]
+    wanted = {"a": [30], "b": [40], "c": [11], "long": [1023, 1499], "p30": [0, 1023, 1024, 1029], "p60": [1059]}
+    plain = {r: plain_forward(cfg, wide, reqs[r], rounder=bf16_round, rows=wanted[r]).numpy() for r in reqs}
+    got = {}
+    for name, choices in (("apart", None), ("one launch", KernelChoices(tail_rows_apart=False))):
+        engine = Engine(None, "bf16", _config=cfg, _tensors=dict(tensors), block_size=16, kernel_choices=choices)
+        cache = engine.new_cache(120, 16, max_requests=4)
+        got[name] = replay.run_trace(engine, cache, steps)
+        for r, places in wanted.items():
+            assert sorted(got[name][r]) == places
+            for i, pos in enumerate(places):
+                ref = plain[r][i]
+                err = np.abs(got[name][r][pos].astype(np.float64) - ref).max() / np.abs(ref).max()
+                assert err < TOL["bf16"], (name, r, pos, err)
+    for r, places in wanted.items():                       # the same sums in the same order, row by row
+        for pos in places:
+            assert np.abs(got["apart"][r][pos] - got["one launch"][r][pos]).max() <= 2e-2 * np.abs(got["one launch"][r][pos]).max()
+
+
 def test_two_heads_of_128_in_a_narrow_model():
     """Case 90 of the random configurations (heads of 128 in a width of 288, two of them, three
     layers): where bfloat16 shows most. The matrix-instruction attention rounds its softmax weights
