@@ -24,6 +24,12 @@ class KernelChoices:
     join_project: bool = True
     # decoding, 17 to 64 tokens with the keys in one split: rotation and cache write inside the attention kernel
     decode_rope: bool = True
+    # decoding with heads of 64, the most tokens whose q/k/v product is still cut over k and added into a cleared
+    # buffer, so that the attention kernel rotates and writes the cache (without decode_rope: 64, as for every
+    # other step). Measured at the 1B sizes and a context of 2,048, ms a step with 64 / 128 here: 65 tokens
+    # 2.125 / 2.044, 80: 2.287 / 2.218, 96: 2.504 / 2.473, 112: 2.916 / 2.898; 128: 3.216 / 3.287 on one box and
+    # 3.268 / 3.195 on another; 160 tokens with 64 / 256: 3.630 / 3.697, 256: 5.069 / 5.236.
+    qkv_sum_rows_decoding: int = 96
     # prompt attention: work items of half the rows where a step has few items
     prefill_half_rows: bool = True
     # Workgroups (of four wavefronts) the decode kernel should have at most when it cuts the keys: one

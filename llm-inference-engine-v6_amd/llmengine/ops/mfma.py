@@ -435,6 +435,16 @@ GEMV_NORM_MAX_ROWS = 16
 QKV_SUM_MAX_ROWS = 64
 
 
+def qkv_sum_max_rows(decoded_only: bool, head_dim: int, choices: KernelChoices | None = None) -> int:
+    """The most rows of a step whose q/k/v product is cut over k and added into a cleared buffer. A step of
+    single decoded tokens with heads of 64 keeps that way further (choices.qkv_sum_rows_decoding): the
+    attention kernel then rotates and writes the cache itself (attention_decode_rope)."""
+    ch = choices or DEFAULT
+    if decoded_only and head_dim == 64 and ch.decode_rope:
+        return max(QKV_SUM_MAX_ROWS, ch.qkv_sum_rows_decoding)
+    return QKV_SUM_MAX_ROWS
+
+
 def gemv_norm_supported(h: torch.Tensor, norm_weight: torch.Tensor, w: torch.Tensor, rows_out: int,
                         gated: bool, choices: KernelChoices | None = None) -> bool:
     """Whether a step may take gemv_norm: the kernel takes the operands, and the choices allow it."""

@@ -104,6 +104,7 @@ class Attention(Mixer):
         act = step.act_dtype
         q = step.buffer("attn.q", (T, self.q_dim), act)
         rms = pre_norm.fused_rms() if pre_norm is not None else None
+        sum_rows = ops.mfma.qkv_sum_max_rows(T == step.num_seqs and rot == hd and not applies, hd, step.choices)
 
         def project(weight, dst):
             if rms is not None:
@@ -115,13 +116,13 @@ class Attention(Mixer):
             # decoding: norm, projection, rotation and the cache write are one kernel
             ops.gemv_norm_rope(x, rms[0], rms[1], self.w_qkv_paired, step.positions, step.seq_idx,
                                block_table, cos, sin, q, k_cache, v_cache, n_q, n_kv, hd)
-        elif (write_cache and rms is None and T > ops.mfma.QKV_SUM_MAX_ROWS and cos is not None
+        elif (write_cache and rms is None and T > sum_rows and cos is not None
               and ops.gemm_qkv_rope_supported(x, self.w_qkv, k_cache, hd, rot, step.choices)):
             # many rows (prompts): rotation and the cache write are the projection's epilogue
             ops.gemm_qkv_rope(x, self.w_qkv, cos, sin, step.positions, step.seq_idx, block_table, q, k_cache, v_cache,
                               n_q, n_kv, hd)
         elif write_cache:
-            adds = (rms is None and ops.mfma.GEMV_NORM_MAX_ROWS < T <= ops.mfma.QKV_SUM_MAX_ROWS
+            adds = (rms is None and ops.mfma.GEMV_NORM_MAX_ROWS < T <= sum_rows
                     and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16
                     and (T * (self.q_dim + 2 * self.kv_dim)) % 4 == 0)
             # (the product that adds has a buffer that nothing else writes: what it is left holding is known)

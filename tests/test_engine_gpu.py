@@ -350,10 +350,11 @@ def test_decoded_tokens_join_their_splits_inside_the_output_projection(zoo, n_li
             assert np.abs(got[rid][pos].astype(np.float64) - apart[rid][pos]).max() / top < 2e-3, (rid, pos)
 
 
-@pytest.mark.parametrize("name", ["C", "F"])
-def test_twenty_decoded_tokens_are_rotated_inside_the_attention_kernel(zoo, name, monkeypatch):
-    """17 to 64 decoded tokens a step: q/k/v is a product cut over k into a cleared 32-bit buffer, and where
-    the keys are in one split the attention kernel itself rotates, writes the cache and clears the rows.
+@pytest.mark.parametrize("name,n_live", [("C", 20), ("F", 20), ("C", 70)])
+def test_twenty_decoded_tokens_are_rotated_inside_the_attention_kernel(zoo, name, n_live, monkeypatch):
+    """17 to 64 decoded tokens a step (to 96 with heads of 64): q/k/v is a product cut over k into a cleared
+    32-bit buffer, and where the keys are in one split the attention kernel itself rotates, writes the cache
+    and clears the rows.
     It must have run, match the plain implementation, and give exactly what the rotation kernel and the
     decode kernel give apart (also on the steps after the first, which find the buffer cleared)."""
     from llmengine.ops import mfma
@@ -370,7 +371,7 @@ def test_twenty_decoded_tokens_are_rotated_inside_the_attention_kernel(zoo, name
     # few kv heads of these models it would cut the keys; models with 8 kv heads do not from 17 requests on)
     model_dir, _, _, page = zoo[name]
     cfg = TINY_C if name == "C" else TINY_F
-    reqs = {f"s{i}": random_tokens(60 + 3 * i, cfg["vocab_size"], 190 + i) for i in range(20)}
+    reqs = {f"s{i}": random_tokens(60 + 3 * i, cfg["vocab_size"], 190 + i) for i in range(n_live)}
     pcfg, pw = load_plain_model(model_dir)
     engine = engine_for(model_dir, "bf16")
     monkeypatch.setattr(engine.runner.choices, "decode_blocks_wanted", 1)
@@ -381,7 +382,7 @@ def test_twenty_decoded_tokens_are_rotated_inside_the_attention_kernel(zoo, name
     pages = replay.trace_peak_tokens(steps, round_to=page) // page
 
     def run():
-        cache = engine.new_cache(pages, page, max_requests=20)
+        cache = engine.new_cache(pages, page, max_requests=n_live)
         return replay.run_trace(engine, cache, steps)
     got = run()
     assert calls and all(calls), "the decode steps did not rotate inside the attention kernel"
