@@ -28,6 +28,7 @@ requests' cache, over its time, against 8 TB/s), `points` (decode at batch 1 and
 from __future__ import annotations
 
 import argparse
+import random
 import json
 import os
 import sys
@@ -234,6 +235,11 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096, help="context length the decode steps run at")
+    ap.add_argument("--context-range", default="", help="decode: contexts drawn uniformly from [a, b] (seeded) instead "
+                                                        "of --context for every request")
+    ap.add_argument("--decode-order", default="as-drawn", choices=["as-drawn", "longest-first"],
+                    help="decode with --context-range: the order of the requests in the batch (the scheduler puts "
+                         "the longest first)")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes: Llama 3.2 1B (the default), 3.2 3B, 3.1 8B")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (named in config)")
@@ -311,10 +317,15 @@ def main() -> int:
 
     # ---- decode ----
     def decode_run(batch: int, steps: int, warmup: int):
-        start_ctx = args.context - steps - warmup
-        if start_ctx < 1:
+        if args.context_range:
+            lo, hi = (int(x) for x in args.context_range.split(","))
+            rnd = random.Random(args.seed * 1000 + batch)
+            starts = [rnd.randint(lo, hi) for _ in range(batch)]
+        else:
+            starts = [args.context - steps - warmup] * batch
+        if min(starts) < 1:
             raise SystemExit("--context must exceed --steps + --warmup")
-        pages = batch * ((args.context + page - 1) // page)
+        pages = sum((st + steps + warmup + page - 1) // page + 1 for st in starts)
         cache = engine.new_cache(pages, page, batch)
         ids = [f"r{i}" for i in range(batch)]
         for rid in ids:
@@ -322,14 +333,16 @@ def main() -> int:
         chunk = 8192
         sync()
         t_fill = time.perf_counter()
-        for rid in ids:                                        # real prefill fills the pages
+        for rid, start_ctx in zip(ids, starts):                # real prefill fills the pages
             toks = torch.randint(0, V, (start_ctx,), generator=gen).tolist()
             for s in range(0, start_ctx, chunk):
                 engine.step(cache, [StepEntry(rid, toks[s:s + chunk], [])])
         sync()
         t_fill = time.perf_counter() - t_fill
-        log(f"filled the cache: {batch} x {start_ctx} tokens in portions of {chunk} in {t_fill:.2f} s "
-            f"({batch * start_ctx / t_fill:.0f} tok/s, token generation on the host included)")
+        log(f"filled the cache: {batch} requests, {sum(starts)} tokens in portions of {chunk} in {t_fill:.2f} s "
+            f"({sum(starts) / t_fill:.0f} tok/s, token generation on the host included)")
+        if args.decode_order == "longest-first":
+            ids = [rid for _, rid in sorted(zip(starts, ids), key=lambda p: -p[0])]
         last = torch.randint(0, V, (batch,), generator=gen).tolist()
 
         # greedy decoding as `Engine.generate` runs it: every step's tokens feed the next on the device, and
@@ -343,7 +356,7 @@ def main() -> int:
         assert len(chosen) == steps and all(len(c) == batch for c in chosen)
         for rid in ids:
             cache.release(rid)
-        mean_ctx = start_ctx + warmup + (steps + 1) / 2.0
+        mean_ctx = sum(starts) / batch + warmup + (steps + 1) / 2.0
         return dt / steps, mean_ctx
 
     log(f"decode: batch {args.batch}, context {args.context}")
@@ -373,7 +386,7 @@ def main() -> int:
             "num_attention_heads": cfg["num_attention_heads"], "num_key_value_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "vocab_size": V, "tie_word_embeddings": cfg["tie_word_embeddings"],
             "rope": f"theta 5e5, llama3 scaling {cfg['rope_scaling']['factor']:g}/1/4/8192", "page_size": page,
-            "prefill_tokens": T, "decode_context": args.context, "sampling": "greedy",
+            "prefill_tokens": T, "decode_context": args.context_range or args.context, "sampling": "greedy",
         },
         "prefill": prefill, "roofline": roofline, "points": points,
     }

@@ -20,8 +20,12 @@
 //
 // Two kernels share this tile code:
 //  * decode: requests that bring one token. The 16 rows are the query heads of one kv
-//    head; grid (request, kv head x head tile, split of the keys); partial results of the
-//    splits are joined by a small second kernel.
+//    head; grid (kv head x head tile, request, split of the keys); partial results of the
+//    splits are joined by a small second kernel. The kv head runs fastest because workgroups
+//    go to the chip's 8 dies in turn: with the request fastest and a number of requests that
+//    is a multiple of 8, a die got all heads of every eighth request, and the dies' loads
+//    differed as the requests' lengths do (44 requests of 256 to 6,144 tokens at the 1B
+//    sizes: 2.45 -> 2.18 ms a step; requests of one length: no difference).
 //  * prefill: requests that bring several tokens. The rows are 16 consecutive tokens of one
 //    query head; a wavefront takes QT such tiles so that every K and V load is used QT
 //    times; a workgroup's four wavefronts take four neighbouring heads of the same tokens,
@@ -48,7 +52,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_kernel(
     int max_blocks, int n_q, int n_kv, int page, float scale, int window, int split_len, int nsplit) {
     __shared__ float sh[decode_lds_floats(HD)];
     decode_item<HD, STREAM>(q, k_cache, v_cache, out, part_o, part_ml, q_start, ctx_len, block_table, max_blocks, n_q,
-                            n_kv, page, scale, window, split_len, nsplit, blockIdx.x, blockIdx.y, blockIdx.z, sh);
+                            n_kv, page, scale, window, split_len, nsplit, blockIdx.y, blockIdx.x, blockIdx.z, sh);
 }
 
 // The same for a step whose q/k/v rows are still as the projection left them (RAW in attention_tiles.h):
@@ -62,7 +66,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void attention_decode_raw_kernel(
     __shared__ float sh[decode_lds_floats(HD)];
     const RawQkv raw{qkv, cos_t, sin_t, k_cache, v_cache};
     decode_item<HD, true, true>(nullptr, k_cache, v_cache, out, nullptr, nullptr, q_start, ctx_len, block_table,
-                                max_blocks, n_q, n_kv, page, scale, window, split_len, 1, blockIdx.x, blockIdx.y, 0, sh,
+                                max_blocks, n_q, n_kv, page, scale, window, split_len, 1, blockIdx.y, blockIdx.x, 0, sh,
                                 raw);
 }
 
@@ -305,7 +309,7 @@ static int launch_for_head(const bf16* q, const bf16* kc, const bf16* vc, bf16* 
     // tokens, one after the other they took 17.8 + 21.4 us a layer).
     const bool together = n_decode > 0 && prefill_groups > 0 && shared_rows > 0 && decode_reads_once(tuning);
     if (n_decode > 0 && !together) {
-        const dim3 grid(n_seq, head_tiles, nsplit);
+        const dim3 grid(head_tiles, n_seq, nsplit);
         if (decode_reads_once(tuning))
             hipLaunchKernelGGL((attention_decode_kernel<HD, true>), grid, dim3(DEC_WAVES * 64), 0, stream, q, kc, vc, out,
                                part_o, part_ml, q_start, ctx_len, table, max_blocks, n_q, n_kv, page, scale, window,
@@ -422,6 +426,7 @@ extern "C" int llme_attention_bf16(const void* q, const void* k_cache, const voi
     if (static_cast<double>(max_blocks) * (page / 16) * (page / 16) >= 4294967296.0) return kErrUnsupported;
     if (static_cast<double>(n_kv) * page * hd >= 4294967296.0) return kErrUnsupported;   // a page's elements: 32 bits
     if (n_decode > 0 && (split_len <= 0 || split_len % 32 != 0 || nsplit <= 0 || nsplit > 64)) return kErrBadArgument;
+    if (n_decode > 0 && n_seq > 65535) return kErrUnsupported;      // (the decode grid counts requests in y)
     if (tune.no_join && prefill_groups > 0) return kErrBadArgument;
     const int qt = direct_rows(hd, tune) / 16;
     const int shared_rows = shared_rows_for(hd, n_q, n_kv, tune);
@@ -456,12 +461,13 @@ extern "C" int llme_attention_decode_rope_bf16(float* qkv, const float* cos_t, c
     if (!qkv || !cos_t || !sin_t || !k_cache || !v_cache || !out || !q_start || !ctx_len || !block_table) return kErrBadArgument;
     if ((hd != 64 && hd != 128) || page % 16 != 0 || n_kv <= 0 || n_q % n_kv != 0 || n_q / n_kv > 16) return kErrUnsupported;
     if (!(scale > 0.f) || split_len <= 0 || split_len % 32 != 0) return kErrBadArgument;
+    if (n_seq > 65535) return kErrUnsupported;                      // (the grid counts requests in y)
     if (static_cast<double>(max_blocks) * (page / 16) * (page / 16) >= 4294967296.0) return kErrUnsupported;
     if (static_cast<double>(n_kv) * page * hd >= 4294967296.0) return kErrUnsupported;
     if (reinterpret_cast<uintptr_t>(qkv) % 16 != 0 || reinterpret_cast<uintptr_t>(cos_t) % 16 != 0 ||
         reinterpret_cast<uintptr_t>(sin_t) % 16 != 0 || reinterpret_cast<uintptr_t>(k_cache) % 16 != 0)
         return kErrUnsupported;
-    const dim3 grid(n_seq, n_kv);
+    const dim3 grid(n_kv, n_seq);
     if (hd == 64)
         hipLaunchKernelGGL(attention_decode_raw_kernel<64>, grid, dim3(DEC_WAVES * 64), 0, stream, qkv, cos_t, sin_t,
                            static_cast<bf16*>(k_cache), static_cast<bf16*>(v_cache), static_cast<bf16*>(out), q_start,

@@ -146,7 +146,14 @@ public:
             portions_.push_back({&s, n});             // (the prompt moves on in complete(), once the portion has run)
             budget -= n;
         }
-        // one token for every decoding request
+        // one token for every decoding request: pages are taken in the order in which the prompts ended;
+        // the entries then stand in the order of the requests' lengths, the longest first (which stays the
+        // same from step to step while nobody joins or leaves: every request grows by one). The decode
+        // kernels deal a step's requests out to the compute units in turn, so that where there are more
+        // requests than units a unit gets one of the longest together with one of the shortest (measured at
+        // the 1B sizes, lengths uniform in 256 .. 6,144: 44 requests 2.54 -> 2.16 ms a step, 72 requests
+        // 3.04 -> 2.79; up to 32 requests the order makes no difference).
+        decoding_.clear();
         for (auto& sp : running_) {
             Seq& s = *sp;
             if (s.state != kRunning) continue;
@@ -154,8 +161,12 @@ public:
                 finish(s, kCapacity);
                 continue;
             }
-            if (!add_entry(s, static_cast<long>(s.tokens.size()) - 1, 1, true, s.generated())) return LLME_HOST_BAD_ARGUMENT;
+            decoding_.push_back(&s);
         }
+        std::stable_sort(decoding_.begin(), decoding_.end(),
+                         [](const Seq* a, const Seq* b) { return a->tokens.size() > b->tokens.size(); });
+        for (Seq* s : decoding_)
+            if (!add_entry(*s, static_cast<long>(s->tokens.size()) - 1, 1, true, s->generated())) return LLME_HOST_BAD_ARGUMENT;
         planned_ = true;
         return E;
     }
@@ -257,6 +268,7 @@ private:
     std::deque<std::unique_ptr<Seq>> waiting_;
     std::vector<std::unique_ptr<Seq>> prefilling_, running_, results_;
     std::vector<Seq*> owners_, prompt_ends_, batch_;   // between plan() and complete(): who gets a token, whose prompt ends, who takes part
+    std::vector<Seq*> decoding_;                       // plan()'s own: the step's decoding requests while they are put in order
     std::vector<std::pair<Seq*, long>> portions_;  // prompt tokens that the planned step carries
 };
 

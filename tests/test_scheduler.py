@@ -112,6 +112,29 @@ def test_budget_is_shared_in_admission_order_and_excludes_decoding():
         assert sum(n for _, n in b) - decoding <= 7
 
 
+def test_decoding_requests_stand_longest_first_and_pages_go_in_admission_order():
+    """A step's decoded tokens come in the order of the requests' lengths (the decode kernels deal the
+    requests out in turn); the streams are the same, and when pages run out it is still the request that
+    came later which ends."""
+    prompts = [[1, 2], list(range(1, 12)), [3, 4, 5, 6], list(range(2, 9))]
+    s, eng, _ = run(prompts, 5)
+    seen = 0
+    for b in eng.batches:
+        decoding = [rid for rid, n in b if n == 1 and len(eng.history[rid]) > len(prompts[rid])]
+        if len(decoding) == 4:
+            assert decoding == [1, 3, 2, 0]
+            seen += 1
+    assert seen >= 3
+    for r, p in zip(s.results, prompts):
+        assert (r.token_ids, r.finish_reason) == single_generate(p, 5)
+    # 8 pages of 4, two requests that need their next page in the same steps (3 + t and 7 + t tokens): when one
+    # page is left, the request that came first takes it, though the other is longer and stands in front
+    s, eng, bm = run([[1, 2, 3], list(range(1, 8))], 12, blocks=(8, 4))
+    assert [r.finish_reason for r in s.results] == ["length", "capacity"]
+    assert s.results[0].token_ids == single_generate([1, 2, 3], 12)[0]
+    assert bm.free_blocks == bm.num_blocks
+
+
 @pytest.mark.parametrize("max_new", [0, 1, 2, 5])               # tests/test_scheduler.py:220-280
 def test_exact_counts(max_new):
     s, _, bm = run([[4, 5, 6]], max_new)
