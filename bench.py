@@ -237,9 +237,10 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096, help="context length the decode steps run at")
     ap.add_argument("--context-range", default="", help="decode: contexts drawn uniformly from [a, b] (seeded) instead "
                                                         "of --context for every request")
-    ap.add_argument("--decode-order", default="as-drawn", choices=["as-drawn", "longest-first"],
+    ap.add_argument("--decode-order", default="as-drawn", choices=["as-drawn", "longest-first", "rounds"],
                     help="decode with --context-range: the order of the requests in the batch (the scheduler puts "
                          "the longest first)")
+    ap.add_argument("--round", type=int, default=32, help="decode order 'rounds': requests per round")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes: Llama 3.2 1B (the default), 3.2 3B, 3.1 8B")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (named in config)")
@@ -343,6 +344,10 @@ def main() -> int:
             f"({sum(starts) / t_fill:.0f} tok/s, token generation on the host included)")
         if args.decode_order == "longest-first":
             ids = [rid for _, rid in sorted(zip(starts, ids), key=lambda p: -p[0])]
+        elif args.decode_order == "rounds":
+            from llmengine.engine.scheduler import rounds_order
+            by_length = sorted(range(batch), key=lambda i: -starts[i])
+            ids = [ids[by_length[i]] for i in rounds_order(batch, args.round)]
         last = torch.randint(0, V, (batch,), generator=gen).tolist()
 
         # greedy decoding as `Engine.generate` runs it: every step's tokens feed the next on the device, and

@@ -66,6 +66,7 @@ public:
     Scheduler(void* cm, int max_concurrent, long budget) : cm_(cm), max_concurrent_(max_concurrent), budget_(budget) {}
 
     void set_budget(long b) { budget_ = b; }
+    void set_decode_round(int requests) { decode_round_ = requests; }
     long budget() const { return budget_; }
     int max_concurrent() const { return max_concurrent_; }
 
@@ -165,6 +166,20 @@ public:
         }
         std::stable_sort(decoding_.begin(), decoding_.end(),
                          [](const Seq* a, const Seq* b) { return a->tokens.size() > b->tokens.size(); });
+        // Where the engine has said after how many requests its decode kernel has given every compute unit one
+        // (decode_round_), the requests are cut into such rounds and every other round, counted from the last,
+        // is reversed: the unit that got the shortest request of one round gets the longest of the next, and
+        // the last round, which may be short and so lands on the first units, meets the short end of the round
+        // before it (measured as above: 44 requests 2.03 -> 1.87 ms a step, 64: 2.30 -> 2.09, 96: 3.04 -> 2.89).
+        const size_t n_dec = decoding_.size(), per_round = static_cast<size_t>(decode_round_);
+        if (per_round > 0 && n_dec > per_round) {
+            const size_t rounds = (n_dec + per_round - 1) / per_round;
+            for (size_t back = 1; back < rounds; back += 2) {
+                const size_t r = rounds - 1 - back;      // (a full round: only the last can be short)
+                std::reverse(decoding_.begin() + static_cast<long>(r * per_round),
+                             decoding_.begin() + static_cast<long>((r + 1) * per_round));
+            }
+        }
         for (Seq* s : decoding_)
             if (!add_entry(*s, static_cast<long>(s->tokens.size()) - 1, 1, true, s->generated())) return LLME_HOST_BAD_ARGUMENT;
         planned_ = true;
@@ -263,6 +278,7 @@ private:
     void* cm_;
     int max_concurrent_;
     long budget_;
+    int decode_round_ = 0;                             // see set_decode_round
     int64_t next_id_ = 0;
     bool planned_ = false;
     std::deque<std::unique_ptr<Seq>> waiting_;
@@ -283,6 +299,13 @@ void* llme_sched_create(void* cache_manager, int max_concurrent, long budget) {
     return new Scheduler(cache_manager, max_concurrent, budget);
 }
 void llme_sched_destroy(void* h) { delete static_cast<Scheduler*>(h); }
+// requests > 0: the order of a step's decoding requests is made for a kernel that deals them out to that many
+// places in turn (see plan()); 0: longest first.
+int llme_sched_set_decode_round(void* h, int requests) {
+    if (requests < 0) return LLME_HOST_BAD_ARGUMENT;
+    static_cast<Scheduler*>(h)->set_decode_round(requests);
+    return 0;
+}
 int llme_sched_set_budget(void* h, long budget) {
     if (budget <= 0) return LLME_HOST_BAD_ARGUMENT;
     static_cast<Scheduler*>(h)->set_budget(budget);

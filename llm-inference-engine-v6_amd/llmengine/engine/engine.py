@@ -185,6 +185,16 @@ class Engine:
     def model(self):
         return self.runner.model
 
+    @property
+    def decode_round(self) -> int:
+        """What the scheduler orders a step's decoding requests by: the number that the model's first mixer
+        with such a number gives (Mixer.decode_round), 0 if none has one."""
+        for layer in self.model.layers:
+            n = int(getattr(layer, "mixer", None).decode_round()) if getattr(layer, "mixer", None) is not None else 0
+            if n > 0:
+                return n
+        return 0
+
     # ---- caches ----
     def new_cache(self, num_blocks: int, block_size: int | None = None, max_requests: int = 64) -> CacheContext:
         with torch.cuda.device(self.runner.device):

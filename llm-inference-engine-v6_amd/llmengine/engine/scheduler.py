@@ -33,6 +33,21 @@ from .step import StepCommittedError, StepEntry
 _REASONS = {1: "stop", 2: "length", 3: "capacity", 4: "error"}
 
 
+def rounds_order(n: int, per_round: int) -> list[int]:
+    """For n items ranked by size (rank 0 the largest) that are dealt out to per_round places in turn
+    (item at position p goes to place p % per_round): the rank to put at each position so that the places'
+    sums come out even. The ranks are cut into rounds of per_round; the last round, which may be short and so
+    lands on the first places, stands in its own order, the round before it reversed, and so on in turns: a
+    place that got the smallest of one round gets the largest of the next."""
+    if per_round <= 0 or n <= per_round:
+        return list(range(n))
+    rounds = [list(range(a, min(a + per_round, n))) for a in range(0, n, per_round)]
+    for back, ranks in enumerate(reversed(rounds)):
+        if back % 2 == 1:
+            ranks.reverse()
+    return [rank for ranks in rounds for rank in ranks]
+
+
 @dataclass
 class SequenceResult:
     seq_id: int
@@ -94,6 +109,9 @@ class ContinuousBatchScheduler:
         self._h = self._lib.llme_sched_create(self._cache.manager.handle, self.max_concurrent, self._budget)
         if not self._h:
             raise ValueError("ContinuousBatchScheduler: the scheduler refused its sizes")
+        # an engine whose decode kernel deals a step's requests out to the compute units in turn says after
+        # how many it has been round once (rounds_order)
+        self._lib.llme_sched_set_decode_round(self._h, max(0, int(getattr(engine, "decode_round", 0) or 0)))
         n = self.max_concurrent
         self._admitted = (ctypes.c_int * n)()
         self._entry_seq = (ctypes.c_int64 * n)()

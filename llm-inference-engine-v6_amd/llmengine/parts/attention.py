@@ -82,6 +82,12 @@ class Attention(Mixer):
                          paged={"k": (self.num_kv_heads, PAGE, self.head_dim),
                                 "v": (self.num_kv_heads, self.head_dim, PAGE)})
 
+    def decode_round(self) -> int:
+        # the decode kernels have a workgroup per request, kv head and 16 query heads of it, and workgroups
+        # go to the compute units in turn
+        tiles = self.num_kv_heads * ((self.num_heads // self.num_kv_heads + 15) // 16)
+        return max(1, ops.mfma.compute_units() // tiles)
+
     def fuses_norm(self, h, norm, step):
         # A few rows (decoding): the q/k/v projection applies the norm itself.
         rms = norm.fused_rms()

@@ -243,6 +243,12 @@ class Mixer(Part):
         norm. Parts that do not know about this are always given normed activations."""
         return False
 
+    def decode_round(self) -> int:
+        """After how many requests of a step of single decoded tokens the part's kernel has given every
+        compute unit one piece of work, where it deals the requests out in turn (a scheduler that knows
+        this can put long and short requests together); 0: no such number."""
+        return 0
+
     def forward(self, x: torch.Tensor, step, cache: LayerCache | None, out: torch.Tensor,
                 accumulate: bool, write_cache: bool = True) -> None:
         raise NotImplementedError

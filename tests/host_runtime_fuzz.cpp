@@ -35,6 +35,7 @@ long llme_cm_fill_step(void* h, int S, const int64_t* keys, const int* new_lens,
                        int* seq_idx, int* q_start, int* ctx_len, int* slots, int* tables);
 void* llme_sched_create(void* cache_manager, int max_concurrent, long budget);
 void llme_sched_destroy(void* h);
+int llme_sched_set_decode_round(void* h, int requests);
 long llme_sched_enqueue(void* h, const int* prompt, long n, long max_new_tokens);
 int llme_sched_idle(void* h);
 int llme_sched_plan(void* h, int* n_admitted, int* admitted_slots, int64_t* entry_seq, int* entry_count, int* entry_want,
@@ -170,6 +171,7 @@ static void fuzz_scheduler(int rounds) {
         void* cm = llme_cm_create(1, is_window, win, pages, page, max_concurrent);
         void* sc = llme_sched_create(cm, max_concurrent, budget);
         REQUIRE(cm && sc);
+        REQUIRE(llme_sched_set_decode_round(sc, -1) < 0 && llme_sched_set_decode_round(sc, pick(0, 4)) == 0);
         const int n_requests = pick(1, 14);
         std::vector<std::vector<int>> prompts;
         std::vector<long> max_new;

@@ -135,6 +135,43 @@ def test_decoding_requests_stand_longest_first_and_pages_go_in_admission_order()
     assert bm.free_blocks == bm.num_blocks
 
 
+def test_rounds_order_pairs_long_with_short():
+    from llmengine.engine.scheduler import rounds_order
+    assert rounds_order(3, 4) == [0, 1, 2] and rounds_order(4, 4) == [0, 1, 2, 3] and rounds_order(5, 0) == list(range(5))
+    assert rounds_order(7, 4) == [3, 2, 1, 0, 4, 5, 6]
+    assert rounds_order(10, 4) == [0, 1, 2, 3, 7, 6, 5, 4, 8, 9]
+    for n, per in [(44, 32), (64, 32), (72, 32), (9, 2), (100, 7)]:
+        order = rounds_order(n, per)
+        assert sorted(order) == list(range(n))
+        sizes = [1000 - 7 * r for r in range(n)]                      # rank 0 the largest
+        places = [sum(sizes[order[p]] for p in range(j, n, per)) for j in range(per)]
+        plain = [sum(sizes[p] for p in range(j, n, per)) for j in range(per)]
+        assert max(places) <= max(plain) and max(places) - min(places) <= max(plain) - min(plain)
+
+
+def test_the_engine_names_the_round_and_the_scheduler_orders_by_it():
+    """An engine that says after how many requests its decode kernel has been round the compute units once gets
+    its decoding requests in rounds_order of their lengths; the streams do not change."""
+    from llmengine.engine.scheduler import rounds_order
+    prompts = [list(range(1, 2 + 2 * i)) for i in range(7)]           # lengths 1, 3, .. 13: request 6 the longest
+    eng = FakeEngine()
+    eng.decode_round = 3
+    s = ContinuousBatchScheduler(eng, FakeBlocks(64, 4))
+    for p in prompts:
+        s.enqueue(p, 6)
+    s.run_until_idle()
+    by_length = [6, 5, 4, 3, 2, 1, 0]
+    seen = 0
+    for b in eng.batches:
+        decoding = [rid for rid, n in b if n == 1 and len(eng.history[rid]) > len(prompts[rid])]
+        if len(decoding) == 7:
+            assert decoding == [by_length[r] for r in rounds_order(7, 3)]
+            seen += 1
+    assert seen >= 3
+    for r, p in zip(s.results, prompts):
+        assert (r.token_ids, r.finish_reason) == single_generate(p, 6)
+
+
 @pytest.mark.parametrize("max_new", [0, 1, 2, 5])               # tests/test_scheduler.py:220-280
 def test_exact_counts(max_new):
     s, _, bm = run([[4, 5, 6]], max_new)
