@@ -259,6 +259,8 @@ def main() -> int:
     ap.add_argument("--prefill-budget", type=int, default=2048, help="serve: max_prefill_tokens_per_step")
     ap.add_argument("--max-concurrent", type=int, default=32, help="serve: live requests at a time")
     ap.add_argument("--temperature", type=float, default=0.0, help="serve: sampling temperature (0 is greedy)")
+    ap.add_argument("--choices", default="", help="fields of llmengine.ops.KernelChoices to set, name=value,... "
+                                                  "(for comparisons: which kernels and launch plans the steps may use)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -273,7 +275,19 @@ def main() -> int:
     wbytes = 2 if args.dtype == "bf16" else 4
     t0 = time.time()
     log(f"building the model ({args.layers} layers, {args.dtype}) with random weights")
-    engine = Engine.from_random(cfg, args.seed, args.dtype, std=0.02)
+    choices = None
+    if args.choices:
+        from llmengine.ops import KernelChoices
+        choices = KernelChoices()
+        for item in args.choices.split(","):
+            name, _, value = item.partition("=")
+            if not hasattr(choices, name.strip()):
+                raise SystemExit(f"--choices: KernelChoices has no field {name.strip()!r}")
+            old = getattr(choices, name.strip())
+            value = value.strip()
+            setattr(choices, name.strip(), None if value == "None" else (value == "True") if isinstance(old, bool)
+                    else float(value) if isinstance(old, float) else int(value))
+    engine = Engine.from_random(cfg, args.seed, args.dtype, std=0.02, kernel_choices=choices)
     runner = engine.runner
     log(f"model on the device after {time.time() - t0:.1f} s")
     gen = torch.Generator().manual_seed(args.seed + 1)

@@ -173,6 +173,8 @@ class StepContext:
     # sum has one fixed order, and a step gives the same bits every time it runs.
     fixed_order: bool = False
     extra: dict = field(default_factory=dict)          # per-step notes of kernels (launch plans)
+    # a recorded step: what the parts said of their plans when the runner chose the recording (Mixer.decode_plan_hint)
+    plan_hints: dict = field(default_factory=dict)
     choices: "ops.KernelChoices | None" = None          # which kernels the operations may choose (the runner's)
 
     def buffer(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
@@ -404,20 +406,31 @@ class ModelRunner:
         recorded once as a HIP graph and replayed; only the integer arrays change."""
         mgr = cache.manager
         lengths = [mgr.length(e.request_id) for e in entries]
-        rec = self._decode_record(cache, entries, max(lengths), choose=None)
+        hints = self._decode_hints(cache, lengths)
+        rec = self._decode_record(cache, entries, max(lengths), choose=None, hints=hints)
         rec.refresh(mgr, entries)
         rec.graph.replay()
         self.graph_replays += 1
         return rec.logits
 
-    def _decode_key(self, cache: CacheContext, S: int, longest: int, choose: str | None):
+    def _decode_width(self, cache: CacheContext, longest: int) -> int:
         need = (longest + cache.page_size) // cache.page_size
         bucket = self.GRAPH_BLOCK_BUCKET
-        # (a recording holds the launches that the choices of its time led to)
-        return (S, (need + bucket - 1) // bucket * bucket, choose, self.choices.key())
+        return (need + bucket - 1) // bucket * bucket
+
+    def _decode_hints(self, cache: CacheContext, lengths: Sequence[int]) -> tuple:
+        """What the parts' launch plans make of these lengths (tokens cached before the step), for a step
+        recorded at the width of block table that the longest needs."""
+        width = self._decode_width(cache, max(lengths))
+        return self.model.decode_plan_hints([int(n) + 1 for n in lengths], width * cache.page_size, self.choices)
+
+    def _decode_key(self, cache: CacheContext, S: int, longest: int, choose: str | None, hints: tuple = ()):
+        # (a recording holds the launches that the choices of its time led to, and those that the parts
+        # planned from the requests' lengths: hints)
+        return (S, self._decode_width(cache, longest), choose, self.choices.key(), hints)
 
     def _decode_record(self, cache: CacheContext, entries: Sequence[StepEntry] | None, longest: int,
-                       choose: str | None, S: int | None = None):
+                       choose: str | None, S: int | None = None, hints: tuple = ()):
         """The recording for this many requests and this width of block tables. choose None: it ends
         at the logits. "greedy": the argmax is behind the model, its result written into pinned host
         memory. "sampled": the sampling kernels instead, with a temperature and a uniform draw per
@@ -426,7 +439,7 @@ class ModelRunner:
         page = cache.page_size
         mgr = cache.manager
         S = len(entries) if S is None else S
-        key = self._decode_key(cache, S, longest, choose)
+        key = self._decode_key(cache, S, longest, choose, hints)
         width = key[1]
         rec = cache.graphs.pop(key, None)
         if rec is not None:
@@ -444,6 +457,7 @@ class ModelRunner:
             total = 7 * S + 1 + groups * S * width
             meta = torch.zeros(total + 1 + 2 * S + 64, dtype=torch.int32, device=self.device)
             ctx, logit_rows = self._build_context(cache, entries, max_blocks=width, plan_len=width * page, dev=meta)
+            ctx.plan_hints = dict(hints)
             tok_host = scratch = temp_dev = uni_dev = None
             if choose == "sampled":
                 temp_dev = meta[total + 1:total + 1 + S].view(torch.float32)
@@ -544,7 +558,9 @@ class ModelRunner:
             if last is None or last[1] != list(ids):
                 return None
             longest = max(mgr.length(r) for r in ids)
-            if self._decode_key(cache, S, longest, choose) != last[2] or cache.graphs.get(last[2]) is not last[0]:
+            # (the chain keeps the plan it began with: every request has grown by one since)
+            if (self._decode_key(cache, S, longest, choose, last[2][-1]) != last[2]
+                    or cache.graphs.get(last[2]) is not last[0]):
                 return None
         # lengths, the position limit and the pages in one call; a call that fails has changed nothing
         rc = mgr._lib.llme_cm_decode_begin(mgr.handle, S, keys, lengths, int(max_position or 0))
@@ -557,11 +573,13 @@ class ModelRunner:
             need = {g: sum(mgr.pages_needed(r, 1)[g] for r in ids) for g in mgr.groups}
             raise CapacityError(f"the step needs {need} more pages, free are "
                                 f"{({g: mgr.free_pages(g) for g in mgr.groups})}")
-        key = self._decode_key(cache, S, longest, choose)
+        hints = cache.chain[2][-1] if tokens is None else self._decode_hints(cache, lengths)
+        key = self._decode_key(cache, S, longest, choose, hints)
         if key in cache.graphs or tokens is None:
-            rec = self._decode_record(cache, None, longest, choose, S=S)
+            rec = self._decode_record(cache, None, longest, choose, S=S, hints=hints)
         else:                                   # (a new recording is made from entries)
-            rec = self._decode_record(cache, [StepEntry(r, [t], [0]) for r, t in zip(ids, tokens)], longest, choose)
+            rec = self._decode_record(cache, [StepEntry(r, [t], [0]) for r, t in zip(ids, tokens)], longest, choose,
+                                      hints=hints)
         slot = 1 - rec.slot
         rec.refresh(mgr, None, keys, slot=slot, tokens=tokens, temperature=float(temperature or 0.0), uniforms=uniforms)
         rec.graph.replay()

@@ -80,6 +80,26 @@ class DecoderModel(Part):
     def hidden_size(self) -> int:
         return self.embedding.hidden_size
 
+    def decode_plan_hints(self, lens: list[int], plan_len: int, choices) -> tuple:
+        """What of the layers' launch plans for a step of single decoded tokens depends on the requests'
+        lengths: the mixers' hints (Mixer.decode_plan_hint), each name once, in a fixed order."""
+        hints: dict = {}
+        asked = set()
+        for call in self.schedule:
+            mixer = getattr(self.layers[call.layer], "mixer", None)
+            if mixer is None or id(mixer) in asked:
+                continue
+            asked.add(id(mixer))
+            sig = getattr(mixer, "plan_signature", None)
+            if sig is not None:
+                if sig in asked:
+                    continue
+                asked.add(sig)
+            hint = mixer.decode_plan_hint(lens, plan_len, choices)
+            if hint is not None:
+                hints[hint[0]] = hint[1]
+        return tuple(sorted(hints.items()))
+
     # ---- the forward pass of one step ----
     def forward(self, step, caches, logit_rows: torch.Tensor | None) -> torch.Tensor | None:
         """Runs the step's tokens through the schedule; returns 32-bit logits

@@ -37,6 +37,22 @@ class KernelChoices:
     # of an MI355X at batch 8 and a context of 4,096: 0.948 ms a step with 256, 0.969 with 512, 0.998
     # with 1,024, 1.036 with 128; with 384 (one and a half per compute unit) 1.000.
     decode_blocks_wanted: int | None = None
+    # Decoding with more workgroups than half the compute units (from 17 requests on with 8 kv heads), where one
+    # per compute unit leaves the keys whole: the keys are cut where the host runtime's estimate says so
+    # (ops.mfma.decode_cut, csrc/host/decode_plan.cpp). Measured at the 1B sizes (ms a step, keys whole / cut),
+    # requests of one length: a context of 8,192: 17 requests 2.061 / 1.840 (5 splits), 20: 2.103 / 1.954 (3),
+    # 24: 2.129 / 2.088 (4), 28 and 32: whole is best, 33: 3.170 / 2.618 (6), 40: 3.384 / 2.889 (4), 48: 3.681 /
+    # 3.179 (2), 56 and 64: whole, 72: 5.071 / 4.664 (3); a context of 2,048: whole is best or equal everywhere
+    # (17 requests 1.186 / 1.218, 33: 1.511 / 1.496); 16,384: 17 requests 3.171 / 2.556, 33: 5.440 / 4.049.
+    decode_cut_most: int = 8            # splits at most (1: never cut)
+    decode_cut_tbs: float = 6.0         # TB/s the keys stream at where the compute units share them evenly
+    decode_cut_key_ns: float = 9.5      # ns a compute unit needs per key of a head of 64 that it is given
+    decode_cut_lone_ns: float = 8.3     # the same for a unit's only piece where others hold two (it ends on a draining chip)
+    decode_cut_piece_us: float = 0.5    # and per piece
+    decode_cut_join_us: float = 4.6     # a cut costs the join kernel (17 requests and more)
+    decode_cut_rope_us: float = 4.8     # and the rotation kernel, where the single split would have rotated itself
+    decode_cut_each_us: float = 1.0     # and this per split
+    decode_cut_gain: float = 0.05       # and must promise this fraction of the whole keys' time
     # Portions of prompts: work items (a span of rows x a group of heads) the prefill kernel should
     # have at least (None: two per compute unit, three where the step has more than half a compute unit's
     # number already); with prefill_cut_items or fewer (None: three quarters of the compute units' number;

@@ -208,11 +208,12 @@ def attention_bf16_supported(q, k_cache, head_dim: int) -> bool:
 
 
 def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_len: int | None = None,
-                   tuning: int = 0, choices: KernelChoices | None = None) -> dict:
+                   tuning: int = 0, choices: KernelChoices | None = None, cut: int | None = None) -> dict:
     """Launch sizes for a step, from how its batch is cut (host-side numbers only). plan_len:
     plan the decode splits for requests of up to this many tokens, whatever their length now
     (a recorded step is replayed while the requests grow). tuning: see attention_tuning. choices:
-    the sizes at which the plan changes its shape."""
+    the sizes at which the plan changes its shape. cut: what decode_cut said for this step, where the caller
+    has asked already (a recorded step is kept under it)."""
     ch = choices or DEFAULT
     rows = entry("llme_attention_bf16_rows")(head_dim, n_q, n_kv, tuning)
     if rows <= 0:
@@ -255,9 +256,58 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
         longest = max(decode) if plan_len is None else max(plan_len, max(decode))
         pairs = len(decode) * n_kv * ((n_q // n_kv + 15) // 16)
         nsplit = max(1, min((ch.decode_blocks_wanted or compute_units()) // pairs, (longest + MIN_SPLIT - 1) // MIN_SPLIT, MAX_SPLITS))
+        if not groups:
+            # (a step of decoded tokens only, many of them: by where the pieces land)
+            n = cut if cut is not None else decode_cut(decode, n_q, n_kv, head_dim, plan_len, ch)
+            if n is not None:
+                nsplit = max(1, min(n, (longest + MIN_SPLIT - 1) // MIN_SPLIT, MAX_SPLITS))
         split_len = ((longest + nsplit - 1) // nsplit + 31) // 32 * 32
         plan["split_len"] = split_len
         plan["nsplit"] = (longest + split_len - 1) // split_len
+    return plan
+
+
+def decode_cut(lens, n_q: int, n_kv: int, head_dim: int, plan_len: int | None = None,
+               choices: KernelChoices | None = None) -> int | None:
+    """Into how many splits a step of single decoded tokens cuts its keys (lens: the keys each request sees,
+    in the step's order), where a workgroup per request, kv head and 16 query heads is more than half the
+    compute units, so that filling the units once would leave the keys whole: the host runtime's estimate
+    (csrc/host/decode_plan.cpp) from where the pieces land. None where the units fill without it (fewer
+    workgroups: plan_attention cuts to one workgroup per unit)."""
+    ch = choices or DEFAULT
+    units = ch.decode_blocks_wanted or compute_units()
+    tiles = n_kv * ((n_q // n_kv + 15) // 16)
+    S = len(lens)
+    if S == 0 or 2 * S * tiles <= units:
+        return None
+    longest = max(lens)
+    rotates = (ch.decode_rope and GEMV_NORM_MAX_ROWS < S <= qkv_sum_max_rows(True, head_dim, ch)
+               and (head_dim == 64 or (head_dim == 128 and S * tiles <= compute_units())))
+    apart_us = (ch.decode_cut_join_us if S > GEMV_NORM_MAX_ROWS else 0.0) + (ch.decode_cut_rope_us if rotates else 0.0)
+    from ..runtime import native
+    n = native.library().llme_decode_cut((ctypes.c_int * S)(*lens), S, tiles, units, head_dim,
+                                         max(longest, plan_len or 0), ch.decode_cut_most, ch.decode_cut_tbs,
+                                         ch.decode_cut_key_ns, ch.decode_cut_lone_ns, ch.decode_cut_piece_us, apart_us,
+                                         ch.decode_cut_each_us,
+                                         ch.decode_cut_gain)
+    if n < 1:
+        raise kernels.KernelError(f"decode_cut: the host runtime refused its arguments (code {n})")
+    return n
+
+
+def cut_hint_name(n_q: int, n_kv: int, head_dim: int) -> tuple:
+    """The name under which a recorded step is told its decode_cut (step.plan_hints)."""
+    return ("attention_cut", n_q, n_kv, head_dim)
+
+
+def _step_plan(step, n_q: int, n_kv: int, head_dim: int) -> dict:
+    """The step's attention plan for these head counts, made once per step."""
+    key = ("attention_plan", n_q, n_kv, head_dim)
+    plan = step.extra.get(key)
+    if plan is None:
+        cut = (getattr(step, "plan_hints", None) or {}).get(cut_hint_name(n_q, n_kv, head_dim))
+        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len,
+                                                choices=choices_of(step), cut=cut)
     return plan
 
 
@@ -306,11 +356,7 @@ def attention_bf16(q, k_cache, v_cache, out, q_start, ctx_len, block_table, n_q:
 def _fast_attention(q, k_cache, v_cache, out, step, block_table, n_q, n_kv, head_dim, scale, window) -> bool:
     if not attention_bf16_supported(q, k_cache, head_dim) or out.dtype != torch.bfloat16:
         return False
-    key = ("attention_plan", n_q, n_kv, head_dim)
-    plan = step.extra.get(key)
-    if plan is None:
-        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len,
-                                                      choices=choices_of(step))
+    plan = _step_plan(step, n_q, n_kv, head_dim)
     part_o = part_ml = None
     if plan["n_decode"] and plan["nsplit"] > 1:
         S = step.num_seqs
@@ -360,11 +406,7 @@ def _fast_attention_project(q, k_cache, v_cache, o, step, block_table, n_q, n_kv
             or out.dtype != torch.float32 or w_o.dtype != torch.bfloat16 or not kernels.is_blocked(w_o)
             or not attention_bf16_supported(q, k_cache, head_dim) or o.dtype != torch.bfloat16):
         return False
-    key = ("attention_plan", n_q, n_kv, head_dim)
-    plan = step.extra.get(key)
-    if plan is None:
-        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len,
-                                                      choices=choices_of(step))
+    plan = _step_plan(step, n_q, n_kv, head_dim)
     N, K = kernels.weight_shape(w_o)
     if (plan["n_decode"] != T or plan["groups"] or plan["nsplit"] <= 1 or K != n_q * head_dim
             or not entry("llme_attention_join_project_pays")(T, n_q, head_dim, plan["nsplit"], N)):
@@ -397,11 +439,7 @@ def attention_decode_rope(qkv, cos, sin, k_cache, v_cache, out, step, block_tabl
             or k_cache.shape[2] % 16 or qkv.data_ptr() % 16 or cos.data_ptr() % 16 or sin.data_ptr() % 16
             or k_cache.data_ptr() % 16):
         return False
-    key = ("attention_plan", n_q, n_kv, head_dim)
-    plan = step.extra.get(key)
-    if plan is None:
-        plan = step.extra[key] = plan_attention(step.new_lens, step.ctx_lens, n_q, n_kv, head_dim, step.plan_len,
-                                                      choices=choices_of(step))
+    plan = _step_plan(step, n_q, n_kv, head_dim)
     if plan["n_decode"] != T or plan["groups"] or plan["nsplit"] != 1:
         return False
     # (measured, ms a decode step at a context of 2,048, apart / inside: 1B sizes 1.238 / 1.203 at 17 requests,

@@ -33,6 +33,8 @@ class Attention(Mixer):
         self.position = position
         self.scale = float(scale) if scale is not None else float(head_dim) ** -0.5
         self.window = int(window)
+        # (layers with the same head counts have the same launch plans: a model asks one of them)
+        self.plan_signature = ("attention", int(num_heads), int(num_kv_heads), int(head_dim))
         self.q_dim = self.num_heads * self.head_dim
         self.kv_dim = self.num_kv_heads * self.head_dim
         self.w_qkv: torch.Tensor | None = None
@@ -87,6 +89,10 @@ class Attention(Mixer):
         # go to the compute units in turn
         tiles = self.num_kv_heads * ((self.num_heads // self.num_kv_heads + 15) // 16)
         return max(1, ops.mfma.compute_units() // tiles)
+
+    def decode_plan_hint(self, lens, plan_len, choices):
+        n = ops.mfma.decode_cut(lens, self.num_heads, self.num_kv_heads, self.head_dim, plan_len, choices)
+        return None if n is None else (ops.mfma.cut_hint_name(self.num_heads, self.num_kv_heads, self.head_dim), n)
 
     def fuses_norm(self, h, norm, step):
         # A few rows (decoding): the q/k/v projection applies the norm itself.

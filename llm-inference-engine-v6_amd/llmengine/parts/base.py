@@ -249,6 +249,14 @@ class Mixer(Part):
         this can put long and short requests together); 0: no such number."""
         return 0
 
+    def decode_plan_hint(self, lens: list[int], plan_len: int, choices) -> tuple | None:
+        """For a step of single decoded tokens that is recorded once and replayed: what of the part's launch
+        plan depends on the requests' lengths (lens: the keys each sees, in the step's order; plan_len: the
+        length the recording is made for), as a pair (name of the plan, value), both hashable. The runner
+        keeps one recording per value and hands the pair back in `step.plan_hints[name]` when it records.
+        None: the part's launches depend on nothing but the step's shape."""
+        return None
+
     def forward(self, x: torch.Tensor, step, cache: LayerCache | None, out: torch.Tensor,
                 accumulate: bool, write_cache: bool = True) -> None:
         raise NotImplementedError

@@ -36,6 +36,8 @@ long llme_cm_fill_step(void* h, int S, const int64_t* keys, const int* new_lens,
 void* llme_sched_create(void* cache_manager, int max_concurrent, long budget);
 void llme_sched_destroy(void* h);
 int llme_sched_set_decode_round(void* h, int requests);
+int llme_decode_cut(const int* lens, int S, int tiles, int units, int head_dim, long plan_len, int most, double tbs,
+                    double key_ns, double lone_ns, double piece_us, double apart_us, double each_us, double gain);
 long llme_sched_enqueue(void* h, const int* prompt, long n, long max_new_tokens);
 int llme_sched_idle(void* h);
 int llme_sched_plan(void* h, int* n_admitted, int* admitted_slots, int64_t* entry_seq, int* entry_count, int* entry_want,
@@ -277,12 +279,27 @@ static void run_plain_model() {
                                      positions.data(), T, logits.data()) < 0);
 }
 
+// ---- the decode plan: any sizes, a number of splits within its bounds ----
+static void fuzz_decode_plan(int rounds) {
+    for (int round = 0; round < rounds; ++round) {
+        const int S = pick(1, 300), tiles = pick(1, 40), units = pick(1, 400), most = pick(1, 70);
+        std::vector<int> lens(static_cast<size_t>(S));
+        for (int& n : lens) n = pick(0, pick(0, 1) ? 200000 : 700);
+        const long plan_len = pick(0, 1) ? pick(1, 300000) : 1;
+        const int n = llme_decode_cut(lens.data(), S, tiles, units, 16 * pick(1, 8), plan_len, most, 6.0, 9.5, 8.3, 0.5,
+                                      pick(0, 20), 1.0, 0.05);
+        REQUIRE(n >= 1 && n <= most && n <= 64);
+        REQUIRE(n == 1 || static_cast<long>(S) * tiles * n <= 10L * units);
+    }
+}
+
 int main(int argc, char** argv) {
     const int rounds = argc > 1 ? std::atoi(argv[1]) : 40;
     if (argc > 2) rng.seed(static_cast<unsigned>(std::atoi(argv[2])));
     fuzz_cache_manager(rounds);
     fuzz_scheduler(rounds * 5);
     run_plain_model();
+    fuzz_decode_plan(rounds * 20);
     std::printf("ok\n");
     return 0;
 }

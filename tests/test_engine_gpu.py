@@ -396,6 +396,55 @@ def test_twenty_decoded_tokens_are_rotated_inside_the_attention_kernel(zoo, name
             assert np.abs(got[rid][pos].astype(np.float64) - apart[rid][pos]).max() / top < 2e-3, (rid, pos)
 
 
+def test_many_decoded_tokens_with_their_keys_cut_by_the_host_plan(zoo, monkeypatch):
+    """More workgroups than half the compute units: the host runtime decides from the requests' lengths whether
+    the keys are cut (ops.mfma.decode_cut), and a recorded step is kept under what it said. Made to cut here
+    (few units, a cut that costs nothing): the steps must have been planned with several splits, match the plain
+    implementation, and match the same steps with the keys whole."""
+    from llmengine.ops import mfma
+    plans = []
+    planning = mfma.plan_attention
+
+    def noting(*args, **kw):
+        plan = planning(*args, **kw)
+        plans.append((plan["n_decode"], plan["nsplit"]))
+        return plan
+    monkeypatch.setattr(mfma, "plan_attention", noting)
+    model_dir, _, _, page = zoo["C"]
+    cfg = TINY_C
+    reqs = {f"s{i}": random_tokens(300 + 80 * (i % 7) + i, cfg["vocab_size"], 400 + i) for i in range(20)}
+    pcfg, pw = load_plain_model(model_dir)
+    engine = engine_for(model_dir, "bf16")
+    ch = engine.runner.choices
+    for name, value in (("decode_blocks_wanted", 32), ("decode_cut_join_us", 0.0), ("decode_cut_rope_us", 0.0),
+                        ("decode_cut_each_us", 0.0), ("decode_cut_gain", 0.0), ("decode_cut_piece_us", 0.0),
+                        ("decode_cut_lone_ns", ch.decode_cut_key_ns)):
+        monkeypatch.setattr(ch, name, value)
+    steps = [{"step": 0, "entries": [{"id": rid, "tokens": ids[:-10], "want": []} for rid, ids in reqs.items()], "end": []}]
+    for t in range(10, 0, -1):
+        steps.append({"step": len(steps), "end": list(reqs) if t == 1 else [],
+                      "entries": [{"id": rid, "tokens": [ids[-t]], "want": [0]} for rid, ids in reqs.items()]})
+    pages = replay.trace_peak_tokens(steps, round_to=page) // page
+
+    def run():
+        cache = engine.new_cache(pages, page, max_requests=20)
+        return replay.run_trace(engine, cache, steps)
+    got = run()
+    assert any(n == 20 and splits > 1 for n, splits in plans), plans
+    del plans[:]
+    monkeypatch.setattr(ch, "decode_cut_most", 1)
+    whole = run()
+    assert plans and all(splits == 1 for n, splits in plans if n == 20), plans
+    for rid, ids in reqs.items():
+        ref = plain_forward(pcfg, pw, ids, rounder=bf16_round).numpy()
+        for pos in range(len(ids) - 10, len(ids)):
+            top = np.abs(ref[pos]).max()
+            assert np.abs(got[rid][pos].astype(np.float64) - ref[pos]).max() / top < TOL["bf16"], (rid, pos)
+            # (other splits round the softmax weights against other running maxima: a few bfloat16 roundings
+            # apart, far from what a lost or doubled split would do)
+            assert np.abs(got[rid][pos].astype(np.float64) - whole[rid][pos]).max() / top < 1e-2, (rid, pos)
+
+
 @pytest.mark.parametrize("dtype,deterministic", [("fp32", False), ("bf16", True)])
 def test_greedy_chain_equals_steps_fetched_one_by_one(zoo, dtype, deterministic):
     """Steps launched before the tokens of the step before them are fetched (the tokens stay on the
