@@ -28,15 +28,17 @@ extern "C" {
 
 // lens [S]: the keys each request sees in this step, in the step's order. plan_len: the length the
 // splits are laid out for (at least the longest; a recorded step is replayed while its requests grow).
-// tiles: workgroups per request and split; units: compute units. most: splits at most.
+// tiles: workgroups per request and split; units: compute units. first: the number of splits that stands
+// unless another promises more (1: the keys whole); most: splits at most (>= first).
 // tbs: TB/s of the even stream; key_ns: ns a place needs per key of a head of 64 (scaled by the head
 // size), lone_ns: the same for a place's only piece of an uncut step that has more workgroups than units;
 // piece_us: per piece on a place; apart_us: what any cut costs; each_us: what every split costs;
 // gain: a cut must promise this fraction. Returns the number of splits (>= 1), or an error code.
-int llme_decode_cut(const int* lens, int S, int tiles, int units, int head_dim, long plan_len, int most, double tbs,
-                    double key_ns, double lone_ns, double piece_us, double apart_us, double each_us, double gain) {
+int llme_decode_cut(const int* lens, int S, int tiles, int units, int head_dim, long plan_len, int first, int most,
+                    double tbs, double key_ns, double lone_ns, double piece_us, double apart_us, double each_us,
+                    double gain) {
     if (!lens || S <= 0 || tiles <= 0 || units <= 0 || head_dim <= 0 || plan_len <= 0 || !(tbs > 0.0) || !(key_ns > 0.0) ||
-        !(lone_ns > 0.0))
+        !(lone_ns > 0.0) || first < 1 || first > 64)
         return LLME_HOST_BAD_ARGUMENT;
     long longest = 0;
     double total = 0.0;
@@ -71,9 +73,9 @@ int llme_decode_cut(const int* lens, int S, int tiles, int units, int head_dim, 
         }
         return std::max(even_us, busiest) + (n > 1 ? apart_us + each_us * n : 0.0);
     };
-    int best = 1;
-    double best_us = estimate(1) * (1.0 - gain);
-    for (int n = 2; n <= most && n <= 64; ++n) {
+    int best = first;
+    double best_us = estimate(first) * (1.0 - gain);
+    for (int n = first + 1; n <= most && n <= 64; ++n) {
         if (static_cast<long>(S) * tiles * n > 10L * units) break;        // (measured up to 9 workgroups a unit)
         if (plan_len / n < 256) break;                                    // (a split of fewer keys is all start-up)
         const double us = estimate(n);

@@ -270,26 +270,31 @@ def plan_attention(new_lens, ctx_lens, n_q: int, n_kv: int, head_dim: int, plan_
 def decode_cut(lens, n_q: int, n_kv: int, head_dim: int, plan_len: int | None = None,
                choices: KernelChoices | None = None) -> int | None:
     """Into how many splits a step of single decoded tokens cuts its keys (lens: the keys each request sees,
-    in the step's order), where a workgroup per request, kv head and 16 query heads is more than half the
-    compute units, so that filling the units once would leave the keys whole: the host runtime's estimate
-    (csrc/host/decode_plan.cpp) from where the pieces land. None where the units fill without it (fewer
-    workgroups: plan_attention cuts to one workgroup per unit)."""
+    in the step's order): the host runtime's estimate (csrc/host/decode_plan.cpp) from where the pieces land
+    on the compute units. Asked where a workgroup per request, kv head and 16 query heads is more than half
+    the compute units, so that filling the units once would leave the keys whole, and where filling them once
+    takes 2 to 6 splits, which one or two more may beat when the requests differ in length (the short ones'
+    last pieces are empty). None otherwise (few workgroups: plan_attention cuts to one workgroup per unit)."""
     ch = choices or DEFAULT
     units = ch.decode_blocks_wanted or compute_units()
     tiles = n_kv * ((n_q // n_kv + 15) // 16)
     S = len(lens)
-    if S == 0 or 2 * S * tiles <= units:
+    if S == 0 or ch.decode_cut_most <= 1:
         return None
-    longest = max(lens)
-    rotates = (ch.decode_rope and GEMV_NORM_MAX_ROWS < S <= qkv_sum_max_rows(True, head_dim, ch)
+    longest = max(max(lens), plan_len or 0)
+    first = max(1, min(units // (S * tiles), (longest + MIN_SPLIT - 1) // MIN_SPLIT, MAX_SPLITS))
+    if first > 6:
+        return None
+    most = ch.decode_cut_most if first == 1 else min(first + 2, MAX_SPLITS)
+    rotates = (first == 1 and ch.decode_rope and GEMV_NORM_MAX_ROWS < S <= qkv_sum_max_rows(True, head_dim, ch)
                and (head_dim == 64 or (head_dim == 128 and S * tiles <= compute_units())))
-    apart_us = (ch.decode_cut_join_us if S > GEMV_NORM_MAX_ROWS else 0.0) + (ch.decode_cut_rope_us if rotates else 0.0)
+    apart_us = 0.0
+    if first == 1:
+        apart_us = (ch.decode_cut_join_us if S > GEMV_NORM_MAX_ROWS else 0.0) + (ch.decode_cut_rope_us if rotates else 0.0)
     from ..runtime import native
-    n = native.library().llme_decode_cut((ctypes.c_int * S)(*lens), S, tiles, units, head_dim,
-                                         max(longest, plan_len or 0), ch.decode_cut_most, ch.decode_cut_tbs,
-                                         ch.decode_cut_key_ns, ch.decode_cut_lone_ns, ch.decode_cut_piece_us, apart_us,
-                                         ch.decode_cut_each_us,
-                                         ch.decode_cut_gain)
+    n = native.library().llme_decode_cut((ctypes.c_int * S)(*lens), S, tiles, units, head_dim, longest, first, most,
+                                         ch.decode_cut_tbs, ch.decode_cut_key_ns, ch.decode_cut_lone_ns,
+                                         ch.decode_cut_piece_us, apart_us, ch.decode_cut_each_us, ch.decode_cut_gain)
     if n < 1:
         raise kernels.KernelError(f"decode_cut: the host runtime refused its arguments (code {n})")
     return n

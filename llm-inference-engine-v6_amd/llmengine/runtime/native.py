@@ -140,7 +140,7 @@ _SIGNATURES = {
     "llme_sched_result_info": (_i, [_vp, _i, _pi64, _pl, _pl, _pi]), "llme_sched_result_tokens": (_i, [_vp, _i, _pi]),
     "llme_sched_clear_results": (None, [_vp]), "llme_sched_abort": (None, [_vp]), "llme_sched_fail": (_i, [_vp]),
     # launch planning (csrc/host/decode_plan.cpp)
-    "llme_decode_cut": (_i, [_pi, _i, _i, _i, _i, _l, _i, _d, _d, _d, _d, _d, _d, _d]),
+    "llme_decode_cut": (_i, [_pi, _i, _i, _i, _i, _l, _i, _i, _d, _d, _d, _d, _d, _d, _d]),
     # plain C++ twins of the device kernels (csrc/host/plain_kernels.cpp), for tests
     "llme_plain_embed": (_i, [_vp, _vp, _i, _i, _i, _vp]),
     "llme_plain_rmsnorm": (_i, [_vp, _vp, _i, _i, _f, _vp]),

@@ -36,8 +36,9 @@ long llme_cm_fill_step(void* h, int S, const int64_t* keys, const int* new_lens,
 void* llme_sched_create(void* cache_manager, int max_concurrent, long budget);
 void llme_sched_destroy(void* h);
 int llme_sched_set_decode_round(void* h, int requests);
-int llme_decode_cut(const int* lens, int S, int tiles, int units, int head_dim, long plan_len, int most, double tbs,
-                    double key_ns, double lone_ns, double piece_us, double apart_us, double each_us, double gain);
+int llme_decode_cut(const int* lens, int S, int tiles, int units, int head_dim, long plan_len, int first, int most,
+                    double tbs, double key_ns, double lone_ns, double piece_us, double apart_us, double each_us,
+                    double gain);
 long llme_sched_enqueue(void* h, const int* prompt, long n, long max_new_tokens);
 int llme_sched_idle(void* h);
 int llme_sched_plan(void* h, int* n_admitted, int* admitted_slots, int64_t* entry_seq, int* entry_count, int* entry_want,
@@ -286,10 +287,11 @@ static void fuzz_decode_plan(int rounds) {
         std::vector<int> lens(static_cast<size_t>(S));
         for (int& n : lens) n = pick(0, pick(0, 1) ? 200000 : 700);
         const long plan_len = pick(0, 1) ? pick(1, 300000) : 1;
-        const int n = llme_decode_cut(lens.data(), S, tiles, units, 16 * pick(1, 8), plan_len, most, 6.0, 9.5, 8.3, 0.5,
-                                      pick(0, 20), 1.0, 0.05);
-        REQUIRE(n >= 1 && n <= most && n <= 64);
-        REQUIRE(n == 1 || static_cast<long>(S) * tiles * n <= 10L * units);
+        const int first = pick(1, 6);
+        const int n = llme_decode_cut(lens.data(), S, tiles, units, 16 * pick(1, 8), plan_len, first, most, 6.0, 9.5, 8.3,
+                                      0.5, pick(0, 20), 1.0, 0.05);
+        REQUIRE(n >= first && (n == first || n <= most) && n <= 64);
+        REQUIRE(n == first || static_cast<long>(S) * tiles * n <= 10L * units);
     }
 }
 

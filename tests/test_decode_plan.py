@@ -10,7 +10,7 @@ from llmengine.runtime import native
 
 # the constants of ops.choices.KernelChoices, heads of 64, 8 tiles a request, 256 compute units; a cut costs
 # the join and the rotation kernel
-ARGS = dict(tiles=8, units=256, head_dim=64, most=8, tbs=6.0, key_ns=9.5, lone_ns=8.3, piece_us=0.5, apart_us=9.4,
+ARGS = dict(tiles=8, units=256, head_dim=64, first=1, most=8, tbs=6.0, key_ns=9.5, lone_ns=8.3, piece_us=0.5, apart_us=9.4,
             each_us=1.0, gain=0.05)
 
 
@@ -18,7 +18,7 @@ def cut(lens, plan_len=0, **kw):
     a = dict(ARGS, **kw)
     lib = native.library()
     return lib.llme_decode_cut((ctypes.c_int * len(lens))(*lens), len(lens), a["tiles"], a["units"], a["head_dim"],
-                               max(plan_len, max(lens)), a["most"], a["tbs"], a["key_ns"], a["lone_ns"], a["piece_us"],
+                               max(plan_len, max(lens)), a["first"], a["most"], a["tbs"], a["key_ns"], a["lone_ns"], a["piece_us"],
                                a["apart_us"], a["each_us"], a["gain"])
 
 
@@ -50,15 +50,27 @@ def test_requests_of_different_lengths():
     assert cut([16000] + [300] * 19) > 1
 
 
+def test_few_requests_whose_splits_fill_the_units_once():
+    """12 requests, 96 workgroups a split: two splits fill the units once (first=2). Requests of one length keep
+    them; with different lengths the short requests' last pieces are empty and a third split is better."""
+    free = dict(first=2, most=4, apart_us=0.0)
+    assert cut([8192] * 12, **free) == 2 and cut([2048] * 12, **free) == 2
+    rnd = random.Random(12)
+    lens = sorted((rnd.randint(1024, 16384) for _ in range(12)), reverse=True)
+    assert cut(lens, **free) == 3
+    assert cut([8192] * 8, first=4, most=6, apart_us=0.0) == 4
+    assert cut([300] * 12, first=2, most=4, apart_us=0.0) == 2     # nothing to cut into
+
+
 def test_limits_and_refusals():
     assert cut([300] * 40) == 1                          # nothing to cut into
     assert cut([100000] * 200) == 1                      # more than ten workgroups a unit
     assert 1 <= cut([100000] * 17) <= 8
     lib = native.library()
     one = (ctypes.c_int * 1)(5)
-    assert lib.llme_decode_cut(one, 0, 8, 256, 64, 5, 8, 6.0, 9.5, 8.3, 0.5, 9.4, 1.0, 0.05) == native.BAD_ARGUMENT
-    assert lib.llme_decode_cut(one, 1, 0, 256, 64, 5, 8, 6.0, 9.5, 8.3, 0.5, 9.4, 1.0, 0.05) == native.BAD_ARGUMENT
-    assert lib.llme_decode_cut(one, 1, 8, 256, 64, 5, 8, 0.0, 9.5, 8.3, 0.5, 9.4, 1.0, 0.05) == native.BAD_ARGUMENT
-    assert lib.llme_decode_cut(None, 1, 8, 256, 64, 5, 8, 6.0, 9.5, 8.3, 0.5, 9.4, 1.0, 0.05) == native.BAD_ARGUMENT
+    assert lib.llme_decode_cut(one, 0, 8, 256, 64, 5, 1, 8, 6.0, 9.5, 8.3, 0.5, 9.4, 1.0, 0.05) == native.BAD_ARGUMENT
+    assert lib.llme_decode_cut(one, 1, 0, 256, 64, 5, 1, 8, 6.0, 9.5, 8.3, 0.5, 9.4, 1.0, 0.05) == native.BAD_ARGUMENT
+    assert lib.llme_decode_cut(one, 1, 8, 256, 64, 5, 1, 8, 0.0, 9.5, 8.3, 0.5, 9.4, 1.0, 0.05) == native.BAD_ARGUMENT
+    assert lib.llme_decode_cut(None, 1, 8, 256, 64, 5, 1, 8, 6.0, 9.5, 8.3, 0.5, 9.4, 1.0, 0.05) == native.BAD_ARGUMENT
     bad = (ctypes.c_int * 2)(5, -1)
-    assert lib.llme_decode_cut(bad, 2, 8, 256, 64, 5, 8, 6.0, 9.5, 8.3, 0.5, 9.4, 1.0, 0.05) == native.BAD_ARGUMENT
+    assert lib.llme_decode_cut(bad, 2, 8, 256, 64, 5, 1, 8, 6.0, 9.5, 8.3, 0.5, 9.4, 1.0, 0.05) == native.BAD_ARGUMENT
