@@ -44,7 +44,10 @@ class KernelChoices:
     # 24: 2.129 / 2.088 (4), 28 and 32: whole is best, 33: 3.170 / 2.618 (6), 40: 3.384 / 2.889 (4), 48: 3.681 /
     # 3.179 (2), 56 and 64: whole, 72: 5.071 / 4.664 (3); a context of 2,048: whole is best or equal everywhere
     # (17 requests 1.186 / 1.218, 33: 1.511 / 1.496); 16,384: 17 requests 3.171 / 2.556, 33: 5.440 / 4.049.
-    decode_cut_most: int = 8            # splits at most (1: never cut)
+    # The same estimate judges one or two splits more where one workgroup per compute unit takes 2 to 6 splits
+    # (5 to 16 requests): requests of one length keep that plan, requests of different lengths gain (12 requests
+    # of 1,024 to 16,384 tokens 1.539 / 1.336, 11: 1.882 / 1.582).
+    decode_cut_most: int = 8            # splits at most where the keys would be whole (1: the estimate is not asked)
     decode_cut_tbs: float = 6.0         # TB/s the keys stream at where the compute units share them evenly
     decode_cut_key_ns: float = 9.5      # ns a compute unit needs per key of a head of 64 that it is given
     decode_cut_lone_ns: float = 8.3     # the same for a unit's only piece where others hold two (it ends on a draining chip)
