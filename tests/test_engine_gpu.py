@@ -445,6 +445,44 @@ def test_many_decoded_tokens_with_their_keys_cut_by_the_host_plan(zoo, monkeypat
             assert np.abs(got[rid][pos].astype(np.float64) - whole[rid][pos]).max() / top < 1e-2, (rid, pos)
 
 
+def test_recorded_steps_of_one_shape_are_kept_apart_by_what_the_parts_planned(zoo, monkeypatch):
+    """20 long requests decode and end, 20 short ones take their places and decode: the same number of requests
+    and the same width of block table, but the host's plan for the keys differs (cut for the long ones, whole
+    for the short), so the second kind of step must get a recording of its own (a recording replays the
+    launches of its plan), and every row must match the plain implementation."""
+    model_dir, _, _, page = zoo["C"]
+    cfg = TINY_C
+    long_ones = {f"a{i}": random_tokens(620 + 7 * i, cfg["vocab_size"], 500 + i) for i in range(20)}
+    short_ones = {f"b{i}": random_tokens(30 + i, cfg["vocab_size"], 600 + i) for i in range(20)}
+    pcfg, pw = load_plain_model(model_dir)
+    engine = engine_for(model_dir, "bf16")
+    ch = engine.runner.choices
+    for name, value in (("decode_blocks_wanted", 32), ("decode_cut_join_us", 0.0), ("decode_cut_rope_us", 0.0),
+                        ("decode_cut_each_us", 0.0), ("decode_cut_gain", 0.0), ("decode_cut_piece_us", 0.0),
+                        ("decode_cut_lone_ns", ch.decode_cut_key_ns)):
+        monkeypatch.setattr(ch, name, value)
+    steps = []
+    for reqs in (long_ones, short_ones):
+        steps.append({"step": len(steps), "end": [],
+                      "entries": [{"id": r, "tokens": ids[:-4], "want": []} for r, ids in reqs.items()]})
+        for t in range(4, 0, -1):
+            steps.append({"step": len(steps), "end": list(reqs) if t == 1 else [],
+                          "entries": [{"id": r, "tokens": [ids[-t]], "want": [0]} for r, ids in reqs.items()]})
+    pages = replay.trace_peak_tokens(steps, round_to=page) // page
+    cache = engine.new_cache(pages, page, max_requests=20)
+    got = replay.run_trace(engine, cache, steps)
+    kept = [k for k in cache.graphs if k[0] == 20]
+    assert len(kept) == 2 and kept[0][:4] == kept[1][:4] and kept[0][4] != kept[1][4], kept
+    assert sorted(max(dict(k[4]).values(), default=1) > 1 for k in kept) == [False, True], kept
+    for reqs in (long_ones, short_ones):
+        for rid, ids in reqs.items():
+            ref = plain_forward(pcfg, pw, ids, rounder=bf16_round).numpy()
+            assert len(got[rid]) == 4
+            for pos in got[rid]:
+                top = np.abs(ref[pos]).max()
+                assert np.abs(got[rid][pos].astype(np.float64) - ref[pos]).max() / top < TOL["bf16"], (rid, pos)
+
+
 @pytest.mark.parametrize("dtype,deterministic", [("fp32", False), ("bf16", True)])
 def test_greedy_chain_equals_steps_fetched_one_by_one(zoo, dtype, deterministic):
     """Steps launched before the tokens of the step before them are fetched (the tokens stay on the
