@@ -190,7 +190,8 @@ class Engine:
         """What the scheduler orders a step's decoding requests by: the number that the model's first mixer
         with such a number gives (Mixer.decode_round), 0 if none has one."""
         for layer in self.model.layers:
-            n = int(getattr(layer, "mixer", None).decode_round()) if getattr(layer, "mixer", None) is not None else 0
+            mixer = getattr(layer, "mixer", None)
+            n = int(mixer.decode_round()) if mixer is not None else 0
             if n > 0:
                 return n
         return 0

@@ -91,6 +91,10 @@ class Attention(Mixer):
         return max(1, ops.mfma.compute_units() // tiles)
 
     def decode_plan_hint(self, lens, plan_len, choices):
+        # (only the bfloat16 kernels on the matrix cores cut their keys by a plan)
+        if (self.w_qkv is None or self.w_qkv.dtype != torch.bfloat16 or self.head_dim > 128 or self.head_dim % 16
+                or (choices is not None and not choices.fast_attention)):
+            return None
         n = ops.mfma.decode_cut(lens, self.num_heads, self.num_kv_heads, self.head_dim, plan_len, choices)
         return None if n is None else (ops.mfma.cut_hint_name(self.num_heads, self.num_kv_heads, self.head_dim), n)
 
