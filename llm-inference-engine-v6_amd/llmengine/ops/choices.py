@@ -30,6 +30,11 @@ class KernelChoices:
     # 2.125 / 2.044, 80: 2.287 / 2.218, 96: 2.504 / 2.473, 112: 2.916 / 2.898; 128: 3.216 / 3.287 on one box and
     # 3.268 / 3.195 on another; 160 tokens with 64 / 256: 3.630 / 3.697, 256: 5.069 / 5.236.
     qkv_sum_rows_decoding: int = 96
+    # The same with heads of 128 (the rotation kernel behind the product, not the attention kernel). Measured at a
+    # context of 2,048 over 8 layers, ms a step with 64 / 96 / 128 here: 3B sizes 65 tokens 1.921 / 1.840 / 1.847, 96:
+    # 2.151 / 2.053 / 2.057, 112: 2.432 / 2.403 / 2.340, 128: 2.564 / 2.556 / 2.498; 8B sizes 65: 2.313 / 2.223 / 2.218,
+    # 96: 2.568 / 2.466 / 2.467, 112: 2.879 / 2.864 / 2.806, 128: 3.014 / 3.030 / 2.984.
+    qkv_sum_rows_decoding_128: int = 128
     # prompt attention: work items of half the rows where a step has few items
     prefill_half_rows: bool = True
     # Workgroups (of four wavefronts) the decode kernel should have at most when it cuts the keys: one

@@ -480,11 +480,15 @@ QKV_SUM_MAX_ROWS = 64
 
 def qkv_sum_max_rows(decoded_only: bool, head_dim: int, choices: KernelChoices | None = None) -> int:
     """The most rows of a step whose q/k/v product is cut over k and added into a cleared buffer. A step of
-    single decoded tokens with heads of 64 keeps that way further (choices.qkv_sum_rows_decoding): the
-    attention kernel then rotates and writes the cache itself (attention_decode_rope)."""
+    single decoded tokens keeps that way further: with heads of 64 (choices.qkv_sum_rows_decoding) the
+    attention kernel then rotates and writes the cache itself (attention_decode_rope); with heads of 128
+    (choices.qkv_sum_rows_decoding_128) the rotation kernel does, and the product's tiles of 96 or 128 rows
+    with the rotation in their epilogue are the slower way until then."""
     ch = choices or DEFAULT
     if decoded_only and head_dim == 64 and ch.decode_rope:
         return max(QKV_SUM_MAX_ROWS, ch.qkv_sum_rows_decoding)
+    if decoded_only and head_dim == 128:
+        return max(QKV_SUM_MAX_ROWS, ch.qkv_sum_rows_decoding_128)
     return QKV_SUM_MAX_ROWS
 
 
