@@ -196,6 +196,17 @@ class Engine:
                 return n
         return 0
 
+    @property
+    def step_rows_round(self) -> tuple[int, int]:
+        """(rows, most): steps of up to `most` rows more than a multiple of `rows` run those rows through the
+        matrix products in launches of their own (ops.mfma.tail_rows); the scheduler avoids such steps.
+        (0, 0) where the products do no such thing."""
+        ch = self.runner.choices
+        if self._torch_dtype != torch.bfloat16 or not ch.fast_gemm or not ch.tail_rows_apart:
+            return (0, 0)
+        from ..ops import mfma
+        return (mfma.TAIL_ROWS_ROUND, int(ch.tail_rows_most))
+
     # ---- caches ----
     def new_cache(self, num_blocks: int, block_size: int | None = None, max_requests: int = 64) -> CacheContext:
         with torch.cuda.device(self.runner.device):

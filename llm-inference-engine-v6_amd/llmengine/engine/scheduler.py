@@ -112,6 +112,12 @@ class ContinuousBatchScheduler:
         # an engine whose decode kernel deals a step's requests out to the compute units in turn says after
         # how many it has been round once (rounds_order)
         self._lib.llme_sched_set_decode_round(self._h, max(0, int(getattr(engine, "decode_round", 0) or 0)))
+        # and an engine whose products run a few rows more than a multiple of some number of rows in launches
+        # of their own says which (rows, most): the step's last prompt portion then leaves those few for the
+        # next step
+        rows, over = getattr(engine, "step_rows_round", None) or (0, 0)
+        if rows > 0 and 0 < over < rows:
+            self._lib.llme_sched_set_row_round(self._h, int(rows), int(over))
         n = self.max_concurrent
         self._admitted = (ctypes.c_int * n)()
         self._entry_seq = (ctypes.c_int64 * n)()

@@ -120,6 +120,9 @@ def gemm_qkv_rope(x: torch.Tensor, w_qkv: torch.Tensor, cos: torch.Tensor, sin: 
         int(tile), stream()), "gemm_qkv_rope")
 
 
+TAIL_ROWS_ROUND = 1024              # rows that the tile kernels cover in full rounds of workgroups (tail_rows)
+
+
 def tail_rows(M: int, choices: KernelChoices | None = None) -> int:
     """Rows at the end of a product of M rows that a launch of their own takes (0: none). The tile kernels
     cover whole multiples of 1,024 rows in full rounds of workgroups over the chip at the widths of the Llama
@@ -130,8 +133,8 @@ def tail_rows(M: int, choices: KernelChoices | None = None) -> int:
     no round exactly) 9.14 / 9.14 and 15.7 / 15.1. Anywhere else two launches lose (1B sizes, 1,160 tokens 3.83 /
     4.24; 1,550 tokens 4.76 / 4.97)."""
     ch = choices or DEFAULT
-    r = M % 1024
-    return r if ch.tail_rows_apart and M > 1024 and 0 < r <= ch.tail_rows_most else 0
+    r = M % TAIL_ROWS_ROUND
+    return r if ch.tail_rows_apart and M > TAIL_ROWS_ROUND and 0 < r <= ch.tail_rows_most else 0
 
 
 def _fast_gemm(a, w, out, accumulate, fixed_order=False, choices: KernelChoices | None = None) -> bool:

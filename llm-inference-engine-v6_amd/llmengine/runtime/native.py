@@ -133,7 +133,8 @@ _SIGNATURES = {
     "llme_cm_lengths": (_i, [_vp, _i, _pi64, _pl]),
     "llme_cm_fill_step": (_l, [_vp, _i, _pi64, _pi, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "llme_sched_create": (_vp, [_vp, _i, _l]), "llme_sched_destroy": (None, [_vp]),
-    "llme_sched_set_budget": (_i, [_vp, _l]), "llme_sched_set_decode_round": (_i, [_vp, _i]), "llme_sched_enqueue": (_l, [_vp, _pi, _l, _l]),
+    "llme_sched_set_budget": (_i, [_vp, _l]), "llme_sched_set_decode_round": (_i, [_vp, _i]),
+    "llme_sched_set_row_round": (_i, [_vp, _l, _l]), "llme_sched_enqueue": (_l, [_vp, _pi, _l, _l]),
     "llme_sched_idle": (_i, [_vp]), "llme_sched_counts": (None, [_vp, _pi]),
     "llme_sched_plan": (_i, [_vp, _pi, _pi, _pi64, _pi, _pi, _pl, _pi, _l]),
     "llme_sched_complete": (_i, [_vp, _pi, _i, _pi, _i]), "llme_sched_num_results": (_i, [_vp]),

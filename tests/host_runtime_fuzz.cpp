@@ -36,6 +36,7 @@ long llme_cm_fill_step(void* h, int S, const int64_t* keys, const int* new_lens,
 void* llme_sched_create(void* cache_manager, int max_concurrent, long budget);
 void llme_sched_destroy(void* h);
 int llme_sched_set_decode_round(void* h, int requests);
+int llme_sched_set_row_round(void* h, long rows, long over);
 int llme_decode_cut(const int* lens, int S, int tiles, int units, int head_dim, long plan_len, int first, int most,
                     double tbs, double key_ns, double lone_ns, double piece_us, double apart_us, double each_us,
                     double gain);
@@ -175,6 +176,7 @@ static void fuzz_scheduler(int rounds) {
         void* sc = llme_sched_create(cm, max_concurrent, budget);
         REQUIRE(cm && sc);
         REQUIRE(llme_sched_set_decode_round(sc, -1) < 0 && llme_sched_set_decode_round(sc, pick(0, 4)) == 0);
+        REQUIRE(llme_sched_set_row_round(sc, 4, 4) < 0 && llme_sched_set_row_round(sc, pick(0, 1) * pick(2, 12), 1) == 0);
         const int n_requests = pick(1, 14);
         std::vector<std::vector<int>> prompts;
         std::vector<long> max_new;

@@ -172,6 +172,40 @@ def test_the_engine_names_the_round_and_the_scheduler_orders_by_it():
         assert (r.token_ids, r.finish_reason) == single_generate(p, 6)
 
 
+def test_a_few_rows_past_a_round_are_left_for_the_next_step():
+    """An engine whose products run a few rows past a multiple of some number apart (step_rows_round): the
+    portion that uses the budget up gives those few tokens back; streams, and everything else, stay."""
+    prompts = [[1, 2, 3], [4, 5], list(range(1, 60))]
+    eng = FakeEngine()
+    eng.step_rows_round = (16, 4)
+    s = ContinuousBatchScheduler(eng, FakeBlocks(64, 4), max_prefill_tokens_per_step=16)
+    for p in prompts:
+        s.enqueue(p, 8)
+    s.run_until_idle()
+    # step 0: 3 + 2 + 11 prompt tokens, nobody decodes yet: 16 rows. step 1: 16 prompt tokens + 2 decoding = 18 rows,
+    # two more than a round: the portion is 14. then 16 rows every step while the long prompt lasts
+    assert eng.batches[0] == [(0, 3), (1, 2), (2, 11)]
+    assert eng.batches[1][0] == (2, 14) and sorted(eng.batches[1][1:]) == [(0, 1), (1, 1)]
+    assert eng.batches[2][0] == (2, 14) and eng.batches[3][0] == (2, 14)
+    assert eng.batches[4][0] == (2, 6)                      # the prompt's end is never cut short
+    for r, p in zip(s.results, prompts):
+        assert (r.token_ids, r.finish_reason) == single_generate(p, 8)
+    # without the hint, and where the rows past the round are more than the engine runs apart: the whole budget
+    eng = FakeEngine()
+    s = ContinuousBatchScheduler(eng, FakeBlocks(64, 4), max_prefill_tokens_per_step=16)
+    for p in prompts:
+        s.enqueue(p, 8)
+    s.run_until_idle()
+    assert eng.batches[1][0] == (2, 16)
+    eng = FakeEngine()
+    eng.step_rows_round = (16, 1)
+    s = ContinuousBatchScheduler(eng, FakeBlocks(64, 4), max_prefill_tokens_per_step=16)
+    for p in prompts:
+        s.enqueue(p, 8)
+    s.run_until_idle()
+    assert eng.batches[1][0] == (2, 16)
+
+
 @pytest.mark.parametrize("max_new", [0, 1, 2, 5])               # tests/test_scheduler.py:220-280
 def test_exact_counts(max_new):
     s, _, bm = run([[4, 5, 6]], max_new)
