@@ -242,6 +242,7 @@ def main() -> int:
                          "the longest first)")
     ap.add_argument("--round", type=int, default=32, help="decode order 'rounds': requests per round")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--page-size", type=int, default=16, help="tokens per cache page (a multiple of 16 for the bf16 kernels)")
     ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes: Llama 3.2 1B (the default), 3.2 3B, 3.1 8B")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (named in config)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
@@ -292,7 +293,7 @@ def main() -> int:
     log(f"model on the device after {time.time() - t0:.1f} s")
     gen = torch.Generator().manual_seed(args.seed + 1)
     V = cfg["vocab_size"]
-    page = 16
+    page = args.page_size
 
     def sync():
         torch.cuda.synchronize()
