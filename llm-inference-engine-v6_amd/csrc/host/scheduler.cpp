@@ -150,7 +150,10 @@ public:
             // every weight again: a step of 1,024 + 8 rows took 3.84 ms at the 1B sizes, one of 1,024 3.30.)
             if (row_round_ > 0 && n == budget && n < s.prompt_len - s.cursor) {
                 const long rows = (budget_ - budget) + n + decoding, over = rows % row_round_;
-                if (rows > row_round_ && over > 0 && over <= row_over_ && over < n) n -= over;
+                if (rows > row_round_ && over > 0 && over <= row_over_ && over < n) {
+                    n -= over;
+                    budget = n;                       // (what is given back is nobody else's either)
+                }
             }
             if (!take_pages(s, n)) {
                 finish(s, kCapacity);

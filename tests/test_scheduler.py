@@ -190,6 +190,18 @@ def test_a_few_rows_past_a_round_are_left_for_the_next_step():
     assert eng.batches[4][0] == (2, 6)                      # the prompt's end is never cut short
     for r, p in zip(s.results, prompts):
         assert (r.token_ids, r.finish_reason) == single_generate(p, 8)
+    # what a portion gives back does not go to the prompt behind it
+    eng = FakeEngine()
+    eng.step_rows_round = (16, 4)
+    s = ContinuousBatchScheduler(eng, FakeBlocks(128, 4), max_prefill_tokens_per_step=16)
+    two = [[1, 2, 3], list(range(1, 50)), list(range(2, 40))]
+    for p in two:
+        s.enqueue(p, 4)
+    s.run_until_idle()
+    assert eng.batches[0] == [(0, 3), (1, 13)] and eng.batches[1][:1] == [(1, 15)] and (2, 1) not in eng.batches[1]
+    assert sum(n for _, n in eng.batches[1]) == 16
+    for r, p in zip(s.results, two):
+        assert (r.token_ids, r.finish_reason) == single_generate(p, 4)
     # without the hint, and where the rows past the round are more than the engine runs apart: the whole budget
     eng = FakeEngine()
     s = ContinuousBatchScheduler(eng, FakeBlocks(64, 4), max_prefill_tokens_per_step=16)
