@@ -172,13 +172,13 @@ def portion(args, engine, cfg: dict, gen, page: int) -> int:
 def mixed(args, engine, cfg: dict, gen, page: int) -> int:
     """The step that continuous batching runs most: a prompt portion of --portion tokens of one
     request (behind --context cached tokens) beside one decoded token of --batch other requests
-    (700 to 1,500 tokens each). Timed as the engine launches it, and once more with the same
+    (--decode-len tokens and up to 800 more each, 700 to 1,500 by default). Timed as the engine launches it, and once more with the same
     launches recorded as a HIP graph and replayed, which is the GPU's time alone."""
     import torch
     from llmengine import StepEntry
     V, n, nd = cfg["vocab_size"], args.portion, args.batch
     steps = max(4, min(args.steps, 32))
-    lens = [700 + (800 * i) // max(nd, 1) for i in range(nd)]
+    lens = [args.decode_len + (800 * i) // max(nd, 1) for i in range(nd)]
     cache = engine.new_cache((args.context + n + sum(lens)) // page + nd + 4, page, nd + 1)
     for i, ln in enumerate(lens):
         cache.admit(i)
@@ -254,6 +254,8 @@ def main() -> int:
                          "steps of --portion prompt tokens of one request behind --context tokens; 'mixed': such a "
                          "portion beside one decoded token of --batch other requests")
     ap.add_argument("--portion", type=int, default=256, help="portion: prompt tokens a step")
+    ap.add_argument("--decode-len", type=int, default=700, help="mixed: tokens of the shortest decoding request "
+                                                                "(the longest has 800 more)")
     ap.add_argument("--requests", type=int, default=32, help="serve: number of requests")
     ap.add_argument("--prompt-range", default="64,3072", help="serve: prompt lengths, uniform in [a, b]")
     ap.add_argument("--new-range", default="128,512", help="serve: new tokens per request, uniform in [a, b]")
